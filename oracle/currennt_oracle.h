@@ -1,0 +1,66 @@
+// C entry points of the CPU oracle -- TEST INFRASTRUCTURE ONLY (see oracle_common.h).
+// All buffers are host memory, fp32, laid out exactly as the reference lays them out:
+// an activation of a layer of size D is a column-major D x (T*S) matrix, column (t*S+s).
+#ifndef CURRENNT_ORACLE_H
+#define CURRENNT_ORACLE_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct {
+    int P;      /* size of the preceding layer                                  */
+    int L;      /* layer size (sum over both directions when bidirectional)     */
+    int bidir;  /* 0 unidirectional, 1 bidirectional                            */
+    int S;      /* parallel sequences                                           */
+    int T;      /* curMaxSeqLength of the fraction                              */
+    int Tmin;   /* curMinSeqLength of the fraction                              */
+    float bias; /* the layer's constant bias input                              */
+} orc_lstm_desc;
+
+/* Per-direction state; every buffer is H x (T*S), H = L or L/2. */
+typedef struct {
+    float *ni, *ig, *fg, *og; /* gate activations (pre-activations until the forward pass overwrites them) */
+    float *c;                 /* cell states                                                               */
+    float *h;                 /* block outputs                                                              */
+    float *herr;              /* output errors of this direction, receives the recurrent terms in place     */
+    float *dni, *dig, *dfg, *dog; /* clipped gate deltas                                                    */
+    float *cerr;              /* cell-state errors (unclipped)                                              */
+} orc_lstm_dir;
+
+/* scalar helpers (for unit tests of the scalar semantics) */
+float orc_logistic(float x);
+float orc_tanh(float x);
+float orc_safe_exp(float x);
+float orc_safe_log(float x);
+float orc_log_add(float x, float y);
+
+/* generic column-major product, reference summation order */
+void orc_mat_product(float *C, int m, int n, int k, const float *A, int tA, const float *B, int tB,
+                     int accumulate);
+
+/* LSTM (LstmLayer.cu).  `out` is L x (T*S). For a unidirectional layer fw->h may alias `out`. */
+void orc_lstm_forward(const orc_lstm_desc *d, const float *weights, const char *patTypes, const float *x,
+                      orc_lstm_dir *fw, orc_lstm_dir *bw, float *out);
+/* `outerr` is L x (T*S) (read only; it is split/copied into herr).  `ex` (P x T*S) may be NULL. */
+void orc_lstm_backward(const orc_lstm_desc *d, const float *weights, const char *patTypes, const float *x,
+                       const float *outerr, orc_lstm_dir *fw, orc_lstm_dir *bw, float *ex,
+                       float *weightUpdates);
+long orc_lstm_weight_count(int P, int L, int bidir);
+
+/* Feed-forward layer (FeedForwardLayer.cu). act: 0 identity, 1 tanh, 2 logistic, 3 relu.
+   weights = [P x D col-major | D bias]. */
+void orc_dense_forward(int P, int D, int N, int act, float bias, const float *weights, const float *x,
+                       float *y);
+/* err (D x N) is turned into deltas in place; ex (P x N) may be NULL; dW has P*D + D entries. */
+void orc_dense_backward(int P, int D, int N, int act, float bias, const float *weights, const float *x,
+                        const float *y, float *err, float *ex, float *dW);
+
+/* SSE post output layer (SsePostOutputLayer.cu) */
+float orc_sse_error(int D, int N, const char *patTypes, const float *y, const float *target);
+void orc_sse_backward(int D, int N, const char *patTypes, const float *y, const float *target, float *err);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,112 @@
+"""ctypes binding of the CPU oracle (oracle/_build/liboracle.so).
+
+Only tests, the smoke check and the CPU-baseline leg of the benchmark import this module;
+the oracle is the checker, never the thing that is measured or shipped.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+LIB_PATH = os.path.join(ORACLE_DIR, "_build", "liboracle.so")
+
+FP = C.POINTER(C.c_float)
+
+
+def build(force=False):
+    if force or not os.path.exists(LIB_PATH):
+        subprocess.check_call(["make", "-C", ORACLE_DIR] + (["-B"] if force else []))
+    return LIB_PATH
+
+
+class LstmDesc(C.Structure):
+    _fields_ = [("P", C.c_int), ("L", C.c_int), ("bidir", C.c_int), ("S", C.c_int), ("T", C.c_int),
+                ("Tmin", C.c_int), ("bias", C.c_float)]
+
+
+LSTM_FIELDS = ["ni", "ig", "fg", "og", "c", "h", "herr", "dni", "dig", "dfg", "dog", "cerr"]
+
+
+class LstmDir(C.Structure):
+    _fields_ = [(n, FP) for n in LSTM_FIELDS]
+
+
+def fptr(a):
+    if a is None:
+        return None
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(FP)
+
+
+def cptr(a):
+    assert a.dtype == np.int8 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(C.c_char_p)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(LIB_PATH)
+        L.orc_logistic.restype = C.c_float
+        L.orc_logistic.argtypes = [C.c_float]
+        L.orc_tanh.restype = C.c_float
+        L.orc_tanh.argtypes = [C.c_float]
+        L.orc_safe_exp.restype = C.c_float
+        L.orc_safe_exp.argtypes = [C.c_float]
+        L.orc_safe_log.restype = C.c_float
+        L.orc_safe_log.argtypes = [C.c_float]
+        L.orc_log_add.restype = C.c_float
+        L.orc_log_add.argtypes = [C.c_float, C.c_float]
+        L.orc_lstm_weight_count.restype = C.c_long
+        L.orc_sse_error.restype = C.c_float
+        _lib = L
+    return _lib
+
+
+class LstmState:
+    """Host buffers of one direction: every field is an H x (T*S) column-major matrix."""
+
+    def __init__(self, H, N):
+        self.arr = {n: np.zeros(H * N, dtype=np.float32) for n in LSTM_FIELDS}
+        self.c = LstmDir(**{n: fptr(a) for n, a in self.arr.items()})
+
+    def __getitem__(self, k):
+        return self.arr[k]
+
+
+def lstm_forward(desc, W, pat, x, fw, bw, out):
+    lib().orc_lstm_forward(C.byref(desc), fptr(W), cptr(pat), fptr(x), C.byref(fw.c),
+                           C.byref(bw.c) if bw is not None else None, fptr(out))
+
+
+def lstm_backward(desc, W, pat, x, outerr, fw, bw, ex, dW):
+    lib().orc_lstm_backward(C.byref(desc), fptr(W), cptr(pat), fptr(x), fptr(outerr), C.byref(fw.c),
+                            C.byref(bw.c) if bw is not None else None, fptr(ex), fptr(dW))
+
+
+def mat_product(Cm, m, n, k, A, tA, B, tB, acc):
+    lib().orc_mat_product(fptr(Cm), m, n, k, fptr(A), int(tA), fptr(B), int(tB), int(acc))
+
+
+def dense_forward(P, D, N, act, bias, W, x, y):
+    lib().orc_dense_forward(P, D, N, act, C.c_float(bias), fptr(W), fptr(x), fptr(y))
+
+
+def dense_backward(P, D, N, act, bias, W, x, y, err, ex, dW):
+    lib().orc_dense_backward(P, D, N, act, C.c_float(bias), fptr(W), fptr(x), fptr(y), fptr(err), fptr(ex),
+                             fptr(dW))
+
+
+def sse_error(D, N, pat, y, tgt):
+    return float(lib().orc_sse_error(D, N, cptr(pat), fptr(y), fptr(tgt)))
+
+
+def sse_backward(D, N, pat, y, tgt, err):
+    lib().orc_sse_backward(D, N, cptr(pat), fptr(y), fptr(tgt), fptr(err))
