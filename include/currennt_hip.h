@@ -1,0 +1,109 @@
+/* C ABI of the gfx950 (MI355X) implementation of CURRENNT's backward hot path.
+ *
+ * Every entry point takes plain device pointers and sizes; no C++ or PyTorch types cross this
+ * boundary.  All buffers are fp32 and use the reference's layouts:
+ *   - an activation / error buffer of a layer of size D is a column-major D x (T*S) matrix whose
+ *     column index is t*S + s  (time-major, S parallel sequences interleaved);
+ *   - patTypes is char[T*S], values 0 none (padding), 1 first, 2 normal, 3 last (Types.hpp:35-38);
+ *   - weight vectors keep the reference's order  input | bias | internal.
+ * `stream` is a hipStream_t passed as void*; every call only enqueues work on that stream.
+ * Every function returns CNT_OK or an error code; cnt_last_error() gives the message of the
+ * calling thread's last failure.  A handle must be used by one thread at a time.
+ *
+ * Paths in the comments are relative to CURRENNT_codes/currennt_lib/src of the reference.
+ */
+#ifndef CURRENNT_HIP_H
+#define CURRENNT_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { CNT_OK = 0, CNT_ERR_ARG = 1, CNT_ERR_HIP = 2, CNT_ERR_STATE = 3, CNT_ERR_DEVICE = 4 };
+
+enum { CNT_ACT_IDENTITY = 0, CNT_ACT_TANH = 1, CNT_ACT_LOGISTIC = 2, CNT_ACT_RELU = 3 };
+
+int cnt_version(void);
+const char *cnt_last_error(void);
+
+/* ---- helpers::Matrix product seam -------------------------------------------------------------
+ * Replaces helpers::Matrix<Gpu>::assignProduct / addProduct (helpers/Matrix.cu:353-377, which call
+ * cublas::multiplyMatrices, helpers/cublas.cu:52-84).  Column-major, C is m x n, inner size k.
+ * transA: A is stored k x m;  transB: B is stored n x k.  (transA && transB) is rejected, as in
+ * the reference.  accumulate != 0 adds to C. */
+int cnt_matrix_product(void *stream, float *C, int m, int n, int k, const float *A, int transA,
+                       const float *B, int transB, int accumulate);
+
+/* ---- feed-forward layer ------------------------------------------------------------------------
+ * FeedForwardLayer<TDevice,TActFn>::computeForwardPass  (layers/FeedForwardLayer.cu:1060-1101)
+ * weights = [P x D column-major | D bias weights];  y = act(W^T x + bias * b). N = T*S columns. */
+int cnt_dense_forward(void *stream, int P, int D, int N, int act, float bias, const float *weights,
+                      const float *x, float *y);
+/* FeedForwardLayer::computeBackwardPass (layers/FeedForwardLayer.cu:1633-1738, functors :105-138).
+ * err (D x N) holds the output errors on entry and the deltas act'(y)*err on return (all slots,
+ * padding included, as the reference does); prev_err (P x N) is overwritten with W*delta and may
+ * be NULL; weight_updates (P*D + D) is overwritten with [x * delta^T | bias * sum delta]. */
+int cnt_dense_backward(void *stream, int P, int D, int N, int act, float bias, const float *weights,
+                       const float *x, const float *y, float *err, float *prev_err,
+                       float *weight_updates);
+
+/* ---- SSE post-output layer ---------------------------------------------------------------------
+ * SsePostOutputLayer::computeBackwardPass (layers/SsePostOutputLayer.cu:224-267):
+ * err = y - target, exactly 0 on padding slots. */
+int cnt_sse_backward(void *stream, int D, int N, const char *patTypes, const float *y,
+                     const float *target, float *err);
+/* SsePostOutputLayer::calculateError (layers/SsePostOutputLayer.cu:166-210): 0.5 * sum (t-y)^2 over
+ * non-padding slots, written to *result_dev (device memory, one float). */
+int cnt_sse_error(void *stream, int D, int N, const char *patTypes, const float *y,
+                  const float *target, float *result_dev);
+
+/* ---- LSTM layer --------------------------------------------------------------------------------
+ * LstmLayer<TDevice> (layers/LstmLayer.cu).  The handle owns what the reference keeps in its two
+ * forward_backward_info_t members (layers/LstmLayer.hpp:99-133): per direction the gate
+ * activations, cell states, block outputs, output errors, gate deltas and cell-state errors, each
+ * H x (maxT*S).  The caller owns weights, weight updates, inputs, outputs and error buffers. */
+typedef struct cnt_lstm cnt_lstm;
+
+typedef struct {
+    int P;       /* preceding layer size                                    */
+    int L;       /* layer size; bidirectional layers use L/2 per direction  */
+    int bidir;   /* 0 "lstm", 1 "blstm" (LayerFactory.cu:104-110)           */
+    int S;       /* parallel sequences                                      */
+    int maxT;    /* maxSeqLength the buffers are allocated for              */
+    float bias;  /* the layer's constant bias input ("bias" in the JSON)    */
+} cnt_lstm_desc;
+
+/* LstmLayer::LstmLayer (layers/LstmLayer.cu:1078-1268): allocates the per-direction state. */
+int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out);
+int cnt_lstm_destroy(cnt_lstm *h);
+/* LstmLayer::loadSequences (layers/LstmLayer.cu:1488-1533): records the fraction's geometry and
+ * zero-fills the stored output-gate deltas.  patTypes is device memory, char[curMaxT*S], and must
+ * stay valid until the next call of this function. */
+int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int curMaxT, int curMinT);
+/* LstmLayer::computeForwardPass(nnState) (layers/LstmLayer.cu:1743-1949).
+ * x is P x (T*S); outputs is L x (T*S). */
+int cnt_lstm_forward(cnt_lstm *h, void *stream, const float *weights, const float *x, float *outputs);
+/* LstmLayer::computeBackwardPass(nnState) (layers/LstmLayer.cu:2066-2382).
+ * output_errors is L x (T*S).  For a unidirectional layer the recurrent error terms are added to
+ * it in place, which is what the reference's buffer swap (:2086-2087, :2378-2381) leaves behind.
+ * prev_errors (P x T*S) is overwritten and may be NULL.  weight_updates has the size and layout of
+ * the weight vector and is overwritten.  `outputs` is the buffer cnt_lstm_forward filled. */
+int cnt_lstm_backward(cnt_lstm *h, void *stream, const float *weights, const float *x,
+                      const float *outputs, float *output_errors, float *prev_errors,
+                      float *weight_updates);
+/* Device pointer to one internal buffer.  dir: 0 forward, 1 backward states.  which:
+ * 0 niActs 1 igActs 2 fgActs 3 ogActs 4 cellStates 5 tmpOutputs 6 tmpOutputErrors
+ * 7 niDeltas 8 igDeltas 9 fgDeltas 10 ogDeltas 11 cellStateErrors.  NULL if out of range. */
+float *cnt_lstm_state(cnt_lstm *h, int dir, int which);
+long cnt_lstm_weight_count(int P, int L, int bidir);
+/* Waits for the stream and reports whether a recursion kernel of this handle gave up waiting for a
+ * neighbouring workgroup (CNT_ERR_DEVICE; the results of that pass are invalid).  The reference has
+ * no counterpart: its per-step launches cannot stall on each other. */
+int cnt_lstm_check(cnt_lstm *h, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,160 @@
+"""ctypes binding of libcurrennt_hip.so.  Device buffers are passed as raw pointers (torch tensors'
+data_ptr()); every call checks the returned status and raises RuntimeError with cnt_last_error()."""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libcurrennt_hip.so")
+
+CNT_OK = 0
+ACT = {"identity": 0, "tanh": 1, "logistic": 2, "relu": 3}
+
+LSTM_STATE = {"ni": 0, "ig": 1, "fg": 2, "og": 3, "c": 4, "h": 5, "herr": 6, "dni": 7, "dig": 8, "dfg": 9,
+              "dog": 10, "cerr": 11}
+
+
+class LstmDesc(C.Structure):
+    _fields_ = [("P", C.c_int), ("L", C.c_int), ("bidir", C.c_int), ("S", C.c_int), ("maxT", C.c_int),
+                ("bias", C.c_float)]
+
+
+_lib = None
+
+VP = C.c_void_p
+I = C.c_int
+F = C.c_float
+
+_SIGNATURES = {
+    "cnt_version": (I, []),
+    "cnt_last_error": (C.c_char_p, []),
+    "cnt_matrix_product": (I, [VP, VP, I, I, I, VP, I, VP, I, I]),
+    "cnt_dense_forward": (I, [VP, I, I, I, I, F, VP, VP, VP]),
+    "cnt_dense_backward": (I, [VP, I, I, I, I, F, VP, VP, VP, VP, VP, VP]),
+    "cnt_sse_backward": (I, [VP, I, I, VP, VP, VP, VP]),
+    "cnt_sse_error": (I, [VP, I, I, VP, VP, VP, VP]),
+    "cnt_lstm_create": (I, [C.POINTER(LstmDesc), C.POINTER(VP)]),
+    "cnt_lstm_destroy": (I, [VP]),
+    "cnt_lstm_load_sequences": (I, [VP, VP, VP, I, I]),
+    "cnt_lstm_forward": (I, [VP, VP, VP, VP, VP]),
+    "cnt_lstm_backward": (I, [VP, VP, VP, VP, VP, VP, VP, VP]),
+    "cnt_lstm_state": (VP, [VP, I, I]),
+    "cnt_lstm_weight_count": (C.c_long, [I, I, I]),
+    "cnt_lstm_check": (I, [VP, VP]),
+}
+
+
+def exported_symbols():
+    return sorted(_SIGNATURES)
+
+
+def lib():
+    """Loads the library; raises if it has not been built (there is no fallback path)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libcurrennt_hip.so is not built (%s); run __graft_entry__.build()" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(status):
+    if status != CNT_OK:
+        raise RuntimeError("currennt_hip error %d: %s" % (status, lib().cnt_last_error().decode()))
+
+
+def ptr(t):
+    """Raw device pointer of a torch tensor (or None)."""
+    if t is None:
+        return None
+    return C.c_void_p(t.data_ptr())
+
+
+def stream_ptr(stream=None):
+    import torch
+
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return C.c_void_p(s.cuda_stream)
+
+
+def matrix_product(Cm, m, n, k, A, tA, B, tB, accumulate, stream=None):
+    check(lib().cnt_matrix_product(stream_ptr(stream), ptr(Cm), m, n, k, ptr(A), int(tA), ptr(B), int(tB),
+                                   int(accumulate)))
+
+
+def dense_forward(P, D, N, act, bias, W, x, y, stream=None):
+    check(lib().cnt_dense_forward(stream_ptr(stream), P, D, N, act, bias, ptr(W), ptr(x), ptr(y)))
+
+
+def dense_backward(P, D, N, act, bias, W, x, y, err, prev_err, dW, stream=None):
+    check(lib().cnt_dense_backward(stream_ptr(stream), P, D, N, act, bias, ptr(W), ptr(x), ptr(y), ptr(err),
+                                   ptr(prev_err), ptr(dW)))
+
+
+def sse_backward(D, N, pat, y, tgt, err, stream=None):
+    check(lib().cnt_sse_backward(stream_ptr(stream), D, N, ptr(pat), ptr(y), ptr(tgt), ptr(err)))
+
+
+def sse_error(D, N, pat, y, tgt, result, stream=None):
+    check(lib().cnt_sse_error(stream_ptr(stream), D, N, ptr(pat), ptr(y), ptr(tgt), ptr(result)))
+
+
+class Lstm:
+    """Thin owner of a cnt_lstm handle."""
+
+    def __init__(self, P, L, bidir, S, maxT, bias=1.0):
+        self.P, self.L, self.bidir, self.S, self.maxT = P, L, bool(bidir), S, maxT
+        self.H = L // (2 if bidir else 1)
+        self.handle = VP()
+        desc = LstmDesc(P, L, int(bidir), S, maxT, bias)
+        check(lib().cnt_lstm_create(C.byref(desc), C.byref(self.handle)))
+        self.T = 0
+
+    def close(self):
+        if self.handle:
+            lib().cnt_lstm_destroy(self.handle)
+            self.handle = VP()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def load_sequences(self, pat, T, Tmin, stream=None):
+        self._pat = pat  # keep the device buffer alive
+        self.T = T
+        check(lib().cnt_lstm_load_sequences(self.handle, stream_ptr(stream), ptr(pat), T, Tmin))
+
+    def forward(self, W, x, out, stream=None):
+        check(lib().cnt_lstm_forward(self.handle, stream_ptr(stream), ptr(W), ptr(x), ptr(out)))
+
+    def backward(self, W, x, out, outerr, prev_err, dW, stream=None):
+        check(lib().cnt_lstm_backward(self.handle, stream_ptr(stream), ptr(W), ptr(x), ptr(out), ptr(outerr),
+                                      ptr(prev_err), ptr(dW)))
+
+    def check(self, stream=None):
+        check(lib().cnt_lstm_check(self.handle, stream_ptr(stream)))
+
+    def state(self, direction, name):
+        """Copy of one internal H x (T*S) buffer as a torch tensor."""
+        import torch
+
+        p = lib().cnt_lstm_state(self.handle, direction, LSTM_STATE[name])
+        if not p:
+            raise RuntimeError("no such LSTM state buffer: %r direction %d" % (name, direction))
+        n = self.H * self.T * self.S
+        torch.cuda.synchronize()
+        return torch.as_tensor(_DeviceArray(p, n), device="cuda").clone()
+
+
+class _DeviceArray:
+    """Exposes a raw device pointer of n floats through __cuda_array_interface__."""
+
+    def __init__(self, pointer, n):
+        self.__cuda_array_interface__ = {"shape": (n,), "typestr": "<f4", "data": (int(pointer), False),
+                                         "version": 2}

@@ -1,0 +1,135 @@
+// Shared declarations of the gfx950 backward-pass library: error plumbing, scalar device
+// functions with the reference's exact clamping rules, and the internal kernel launch API.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/currennt_hip.h"
+
+namespace cnt {
+
+// ----- error plumbing: nothing throws across the C ABI ------------------------------------------
+void set_error(const char *fmt, ...);
+const char *last_error();
+
+#define CNT_HIP(expr)                                                                        \
+    do {                                                                                     \
+        hipError_t _e = (expr);                                                              \
+        if (_e != hipSuccess) {                                                              \
+            ::cnt::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, \
+                             __LINE__);                                                      \
+            return CNT_ERR_HIP;                                                              \
+        }                                                                                    \
+    } while (0)
+
+#define CNT_REQUIRE(cond, ...)           \
+    do {                                 \
+        if (!(cond)) {                   \
+            ::cnt::set_error(__VA_ARGS__); \
+            return CNT_ERR_ARG;          \
+        }                                \
+    } while (0)
+
+#define CNT_TRY(expr)            \
+    do {                         \
+        int _s = (expr);         \
+        if (_s != CNT_OK) return _s; \
+    } while (0)
+
+// ----- scalar semantics ---------------------------------------------------------------------------
+// Reference: activation_functions/{Logistic,Maxmin1,Tanh}.cuh, helpers/{limitedError,safeExp,
+// NumericLimits}.cuh.  tanh is 2*logistic(2x)-1 and the logistic saturates outside +-88.722839.
+namespace lim {
+constexpr float kMin = 1.1754944e-038f;
+constexpr float kMax = 3.4028235e+038f;
+constexpr float kExpLimit = 88.722839f;
+constexpr float kLogZero = -1e30f;
+constexpr float kLSmall = -0.5e10f;
+constexpr float kMinLarg = 1.1754944e-038f;
+constexpr float kMinLogExp = -69.0776f;
+}  // namespace lim
+
+__device__ __forceinline__ float logistic(float x) {
+    if (x < lim::kExpLimit) {
+        if (x > -lim::kExpLimit) return 1.0f / (1.0f + expf(-x));
+        return 0.0f;
+    }
+    return 1.0f;
+}
+__device__ __forceinline__ float logistic_deriv(float y) { return y * (1.0f - y); }
+__device__ __forceinline__ float tanh_act(float x) { return 2.0f * logistic(2.0f * x) - 1.0f; }
+__device__ __forceinline__ float tanh_deriv(float y) { return 1.0f - y * y; }
+__device__ __forceinline__ float clip1(float e) { return e < -1.0f ? -1.0f : (e > 1.0f ? 1.0f : e); }
+__device__ __forceinline__ float safe_exp(float x) {
+    if (x <= lim::kLogZero) return 0.0f;
+    if (x >= lim::kExpLimit) return lim::kMax;
+    return expf(x);
+}
+__device__ __forceinline__ float safe_log(float x) { return x < lim::kMinLarg ? lim::kLogZero : logf(x); }
+__device__ __forceinline__ float log_add(float x, float y) {
+    const float hi = x > y ? x : y;
+    const float lo = x > y ? y : x;
+    if ((lo - hi) < lim::kMinLogExp) return hi < lim::kLSmall ? lim::kLogZero : hi;
+    return (float)((double)hi + log(1.0 + (double)expf(lo - hi)));
+}
+
+enum Act { ACT_IDENTITY = 0, ACT_TANH = 1, ACT_LOGISTIC = 2, ACT_RELU = 3 };
+__device__ __forceinline__ float act_fn(int act, float a) {
+    switch (act) {
+        case ACT_TANH: return tanh_act(a);
+        case ACT_LOGISTIC: return logistic(a);
+        case ACT_RELU: return a > 0.0f ? a : 0.0f;
+        default: return a;
+    }
+}
+__device__ __forceinline__ float act_deriv(int act, float y) {
+    switch (act) {
+        case ACT_TANH: return tanh_deriv(y);
+        case ACT_LOGISTIC: return logistic_deriv(y);
+        case ACT_RELU: return y > 0.0f ? 1.0f : 0.0f;
+        default: return 1.0f;
+    }
+}
+
+// ----- GEMM (gemm.hip) ------------------------------------------------------------------------------
+// C (m x n, column-major, ldc) = sum over segments of opA(A_i) * opB(B_i), optionally added to C.
+// An operand is described by where element (row, kk) lives: row-contiguous (ptr[kk*ld + row]) or
+// k-contiguous (ptr[row*ld + kk]).
+constexpr int kGemmMaxSeg = 8;
+constexpr int kGemmMaxProb = 8;
+
+enum GemmEpilogue { EPI_STORE = 0, EPI_ADD = 1, EPI_ATOMIC = 2, EPI_BIAS_ACT = 3 };
+
+struct GemmProblem {
+    const float *A[kGemmMaxSeg];
+    const float *B[kGemmMaxSeg];
+    float *C;
+    const float *bias_vec;  // EPI_BIAS_ACT: C = act(acc + bias_scale * bias_vec[row])
+};
+
+struct GemmArgs {
+    int m, n, k;
+    int lda, ldb, ldc;
+    int a_kcontig, b_kcontig;  // 1: element (row,kk) at ptr[row*ld+kk]; 0: ptr[kk*ld+row]
+    int nseg, nprob, splitk;
+    int epilogue, act;
+    float bias_scale;
+    GemmProblem prob[kGemmMaxProb];
+};
+
+int gemm_launch(hipStream_t stream, const GemmArgs &args);
+
+// Convenience: single problem, BLAS-like transposes on column-major matrices.
+int gemm_simple(hipStream_t stream, float *C, int m, int n, int k, const float *A, bool transA,
+                const float *B, bool transB, bool accumulate);
+
+// ----- small streaming kernels (elementwise.hip) ----------------------------------------------------
+int fill_zero(hipStream_t stream, float *p, size_t count);
+// out[d] += scale * sum over the N columns of a D x N column-major matrix (out pre-zeroed by the caller)
+int column_sum(hipStream_t stream, const float *v, int D, int N, float scale, float *out);
+
+}  // namespace cnt

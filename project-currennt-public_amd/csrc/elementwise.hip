@@ -1,0 +1,163 @@
+// Streaming kernels of the dense and SSE layers plus small utilities.
+//
+// Reference behaviour: layers/FeedForwardLayer.cu (:105-138 functors, :1633-1738 backward driver,
+// :1060-1101 forward) and layers/SsePostOutputLayer.cu (:94-136, :166-267).
+#include "common.hpp"
+
+namespace cnt {
+namespace {
+
+__global__ void fill_zero_kernel(float *__restrict__ p, size_t count) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) p[i] = 0.0f;
+}
+
+// delta = act'(y) * err in place, on every slot (the reference does not mask padding here)
+__global__ void dense_delta_kernel(float *__restrict__ err, const float *__restrict__ y, size_t count, int act) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) err[i] = act_deriv(act, y[i]) * err[i];
+}
+
+// out[d] += scale * sum_i v[d + i*D] over a chunk of columns; out is zeroed by the caller
+__global__ void column_sum_kernel(const float *__restrict__ v, int D, int N, int chunk, float scale,
+                                  float *__restrict__ out) {
+    const int d = blockIdx.x * blockDim.x + threadIdx.x;
+    if (d >= D) return;
+    const int i0 = blockIdx.y * chunk, i1 = min(N, i0 + chunk);
+    float acc = 0.0f;
+    for (int i = i0; i < i1; ++i) acc += scale * v[(size_t)i * D + d];
+    atomicAdd(out + d, acc);
+}
+
+__global__ void sse_backward_kernel(int D, size_t count, const char *__restrict__ pat, const float *__restrict__ y,
+                                    const float *__restrict__ tgt, float *__restrict__ err) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) err[i] = (pat[i / D] == 0) ? 0.0f : (y[i] - tgt[i]);
+}
+
+__global__ void sse_error_kernel(int D, size_t count, const char *__restrict__ pat, const float *__restrict__ y,
+                                 const float *__restrict__ tgt, float *__restrict__ result) {
+    __shared__ float part[4];
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    float acc = 0.0f;
+    for (; i < count; i += stride) {
+        if (pat[i / D] == 0) continue;
+        const float diff = tgt[i] - y[i];
+        acc += diff * diff;
+    }
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicAdd(result, 0.5f * (part[0] + part[1] + part[2] + part[3]));
+}
+
+inline int stream_blocks(size_t count) {
+    size_t b = (count + 255) / 256;
+    if (b > 4096) b = 4096;
+    if (b < 1) b = 1;
+    return (int)b;
+}
+
+}  // namespace
+
+int fill_zero(hipStream_t stream, float *p, size_t count) {
+    if (count == 0) return CNT_OK;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, p, count);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+int column_sum(hipStream_t stream, const float *v, int D, int N, float scale, float *out) {
+    const int chunk = 64;
+    dim3 grid((D + 255) / 256, (N + chunk - 1) / chunk);
+    hipLaunchKernelGGL(column_sum_kernel, grid, dim3(256), 0, stream, v, D, N, chunk, scale, out);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+}  // namespace cnt
+
+extern "C" {
+
+int cnt_dense_forward(void *stream_, int P, int D, int N, int act, float bias, const float *weights, const float *x,
+                      float *y) {
+    using namespace cnt;
+    CNT_REQUIRE(weights && x && y, "dense_forward: null argument");
+    CNT_REQUIRE(P > 0 && D > 0 && N > 0, "dense_forward: non-positive size");
+    CNT_REQUIRE(act >= 0 && act <= 3, "dense_forward: unknown activation %d", act);
+    GemmArgs ga = {};
+    ga.m = D; ga.n = N; ga.k = P;
+    ga.a_kcontig = 1; ga.lda = P;
+    ga.b_kcontig = 1; ga.ldb = P;
+    ga.ldc = D;
+    ga.nseg = 1; ga.nprob = 1; ga.splitk = 1;
+    ga.epilogue = EPI_BIAS_ACT; ga.act = act; ga.bias_scale = bias;
+    ga.prob[0].A[0] = weights; ga.prob[0].B[0] = x; ga.prob[0].C = y;
+    ga.prob[0].bias_vec = weights + (size_t)P * D;
+    return gemm_launch(static_cast<hipStream_t>(stream_), ga);
+}
+
+int cnt_dense_backward(void *stream_, int P, int D, int N, int act, float bias, const float *weights, const float *x,
+                       const float *y, float *err, float *prev_err, float *weight_updates) {
+    using namespace cnt;
+    CNT_REQUIRE(weights && x && y && err && weight_updates, "dense_backward: null argument");
+    CNT_REQUIRE(P > 0 && D > 0 && N > 0, "dense_backward: non-positive size");
+    CNT_REQUIRE(act >= 0 && act <= 3, "dense_backward: unknown activation %d", act);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const size_t count = (size_t)D * N;
+    if (act != ACT_IDENTITY) {
+        hipLaunchKernelGGL(dense_delta_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, err, y, count, act);
+        CNT_HIP(hipGetLastError());
+    }
+    if (prev_err) CNT_TRY(gemm_simple(stream, prev_err, P, N, D, weights, false, err, false, false));
+    CNT_TRY(fill_zero(stream, weight_updates, (size_t)P * D + D));
+    {
+        GemmArgs ga = {};
+        ga.m = P; ga.n = D; ga.k = N;
+        ga.a_kcontig = 0; ga.lda = P;
+        ga.b_kcontig = 0; ga.ldb = D;
+        ga.ldc = P;
+        ga.nseg = 1; ga.nprob = 1; ga.epilogue = EPI_ATOMIC;
+        const int tiles = ((P + 127) / 128) * ((D + 127) / 128);
+        int s = (512 + tiles - 1) / tiles;
+        const int kt = (N + 15) / 16;
+        ga.splitk = s > kt ? kt : s;
+        ga.prob[0].A[0] = x; ga.prob[0].B[0] = err; ga.prob[0].C = weight_updates;
+        CNT_TRY(gemm_launch(stream, ga));
+    }
+    return column_sum(stream, err, D, N, bias, weight_updates + (size_t)P * D);
+}
+
+int cnt_sse_backward(void *stream_, int D, int N, const char *patTypes, const float *y, const float *target,
+                     float *err) {
+    using namespace cnt;
+    CNT_REQUIRE(patTypes && y && target && err, "sse_backward: null argument");
+    CNT_REQUIRE(D > 0 && N > 0, "sse_backward: non-positive size");
+    const size_t count = (size_t)D * N;
+    hipLaunchKernelGGL(sse_backward_kernel, dim3(stream_blocks(count)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream_), D, count, patTypes, y, target, err);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+int cnt_sse_error(void *stream_, int D, int N, const char *patTypes, const float *y, const float *target,
+                  float *result_dev) {
+    using namespace cnt;
+    CNT_REQUIRE(patTypes && y && target && result_dev, "sse_error: null argument");
+    CNT_REQUIRE(D > 0 && N > 0, "sse_error: non-positive size");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    CNT_TRY(fill_zero(stream, result_dev, 1));
+    const size_t count = (size_t)D * N;
+    int blocks = stream_blocks(count);
+    if (blocks > 512) blocks = 512;
+    hipLaunchKernelGGL(sse_error_kernel, dim3(blocks), dim3(256), 0, stream, D, count, patTypes, y, target,
+                       result_dev);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+}  // extern "C"

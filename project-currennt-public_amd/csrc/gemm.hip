@@ -1,0 +1,291 @@
+// fp32 MFMA matrix product for gfx950.
+//
+// This is the seam that the reference reaches through helpers::Matrix::assignProduct/addProduct
+// (helpers/Matrix.cu:353-377 -> helpers/cublas.cu:52-84).  One kernel covers every operand
+// orientation, K-concatenated accumulation over several operand pairs (the eight W_in * delta
+// products of a BLSTM become one pass), several independent problems per launch, split-K for the
+// long-K weight-gradient shapes, and a fused bias + activation epilogue for the dense forward.
+//
+// Tiling: 128 x 128 x 16 per workgroup, four 64-lane waves in a 2 x 2 arrangement, each wave owning
+// a 64 x 64 block as 2 x 2 tiles of v_mfma_f32_32x32x2_f32.  Both operand tiles sit in LDS as
+// [row][k] with a 20-float row pitch so that the 16-byte fragment reads are bank-conflict free.
+// The MFMA operands are swapped (the B tile feeds the instruction's A port) so that lane%32 walks
+// along the column-major output's contiguous dimension and every store is a 128-byte segment.
+#include "common.hpp"
+
+namespace cnt {
+namespace {
+
+constexpr int BM = 128, BN = 128, BK = 16;
+constexpr int PITCH = BK + 4;
+constexpr int NTHREADS = 256;
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <int V>
+struct VecT;
+template <>
+struct VecT<1> { typedef float type; };
+template <>
+struct VecT<2> { typedef float2 type; };
+template <>
+struct VecT<4> { typedef float4 type; };
+
+// Stages one 128-row x 16-k operand tile: global -> registers -> LDS [row][k].
+template <int VEC, bool KCONTIG>
+struct TileStage {
+    static constexpr int NLOAD = (128 * BK) / (NTHREADS * VEC);
+    typename VecT<VEC>::type r[NLOAD];
+
+    __device__ __forceinline__ void load(const float *__restrict__ base, int ld, int row0, int k0,
+                                         int rows_total, int k_total, int tid) {
+        if (KCONTIG) {
+            constexpr int TPR = BK / VEC;        // threads per row
+            constexpr int RPP = NTHREADS / TPR;  // rows per pass
+            const int kq = (tid % TPR) * VEC;
+            const int rr = tid / TPR;
+#pragma unroll
+            for (int p = 0; p < NLOAD; ++p) {
+                const int row = row0 + rr + p * RPP;
+                typename VecT<VEC>::type v = {};
+                if (row < rows_total && (k0 + kq) < k_total)
+                    v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)row * ld + k0 + kq);
+                r[p] = v;
+            }
+        } else {
+            constexpr int TPK = 128 / VEC;       // threads per k line
+            constexpr int KPP = NTHREADS / TPK;  // k lines per pass
+            const int rq = (tid % TPK) * VEC;
+            const int kk = tid / TPK;
+#pragma unroll
+            for (int p = 0; p < NLOAD; ++p) {
+                const int k = k0 + kk + p * KPP;
+                typename VecT<VEC>::type v = {};
+                if (k < k_total && (row0 + rq) < rows_total)
+                    v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)k * ld + row0 + rq);
+                r[p] = v;
+            }
+        }
+    }
+
+    __device__ __forceinline__ void store(float *__restrict__ lds, int tid) const {
+        if (KCONTIG) {
+            constexpr int TPR = BK / VEC;
+            constexpr int RPP = NTHREADS / TPR;
+            const int kq = (tid % TPR) * VEC;
+            const int rr = tid / TPR;
+#pragma unroll
+            for (int p = 0; p < NLOAD; ++p)
+                *reinterpret_cast<typename VecT<VEC>::type *>(lds + (rr + p * RPP) * PITCH + kq) = r[p];
+        } else {
+            constexpr int TPK = 128 / VEC;
+            constexpr int KPP = NTHREADS / TPK;
+            const int rq = (tid % TPK) * VEC;
+            const int kk = tid / TPK;
+#pragma unroll
+            for (int p = 0; p < NLOAD; ++p) {
+                const float *e = reinterpret_cast<const float *>(&r[p]);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) lds[(rq + j) * PITCH + kk + p * KPP] = e[j];
+            }
+        }
+    }
+};
+
+template <int VA, bool AK, int VB, bool BK_>
+__global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args) {
+    __shared__ __attribute__((aligned(16))) float lds_a[2][BM * PITCH];
+    __shared__ __attribute__((aligned(16))) float lds_b[2][BN * PITCH];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave & 1, wn = wave >> 1;
+
+    const int tiles_m = (args.m + BM - 1) / BM;
+    const int tile = blockIdx.x;
+    const int m0 = (tile % tiles_m) * BM;
+    const int n0 = (tile / tiles_m) * BN;
+    const GemmProblem &pb = args.prob[blockIdx.z];
+
+    // iteration space: segments x k-tiles, cut into splitk contiguous ranges
+    const int kt_per_seg = (args.k + BK - 1) / BK;
+    const int total_it = kt_per_seg * args.nseg;
+    const int per_split = (total_it + args.splitk - 1) / args.splitk;
+    const int it_begin = blockIdx.y * per_split;
+    const int it_end = min(total_it, it_begin + per_split);
+    if (it_begin >= it_end) return;
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    TileStage<VA, AK> sa;
+    TileStage<VB, BK_> sb;
+
+    {
+        const int seg = it_begin / kt_per_seg;
+        const int k0 = (it_begin % kt_per_seg) * BK;
+        sa.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
+        sb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid);
+        sa.store(lds_a[0], tid);
+        sb.store(lds_b[0], tid);
+    }
+    __syncthreads();
+
+    const int frag_row = lane & 31;
+    const int frag_k = (lane >> 5) * 8;
+
+    for (int it = it_begin; it < it_end; ++it) {
+        const int cur = (it - it_begin) & 1;
+        const bool has_next = (it + 1) < it_end;
+        if (has_next) {
+            const int seg = (it + 1) / kt_per_seg;
+            const int k0 = ((it + 1) % kt_per_seg) * BK;
+            sa.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
+            sb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid);
+        }
+
+        float4 fa[2][2], fb[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const float *pa = &lds_a[cur][(wm * 64 + i * 32 + frag_row) * PITCH + frag_k];
+            fa[i][0] = *reinterpret_cast<const float4 *>(pa);
+            fa[i][1] = *reinterpret_cast<const float4 *>(pa + 4);
+            const float *pbq = &lds_b[cur][(wn * 64 + i * 32 + frag_row) * PITCH + frag_k];
+            fb[i][0] = *reinterpret_cast<const float4 *>(pbq);
+            fb[i][1] = *reinterpret_cast<const float4 *>(pbq + 4);
+        }
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const float av = reinterpret_cast<const float *>(&fa[i][0])[kk];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const float bv = reinterpret_cast<const float *>(&fb[j][0])[kk];
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv, av, acc[i][j], 0, 0, 0);
+                }
+            }
+        }
+
+        if (has_next) {
+            sa.store(lds_a[cur ^ 1], tid);
+            sb.store(lds_b[cur ^ 1], tid);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: lane%32 runs along m (contiguous), the 16 accumulators along n
+    float *__restrict__ C = pb.C;
+    const int half = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int m = m0 + wm * 64 + i * 32 + frag_row;
+        if (m >= args.m) continue;
+        float bterm = 0.0f;
+        if (args.epilogue == EPI_BIAS_ACT) bterm = args.bias_scale * pb.bias_vec[m];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int n = n0 + wn * 64 + j * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (n >= args.n) continue;
+                float *dst = C + (size_t)n * args.ldc + m;
+                const float v = acc[i][j][r];
+                switch (args.epilogue) {
+                    case EPI_STORE: *dst = v; break;
+                    case EPI_ADD: *dst = *dst + v; break;
+                    case EPI_ATOMIC: atomicAdd(dst, v); break;
+                    default: *dst = act_fn(args.act, v + bterm); break;
+                }
+            }
+        }
+    }
+}
+
+inline int pick_vec(const GemmArgs &a, bool for_a) {
+    const int ld = for_a ? a.lda : a.ldb;
+    const bool kc = for_a ? a.a_kcontig : a.b_kcontig;
+    const int extent = kc ? a.k : (for_a ? a.m : a.n);
+    int v = 4;
+    while (v > 1) {
+        bool ok = (ld % v == 0) && (extent % v == 0);
+        for (int p = 0; ok && p < a.nprob; ++p)
+            for (int s = 0; ok && s < a.nseg; ++s) {
+                const float *ptr = for_a ? a.prob[p].A[s] : a.prob[p].B[s];
+                ok = (reinterpret_cast<uintptr_t>(ptr) % (4 * v)) == 0;
+            }
+        if (ok) break;
+        v >>= 1;
+    }
+    return v;
+}
+
+template <int VA, bool AK, int VB>
+void launch_b(const GemmArgs &a, dim3 grid, hipStream_t s, bool bk) {
+    if (bk) hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, true>), grid, dim3(NTHREADS), 0, s, a);
+    else hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, false>), grid, dim3(NTHREADS), 0, s, a);
+}
+template <int VA, bool AK>
+void launch_vb(const GemmArgs &a, dim3 grid, hipStream_t s, int vb, bool bk) {
+    if (vb == 4) launch_b<VA, AK, 4>(a, grid, s, bk);
+    else if (vb == 2) launch_b<VA, AK, 2>(a, grid, s, bk);
+    else launch_b<VA, AK, 1>(a, grid, s, bk);
+}
+template <int VA>
+void launch_ak(const GemmArgs &a, dim3 grid, hipStream_t s, bool ak, int vb, bool bk) {
+    if (ak) launch_vb<VA, true>(a, grid, s, vb, bk);
+    else launch_vb<VA, false>(a, grid, s, vb, bk);
+}
+
+}  // namespace
+
+int gemm_launch(hipStream_t stream, const GemmArgs &args) {
+    CNT_REQUIRE(args.m > 0 && args.n > 0 && args.k > 0, "gemm: empty problem %d x %d x %d", args.m, args.n,
+                args.k);
+    CNT_REQUIRE(args.nseg >= 1 && args.nseg <= kGemmMaxSeg, "gemm: %d operand pairs, supported 1..%d",
+                args.nseg, kGemmMaxSeg);
+    CNT_REQUIRE(args.nprob >= 1 && args.nprob <= kGemmMaxProb, "gemm: %d problems, supported 1..%d",
+                args.nprob, kGemmMaxProb);
+    CNT_REQUIRE(args.splitk >= 1 && (args.splitk == 1 || args.epilogue == EPI_ATOMIC),
+                "gemm: split-K needs the atomic epilogue");
+    for (int p = 0; p < args.nprob; ++p) {
+        CNT_REQUIRE(args.prob[p].C != nullptr, "gemm: null output");
+        for (int s = 0; s < args.nseg; ++s)
+            CNT_REQUIRE(args.prob[p].A[s] && args.prob[p].B[s], "gemm: null operand");
+    }
+    const int va = pick_vec(args, true), vb = pick_vec(args, false);
+    const int tiles = ((args.m + BM - 1) / BM) * ((args.n + BN - 1) / BN);
+    dim3 grid(tiles, args.splitk, args.nprob);
+    if (va == 4) launch_ak<4>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig);
+    else if (va == 2) launch_ak<2>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig);
+    else launch_ak<1>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+int gemm_simple(hipStream_t stream, float *C, int m, int n, int k, const float *A, bool transA,
+                const float *B, bool transB, bool accumulate) {
+    GemmArgs a = {};
+    a.m = m; a.n = n; a.k = k;
+    // column-major A (m x k, lda=m) is row-contiguous; transposed storage (k x m, lda=k) is k-contiguous
+    a.a_kcontig = transA ? 1 : 0;
+    a.lda = transA ? k : m;
+    // column-major B (k x n, ldb=k) is k-contiguous; transposed storage (n x k, ldb=n) is row-contiguous
+    a.b_kcontig = transB ? 0 : 1;
+    a.ldb = transB ? n : k;
+    a.ldc = m;
+    a.nseg = 1; a.nprob = 1; a.splitk = 1;
+    a.epilogue = accumulate ? EPI_ADD : EPI_STORE;
+    a.prob[0].A[0] = A;
+    a.prob[0].B[0] = B;
+    a.prob[0].C = C;
+    return gemm_launch(stream, a);
+}
+
+}  // namespace cnt

@@ -1,0 +1,779 @@
+// LSTM layer for gfx950: forward recursion, BPTT error recursion, and the batched contractions.
+//
+// Reference behaviour: layers/LstmLayer.cu  (forward :57-208, :1743-1949; backward :210-648,
+// :2066-2382; sequence loading :1488-1533; weight layout :1136-1169, :1218-1268).
+//
+// The reference launches four small matrix products and one elementwise functor per time step and
+// direction.  Here each direction is ONE persistent kernel ("chain"): G = H/JB workgroups each own
+// JB cells for the whole sequence, keep their slice of the recurrent weight matrix in registers as
+// MFMA operands for all T steps, carry the per-cell recurrent state (cell error, forget-gate
+// activation, gate deltas) in registers, and exchange the only truly shared quantity of a step
+// through a small device-memory mailbox:
+//   forward : block outputs h[t] (H x S), gathered by every workgroup;
+//   backward: each workgroup multiplies its own 4*JB gate deltas with its weight slice and
+//             scatters partial output errors to the owners of the receiving cells (H x S words per
+//             workgroup instead of the 4H x S a gather of the deltas would need).
+// Mailbox words are 8 bytes, (value, tag), written and polled with relaxed agent-scope atomics; the
+// tag carries launch epoch and step, so a word validates itself and no fence sits on the critical
+// path.  Two mailbox slots alternate by step parity.  Every poll loop is bounded: when the bound is
+// hit the workgroup raises a device flag and every workgroup drains out.
+//
+// The dense work that does not sit on the recursion is batched over all time steps on the MFMA
+// GEMM: input projections (8 problems, one launch), the error to the preceding layer
+// (one K-concatenated product), input and recurrent weight gradients (split-K), and one streaming
+// reduction for bias and peephole gradients.
+#include "common.hpp"
+
+#include <cstdlib>
+#include <cstring>
+#include <new>
+
+namespace cnt {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned long long u64;
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr unsigned kStepBits = 20;  // tag = epoch << 20 | (step + 1)
+
+struct DirPtrs {
+    float *ni, *ig, *fg, *og, *c, *h;
+    float *herr, *dni, *dig, *dfg, *dog, *cerr;
+    const float *w_int;    // gate 0 block of this direction; gate g at + g*L*H
+    const float *b[4];     // bias weights per gate
+    const float *peep[3];  // ig, fg, og peepholes
+    u64 *mailbox;          // 2 slots
+};
+
+struct ChainParams {
+    int H, L, S, T, Tmin, ndir;
+    float bias;
+    const char *pat;
+    DirPtrs d[2];
+    float *out;           // forward: L x (T*S) layer outputs (NULL when it aliases d[0].h)
+    const float *outerr;  // backward: L x (T*S) output errors
+    float *herr_out;      // backward, unidirectional: where the summed error is written back
+    unsigned tag_base;
+    unsigned spin_limit;
+    int *abort_flag;
+    int xcd_pack;
+};
+
+__device__ __forceinline__ u64 mb_load(const u64 *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void mb_store(u64 *p, float v, unsigned tag) {
+    const u64 w = ((u64)tag << 32) | (u64)__float_as_uint(v);
+    __hip_atomic_store(p, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Polls N mailbox words until each carries `tag`.  Returns false when the spin bound is hit or
+// another workgroup has raised the abort flag.
+template <int N>
+__device__ __forceinline__ bool mb_wait(const u64 *const (&addr)[N], float (&val)[N], unsigned tag,
+                                        unsigned spin_limit, const int *abort_flag) {
+    u64 w[N];
+#pragma unroll
+    for (int q = 0; q < N; ++q) w[q] = mb_load(addr[q]);
+    unsigned spins = 0;
+    bool ok = true;
+#pragma unroll
+    for (int q = 0; q < N; ++q) {
+        while ((unsigned)(w[q] >> 32) != tag) {
+            if (++spins > spin_limit) { ok = false; break; }
+            if ((spins & 255u) == 0u &&
+                __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+                ok = false;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+            w[q] = mb_load(addr[q]);
+        }
+        val[q] = __uint_as_float((unsigned)w[q]);
+    }
+    return ok;
+}
+
+__device__ __forceinline__ bool map_block(const ChainParams &p, int G, int &dir, int &me) {
+    const int b = blockIdx.x;
+    if (p.xcd_pack) {
+        // workgroups are dealt round-robin to the 8 XCDs; keep one chain inside one XCD's L2
+        const int xcd = b & 7;
+        if (xcd >= p.ndir) return false;
+        dir = xcd;
+        me = b >> 3;
+    } else {
+        dir = b % p.ndir;
+        me = b / p.ndir;
+    }
+    return me < G;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Forward recursion.  HT = H/64, JB = cells per workgroup, NT = ceil(S/16).
+// ---------------------------------------------------------------------------------------------------
+template <int HT, int JB, int NT>
+__global__ __launch_bounds__(kThreads) void lstm_forward_chain(const ChainParams p) {
+    constexpr int H = 64 * HT;
+    constexpr int G = H / JB;
+    constexpr int NS = 16 * NT;
+    constexpr int MT = (4 * JB) / 16;  // output tiles: rows are (gate, cell)
+    constexpr int KS = H / 16;         // k-steps of 4 per wave (each wave covers H/4 source cells)
+    static_assert((4 * JB) % 16 == 0, "JB must be a multiple of 4");
+    static_assert(JB * NS <= kThreads, "cell phase needs one thread per (cell, sequence)");
+
+    int dir, me;
+    if (!map_block(p, G, dir, me)) return;
+    const DirPtrs &D = p.d[dir];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int S = p.S, T = p.T;
+    const int j0 = me * JB;
+    const int n = S * H;
+
+    __shared__ float red[kWaves][4 * JB][NS + 1];
+
+    // recurrent weights as MFMA A operands: row (gate, cell), k = source cell
+    float wA[MT][KS];
+    {
+        const int i = lane & 15, kq = lane >> 4;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int o = mt * 16 + i, g = o / JB, jj = o % JB;
+            const float *wg = D.w_int + (size_t)g * p.L * H + (size_t)(j0 + jj) * H;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) wA[mt][ks] = wg[wave * (H / 4) + 4 * ks + kq];
+        }
+    }
+
+    // cell phase thread: one (sequence, cell) pair
+    const bool cell_thread = tid < JB * NS;
+    const int cs = tid / JB, cj = tid % JB;
+    const bool cell_valid = cell_thread && cs < S;
+    float b_ni = 0, b_ig = 0, b_fg = 0, b_og = 0, p_ig = 0, p_fg = 0, p_og = 0;
+    if (cell_valid) {
+        b_ni = p.bias * D.b[0][j0 + cj]; b_ig = p.bias * D.b[1][j0 + cj];
+        b_fg = p.bias * D.b[2][j0 + cj]; b_og = p.bias * D.b[3][j0 + cj];
+        p_ig = D.peep[0][j0 + cj]; p_fg = D.peep[1][j0 + cj]; p_og = D.peep[2][j0 + cj];
+    }
+    float c_prev = 0.0f;
+
+    for (int step = 0; step < T; ++step) {
+        const int t = dir ? (T - 1 - step) : step;
+        const bool first = (step == 0);
+        const size_t gi = (size_t)t * n + (size_t)cs * H + j0 + cj;
+
+        // pre-activations from the input projection: independent of the recursion, issued early
+        float a_ni = 0, a_ig = 0, a_fg = 0, a_og = 0;
+        bool dummy = false;
+        if (cell_valid) {
+            a_ni = D.ni[gi]; a_ig = D.ig[gi]; a_fg = D.fg[gi]; a_og = D.og[gi];
+            dummy = (t >= p.Tmin) && (p.pat[t * S + cs] == 0);
+        }
+
+        if (!first) {
+            // gather h of the previous step straight into MFMA B operands
+            const unsigned tag = p.tag_base + (unsigned)step;  // published at the end of step-1
+            const u64 *slot = D.mailbox + (size_t)((step - 1) & 1) * H * NS;
+            f32x4 acc[MT][NT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0, 0, 0, 0};
+            bool ok = true;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const int s = nt * 16 + (lane & 15);
+                float hv[KS];
+                if (s < S) {
+                    const u64 *addr[KS];
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+                        addr[ks] = slot + ((size_t)(wave * KS + ks) * NS + s) * 4 + (lane >> 4);
+                    ok = mb_wait<KS>(addr, hv, tag, p.spin_limit, p.abort_flag) && ok;
+                } else {
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) hv[ks] = 0.0f;
+                }
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wA[mt][ks], hv[ks], acc[mt][nt], 0, 0, 0);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        red[wave][mt * 16 + 4 * (lane >> 4) + r][nt * 16 + (lane & 15)] = acc[mt][nt][r];
+            if (__syncthreads_or(ok ? 0 : 1)) {
+                if (tid == 0) __hip_atomic_store(p.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return;
+            }
+        }
+
+        if (cell_valid) {
+            if (!first) {
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) {
+                    a_ni += red[w][0 * JB + cj][cs];
+                    a_ig += red[w][1 * JB + cj][cs];
+                    a_fg += red[w][2 * JB + cj][cs];
+                    a_og += red[w][3 * JB + cj][cs];
+                }
+            }
+            float hval = 0.0f;
+            if (dummy) {
+                // the reference leaves the summed pre-activations in place on padding slots, clears the
+                // cell only in the time-reversed direction and emits a zero output
+                if (!first) { D.ni[gi] = a_ni; D.ig[gi] = a_ig; D.fg[gi] = a_fg; D.og[gi] = a_og; }
+                if (dir) { D.c[gi] = 0.0f; c_prev = 0.0f; }
+                else c_prev = D.c[gi];
+            } else {
+                float x_ni = a_ni + b_ni, x_ig = a_ig + b_ig, x_fg = a_fg + b_fg, x_og = a_og + b_og;
+                if (!first) { x_ig += c_prev * p_ig; x_fg += c_prev * p_fg; }
+                const float ni = tanh_act(x_ni), ig = logistic(x_ig), fg = logistic(x_fg);
+                float c = ni * ig;
+                if (!first) c += c_prev * fg;
+                x_og += c * p_og;
+                const float og = logistic(x_og);
+                hval = tanh_act(c) * og;
+                D.ni[gi] = ni; D.ig[gi] = ig; D.fg[gi] = fg; D.og[gi] = og; D.c[gi] = c;
+                c_prev = c;
+            }
+            if (step + 1 < T) {
+                const int from = j0 + cj;
+                u64 *slot = D.mailbox + (size_t)(step & 1) * H * NS;
+                mb_store(slot + ((size_t)(from >> 2) * NS + cs) * 4 + (from & 3), hval,
+                         p.tag_base + (unsigned)step + 1u);
+            }
+            D.h[gi] = hval;
+            if (p.out) p.out[((size_t)t * S + cs) * p.L + dir * H + j0 + cj] = hval;
+        }
+        __syncthreads();  // `red` is rewritten in the next step
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Backward (error) recursion.
+// ---------------------------------------------------------------------------------------------------
+template <int HT, int JB, int NT>
+__global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParams p) {
+    constexpr int H = 64 * HT;
+    constexpr int G = H / JB;
+    constexpr int NS = 16 * NT;
+    constexpr int MT = H / 64;  // 16-row tiles of receiving cells per wave (each wave covers H/4)
+    constexpr int KS = JB;      // k = (gate, own cell): 4*JB values, 4 per MFMA
+    constexpr int EL = JB * NS; // (cell, sequence) pairs of this workgroup, padded
+    constexpr int NPART = kThreads / EL;
+    constexpr int NPOLL = G / NPART;
+    static_assert(kThreads % EL == 0 && G % NPART == 0, "mailbox polling layout");
+
+    int dir, me;
+    if (!map_block(p, G, dir, me)) return;
+    const DirPtrs &D = p.d[dir];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int S = p.S, T = p.T;
+    const int j0 = me * JB;
+    const int n = S * H;
+
+    __shared__ float psum[NPART][JB][NS + 1];
+    __shared__ float dl[4 * JB][NS + 1];
+
+    // recurrent weights as MFMA A operands: row = receiving ("from") cell, k = (gate, own cell)
+    float wA[MT][KS];
+    {
+        const int i = lane & 15, kq = lane >> 4;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int k = 4 * ks + kq, g = k / JB, jj = k % JB;
+            const float *wg = D.w_int + (size_t)g * p.L * H + (size_t)(j0 + jj) * H;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) wA[mt][ks] = wg[wave * (H / 4) + mt * 16 + i];
+        }
+    }
+
+    // polling role: element (cell pj, sequence ps), sources part, part+NPART, ...
+    const int pe = tid % EL, part = tid / EL;
+    const int pj = pe / NS, ps = pe % NS;
+    // cell-phase role: jj fastest so that global accesses of neighbouring lanes touch one segment
+    const bool cell_thread = tid < EL;
+    const int cs = tid / JB, cj = tid % JB;
+    const bool cell_valid = cell_thread && cs < S;
+    float p_ig = 0, p_fg = 0, p_og = 0;
+    if (cell_valid) { p_ig = D.peep[0][j0 + cj]; p_fg = D.peep[1][j0 + cj]; p_og = D.peep[2][j0 + cj]; }
+    // this cell's values at the slot processed in the previous iteration
+    float fg_later = 0, cerr_later = 0, dig_later = 0, dfg_later = 0;
+
+    for (int step = 0; step < T; ++step) {
+        const int t = dir ? step : (T - 1 - step);
+        const int earlier = dir ? t + 1 : t - 1;
+        const bool first = (step == 0), last = (step == T - 1);
+        const size_t gi = (size_t)t * n + (size_t)cs * H + j0 + cj;
+
+        // everything that does not depend on the recursion is requested before the wait
+        float e = 0, ni = 0, ig = 0, fg = 0, og = 0, c = 0, c_earlier = 0, dog_old = 0;
+        bool dummy = false;
+        if (cell_valid) {
+            e = p.outerr[((size_t)t * S + cs) * p.L + dir * H + j0 + cj];
+            ni = D.ni[gi]; ig = D.ig[gi]; fg = D.fg[gi]; og = D.og[gi]; c = D.c[gi];
+            dog_old = D.dog[gi];
+            if (!last) c_earlier = D.c[(size_t)earlier * n + (size_t)cs * H + j0 + cj];
+            dummy = (t >= p.Tmin) && (p.pat[t * S + cs] == 0);
+        }
+
+        if (!first) {
+            const unsigned tag = p.tag_base + (unsigned)step;
+            const u64 *slot = D.mailbox + (size_t)((step - 1) & 1) * G * G * EL;
+            float part_sum = 0.0f;
+            bool ok = true;
+            if (ps < S) {
+                const u64 *addr[NPOLL];
+                float v[NPOLL];
+#pragma unroll
+                for (int q = 0; q < NPOLL; ++q)
+                    addr[q] = slot + ((size_t)(me * G + part + NPART * q) * JB + pj) * NS + ps;
+                ok = mb_wait<NPOLL>(addr, v, tag, p.spin_limit, p.abort_flag);
+#pragma unroll
+                for (int q = 0; q < NPOLL; ++q) part_sum += v[q];
+            }
+            psum[part][pj][ps] = part_sum;
+            if (__syncthreads_or(ok ? 0 : 1)) {
+                if (tid == 0) __hip_atomic_store(p.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return;
+            }
+        }
+
+        if (cell_valid) {
+            if (!first) {
+#pragma unroll
+                for (int q = 0; q < NPART; ++q) e += psum[q][cj][cs];
+            }
+            float s_ni = 0, s_ig = 0, s_fg = 0, s_og = 0, ce = 0;
+            if (!dummy) {
+                const float tc = tanh_act(c);
+                const float d_og = (logistic_deriv(og) * tc * e) + dog_old;
+                ce = og * tanh_deriv(tc) * e + p_og * d_og;
+                if (!first) ce += (fg_later * cerr_later + p_ig * dig_later + p_fg * dfg_later);
+                const float d_ni = ig * tanh_deriv(ni) * ce;
+                const float d_fg = last ? 0.0f : logistic_deriv(fg) * c_earlier * ce;
+                const float d_ig = logistic_deriv(ig) * ni * ce;
+                s_ni = clip1(d_ni); s_ig = clip1(d_ig); s_fg = clip1(d_fg); s_og = clip1(d_og);
+            }
+            D.dni[gi] = s_ni; D.dig[gi] = s_ig; D.dfg[gi] = s_fg; D.dog[gi] = s_og; D.cerr[gi] = ce;
+            if (p.herr_out) p.herr_out[gi] = e;
+            else D.herr[gi] = e;
+            dl[0 * JB + cj][cs] = s_ni; dl[1 * JB + cj][cs] = s_ig;
+            dl[2 * JB + cj][cs] = s_fg; dl[3 * JB + cj][cs] = s_og;
+            fg_later = fg; cerr_later = ce; dig_later = s_ig; dfg_later = s_fg;
+        }
+        __syncthreads();
+
+        if (!last) {
+            // partial output errors of every receiving cell from this workgroup's deltas
+            const unsigned tag = p.tag_base + (unsigned)step + 1u;
+            u64 *slot = D.mailbox + (size_t)(step & 1) * G * G * EL;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const int s = nt * 16 + (lane & 15);
+                f32x4 acc[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0, 0, 0, 0};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const float bv = dl[4 * ks + (lane >> 4)][s];
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wA[mt][ks], bv, acc[mt], 0, 0, 0);
+                }
+                if (s < S) {
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int from = wave * (H / 4) + mt * 16 + 4 * (lane >> 4) + r;
+                            const int dst = from / JB, jd = from % JB;
+                            mb_store(slot + ((size_t)(dst * G + me) * JB + jd) * NS + s, acc[mt][r], tag);
+                        }
+                }
+            }
+        }
+        // `dl` and `psum` are rewritten only after the next step's barrier
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Bias and peephole gradients: per (direction, gate, cell) sums over all patterns
+// (LstmLayer.cu:524-541, 574-610, 625-646).  One thread per cell, a chunk of patterns per block.
+// ---------------------------------------------------------------------------------------------------
+struct SmallGradParams {
+    int H, L, S, N;  // N = T*S patterns
+    float bias;
+    const float *dni, *dig, *dfg, *dog, *c;
+    float *g_bias;  // + g*L + u
+    float *g_peep;  // + k*L + u
+    int dir;
+    int chunk;
+};
+
+__global__ void lstm_small_grads(const SmallGradParams p) {
+    const int u = blockIdx.x * blockDim.x + threadIdx.x;
+    if (u >= p.H) return;
+    const int i0 = blockIdx.y * p.chunk;
+    const int i1 = min(p.N, i0 + p.chunk);
+    const int H = p.H, S = p.S;
+    float b0 = 0, b1 = 0, b2 = 0, b3 = 0, q_ig = 0, q_fg = 0, q_og = 0;
+    for (int i = i0; i < i1; ++i) {
+        const size_t o = (size_t)i * H + u;
+        const float d_ni = p.dni[o], d_ig = p.dig[o], d_fg = p.dfg[o], d_og = p.dog[o];
+        b0 += p.bias * d_ni; b1 += p.bias * d_ig; b2 += p.bias * d_fg; b3 += p.bias * d_og;
+        q_og += p.c[o] * d_og;
+        // input/forget peepholes look at the cell state one step earlier in processing order
+        const int ie = p.dir ? i + S : i - S;
+        if (ie >= 0 && ie < p.N) {
+            const float ce = p.c[(size_t)ie * H + u];
+            q_ig += ce * d_ig;
+            q_fg += ce * d_fg;
+        }
+    }
+    const int L = p.L;
+    atomicAdd(p.g_bias + 0 * L + u, b0); atomicAdd(p.g_bias + 1 * L + u, b1);
+    atomicAdd(p.g_bias + 2 * L + u, b2); atomicAdd(p.g_bias + 3 * L + u, b3);
+    atomicAdd(p.g_peep + 0 * L + u, q_ig); atomicAdd(p.g_peep + 1 * L + u, q_fg);
+    atomicAdd(p.g_peep + 2 * L + u, q_og);
+}
+
+}  // namespace
+}  // namespace cnt
+
+// ---------------------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------------------
+struct cnt_lstm {
+    cnt_lstm_desc desc;
+    int ndir, H;
+    int T, Tmin;  // current fraction
+    const char *pat;
+    float *state[2][12];
+    cnt::u64 *mailbox[2];
+    size_t mailbox_bytes;
+    int *abort_flag;
+    unsigned epoch;
+    int device;
+    int JB, NT;
+    unsigned spin_limit;
+    int xcd_pack;
+};
+
+namespace cnt {
+namespace {
+
+typedef void (*chain_kernel_t)(const ChainParams);
+
+template <int HT, int JB>
+chain_kernel_t pick_nt(bool fwd, int NT) {
+    if (NT == 1) return fwd ? (chain_kernel_t)lstm_forward_chain<HT, JB, 1> : (chain_kernel_t)lstm_backward_chain<HT, JB, 1>;
+    if (NT == 2) return fwd ? (chain_kernel_t)lstm_forward_chain<HT, JB, 2> : (chain_kernel_t)lstm_backward_chain<HT, JB, 2>;
+    return nullptr;
+}
+
+chain_kernel_t pick_kernel(bool fwd, int H, int JB, int NT) {
+    if (H == 64 && JB == 4) return pick_nt<1, 4>(fwd, NT);
+    if (H == 128 && JB == 4) return pick_nt<2, 4>(fwd, NT);
+    if (H == 128 && JB == 8) return pick_nt<2, 8>(fwd, NT);
+    if (H == 256 && JB == 4) return pick_nt<4, 4>(fwd, NT);
+    if (H == 256 && JB == 8) return pick_nt<4, 8>(fwd, NT);
+    if (H == 512 && JB == 8) return pick_nt<8, 8>(fwd, NT);
+    return nullptr;
+}
+
+int default_jb(int H) { return H >= 256 ? 8 : 4; }
+
+size_t weight_count(int P, int L, int bidir) {
+    const size_t H = L / (bidir ? 2 : 1);
+    return (size_t)4 * P * L + (size_t)4 * L + (size_t)4 * L * H + (size_t)3 * L;
+}
+
+void fill_chain_params(const cnt_lstm *h, const float *weights, ChainParams &p) {
+    const cnt_lstm_desc &d = h->desc;
+    const int P = d.P, L = d.L, H = h->H;
+    std::memset(&p, 0, sizeof(p));
+    p.H = H; p.L = L; p.S = d.S; p.T = h->T; p.Tmin = h->Tmin; p.ndir = h->ndir; p.bias = d.bias;
+    p.pat = h->pat;
+    const size_t off_bias = (size_t)4 * P * L, off_int = off_bias + (size_t)4 * L;
+    const size_t off_peep = off_int + (size_t)4 * L * H;
+    for (int dir = 0; dir < h->ndir; ++dir) {
+        DirPtrs &D = p.d[dir];
+        float *const *s = h->state[dir];
+        D.ni = s[0]; D.ig = s[1]; D.fg = s[2]; D.og = s[3]; D.c = s[4]; D.h = s[5];
+        D.herr = s[6]; D.dni = s[7]; D.dig = s[8]; D.dfg = s[9]; D.dog = s[10]; D.cerr = s[11];
+        D.w_int = weights + off_int + (size_t)dir * H * H;
+        for (int g = 0; g < 4; ++g) D.b[g] = weights + off_bias + (size_t)g * L + dir * H;
+        for (int k = 0; k < 3; ++k) D.peep[k] = weights + off_peep + (size_t)k * L + dir * H;
+        D.mailbox = h->mailbox[dir];
+    }
+    p.spin_limit = h->spin_limit;
+    p.abort_flag = h->abort_flag;
+    p.xcd_pack = h->xcd_pack;
+}
+
+int next_epoch(cnt_lstm *h, hipStream_t stream, unsigned &tag_base) {
+    // tags are epoch << 20 | step+1; when the 12-bit epoch wraps the mailboxes are wiped so that a
+    // word of an old launch can never validate
+    h->epoch += 1;
+    if (h->epoch >= (1u << (32 - kStepBits))) {
+        for (int dir = 0; dir < h->ndir; ++dir)
+            CNT_TRY(fill_zero(stream, reinterpret_cast<float *>(h->mailbox[dir]), h->mailbox_bytes / 4));
+        h->epoch = 1;
+    }
+    tag_base = h->epoch << kStepBits;
+    return CNT_OK;
+}
+
+int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
+    chain_kernel_t k = pick_kernel(fwd, h->H, h->JB, h->NT);
+    CNT_REQUIRE(k != nullptr, "lstm: no recursion kernel for H=%d JB=%d S=%d", h->H, h->JB, h->desc.S);
+    CNT_TRY(next_epoch(h, stream, p.tag_base));
+    const int G = h->H / h->JB;
+    const int blocks = h->xcd_pack ? 8 * G : h->ndir * G;
+    hipLaunchKernelGGL(k, dim3(blocks), dim3(kThreads), 0, stream, p);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+}  // namespace
+}  // namespace cnt
+
+extern "C" {
+
+long cnt_lstm_weight_count(int P, int L, int bidir) { return (long)cnt::weight_count(P, L, bidir); }
+
+int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
+    using namespace cnt;
+    CNT_REQUIRE(desc && out, "lstm_create: null argument");
+    CNT_REQUIRE(desc->P > 0 && desc->L > 0 && desc->S > 0 && desc->maxT > 0, "lstm_create: non-positive size");
+    // the reference refuses odd bidirectional sizes (LstmLayer.cu:1091-1092)
+    CNT_REQUIRE(!desc->bidir || desc->L % 2 == 0, "Cannot create a bidirectional layer with an odd layer size");
+    const int ndir = desc->bidir ? 2 : 1;
+    const int H = desc->L / ndir;
+    CNT_REQUIRE(desc->maxT < (1 << kStepBits) - 2, "lstm_create: maxT %d too long", desc->maxT);
+    const int NT = (desc->S + 15) / 16;
+    int JB = default_jb(H);
+    if (const char *e = std::getenv("CNT_LSTM_JB")) JB = std::atoi(e);
+    CNT_REQUIRE(pick_kernel(true, H, JB, NT) != nullptr,
+                "lstm_create: cells per direction H=%d with S=%d parallel sequences has no recursion kernel "
+                "(H in {64,128,256,512}, S <= 32)", H, desc->S);
+
+    cnt_lstm *h = new (std::nothrow) cnt_lstm();
+    CNT_REQUIRE(h != nullptr, "lstm_create: out of host memory");
+    std::memset(h, 0, sizeof(*h));
+    h->desc = *desc; h->ndir = ndir; h->H = H; h->JB = JB; h->NT = NT;
+    h->spin_limit = 1u << 22;
+    if (const char *e = std::getenv("CNT_LSTM_SPIN_LIMIT")) h->spin_limit = (unsigned)std::strtoul(e, nullptr, 10);
+    h->xcd_pack = 0;
+    if (const char *e = std::getenv("CNT_LSTM_XCD_PACK")) h->xcd_pack = std::atoi(e) != 0;
+    hipError_t err = hipGetDevice(&h->device);
+    const size_t nstate = (size_t)H * desc->maxT * desc->S;
+    const int G = H / JB, NS = 16 * NT;
+    // forward needs H*NS words per slot, backward G*G*JB*NS = H*G*NS
+    h->mailbox_bytes = (size_t)2 * H * G * NS * sizeof(u64);
+    for (int dir = 0; dir < ndir && err == hipSuccess; ++dir) {
+        for (int w = 0; w < 12 && err == hipSuccess; ++w) {
+            err = hipMalloc(reinterpret_cast<void **>(&h->state[dir][w]), nstate * sizeof(float));
+            if (err == hipSuccess) err = hipMemset(h->state[dir][w], 0, nstate * sizeof(float));
+        }
+        if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->mailbox[dir]), h->mailbox_bytes);
+        if (err == hipSuccess) err = hipMemset(h->mailbox[dir], 0, h->mailbox_bytes);
+    }
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->abort_flag), sizeof(int));
+    if (err == hipSuccess) err = hipMemset(h->abort_flag, 0, sizeof(int));
+    if (err != hipSuccess) {
+        set_error("lstm_create: %s", hipGetErrorString(err));
+        cnt_lstm_destroy(h);
+        return CNT_ERR_HIP;
+    }
+    *out = h;
+    return CNT_OK;
+}
+
+int cnt_lstm_destroy(cnt_lstm *h) {
+    if (!h) return CNT_OK;
+    for (int dir = 0; dir < 2; ++dir) {
+        for (int w = 0; w < 12; ++w)
+            if (h->state[dir][w]) (void)hipFree(h->state[dir][w]);
+        if (h->mailbox[dir]) (void)hipFree(h->mailbox[dir]);
+    }
+    if (h->abort_flag) (void)hipFree(h->abort_flag);
+    delete h;
+    return CNT_OK;
+}
+
+int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int curMaxT, int curMinT) {
+    using namespace cnt;
+    CNT_REQUIRE(h && patTypes, "lstm_load_sequences: null argument");
+    CNT_REQUIRE(curMaxT >= 1 && curMaxT <= h->desc.maxT, "lstm_load_sequences: curMaxT %d outside 1..%d", curMaxT,
+                h->desc.maxT);
+    CNT_REQUIRE(curMinT >= 0 && curMinT <= curMaxT, "lstm_load_sequences: curMinT %d outside 0..%d", curMinT, curMaxT);
+    h->T = curMaxT; h->Tmin = curMinT; h->pat = patTypes;
+    const size_t nstate = (size_t)h->H * h->desc.maxT * h->desc.S;
+    for (int dir = 0; dir < h->ndir; ++dir)
+        CNT_TRY(fill_zero(static_cast<hipStream_t>(stream), h->state[dir][10], nstate));
+    return CNT_OK;
+}
+
+float *cnt_lstm_state(cnt_lstm *h, int dir, int which) {
+    if (!h || dir < 0 || dir >= h->ndir || which < 0 || which >= 12) return nullptr;
+    return h->state[dir][which];
+}
+
+int cnt_lstm_check(cnt_lstm *h, void *stream) {
+    using namespace cnt;
+    CNT_REQUIRE(h, "lstm_check: null handle");
+    int flag = 0;
+    CNT_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    CNT_HIP(hipMemcpy(&flag, h->abort_flag, sizeof(int), hipMemcpyDeviceToHost));
+    if (flag != 0) {
+        CNT_HIP(hipMemset(h->abort_flag, 0, sizeof(int)));
+        set_error("lstm: a recursion kernel gave up waiting for a neighbouring workgroup; results are invalid");
+        return CNT_ERR_DEVICE;
+    }
+    return CNT_OK;
+}
+
+int cnt_lstm_forward(cnt_lstm *h, void *stream_, const float *weights, const float *x, float *outputs) {
+    using namespace cnt;
+    CNT_REQUIRE(h && weights && x && outputs, "lstm_forward: null argument");
+    CNT_REQUIRE(h->T > 0, "lstm_forward: load_sequences has not been called");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const cnt_lstm_desc &d = h->desc;
+    const int P = d.P, L = d.L, H = h->H, N = h->T * d.S;
+
+    // input projections of all gates and directions in one launch: a_g = W_in[g]^T x
+    GemmArgs ga = {};
+    ga.m = H; ga.n = N; ga.k = P;
+    ga.a_kcontig = 1; ga.lda = P;  // W_in block is P x H column-major: element (unit, p) at [unit*P + p]
+    ga.b_kcontig = 1; ga.ldb = P;
+    ga.ldc = H;
+    ga.nseg = 1; ga.splitk = 1; ga.epilogue = EPI_STORE;
+    ga.nprob = 4 * h->ndir;
+    for (int dir = 0; dir < h->ndir; ++dir)
+        for (int g = 0; g < 4; ++g) {
+            GemmProblem &pb = ga.prob[dir * 4 + g];
+            pb.A[0] = weights + (size_t)g * P * L + (size_t)dir * P * H;
+            pb.B[0] = x;
+            pb.C = h->state[dir][g];
+        }
+    CNT_TRY(gemm_launch(stream, ga));
+
+    ChainParams p;
+    fill_chain_params(h, weights, p);
+    // the reference lets a unidirectional layer write its outputs directly (buffer swap, :1747-1749)
+    p.out = outputs;
+    return launch_chain(h, stream, true, p);
+}
+
+int cnt_lstm_backward(cnt_lstm *h, void *stream_, const float *weights, const float *x, const float *outputs,
+                      float *output_errors, float *prev_errors, float *weight_updates) {
+    using namespace cnt;
+    CNT_REQUIRE(h && weights && x && outputs && output_errors && weight_updates, "lstm_backward: null argument");
+    CNT_REQUIRE(h->T > 0, "lstm_backward: load_sequences has not been called");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const cnt_lstm_desc &d = h->desc;
+    const int P = d.P, L = d.L, H = h->H, S = d.S, N = h->T * S;
+    (void)outputs;
+
+    // 1. error recursion (splits the interleaved output errors on the fly)
+    ChainParams p;
+    fill_chain_params(h, weights, p);
+    p.outerr = output_errors;
+    p.herr_out = (h->ndir == 1) ? output_errors : nullptr;
+    CNT_TRY(launch_chain(h, stream, false, p));
+
+    // 2. error to the preceding layer: e_x = sum_{dir,g} W_in[g,dir] * delta[g,dir]  (overwrite)
+    if (prev_errors) {
+        GemmArgs ga = {};
+        ga.m = P; ga.n = N; ga.k = H;
+        ga.a_kcontig = 0; ga.lda = P;
+        ga.b_kcontig = 1; ga.ldb = H;
+        ga.ldc = P;
+        ga.nseg = 4 * h->ndir; ga.nprob = 1; ga.splitk = 1; ga.epilogue = EPI_STORE;
+        for (int dir = 0; dir < h->ndir; ++dir)
+            for (int g = 0; g < 4; ++g) {
+                ga.prob[0].A[dir * 4 + g] = weights + (size_t)g * P * L + (size_t)dir * P * H;
+                ga.prob[0].B[dir * 4 + g] = h->state[dir][7 + g];
+            }
+        ga.prob[0].C = prev_errors;
+        CNT_TRY(gemm_launch(stream, ga));
+    }
+
+    // 3. weight updates (overwritten every call, as the reference's transform-assign does)
+    const size_t nW = weight_count(P, L, d.bidir);
+    CNT_TRY(fill_zero(stream, weight_updates, nW));
+    const size_t off_bias = (size_t)4 * P * L, off_int = off_bias + (size_t)4 * L;
+    const size_t off_peep = off_int + (size_t)4 * L * H;
+    auto split_for = [](int tiles, int k) {
+        int s = (512 + tiles - 1) / tiles;
+        const int kt = (k + 15) / 16;
+        if (s > kt) s = kt;
+        if (s < 1) s = 1;
+        return s;
+    };
+    {
+        // input weights: dW_in[g,dir] (P x H) = x (P x N) * delta^T
+        GemmArgs ga = {};
+        ga.m = P; ga.n = H; ga.k = N;
+        ga.a_kcontig = 0; ga.lda = P;
+        ga.b_kcontig = 0; ga.ldb = H;
+        ga.ldc = P;
+        ga.nseg = 1; ga.nprob = 4 * h->ndir; ga.epilogue = EPI_ATOMIC;
+        ga.splitk = split_for(((P + 127) / 128) * ((H + 127) / 128) * ga.nprob, N);
+        for (int dir = 0; dir < h->ndir; ++dir)
+            for (int g = 0; g < 4; ++g) {
+                GemmProblem &pb = ga.prob[dir * 4 + g];
+                pb.A[0] = x;
+                pb.B[0] = h->state[dir][7 + g];
+                pb.C = weight_updates + (size_t)g * P * L + (size_t)dir * P * H;
+            }
+        CNT_TRY(gemm_launch(stream, ga));
+    }
+    if (h->T > 1) {
+        // recurrent weights: dW_int[g,dir][src + to*H] = sum h[src] at the earlier step * delta[to]
+        GemmArgs ga = {};
+        ga.m = H; ga.n = H; ga.k = N - S;
+        ga.a_kcontig = 0; ga.lda = H;
+        ga.b_kcontig = 0; ga.ldb = H;
+        ga.ldc = H;
+        ga.nseg = 1; ga.nprob = 4 * h->ndir; ga.epilogue = EPI_ATOMIC;
+        ga.splitk = split_for(((H + 127) / 128) * ((H + 127) / 128) * ga.nprob, N - S);
+        for (int dir = 0; dir < h->ndir; ++dir)
+            for (int g = 0; g < 4; ++g) {
+                GemmProblem &pb = ga.prob[dir * 4 + g];
+                const float *hbuf = h->state[dir][5];
+                const float *dl = h->state[dir][7 + g];
+                // forward states pair delta[t] with h[t-1]; backward states pair delta[t] with h[t+1]
+                pb.A[0] = dir ? hbuf + (size_t)S * H : hbuf;
+                pb.B[0] = dir ? dl : dl + (size_t)S * H;
+                pb.C = weight_updates + off_int + (size_t)g * L * H + (size_t)dir * H * H;
+            }
+        CNT_TRY(gemm_launch(stream, ga));
+    }
+    for (int dir = 0; dir < h->ndir; ++dir) {
+        SmallGradParams sp;
+        sp.H = H; sp.L = L; sp.S = S; sp.N = N; sp.bias = d.bias;
+        sp.dni = h->state[dir][7]; sp.dig = h->state[dir][8]; sp.dfg = h->state[dir][9]; sp.dog = h->state[dir][10];
+        sp.c = h->state[dir][4];
+        sp.g_bias = weight_updates + off_bias + dir * H;
+        sp.g_peep = weight_updates + off_peep + dir * H;
+        sp.dir = dir;
+        sp.chunk = 32;
+        dim3 grid((H + 255) / 256, (N + sp.chunk - 1) / sp.chunk);
+        hipLaunchKernelGGL(lstm_small_grads, grid, dim3(256), 0, stream, sp);
+        CNT_HIP(hipGetLastError());
+    }
+    return CNT_OK;
+}
+
+}  // extern "C"

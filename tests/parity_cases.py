@@ -1,0 +1,203 @@
+"""Shared GPU-vs-oracle parity drivers.  Each function builds seeded inputs, runs the CPU oracle and the
+HIP library (through its C ABI) on the same data and returns the worst L2-normalised error over all
+compared tensors; index / masking properties are asserted bit-exactly on the way."""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+import oracle_lib as O  # noqa: E402
+from torch_models import make_pat_types  # noqa: E402
+
+
+def pkg():
+    from __graft_entry__ import load_package
+
+    return load_package()
+
+
+def relerr(a, b):
+    a = np.asarray(a, dtype=np.float64).ravel()
+    b = np.asarray(b, dtype=np.float64).ravel()
+    d = np.linalg.norm(b)
+    if d == 0:
+        return float(np.linalg.norm(a))
+    return float(np.linalg.norm(a - b) / d)
+
+
+def dev(a):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def lstm_inputs(P, L, bidir, S, T, lengths, seed, wscale=0.1, escale=0.1):
+    rng = np.random.default_rng(seed)
+    nW = O.lib().orc_lstm_weight_count(P, L, int(bidir))
+    W = rng.uniform(-wscale, wscale, nW).astype(np.float32)
+    x = rng.standard_normal((T, S, P)).astype(np.float32)
+    outerr = (escale * rng.standard_normal((T, S, L))).astype(np.float32)
+    for s, n in enumerate(lengths):
+        x[n:, s] = 0
+        outerr[n:, s] = 0
+    return W, x.reshape(-1), outerr.reshape(-1)
+
+
+def run_lstm_case(P, L, bidir, lengths, seed, wscale=0.1, escale=0.1, bias=1.0, repeat_backward=False,
+                  tol=1e-4, verbose=False):
+    import torch
+
+    capi = pkg().capi
+    S, T = len(lengths), max(lengths)
+    nd = 2 if bidir else 1
+    H = L // nd
+    N = T * S
+    W, x, outerr = lstm_inputs(P, L, bidir, S, T, lengths, seed, wscale, escale)
+    pat = make_pat_types(lengths, T)
+
+    # ---- oracle
+    desc = O.LstmDesc(P, L, int(bidir), S, T, min(lengths), bias)
+    fw = O.LstmState(H, N)
+    bw = O.LstmState(H, N) if bidir else None
+    out_o = np.zeros(L * N, dtype=np.float32)
+    O.lstm_forward(desc, W, pat, x, fw, bw, out_o)
+    ex_o = np.zeros(P * N, dtype=np.float32)
+    dW_o = np.zeros_like(W)
+    O.lstm_backward(desc, W, pat, x, outerr, fw, bw, ex_o, dW_o)
+    if repeat_backward:
+        O.lstm_backward(desc, W, pat, x, outerr, fw, bw, ex_o, dW_o)
+
+    # ---- HIP library
+    Wd, xd, pd = dev(W), dev(x), dev(pat)
+    out_d = torch.zeros(L * N, dtype=torch.float32, device="cuda")
+    err_d = dev(outerr)
+    ex_d = torch.full((P * N,), 7.0, dtype=torch.float32, device="cuda")  # must be overwritten
+    dW_d = torch.full((len(W),), 7.0, dtype=torch.float32, device="cuda")
+    layer = capi.Lstm(P, L, bidir, S, T, bias)
+    layer.load_sequences(pd, T, min(lengths))
+    layer.forward(Wd, xd, out_d)
+    layer.check()
+    layer.backward(Wd, xd, out_d, err_d, ex_d, dW_d)
+    layer.check()
+    if repeat_backward:
+        # no load_sequences in between: the stored output-gate deltas are added (read-modify-write)
+        err_d = dev(outerr)
+        layer.backward(Wd, xd, out_d, err_d, ex_d, dW_d)
+        layer.check()
+    torch.cuda.synchronize()
+
+    worst = 0.0
+    report = {}
+
+    def cmp(name, got, want):
+        nonlocal worst
+        e = relerr(got, want)
+        report[name] = e
+        worst = max(worst, e)
+
+    cmp("outputs", out_d.cpu().numpy(), out_o)
+    cmp("prev_errors", ex_d.cpu().numpy(), ex_o)
+    dW_g = dW_d.cpu().numpy()
+    o_b = 4 * P * L
+    o_i = o_b + 4 * L
+    o_p = o_i + 4 * L * H
+    for nm, lo, hi in [("dW_input", 0, o_b), ("dW_bias", o_b, o_i), ("dW_internal", o_i, o_p),
+                       ("dW_peephole", o_p, len(W))]:
+        cmp(nm, dW_g[lo:hi], dW_o[lo:hi])
+    dummy = (pat == 0)
+    for d, st in enumerate([fw] + ([bw] if bidir else [])):
+        for k in ("ni", "ig", "fg", "og", "c", "h", "dni", "dig", "dfg", "dog", "cerr"):
+            got = layer.state(d, k).cpu().numpy()
+            want = st[k]
+            if k in ("ni", "ig", "fg", "og", "c"):
+                # padding slots hold leftovers of the projection in both implementations; compare valid slots
+                got = got.reshape(N, H)[~dummy]
+                want = want.reshape(N, H)[~dummy]
+            cmp("dir%d.%s" % (d, k), got, want)
+        # masking is exact: padding slots hold exact zeros in outputs, deltas and cell errors
+        if dummy.any():
+            for k in ("h", "dni", "dig", "dfg", "dog", "cerr"):
+                assert not layer.state(d, k).cpu().numpy().reshape(N, H)[dummy].any(), "mask leak in " + k
+    if dummy.any():
+        assert not out_d.cpu().numpy().reshape(N, L)[dummy].any()
+        assert not ex_d.cpu().numpy().reshape(N, P)[dummy].any()
+    if not bidir:
+        # the recurrent terms are left in the caller's error buffer, as the reference's swap leaves them
+        cmp("output_errors_inplace", err_d.cpu().numpy(), fw["herr"])
+    layer.close()
+    if verbose or worst > tol:
+        for k, v in sorted(report.items(), key=lambda kv: -kv[1])[:8]:
+            print("   %-26s %.3e" % (k, v))
+    return worst
+
+
+def run_gemm_case(m, n, k, tA, tB, accumulate, seed):
+    import torch
+
+    capi = pkg().capi
+    rng = np.random.default_rng(seed)
+    A = rng.standard_normal(m * k).astype(np.float32)
+    B = rng.standard_normal(k * n).astype(np.float32)
+    C0 = rng.standard_normal(m * n).astype(np.float32)
+    want = C0.copy()
+    O.mat_product(want, m, n, k, A, tA, B, tB, accumulate)
+    Cd = dev(C0)
+    capi.matrix_product(Cd, m, n, k, dev(A), tA, dev(B), tB, accumulate)
+    torch.cuda.synchronize()
+    return relerr(Cd.cpu().numpy(), want)
+
+
+def run_dense_case(P, D, N, act, bias, seed, lengths_frac=0.8):
+    import torch
+
+    capi = pkg().capi
+    rng = np.random.default_rng(seed)
+    W = rng.uniform(-0.1, 0.1, P * D + D).astype(np.float32)
+    x = rng.standard_normal(P * N).astype(np.float32)
+    err = (0.1 * rng.standard_normal(D * N)).astype(np.float32)
+    y_o = np.zeros(D * N, dtype=np.float32)
+    O.dense_forward(P, D, N, act, bias, W, x, y_o)
+    err_o = err.copy()
+    ex_o = np.zeros(P * N, dtype=np.float32)
+    dW_o = np.zeros_like(W)
+    O.dense_backward(P, D, N, act, bias, W, x, y_o, err_o, ex_o, dW_o)
+
+    Wd, xd = dev(W), dev(x)
+    y_d = torch.zeros(D * N, dtype=torch.float32, device="cuda")
+    capi.dense_forward(P, D, N, act, bias, Wd, xd, y_d)
+    err_d = dev(err)
+    ex_d = torch.full((P * N,), 3.0, dtype=torch.float32, device="cuda")
+    dW_d = torch.full((len(W),), 3.0, dtype=torch.float32, device="cuda")
+    capi.dense_backward(P, D, N, act, bias, Wd, xd, y_d, err_d, ex_d, dW_d)
+    torch.cuda.synchronize()
+    worst = 0.0
+    for got, want in [(y_d, y_o), (err_d, err_o), (ex_d, ex_o), (dW_d[:P * D], dW_o[:P * D]), (dW_d[P * D:], dW_o[P * D:])]:
+        worst = max(worst, relerr(got.cpu().numpy(), want))
+    return worst
+
+
+def run_sse_case(D, lengths, seed):
+    import torch
+
+    capi = pkg().capi
+    S, T = len(lengths), max(lengths)
+    N = T * S
+    rng = np.random.default_rng(seed)
+    y = rng.standard_normal(D * N).astype(np.float32)
+    tgt = rng.standard_normal(D * N).astype(np.float32)
+    pat = make_pat_types(lengths, T)
+    err_o = np.zeros(D * N, dtype=np.float32)
+    O.sse_backward(D, N, pat, y, tgt, err_o)
+    e_o = O.sse_error(D, N, pat, y, tgt)
+    err_d = torch.full((D * N,), 5.0, dtype=torch.float32, device="cuda")
+    res = torch.zeros(1, dtype=torch.float32, device="cuda")
+    capi.sse_backward(D, N, dev(pat), dev(y), dev(tgt), err_d)
+    capi.sse_error(D, N, dev(pat), dev(y), dev(tgt), res)
+    torch.cuda.synchronize()
+    # elementwise subtraction and masking are exact
+    assert np.array_equal(err_d.cpu().numpy(), err_o)
+    return abs(float(res.item()) - e_o) / max(abs(e_o), 1e-30)

@@ -1,0 +1,35 @@
+"""CPU-only: the C-ABI library loads and exports every symbol the public header declares."""
+import ctypes
+import os
+import re
+
+from __graft_entry__ import ROOT, load_package
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "currennt_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cnt_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_header_symbols():
+    capi = load_package().capi
+    assert os.path.exists(capi.LIB_PATH), "build the library first: python __graft_entry__.py"
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    names = declared_symbols()
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), "missing export " + n
+    # the ctypes binding covers the same set
+    assert sorted(capi.exported_symbols()) == names
+
+
+def test_version_and_argument_errors_without_gpu():
+    capi = load_package().capi
+    L = capi.lib()
+    assert L.cnt_version() >= 1
+    # argument validation happens before any device call
+    assert L.cnt_matrix_product(None, None, 1, 1, 1, None, 0, None, 0, 0) == 1
+    assert b"null" in L.cnt_last_error()
+    assert L.cnt_lstm_weight_count(382, 256, 0) == 655104
+    assert L.cnt_lstm_weight_count(512, 512, 1) == 1576448
