@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the backward hot path on one MI355X.
+
+Workload: BASELINE config 2, the acoustic model 382 -> 2 x feedforward_tanh 512 -> 2 x blstm 512
+(256 cells per direction) -> feedforward_identity 187 -> sse, T = 600 frames, 10 parallel sequences
+with lengths U{300..600}, fp32, synthetic seeded data, weights U(-0.08, 0.08).
+
+A step is one full backward pass of the network over the resident fraction (all inputs, states and
+weights already in HBM): per-fraction clearing of the stored output-gate deltas, SSE error, dense and
+BLSTM backward including every weight gradient.  `value` is valid frames per second of that pass.
+The forward pass that produces the states is run before the timed region (and timed separately as
+`forward_backward_ms`).
+
+Prints ONE JSON line.  Besides the contract fields it carries
+  roofline      for the kernel family with the largest share of the step, measured live with HIP events
+                on the launch stream (cnt_profile_enable) over a second run of the same K steps;
+  cpu_baseline  the CPU oracle (a sequential restatement of the reference's host path, 1 core) timed on a
+                bounded sample of the same network.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+METRIC = "BLSTM backward frames/sec at 1 MI355X; % HBM/MFMA roofline vs host CPU"
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def make_fraction(seed, S, Tmax, Tlo, in_dim, out_dim):
+    rng = np.random.default_rng(seed)
+    lengths = [int(v) for v in rng.integers(Tlo, Tmax + 1, size=S)]
+    T = max(lengths)
+    x = rng.standard_normal((T, S, in_dim)).astype(np.float32)
+    tgt = rng.standard_normal((T, S, out_dim)).astype(np.float32)
+    pat = np.zeros((T, S), dtype=np.int8)
+    for s, n in enumerate(lengths):
+        x[n:, s] = 0
+        tgt[n:, s] = 0
+        pat[:n, s] = 2
+        pat[0, s] = 1
+        pat[n - 1, s] = 3
+    return lengths, T, x.reshape(-1), tgt.reshape(-1), pat.reshape(-1)
+
+
+def backward_flops_per_slot(input_size, specs):
+    """Algorithmic multiply-add flops of one backward pass per (t, s) slot."""
+    fl, prev = 0.0, input_size
+    for i, sp in enumerate(specs):
+        t, D = sp["type"], sp["size"]
+        if t.startswith("feedforward"):
+            fl += 2.0 * prev * D * (1 if i == 0 else 2)  # dW always, dX unless it feeds the input layer
+        elif t in ("lstm", "blstm"):
+            nd = 2 if t == "blstm" else 1
+            H = D // nd
+            # recurrent 8H^2 + dW_int 8H^2 + dW_in 8HP + e_x 8HP per direction
+            fl += nd * (16.0 * H * H + 16.0 * H * prev)
+        prev = D
+    return fl
+
+
+def cpu_baseline(input_size, specs, S, seed, sample_T):
+    """Times the oracle's backward on a short fraction of the same network (one core, sequential)."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_models as OM
+
+    lengths, T, x, tgt, pat = make_fraction(seed, S, sample_T, max(1, sample_T // 2), input_size, specs[-1]["size"])
+    weights = OM.init_weights(input_size, specs, seed + 1, 0.08)
+    net = OM.OracleNetwork(input_size, specs, S, T, min(lengths), pat, weights)
+    net.forward(x, tgt)
+    t0 = time.perf_counter()
+    net.backward()
+    dt = time.perf_counter() - t0
+    frames = sum(lengths)
+    return {
+        "value": frames / dt, "unit": "frames/s", "cores": 1, "kind": "port",
+        "sample": "same network and weights distribution, one backward pass of a fraction with T=%d, S=%d "
+                  "(%d valid frames, %.1f s); CPU oracle = sequential restatement of the reference's Thrust-host "
+                  "path (naive k-ordered products, one loop per weight), g++ -O2, host has %d cores"
+                  % (T, S, frames, dt, os.cpu_count() or 0),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--cpu-sample-T", type=int, default=160)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path has no multi-GPU part); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from __graft_entry__ import load_package
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    pkg = load_package()
+    capi, networks = pkg.capi, pkg.networks
+
+    S, Tmax, seed = 10, 600, 20240
+    input_size, specs = networks.acoustic_model_spec()
+    lengths, T, x, tgt, pat = make_fraction(seed, S, Tmax, 300, input_size, 187)
+    frames = sum(lengths)
+
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    net = networks.StackedNetwork(input_size, specs, S, T)
+    # weights: seeded U(-0.08, 0.08), generated on the host with the same generator the parity tests use
+    rng = np.random.default_rng(seed + 1)
+    weights, prev = [], input_size
+    for sp in specs:
+        n = networks.layer_weight_count(sp, prev)
+        if n:
+            weights.append(rng.uniform(-0.08, 0.08, n).astype(np.float32))
+        prev = sp["size"]
+    net.set_weights(weights)
+    pat_d = torch.from_numpy(pat).cuda()
+    net.load_sequences(pat_d, T, min(lengths), torch.from_numpy(x).cuda(), torch.from_numpy(tgt).cuda())
+    net.forward()
+    net.check()
+
+    def step():
+        net.load_sequences(pat_d, T, min(lengths))  # per-fraction clearing of the stored output-gate deltas
+        net.backward()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    net.check()
+    ms_per_step = 1e3 * dt / args.steps
+    value = frames * args.steps / dt
+
+    # forward + backward, for information
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        net.load_sequences(pat_d, T, min(lengths))
+        net.forward()
+        net.backward()
+    torch.cuda.synchronize()
+    fb_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+
+    # per-kernel durations over the same K steps, HIP events on the launch stream
+    capi.profile_enable(True)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    prof = capi.profile_read()
+    capi.profile_enable(False)
+    net.check()
+    kernels = {k: {"launches": n, "avg_ms": ms / max(n, 1), "ms_per_step": ms / args.steps}
+               for k, (n, ms) in prof.items()}
+    dom = max(kernels, key=lambda k: kernels[k]["ms_per_step"])
+    dom_avg_s = kernels[dom]["avg_ms"] * 1e-3
+
+    H = 256
+    slots = T * S
+    if dom == "lstm_backward_chain":
+        # one launch = both directions of one BLSTM layer over all T*S slots; the only dense work on the
+        # recursion is the recurrent product, 8*H^2 flops per slot and direction
+        flops = 2 * 8.0 * H * H * slots
+        roof = {"bound": "mfma", "achieved": flops / dom_avg_s / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS,
+                "unit": "TFLOP/s", "traffic": None,
+                "kernel": dom,
+                "note": "latency-bound recursion: T sequential steps, each a 256x1024x%d product spread over "
+                        "32 workgroups per direction plus one mailbox round trip" % S}
+    elif dom.startswith("gemm"):
+        flops = backward_flops_per_slot(input_size, specs) * slots / max(1, len([k for k in kernels if k.startswith("gemm")]))
+        roof = {"bound": "mfma", "achieved": flops / dom_avg_s / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS,
+                "unit": "TFLOP/s", "traffic": None, "kernel": dom}
+    else:
+        nbytes = 40.0 * H * slots
+        roof = {"bound": "hbm", "achieved": nbytes / dom_avg_s / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "traffic": None, "kernel": dom}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+
+    step_flops = backward_flops_per_slot(input_size, specs) * slots
+    out = {
+        "metric": METRIC, "value": value, "unit": "frames/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: acoustic model 382-512t-512t-blstm512-blstm512-187 + sse, full backward "
+                               "pass, T=%d, S=%d, lengths U{300..600}, %d valid frames" % (T, S, frames),
+                   "T": T, "parallel_sequences": S, "valid_frames": frames},
+        "roofline": roof,
+        "step_roofline": {"bound": "mfma", "achieved": step_flops / (ms_per_step * 1e-3) / 1e12,
+                          "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                          "frac": step_flops / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+                          "flops_per_slot": backward_flops_per_slot(input_size, specs)},
+        "forward_backward_ms": fb_ms,
+        "kernels": kernels,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(input_size, specs, S, seed, args.cpu_sample_T)
+    net.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -28,6 +28,14 @@ enum { CNT_ACT_IDENTITY = 0, CNT_ACT_TANH = 1, CNT_ACT_LOGISTIC = 2, CNT_ACT_REL
 int cnt_version(void);
 const char *cnt_last_error(void);
 
+/* ---- per-kernel timing ----------------------------------------------------------------------------
+ * The reference has no profiler hooks (it prints wall-clock per epoch, currennt/src/main.cpp:302-317).
+ * cnt_profile_enable(1) clears earlier records and makes every launch site bracket its kernels with
+ * HIP events on the launch stream; cnt_profile_get(i, ...) waits for the events and returns the i-th
+ * label (order of first use), its launch count and summed duration in ms, or CNT_ERR_ARG past the end. */
+int cnt_profile_enable(int on);
+int cnt_profile_get(int index, char *label, int label_cap, int *launches, float *total_ms);
+
 /* ---- helpers::Matrix product seam -------------------------------------------------------------
  * Replaces helpers::Matrix<Gpu>::assignProduct / addProduct (helpers/Matrix.cu:353-377, which call
  * cublas::multiplyMatrices, helpers/cublas.cu:52-84).  Column-major, C is m x n, inner size k.

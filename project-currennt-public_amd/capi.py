@@ -27,6 +27,8 @@ F = C.c_float
 _SIGNATURES = {
     "cnt_version": (I, []),
     "cnt_last_error": (C.c_char_p, []),
+    "cnt_profile_enable": (I, [I]),
+    "cnt_profile_get": (I, [I, C.c_char_p, I, C.POINTER(I), C.POINTER(F)]),
     "cnt_matrix_product": (I, [VP, VP, I, I, I, VP, I, VP, I, I]),
     "cnt_dense_forward": (I, [VP, I, I, I, I, F, VP, VP, VP]),
     "cnt_dense_backward": (I, [VP, I, I, I, I, F, VP, VP, VP, VP, VP, VP]),
@@ -79,6 +81,24 @@ def stream_ptr(stream=None):
 
     s = stream if stream is not None else torch.cuda.current_stream()
     return C.c_void_p(s.cuda_stream)
+
+
+def profile_enable(on):
+    check(lib().cnt_profile_enable(int(on)))
+
+
+def profile_read():
+    """{label: (launches, total_ms)} of everything recorded since profile_enable(True)."""
+    out = {}
+    i = 0
+    while True:
+        buf = C.create_string_buffer(128)
+        n, ms = I(0), F(0.0)
+        if lib().cnt_profile_get(i, buf, 128, C.byref(n), C.byref(ms)) != CNT_OK:
+            break
+        out[buf.value.decode()] = (n.value, ms.value)
+        i += 1
+    return out
 
 
 def matrix_product(Cm, m, n, k, A, tA, B, tB, accumulate, stream=None):

@@ -95,6 +95,16 @@ __device__ __forceinline__ float act_deriv(int act, float y) {
     }
 }
 
+// ----- optional per-kernel timing (capi.hip) -------------------------------------------------------
+// When enabled through cnt_profile_enable, every ProfileScope brackets the launches made inside it
+// with a pair of HIP events on the launch stream; cnt_profile_get sums them per label.
+struct ProfileScope {
+    ProfileScope(hipStream_t stream, const char *label);
+    ~ProfileScope();
+    hipStream_t stream_;
+    int slot_;
+};
+
 // ----- GEMM (gemm.hip) ------------------------------------------------------------------------------
 // C (m x n, column-major, ldc) = sum over segments of opA(A_i) * opB(B_i), optionally added to C.
 // An operand is described by where element (row, kk) lives: row-contiguous (ptr[kk*ld + row]) or
@@ -119,6 +129,7 @@ struct GemmArgs {
     int epilogue, act;
     float bias_scale;
     GemmProblem prob[kGemmMaxProb];
+    const char *label;  // name under which the launch is timed when profiling is on (may be NULL)
 };
 
 int gemm_launch(hipStream_t stream, const GemmArgs &args);

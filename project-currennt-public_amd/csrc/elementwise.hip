@@ -98,6 +98,7 @@ int cnt_dense_forward(void *stream_, int P, int D, int N, int act, float bias, c
     ga.epilogue = EPI_BIAS_ACT; ga.act = act; ga.bias_scale = bias;
     ga.prob[0].A[0] = weights; ga.prob[0].B[0] = x; ga.prob[0].C = y;
     ga.prob[0].bias_vec = weights + (size_t)P * D;
+    ga.label = "gemm:dense_forward";
     return gemm_launch(static_cast<hipStream_t>(stream_), ga);
 }
 
@@ -113,7 +114,17 @@ int cnt_dense_backward(void *stream_, int P, int D, int N, int act, float bias, 
         hipLaunchKernelGGL(dense_delta_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, err, y, count, act);
         CNT_HIP(hipGetLastError());
     }
-    if (prev_err) CNT_TRY(gemm_simple(stream, prev_err, P, N, D, weights, false, err, false, false));
+    if (prev_err) {
+        GemmArgs ga = {};
+        ga.m = P; ga.n = N; ga.k = D;
+        ga.a_kcontig = 0; ga.lda = P;
+        ga.b_kcontig = 1; ga.ldb = D;
+        ga.ldc = P;
+        ga.nseg = 1; ga.nprob = 1; ga.splitk = 1; ga.epilogue = EPI_STORE;
+        ga.prob[0].A[0] = weights; ga.prob[0].B[0] = err; ga.prob[0].C = prev_err;
+        ga.label = "gemm:dense_prev_errors";
+        CNT_TRY(gemm_launch(stream, ga));
+    }
     CNT_TRY(fill_zero(stream, weight_updates, (size_t)P * D + D));
     {
         GemmArgs ga = {};
@@ -127,6 +138,7 @@ int cnt_dense_backward(void *stream_, int P, int D, int N, int act, float bias, 
         const int kt = (N + 15) / 16;
         ga.splitk = s > kt ? kt : s;
         ga.prob[0].A[0] = x; ga.prob[0].B[0] = err; ga.prob[0].C = weight_updates;
+        ga.label = "gemm:dense_dW";
         CNT_TRY(gemm_launch(stream, ga));
     }
     return column_sum(stream, err, D, N, bias, weight_updates + (size_t)P * D);

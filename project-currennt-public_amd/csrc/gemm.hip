@@ -262,6 +262,7 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args) {
     const int va = pick_vec(args, true), vb = pick_vec(args, false);
     const int tiles = ((args.m + BM - 1) / BM) * ((args.n + BN - 1) / BN);
     dim3 grid(tiles, args.splitk, args.nprob);
+    ProfileScope prof(stream, args.label ? args.label : "gemm");
     if (va == 4) launch_ak<4>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig);
     else if (va == 2) launch_ak<2>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig);
     else launch_ak<1>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig);

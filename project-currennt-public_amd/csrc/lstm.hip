@@ -539,6 +539,7 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     CNT_TRY(next_epoch(h, stream, p.tag_base));
     const int G = h->H / h->JB;
     const int blocks = h->xcd_pack ? 8 * G : h->ndir * G;
+    ProfileScope prof(stream, fwd ? "lstm_forward_chain" : "lstm_backward_chain");
     hipLaunchKernelGGL(k, dim3(blocks), dim3(kThreads), 0, stream, p);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
@@ -666,6 +667,7 @@ int cnt_lstm_forward(cnt_lstm *h, void *stream_, const float *weights, const flo
             pb.B[0] = x;
             pb.C = h->state[dir][g];
         }
+    ga.label = "gemm:lstm_input_projection";
     CNT_TRY(gemm_launch(stream, ga));
 
     ChainParams p;
@@ -706,6 +708,7 @@ int cnt_lstm_backward(cnt_lstm *h, void *stream_, const float *weights, const fl
                 ga.prob[0].B[dir * 4 + g] = h->state[dir][7 + g];
             }
         ga.prob[0].C = prev_errors;
+        ga.label = "gemm:lstm_prev_errors";
         CNT_TRY(gemm_launch(stream, ga));
     }
 
@@ -737,6 +740,7 @@ int cnt_lstm_backward(cnt_lstm *h, void *stream_, const float *weights, const fl
                 pb.B[0] = h->state[dir][7 + g];
                 pb.C = weight_updates + (size_t)g * P * L + (size_t)dir * P * H;
             }
+        ga.label = "gemm:lstm_dW_input";
         CNT_TRY(gemm_launch(stream, ga));
     }
     if (h->T > 1) {
@@ -758,6 +762,7 @@ int cnt_lstm_backward(cnt_lstm *h, void *stream_, const float *weights, const fl
                 pb.B[0] = dir ? dl : dl + (size_t)S * H;
                 pb.C = weight_updates + off_int + (size_t)g * L * H + (size_t)dir * H * H;
             }
+        ga.label = "gemm:lstm_dW_internal";
         CNT_TRY(gemm_launch(stream, ga));
     }
     for (int dir = 0; dir < h->ndir; ++dir) {
@@ -770,6 +775,7 @@ int cnt_lstm_backward(cnt_lstm *h, void *stream_, const float *weights, const fl
         sp.dir = dir;
         sp.chunk = 32;
         dim3 grid((H + 255) / 256, (N + sp.chunk - 1) / sp.chunk);
+        ProfileScope prof(stream, "lstm_small_grads");
         hipLaunchKernelGGL(lstm_small_grads, grid, dim3(256), 0, stream, sp);
         CNT_HIP(hipGetLastError());
     }

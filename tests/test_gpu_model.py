@@ -1,0 +1,70 @@
+"""GPU parity of the whole acoustic model of BASELINE config 2 (382 -> 512t -> 512t -> blstm512 -> blstm512
+-> 187 -> sse) against the CPU oracle on a shortened fraction, every gradient tensor at 1e-4 (L2-normalised)."""
+import numpy as np
+import pytest
+
+import oracle_models as OM
+import parity_cases as PC
+
+pytestmark = pytest.mark.gpu
+
+
+def make_fraction(seed, S, Tmax, Tlo, in_dim, out_dim):
+    rng = np.random.default_rng(seed)
+    lengths = [int(v) for v in rng.integers(Tlo, Tmax + 1, size=S)]
+    T = max(lengths)
+    x = rng.standard_normal((T, S, in_dim)).astype(np.float32)
+    tgt = rng.standard_normal((T, S, out_dim)).astype(np.float32)
+    pat = np.zeros((T, S), dtype=np.int8)
+    for s, n in enumerate(lengths):
+        x[n:, s] = 0
+        tgt[n:, s] = 0
+        pat[:n, s] = 2
+        pat[0, s] = 1
+        pat[n - 1, s] = 3
+    return lengths, T, x.reshape(-1), tgt.reshape(-1), pat.reshape(-1)
+
+
+def test_acoustic_model_forward_backward():
+    import torch
+
+    print("acoustic model parity", flush=True)
+    networks = PC.pkg().networks
+    input_size, specs = networks.acoustic_model_spec()
+    S = 10
+    lengths, T, x, tgt, pat = make_fraction(7, S, 20, 10, input_size, 187)
+    weights = OM.init_weights(input_size, specs, 8, 0.08)
+
+    ref = OM.OracleNetwork(input_size, specs, S, T, min(lengths), pat, [w.copy() for w in weights])
+    ref.forward(x, tgt)
+    ref_loss = ref.error()
+    ref.backward()
+
+    net = networks.StackedNetwork(input_size, specs, S, T)
+    net.set_weights(weights)
+    pat_d = torch.from_numpy(pat).cuda()
+    net.load_sequences(pat_d, T, min(lengths), torch.from_numpy(x).cuda(), torch.from_numpy(tgt).cuda())
+    net.forward()
+    loss = float(net.calculate_error().item())
+    net.backward()
+    net.check()
+    torch.cuda.synchronize()
+
+    assert abs(loss - ref_loss) <= 1e-4 * abs(ref_loss)
+    N = T * S
+    worst = 0.0
+    for i, (g, r) in enumerate(zip(net.layers, ref.layers)):
+        if g["type"] == "sse":
+            continue
+        n = g["size"] * N
+        e = PC.relerr(g["outputs"][:n].cpu().numpy(), r["outputs"])
+        print("layer %d %-22s outputs %.2e" % (i, g["type"], e), flush=True)
+        worst = max(worst, e)
+        e = PC.relerr(g["updates"].cpu().numpy(), r["updates"])
+        print("layer %d %-22s updates %.2e" % (i, g["type"], e), flush=True)
+        worst = max(worst, e)
+        e = PC.relerr(g["errors"][:n].cpu().numpy(), r["errors"])
+        print("layer %d %-22s errors  %.2e" % (i, g["type"], e), flush=True)
+        worst = max(worst, e)
+    net.close()
+    assert worst < 1e-4
