@@ -27,6 +27,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <new>
+#include <vector>
 
 namespace cnt {
 namespace {
@@ -59,6 +60,7 @@ struct ChainParams {
     unsigned spin_limit;
     int *abort_flag;
     int xcd_pack;
+    long long *phase_ticks;  // optional diagnostic: per workgroup 4 accumulated phase durations (100 MHz ticks)
 };
 
 __device__ __forceinline__ u64 mb_load(const u64 *p) {
@@ -94,6 +96,16 @@ __device__ __forceinline__ bool mb_wait(const u64 *const (&addr)[N], float (&val
         val[q] = __uint_as_float((unsigned)w[q]);
     }
     return ok;
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
+// global load and store of the wave, which would put the HBM latency of the look-ahead loads and the
+// acknowledgement of the result stores on the recursion's critical path.  No thread of a workgroup
+// reads global data written by another thread of the same launch except through the mailbox.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 __device__ __forceinline__ bool map_block(const ChainParams &p, int G, int &dir, int &me) {
@@ -133,6 +145,9 @@ __global__ __launch_bounds__(kThreads) void lstm_forward_chain(const ChainParams
     const int n = S * H;
 
     __shared__ float red[kWaves][4 * JB][NS + 1];
+    __shared__ int wait_failed;
+    if (threadIdx.x == 0) wait_failed = 0;
+    lds_barrier();
 
     // recurrent weights as MFMA A operands: row (gate, cell), k = source cell
     float wA[MT][KS];
@@ -159,18 +174,28 @@ __global__ __launch_bounds__(kThreads) void lstm_forward_chain(const ChainParams
     }
     float c_prev = 0.0f;
 
+    // Pre-activations of the input projection do not depend on the recursion: they are requested one
+    // step ahead, right after the wait of the current step, so that their HBM latency is hidden
+    // behind the cell update and the next wait instead of stacking up in front of the mailbox polls.
+    struct StepIn { float a_ni, a_ig, a_fg, a_og; char pat; };  // pat is compared at use, not at load
+    auto load_step = [&](int step) {
+        StepIn v = {0, 0, 0, 0, 1};
+        if (cell_valid) {
+            const int t = dir ? (T - 1 - step) : step;
+            const size_t gi = (size_t)t * n + (size_t)cs * H + j0 + cj;
+            v.a_ni = D.ni[gi]; v.a_ig = D.ig[gi]; v.a_fg = D.fg[gi]; v.a_og = D.og[gi];
+            v.pat = p.pat[t * S + cs];
+        }
+        return v;
+    };
+    StepIn cur = load_step(0);
+
     for (int step = 0; step < T; ++step) {
         const int t = dir ? (T - 1 - step) : step;
         const bool first = (step == 0);
         const size_t gi = (size_t)t * n + (size_t)cs * H + j0 + cj;
-
-        // pre-activations from the input projection: independent of the recursion, issued early
-        float a_ni = 0, a_ig = 0, a_fg = 0, a_og = 0;
-        bool dummy = false;
-        if (cell_valid) {
-            a_ni = D.ni[gi]; a_ig = D.ig[gi]; a_fg = D.fg[gi]; a_og = D.og[gi];
-            dummy = (t >= p.Tmin) && (p.pat[t * S + cs] == 0);
-        }
+        float a_ni = cur.a_ni, a_ig = cur.a_ig, a_fg = cur.a_fg, a_og = cur.a_og;
+        const bool dummy = (t >= p.Tmin) && (cur.pat == 0);
 
         if (!first) {
             // gather h of the previous step straight into MFMA B operands
@@ -209,11 +234,15 @@ __global__ __launch_bounds__(kThreads) void lstm_forward_chain(const ChainParams
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
                         red[wave][mt * 16 + 4 * (lane >> 4) + r][nt * 16 + (lane & 15)] = acc[mt][nt][r];
-            if (__syncthreads_or(ok ? 0 : 1)) {
+            if (!ok) wait_failed = 1;
+            lds_barrier();
+            if (wait_failed) {
                 if (tid == 0) __hip_atomic_store(p.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 return;
             }
         }
+
+        if (step + 1 < T) cur = load_step(step + 1);
 
         if (cell_valid) {
             if (!first) {
@@ -253,7 +282,7 @@ __global__ __launch_bounds__(kThreads) void lstm_forward_chain(const ChainParams
             D.h[gi] = hval;
             if (p.out) p.out[((size_t)t * S + cs) * p.L + dir * H + j0 + cj] = hval;
         }
-        __syncthreads();  // `red` is rewritten in the next step
+        lds_barrier();  // `red` is rewritten in the next step
     }
 }
 
@@ -282,6 +311,9 @@ __global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParam
 
     __shared__ float psum[NPART][JB][NS + 1];
     __shared__ float dl[4 * JB][NS + 1];
+    __shared__ int wait_failed;
+    if (threadIdx.x == 0) wait_failed = 0;
+    lds_barrier();
 
     // recurrent weights as MFMA A operands: row = receiving ("from") cell, k = (gate, own cell)
     float wA[MT][KS];
@@ -307,23 +339,42 @@ __global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParam
     if (cell_valid) { p_ig = D.peep[0][j0 + cj]; p_fg = D.peep[1][j0 + cj]; p_og = D.peep[2][j0 + cj]; }
     // this cell's values at the slot processed in the previous iteration
     float fg_later = 0, cerr_later = 0, dig_later = 0, dfg_later = 0;
+    long long ph0 = 0, ph1 = 0, ph2 = 0, ph3 = 0;
+    const bool timing = p.phase_ticks != nullptr;
+
+    // Everything the cell update reads besides the recursion is requested one step ahead (cell states
+    // two steps ahead, because a step also needs the cell state of the slot processed next), right
+    // after the wait of the current step; see the forward kernel.
+    struct StepIn { float e, ni, ig, fg, og, dog_old; char pat; };
+    auto slot_of = [&](int step) { return dir ? step : (T - 1 - step); };
+    auto load_step = [&](int step) {
+        StepIn v = {0, 0, 0, 0, 0, 0, 1};
+        if (cell_valid) {
+            const int t = slot_of(step);
+            const size_t gi = (size_t)t * n + (size_t)cs * H + j0 + cj;
+            v.e = p.outerr[((size_t)t * S + cs) * p.L + dir * H + j0 + cj];
+            v.ni = D.ni[gi]; v.ig = D.ig[gi]; v.fg = D.fg[gi]; v.og = D.og[gi];
+            v.dog_old = D.dog[gi];
+            v.pat = p.pat[t * S + cs];
+        }
+        return v;
+    };
+    auto load_c = [&](int step) {
+        if (!cell_valid || step >= T) return 0.0f;
+        return D.c[(size_t)slot_of(step) * n + (size_t)cs * H + j0 + cj];
+    };
+    StepIn cur = load_step(0);
+    float c_cur = load_c(0), c_next = load_c(1);
 
     for (int step = 0; step < T; ++step) {
-        const int t = dir ? step : (T - 1 - step);
-        const int earlier = dir ? t + 1 : t - 1;
+        const long long tk0 = timing ? wall_clock64() : 0;
+        const int t = slot_of(step);
         const bool first = (step == 0), last = (step == T - 1);
         const size_t gi = (size_t)t * n + (size_t)cs * H + j0 + cj;
-
-        // everything that does not depend on the recursion is requested before the wait
-        float e = 0, ni = 0, ig = 0, fg = 0, og = 0, c = 0, c_earlier = 0, dog_old = 0;
-        bool dummy = false;
-        if (cell_valid) {
-            e = p.outerr[((size_t)t * S + cs) * p.L + dir * H + j0 + cj];
-            ni = D.ni[gi]; ig = D.ig[gi]; fg = D.fg[gi]; og = D.og[gi]; c = D.c[gi];
-            dog_old = D.dog[gi];
-            if (!last) c_earlier = D.c[(size_t)earlier * n + (size_t)cs * H + j0 + cj];
-            dummy = (t >= p.Tmin) && (p.pat[t * S + cs] == 0);
-        }
+        float e = cur.e;
+        const float ni = cur.ni, ig = cur.ig, fg = cur.fg, og = cur.og, dog_old = cur.dog_old;
+        const float c = c_cur, c_earlier = c_next;
+        const bool dummy = (t >= p.Tmin) && (cur.pat == 0);
 
         if (!first) {
             const unsigned tag = p.tag_base + (unsigned)step;
@@ -341,12 +392,18 @@ __global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParam
                 for (int q = 0; q < NPOLL; ++q) part_sum += v[q];
             }
             psum[part][pj][ps] = part_sum;
-            if (__syncthreads_or(ok ? 0 : 1)) {
+            if (!ok) wait_failed = 1;
+            lds_barrier();
+            if (wait_failed) {
                 if (tid == 0) __hip_atomic_store(p.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 return;
             }
         }
 
+        const long long tk1 = timing ? wall_clock64() : 0;
+        if (!last) cur = load_step(step + 1);
+        c_cur = c_next;
+        c_next = load_c(step + 2);
         if (cell_valid) {
             if (!first) {
 #pragma unroll
@@ -370,7 +427,8 @@ __global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParam
             dl[2 * JB + cj][cs] = s_fg; dl[3 * JB + cj][cs] = s_og;
             fg_later = fg; cerr_later = ce; dig_later = s_ig; dfg_later = s_fg;
         }
-        __syncthreads();
+        lds_barrier();
+        const long long tk2 = timing ? wall_clock64() : 0;
 
         if (!last) {
             // partial output errors of every receiving cell from this workgroup's deltas
@@ -402,6 +460,14 @@ __global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParam
             }
         }
         // `dl` and `psum` are rewritten only after the next step's barrier
+        if (timing) {
+            const long long tk3 = wall_clock64();
+            ph0 += tk1 - tk0; ph1 += tk2 - tk1; ph2 += tk3 - tk2;
+        }
+    }
+    if (timing && tid == 0) {
+        long long *o = p.phase_ticks + (size_t)blockIdx.x * 4;
+        o[0] = ph0; o[1] = ph1; o[2] = ph2; o[3] = ph3;
     }
 }
 
@@ -466,6 +532,7 @@ struct cnt_lstm {
     int JB, NT;
     unsigned spin_limit;
     int xcd_pack;
+    long long *phase_ticks;  // diagnostic buffer, allocated when CNT_LSTM_TIMING is set
 };
 
 namespace cnt {
@@ -518,6 +585,7 @@ void fill_chain_params(const cnt_lstm *h, const float *weights, ChainParams &p) 
     p.spin_limit = h->spin_limit;
     p.abort_flag = h->abort_flag;
     p.xcd_pack = h->xcd_pack;
+    p.phase_ticks = h->phase_ticks;
 }
 
 int next_epoch(cnt_lstm *h, hipStream_t stream, unsigned &tag_base) {
@@ -589,6 +657,8 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
         if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->mailbox[dir]), h->mailbox_bytes);
         if (err == hipSuccess) err = hipMemset(h->mailbox[dir], 0, h->mailbox_bytes);
     }
+    if (err == hipSuccess && std::getenv("CNT_LSTM_TIMING"))
+        err = hipMalloc(reinterpret_cast<void **>(&h->phase_ticks), 8 * 512 * 4 * sizeof(long long));
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->abort_flag), sizeof(int));
     if (err == hipSuccess) err = hipMemset(h->abort_flag, 0, sizeof(int));
     if (err != hipSuccess) {
@@ -608,6 +678,7 @@ int cnt_lstm_destroy(cnt_lstm *h) {
         if (h->mailbox[dir]) (void)hipFree(h->mailbox[dir]);
     }
     if (h->abort_flag) (void)hipFree(h->abort_flag);
+    if (h->phase_ticks) (void)hipFree(h->phase_ticks);
     delete h;
     return CNT_OK;
 }
@@ -636,6 +707,17 @@ int cnt_lstm_check(cnt_lstm *h, void *stream) {
     int flag = 0;
     CNT_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     CNT_HIP(hipMemcpy(&flag, h->abort_flag, sizeof(int), hipMemcpyDeviceToHost));
+    if (h->phase_ticks) {
+        // diagnostic: mean phase durations of the last backward recursion, in 10 ns ticks
+        const int blocks = h->ndir * (h->H / h->JB);
+        std::vector<long long> t((size_t)blocks * 4);
+        CNT_HIP(hipMemcpy(t.data(), h->phase_ticks, t.size() * sizeof(long long), hipMemcpyDeviceToHost));
+        double m[4] = {0, 0, 0, 0};
+        for (int b = 0; b < blocks; ++b)
+            for (int q = 0; q < 4; ++q) m[q] += (double)t[(size_t)b * 4 + q] / blocks;
+        std::fprintf(stderr, "lstm backward phases per step [us]: wait %.3f cell %.3f product+publish %.3f (T=%d)\n",
+                     m[0] * 0.01 / h->T, m[1] * 0.01 / h->T, m[2] * 0.01 / h->T, h->T);
+    }
     if (flag != 0) {
         CNT_HIP(hipMemset(h->abort_flag, 0, sizeof(int)));
         set_error("lstm: a recursion kernel gave up waiting for a neighbouring workgroup; results are invalid");
