@@ -111,6 +111,45 @@ long cnt_lstm_weight_count(int P, int L, int bidir);
  * no counterpart: its per-step launches cannot stall on each other. */
 int cnt_lstm_check(cnt_lstm *h, void *stream);
 
+/* ---- mixture-density post-output layer ----------------------------------------------------------
+ * MDNLayer<TDevice> with MDNUnit_softmax (flat) and MDNUnit_mixture (untied variance) units
+ * (layers/MDNLayer.cu, layers/MDNUnit.cu).  The handle owns what the units keep between calls: the
+ * distribution parameters (m_paraVec) and the per-mixture log-likelihoods and log-sums (m_tmpPat).
+ * `config` is the content of the reference's binary mdn config: [n, (startD, endD, startDOut, endDOut,
+ * type) x n] as floats (layers/MDNLayer.cu:286-324); type -1 = softmax, > 0 = number of Gaussians
+ * (layers/MDNLayer.hpp:35-36).  Other unit types and tied variances are rejected. */
+typedef struct cnt_mdn cnt_mdn;
+
+typedef struct {
+    int Lp;            /* size of the layer feeding the MDN layer            */
+    int Lt;            /* size of the MDN layer = target dimension           */
+    int S;             /* parallel sequences                                 */
+    int maxT;          /* maxSeqLength                                       */
+    int tie_variance;  /* --tieVariance; only 0 is supported                 */
+} cnt_mdn_desc;
+
+/* MDNLayer::MDNLayer (layers/MDNLayer.cu:280-324, 457-545). */
+int cnt_mdn_create(const cnt_mdn_desc *desc, const float *config, int config_len, cnt_mdn **out);
+int cnt_mdn_destroy(cnt_mdn *h);
+/* Variance floor of a mixture unit (MDNUnit.cu:5233-5234 sets it when the network has no trained
+ * weights; it is 0 otherwise). */
+int cnt_mdn_set_var_floor(cnt_mdn *h, int unit, float var_floor);
+/* Layer::loadSequences: records the fraction's pattern types (device memory, char[curMaxT*S]). */
+int cnt_mdn_load_sequences(cnt_mdn *h, void *stream, const char *patTypes, int curMaxT);
+/* MDNLayer::computeForwardPass (layers/MDNLayer.cu:841-852): nn_outputs is Lp x (T*S). */
+int cnt_mdn_forward(cnt_mdn *h, void *stream, const float *nn_outputs);
+/* MDNLayer::calculateError (layers/MDNLayer.cu:797-827): targets is Lt x (T*S); the negative
+ * log-likelihood summed over units and frames is written to *result_dev (device memory).  It also
+ * stores the posteriors' ingredients that cnt_mdn_backward reads, as the reference does. */
+int cnt_mdn_calculate_error(cnt_mdn *h, void *stream, const float *targets, float *result_dev);
+/* MDNLayer::computeBackwardPass (layers/MDNLayer.cu:875-917): prev_errors is the preceding layer's
+ * whole error buffer, Lp x (maxT*S); it is zero-filled and then receives every unit's gradient. */
+int cnt_mdn_backward(cnt_mdn *h, void *stream, const float *targets, float *prev_errors);
+/* Device pointer to a unit's buffer. which: 0 parameters (softmax: F*K probabilities; mixture:
+ * [F*M weights | F*M*D means | F*M*D std]), 1 mixture log-likelihoods [F*M | F].  *count receives the
+ * number of floats in use for the current fraction. */
+float *cnt_mdn_unit_buffer(cnt_mdn *h, int unit, int which, long *count);
+
 #ifdef __cplusplus
 }
 #endif

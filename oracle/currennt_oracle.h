@@ -60,6 +60,24 @@ void orc_dense_backward(int P, int D, int N, int act, float bias, const float *w
 float orc_sse_error(int D, int N, const char *patTypes, const float *y, const float *target);
 void orc_sse_backward(int D, int N, const char *patTypes, const float *y, const float *target, float *err);
 
+/* Mixture-density post-output layer (MDNUnit.cu, MDNLayer.cu).  F = T*S frames, Lp = size of the layer
+   feeding the MDN, Lt = size of the target vector.  A mixture unit with M components over D target
+   dimensions reads columns [startD, startD + M + 2*M*D) of the input: weights, means, log-std.
+   para = [F*M weights | F*M*D means | F*M*D std]; tmp = [F*M log-likelihoods | F log-sums]. */
+void orc_mdn_mixture_forward(int F, int Lp, int startD, int M, int D, float var_floor, const char *pat,
+                             const float *x, float *para);
+float orc_mdn_mixture_error(int F, int Lt, int startDOut, int M, int D, const char *pat, const float *target,
+                            const float *para, float *tmp);
+void orc_mdn_mixture_backward(int F, int Lp, int Lt, int startD, int startDOut, int M, int D, float var_floor,
+                              const char *pat, const float *target, const float *para, const float *tmp,
+                              float *errors);
+void orc_softmax_forward(int F, int Lp, int startD, int K, float temperature, const char *pat, const float *x,
+                         float *prob);
+float orc_softmax_error(int F, int Lt, int startDOut, int K, long prob_capacity, const char *pat,
+                        const float *target, const float *prob);
+void orc_softmax_backward(int F, int Lp, int Lt, int startD, int startDOut, int K, const char *pat,
+                          const float *target, const float *prob, float *errors);
+
 #ifdef __cplusplus
 }
 #endif

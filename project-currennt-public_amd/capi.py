@@ -13,6 +13,10 @@ LSTM_STATE = {"ni": 0, "ig": 1, "fg": 2, "og": 3, "c": 4, "h": 5, "herr": 6, "dn
               "dog": 10, "cerr": 11}
 
 
+class MdnDesc(C.Structure):
+    _fields_ = [("Lp", C.c_int), ("Lt", C.c_int), ("S", C.c_int), ("maxT", C.c_int), ("tie_variance", C.c_int)]
+
+
 class LstmDesc(C.Structure):
     _fields_ = [("P", C.c_int), ("L", C.c_int), ("bidir", C.c_int), ("S", C.c_int), ("maxT", C.c_int),
                 ("bias", C.c_float)]
@@ -42,6 +46,14 @@ _SIGNATURES = {
     "cnt_lstm_state": (VP, [VP, I, I]),
     "cnt_lstm_weight_count": (C.c_long, [I, I, I]),
     "cnt_lstm_check": (I, [VP, VP]),
+    "cnt_mdn_create": (I, [C.POINTER(MdnDesc), C.POINTER(F), I, C.POINTER(VP)]),
+    "cnt_mdn_destroy": (I, [VP]),
+    "cnt_mdn_set_var_floor": (I, [VP, I, F]),
+    "cnt_mdn_load_sequences": (I, [VP, VP, VP, I]),
+    "cnt_mdn_forward": (I, [VP, VP, VP]),
+    "cnt_mdn_calculate_error": (I, [VP, VP, VP, VP]),
+    "cnt_mdn_backward": (I, [VP, VP, VP, VP]),
+    "cnt_mdn_unit_buffer": (VP, [VP, I, I, C.POINTER(C.c_long)]),
 }
 
 
@@ -170,6 +182,53 @@ class Lstm:
         n = self.H * self.T * self.S
         torch.cuda.synchronize()
         return torch.as_tensor(_DeviceArray(p, n), device="cuda").clone()
+
+
+class Mdn:
+    """Thin owner of a cnt_mdn handle.  config: flat list [n, (startD, endD, startDOut, endDOut, type) * n]."""
+
+    def __init__(self, Lp, Lt, S, maxT, config, tie_variance=False):
+        self.handle = VP()
+        desc = MdnDesc(Lp, Lt, S, maxT, int(tie_variance))
+        arr = (F * len(config))(*[float(v) for v in config])
+        check(lib().cnt_mdn_create(C.byref(desc), arr, len(config), C.byref(self.handle)))
+
+    def close(self):
+        if self.handle:
+            lib().cnt_mdn_destroy(self.handle)
+            self.handle = VP()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_var_floor(self, unit, v):
+        check(lib().cnt_mdn_set_var_floor(self.handle, unit, v))
+
+    def load_sequences(self, pat, T, stream=None):
+        self._pat = pat
+        check(lib().cnt_mdn_load_sequences(self.handle, stream_ptr(stream), ptr(pat), T))
+
+    def forward(self, x, stream=None):
+        check(lib().cnt_mdn_forward(self.handle, stream_ptr(stream), ptr(x)))
+
+    def calculate_error(self, targets, result, stream=None):
+        check(lib().cnt_mdn_calculate_error(self.handle, stream_ptr(stream), ptr(targets), ptr(result)))
+
+    def backward(self, targets, prev_errors, stream=None):
+        check(lib().cnt_mdn_backward(self.handle, stream_ptr(stream), ptr(targets), ptr(prev_errors)))
+
+    def unit_buffer(self, unit, which):
+        import torch
+
+        n = C.c_long(0)
+        p = lib().cnt_mdn_unit_buffer(self.handle, unit, which, C.byref(n))
+        if not p:
+            raise RuntimeError("no such MDN unit buffer")
+        torch.cuda.synchronize()
+        return torch.as_tensor(_DeviceArray(p, n.value), device="cuda").clone()
 
 
 class _DeviceArray:

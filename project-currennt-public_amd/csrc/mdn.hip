@@ -1,0 +1,442 @@
+// Mixture-density post-output layer for gfx950: flat softmax units and untied-variance Gaussian
+// mixture units.
+//
+// Reference behaviour: layers/MDNLayer.cu (config parsing :280-324, unit creation :457-545,
+// calculateError :797-827, forward :841-852, backward :875-917) and layers/MDNUnit.cu (functors
+// :227-296, :333-405, :437-470, :503-530, :683-750, :921-1000, :1003-1063, :2096-2325; drivers
+// :4170-4339, :4685-4754, :5249-5420, :6036-6193, :6195-6416).
+//
+// The reference walks the F x Lp activation matrix with 4-6 one-element-per-thread launches per
+// call.  Here every call is one streaming kernel per unit: one 64-lane wave owns one frame, lanes run
+// along the frame's contiguous columns, and the per-frame reductions (offset, normaliser,
+// per-mixture distance, log-sum) are wave shuffles.  HBM traffic per call is one read of the
+// unit's columns plus one write of its result.
+//
+// Kept on purpose: the mixture-weight gradient of a padding frame is "zeroed" at index t*M+m
+// instead of t*Lp+startD+m (MDNUnit.cu:2199-2200); on the reference's sequential host backend that
+// zero lands after the value it collides with, so the colliding mixture-weight gradient of an
+// earlier valid frame reads 0.  The kernels reproduce exactly that outcome without a race.
+#include "common.hpp"
+
+#include <cmath>
+#include <cstring>
+#include <new>
+#include <vector>
+
+namespace cnt {
+namespace {
+
+constexpr float kSkipMarker = lim::kMax;
+constexpr int kFramesPerBlock = 4;
+
+__device__ __forceinline__ float wave_sum(float v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ float wave_min(float v) {
+    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+// offset = (min + max) / 2 with the reference's start values, exp((x - offset)/T), normalise.
+// `in` points at the K inputs of the frame, `out` at its K outputs.
+__device__ __forceinline__ void softmax_frame(const float *__restrict__ in, float *__restrict__ out, int K,
+                                              float temperature, int lane) {
+    float mx = lim::kMin, mn = lim::kMax;
+    for (int k = lane; k < K; k += 64) {
+        const float v = in[k];
+        mn = fminf(mn, v);
+        mx = fmaxf(mx, v);
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    const float offset = 0.5f * (mn + mx);
+    float sum = 0.0f;
+    for (int k = lane; k < K; k += 64) {
+        const float e = safe_exp((in[k] - offset) / temperature);
+        out[k] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    if (sum == kSkipMarker) return;
+    for (int k = lane; k < K; k += 64) out[k] = out[k] / sum;  // each lane re-reads its own writes
+}
+
+struct UnitGeom {
+    int F, Lp, Lt;
+    int startD, startDOut;
+    int M, D;  // softmax unit: M = classes, D unused
+    float var_floor, temperature;
+    long capacity;  // allocated elements of the unit's parameter buffer
+};
+
+// ---- softmax unit -----------------------------------------------------------------------------------
+__global__ void softmax_forward_kernel(UnitGeom g, const char *__restrict__ pat, const float *__restrict__ x,
+                                       float *__restrict__ prob) {
+    const int lane = threadIdx.x & 63;
+    const int f = blockIdx.x * kFramesPerBlock + (threadIdx.x >> 6);
+    if (f >= g.F) return;
+    float *row = prob + (size_t)f * g.M;
+    if (pat[f] == 0) {
+        for (int k = lane; k < g.M; k += 64) row[k] = kSkipMarker;
+        return;
+    }
+    softmax_frame(x + (size_t)f * g.Lp + g.startD, row, g.M, g.temperature, lane);
+}
+
+__global__ void softmax_error_kernel(UnitGeom g, const char *__restrict__ pat, const float *__restrict__ target,
+                                     const float *__restrict__ prob, float *__restrict__ result) {
+    const int f = blockIdx.x * blockDim.x + threadIdx.x;
+    float v = 0.0f;
+    if (f < g.F && pat[f] != 0) {
+        const int ti = (int)target[(size_t)f * g.Lt + g.startDOut];
+        const long idx = (long)f * g.M + ti;
+        float p = 1.0f;
+        if (idx < g.capacity && idx >= 0) p = fmaxf(lim::kMin, prob[idx]);
+        v = -logf(p);
+    }
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0 && v != 0.0f) atomicAdd(result, v);
+}
+
+__global__ void softmax_backward_kernel(UnitGeom g, const char *__restrict__ pat, const float *__restrict__ target,
+                                        const float *__restrict__ prob, float *__restrict__ errors) {
+    const int lane = threadIdx.x & 63;
+    const int f = blockIdx.x * kFramesPerBlock + (threadIdx.x >> 6);
+    if (f >= g.F) return;
+    float *e = errors + (size_t)f * g.Lp + g.startD;
+    if (pat[f] == 0) {
+        // never written by the reference; the layer's zero fill is what remains
+        for (int k = lane; k < g.M; k += 64) e[k] = 0.0f;
+        return;
+    }
+    const float t = target[(size_t)f * g.Lt + g.startDOut];
+    const float *p = prob + (size_t)f * g.M;
+    for (int k = lane; k < g.M; k += 64) {
+        const bool hit = (double)((t - k) * (t - k)) < 0.0001;
+        e[k] = hit ? (-1 + p[k]) : p[k];
+    }
+}
+
+// ---- mixture unit -----------------------------------------------------------------------------------
+// para = [F*M weights | F*M*D means | F*M*D std], offsets by the CURRENT frame count F.
+__global__ void mixture_forward_kernel(UnitGeom g, const char *__restrict__ pat, const float *__restrict__ x,
+                                       float *__restrict__ para) {
+    const int lane = threadIdx.x & 63;
+    const int f = blockIdx.x * kFramesPerBlock + (threadIdx.x >> 6);
+    if (f >= g.F) return;
+    const int MD = g.M * g.D;
+    float *w = para + (size_t)f * g.M;
+    float *mean = para + (size_t)g.F * g.M + (size_t)f * MD;
+    float *sd = para + (size_t)g.F * g.M * (1 + g.D) + (size_t)f * MD;
+    if (pat[f] == 0) {
+        for (int k = lane; k < g.M; k += 64) w[k] = kSkipMarker;
+        for (int i = lane; i < MD; i += 64) sd[i] = kSkipMarker;  // means stay untouched
+        return;
+    }
+    const float *in = x + (size_t)f * g.Lp + g.startD;
+    softmax_frame(in, w, g.M, 1.0f, lane);
+    for (int i = lane; i < MD; i += 64) {
+        mean[i] = in[g.M + i];
+        const float b = safe_exp(in[g.M + MD + i]);
+        sd[i] = b < g.var_floor ? g.var_floor : b;
+    }
+}
+
+// tmp = [F*M per-mixture log-likelihoods | F log-sums]; result accumulates -sum of log-sums
+__global__ void mixture_error_kernel(UnitGeom g, const char *__restrict__ pat, const float *__restrict__ target,
+                                     const float *__restrict__ para, float *__restrict__ tmp,
+                                     float *__restrict__ result) {
+    const int lane = threadIdx.x & 63;
+    const int f = blockIdx.x * kFramesPerBlock + (threadIdx.x >> 6);
+    if (f >= g.F) return;
+    const int M = g.M, D = g.D;
+    if (pat[f] == 0) {
+        for (int m = lane; m < M; m += 64) tmp[(size_t)f * M + m] = 0.0f;  // distance pass writes 0, the rest skips
+        return;
+    }
+    const float *t = target + (size_t)f * g.Lt + g.startDOut;
+    const float *mean = para + (size_t)g.F * M + (size_t)f * M * D;
+    const float *sd = para + (size_t)g.F * M * (1 + D) + (size_t)f * M * D;
+    const float gauss_const = (float)(D * log(2 * 3.141215) / 2.0);  // the reference's own value of pi
+    float lsum = lim::kLogZero;
+    for (int m = 0; m < M; ++m) {
+        float dist = 0.0f, logsd = 0.0f;
+        for (int d = lane; d < D; d += 64) {
+            const float s = sd[m * D + d], diff = t[d] - mean[m * D + d];
+            dist += diff * diff / (s * s) * 0.5f;
+            logsd += safe_log(s);
+        }
+        dist = wave_sum(dist);
+        logsd = wave_sum(logsd);
+        float lp = logf(para[(size_t)f * M + m]) - dist - gauss_const - logsd;
+        if (lp < lim::kLSmall) lp = lim::kLSmall;
+        lsum = log_add(lsum, lp);
+        if (lane == 0) tmp[(size_t)f * M + m] = lp;
+    }
+    if (lane == 0) {
+        tmp[(size_t)g.F * M + f] = lsum;
+        atomicAdd(result, -lsum);
+    }
+}
+
+__global__ void mixture_backward_kernel(UnitGeom g, const char *__restrict__ pat, const float *__restrict__ target,
+                                        const float *__restrict__ para, const float *__restrict__ tmp,
+                                        float *__restrict__ errors) {
+    const int lane = threadIdx.x & 63;
+    const int f = blockIdx.x * kFramesPerBlock + (threadIdx.x >> 6);
+    if (f >= g.F) return;
+    const int M = g.M, D = g.D, MD = M * D, Lp = g.Lp;
+    const int unit_cols = M + 2 * MD;
+    float *e = errors + (size_t)f * Lp + g.startD;
+    if (pat[f] == 0) {
+        // The reference zeroes index f*M+m for this frame's mixture weights.  Where that index is a column
+        // of this unit the outcome is decided by the owner of the column (see below); elsewhere the zero
+        // is written as is.  This frame's own columns end up 0: weights by the layer's zero fill, means and
+        // std by the second pass.
+        for (int m = lane; m < M; m += 64) {
+            const long idx = (long)f * M + m;
+            const int col = (int)(idx % Lp);
+            if (col < g.startD || col >= g.startD + unit_cols) errors[idx] = 0.0f;
+        }
+        for (int i = lane; i < unit_cols; i += 64) e[i] = 0.0f;
+        return;
+    }
+    const float lsum = tmp[(size_t)g.F * M + f];
+    for (int m = lane; m < M; m += 64) {
+        const float post = safe_exp(tmp[(size_t)f * M + m] - lsum);
+        float v = para[(size_t)f * M + m] - post;
+        // a padding frame fd with fd*M + m' == this index overwrites the value with 0 afterwards
+        const long idx = (long)f * Lp + g.startD + m;
+        const long fd = idx / M;
+        if (fd < g.F && pat[fd] == 0) v = 0.0f;
+        e[m] = v;
+    }
+    const float *t = target + (size_t)f * g.Lt + g.startDOut;
+    const float *mean = para + (size_t)g.F * M + (size_t)f * MD;
+    const float *sd = para + (size_t)g.F * M * (1 + D) + (size_t)f * MD;
+    for (int i = lane; i < MD; i += 64) {
+        const int m = i / D, d = i - m * D;
+        const float post = safe_exp(tmp[(size_t)f * M + m] - lsum);
+        const float mu = mean[i], s = sd[i], tv = t[d];
+        const float e_mu = post * (mu - tv) / s / s;
+        e[M + i] = e_mu;
+        e[M + MD + i] = (s > g.var_floor) ? post - e_mu * (mu - tv) : 0.0f;
+    }
+}
+
+}  // namespace
+}  // namespace cnt
+
+// ---------------------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------------------
+struct cnt_mdn_unit {
+    int type;  // >0 mixtures, -1 softmax
+    int startD, endD, startDOut, endDOut;
+    int M, D;
+    float var_floor;
+    float *para, *tmp;
+    long para_capacity, tmp_capacity;
+};
+
+struct cnt_mdn {
+    cnt_mdn_desc desc;
+    std::vector<cnt_mdn_unit> units;
+    const char *pat;
+    int T;
+    bool covers_all_columns;
+};
+
+extern "C" {
+
+int cnt_mdn_destroy(cnt_mdn *h) {
+    if (!h) return CNT_OK;
+    for (auto &u : h->units) {
+        if (u.para) (void)hipFree(u.para);
+        if (u.tmp) (void)hipFree(u.tmp);
+    }
+    delete h;
+    return CNT_OK;
+}
+
+int cnt_mdn_create(const cnt_mdn_desc *desc, const float *config, int config_len, cnt_mdn **out) {
+    using namespace cnt;
+    CNT_REQUIRE(desc && config && out, "mdn_create: null argument");
+    CNT_REQUIRE(desc->Lp > 0 && desc->Lt > 0 && desc->S > 0 && desc->maxT > 0, "mdn_create: non-positive size");
+    CNT_REQUIRE(config_len >= 1, "mdn_create: empty configuration");
+    const int n = (int)config[0];
+    // same consistency rule as the reference's reader (MDNLayer.cu:303-305)
+    CNT_REQUIRE(config_len == n * 5 + 1, "Number of parameter != 1st parameter * 5 + 1");
+    cnt_mdn *h = new (std::nothrow) cnt_mdn();
+    CNT_REQUIRE(h != nullptr, "mdn_create: out of host memory");
+    h->desc = *desc;
+    h->pat = nullptr;
+    h->T = 0;
+    const long maxF = (long)desc->maxT * desc->S;
+    std::vector<char> covered((size_t)desc->Lp, 0);
+    for (int i = 0; i < n; ++i) {
+        cnt_mdn_unit u = {};
+        u.startD = (int)config[1 + i * 5]; u.endD = (int)config[2 + i * 5];
+        u.startDOut = (int)config[3 + i * 5]; u.endDOut = (int)config[4 + i * 5];
+        u.type = (int)config[5 + i * 5];
+        const int cols = u.endD - u.startD, dims = u.endDOut - u.startDOut;
+        bool ok = u.startD >= 0 && u.endD <= desc->Lp && cols > 0 && u.startDOut >= 0 && u.endDOut <= desc->Lt && dims > 0;
+        if (ok && u.type == -1) {
+            u.M = cols; u.D = 1;
+            u.para_capacity = maxF * u.M;
+            u.tmp_capacity = 0;
+            ok = (dims == 1);
+        } else if (ok && u.type > 0) {
+            u.M = u.type; u.D = dims;
+            ok = !desc->tie_variance && cols == u.M * (1 + 2 * u.D);
+            u.para_capacity = maxF * u.M * (1 + 2 * u.D);
+            u.tmp_capacity = maxF * (u.M + 1);
+        } else {
+            ok = false;
+        }
+        if (!ok) {
+            set_error("mdn_create: unit %d (type %d, columns %d..%d, targets %d..%d) is not supported: only flat softmax "
+                      "(-1) and untied-variance mixture units (>0 with columns = M*(1+2*D)) are built",
+                      i, u.type, u.startD, u.endD, u.startDOut, u.endDOut);
+            cnt_mdn_destroy(h);
+            return CNT_ERR_ARG;
+        }
+        hipError_t err = hipMalloc(reinterpret_cast<void **>(&u.para), (size_t)u.para_capacity * sizeof(float));
+        if (err == hipSuccess) err = hipMemset(u.para, 0, (size_t)u.para_capacity * sizeof(float));
+        if (err == hipSuccess && u.tmp_capacity) {
+            err = hipMalloc(reinterpret_cast<void **>(&u.tmp), (size_t)u.tmp_capacity * sizeof(float));
+            if (err == hipSuccess) err = hipMemset(u.tmp, 0, (size_t)u.tmp_capacity * sizeof(float));
+        }
+        h->units.push_back(u);
+        if (err != hipSuccess) {
+            set_error("mdn_create: %s", hipGetErrorString(err));
+            cnt_mdn_destroy(h);
+            return CNT_ERR_HIP;
+        }
+        for (int c = u.startD; c < u.endD; ++c) covered[(size_t)c] = 1;
+    }
+    h->covers_all_columns = true;
+    for (char c : covered) h->covers_all_columns = h->covers_all_columns && c;
+    *out = h;
+    return CNT_OK;
+}
+
+int cnt_mdn_set_var_floor(cnt_mdn *h, int unit, float var_floor) {
+    using namespace cnt;
+    CNT_REQUIRE(h && unit >= 0 && unit < (int)h->units.size(), "mdn_set_var_floor: no such unit");
+    h->units[(size_t)unit].var_floor = var_floor;
+    return CNT_OK;
+}
+
+int cnt_mdn_load_sequences(cnt_mdn *h, void *stream, const char *patTypes, int curMaxT) {
+    using namespace cnt;
+    (void)stream;
+    CNT_REQUIRE(h && patTypes, "mdn_load_sequences: null argument");
+    CNT_REQUIRE(curMaxT >= 1 && curMaxT <= h->desc.maxT, "mdn_load_sequences: curMaxT %d outside 1..%d", curMaxT,
+                h->desc.maxT);
+    h->pat = patTypes;
+    h->T = curMaxT;
+    return CNT_OK;
+}
+
+float *cnt_mdn_unit_buffer(cnt_mdn *h, int unit, int which, long *count) {
+    if (!h || unit < 0 || unit >= (int)h->units.size()) return nullptr;
+    cnt_mdn_unit &u = h->units[(size_t)unit];
+    const long F = (long)h->T * h->desc.S;
+    if (which == 0) {
+        if (count) *count = u.type == -1 ? F * u.M : F * u.M * (1 + 2 * u.D);
+        return u.para;
+    }
+    if (which == 1 && u.tmp) {
+        if (count) *count = F * (u.M + 1);
+        return u.tmp;
+    }
+    return nullptr;
+}
+
+static cnt::UnitGeom unit_geom(const cnt_mdn *h, const cnt_mdn_unit &u) {
+    cnt::UnitGeom g;
+    g.F = h->T * h->desc.S; g.Lp = h->desc.Lp; g.Lt = h->desc.Lt;
+    g.startD = u.startD; g.startDOut = u.startDOut; g.M = u.M; g.D = u.D;
+    g.var_floor = u.var_floor; g.temperature = 1.0f;
+    g.capacity = u.para_capacity;
+    return g;
+}
+
+int cnt_mdn_forward(cnt_mdn *h, void *stream_, const float *nn_outputs) {
+    using namespace cnt;
+    CNT_REQUIRE(h && nn_outputs, "mdn_forward: null argument");
+    CNT_REQUIRE(h->T > 0, "mdn_forward: load_sequences has not been called");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    for (auto &u : h->units) {
+        const UnitGeom g = unit_geom(h, u);
+        const dim3 grid((g.F + kFramesPerBlock - 1) / kFramesPerBlock), block(64 * kFramesPerBlock);
+        if (u.type == -1) {
+            ProfileScope prof(stream, "mdn_softmax_forward");
+            hipLaunchKernelGGL(softmax_forward_kernel, grid, block, 0, stream, g, h->pat, nn_outputs, u.para);
+        } else {
+            ProfileScope prof(stream, "mdn_mixture_forward");
+            hipLaunchKernelGGL(mixture_forward_kernel, grid, block, 0, stream, g, h->pat, nn_outputs, u.para);
+        }
+        CNT_HIP(hipGetLastError());
+    }
+    return CNT_OK;
+}
+
+int cnt_mdn_calculate_error(cnt_mdn *h, void *stream_, const float *targets, float *result_dev) {
+    using namespace cnt;
+    CNT_REQUIRE(h && targets && result_dev, "mdn_calculate_error: null argument");
+    CNT_REQUIRE(h->T > 0, "mdn_calculate_error: load_sequences has not been called");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    CNT_TRY(fill_zero(stream, result_dev, 1));
+    for (auto &u : h->units) {
+        const UnitGeom g = unit_geom(h, u);
+        if (u.type == -1) {
+            ProfileScope prof(stream, "mdn_softmax_error");
+            hipLaunchKernelGGL(softmax_error_kernel, dim3((g.F + 255) / 256), dim3(256), 0, stream, g, h->pat, targets,
+                               u.para, result_dev);
+        } else {
+            ProfileScope prof(stream, "mdn_mixture_error");
+            const dim3 grid((g.F + kFramesPerBlock - 1) / kFramesPerBlock), block(64 * kFramesPerBlock);
+            hipLaunchKernelGGL(mixture_error_kernel, grid, block, 0, stream, g, h->pat, targets, u.para, u.tmp,
+                               result_dev);
+        }
+        CNT_HIP(hipGetLastError());
+    }
+    return CNT_OK;
+}
+
+int cnt_mdn_backward(cnt_mdn *h, void *stream_, const float *targets, float *prev_errors) {
+    using namespace cnt;
+    CNT_REQUIRE(h && targets && prev_errors, "mdn_backward: null argument");
+    CNT_REQUIRE(h->T > 0, "mdn_backward: load_sequences has not been called");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const size_t used = (size_t)h->T * h->desc.S * h->desc.Lp;
+    const size_t cap = (size_t)h->desc.maxT * h->desc.S * h->desc.Lp;
+    // MDNLayer::computeBackwardPass zero-fills the whole preceding error buffer first.  The unit kernels
+    // write every column they own for every current frame, so only what they do not cover is filled.
+    if (!h->covers_all_columns) CNT_TRY(fill_zero(stream, prev_errors, used));
+    if (cap > used) CNT_TRY(fill_zero(stream, prev_errors + used, cap - used));
+    for (auto &u : h->units) {
+        const UnitGeom g = unit_geom(h, u);
+        const dim3 grid((g.F + kFramesPerBlock - 1) / kFramesPerBlock), block(64 * kFramesPerBlock);
+        if (u.type == -1) {
+            ProfileScope prof(stream, "mdn_softmax_backward");
+            hipLaunchKernelGGL(softmax_backward_kernel, grid, block, 0, stream, g, h->pat, targets, u.para,
+                               prev_errors);
+        } else {
+            ProfileScope prof(stream, "mdn_mixture_backward");
+            hipLaunchKernelGGL(mixture_backward_kernel, grid, block, 0, stream, g, h->pat, targets, u.para, u.tmp,
+                               prev_errors);
+        }
+        CNT_HIP(hipGetLastError());
+    }
+    return CNT_OK;
+}
+
+}  // extern "C"

@@ -66,6 +66,8 @@ def lib():
         L.orc_log_add.argtypes = [C.c_float, C.c_float]
         L.orc_lstm_weight_count.restype = C.c_long
         L.orc_sse_error.restype = C.c_float
+        L.orc_mdn_mixture_error.restype = C.c_float
+        L.orc_softmax_error.restype = C.c_float
         _lib = L
     return _lib
 
@@ -110,3 +112,28 @@ def sse_error(D, N, pat, y, tgt):
 
 def sse_backward(D, N, pat, y, tgt, err):
     lib().orc_sse_backward(D, N, cptr(pat), fptr(y), fptr(tgt), fptr(err))
+
+
+def mdn_mixture_forward(F, Lp, startD, M, D, var_floor, pat, x, para):
+    lib().orc_mdn_mixture_forward(F, Lp, startD, M, D, C.c_float(var_floor), cptr(pat), fptr(x), fptr(para))
+
+
+def mdn_mixture_error(F, Lt, startDOut, M, D, pat, target, para, tmp):
+    return float(lib().orc_mdn_mixture_error(F, Lt, startDOut, M, D, cptr(pat), fptr(target), fptr(para), fptr(tmp)))
+
+
+def mdn_mixture_backward(F, Lp, Lt, startD, startDOut, M, D, var_floor, pat, target, para, tmp, errors):
+    lib().orc_mdn_mixture_backward(F, Lp, Lt, startD, startDOut, M, D, C.c_float(var_floor), cptr(pat),
+                                   fptr(target), fptr(para), fptr(tmp), fptr(errors))
+
+
+def softmax_forward(F, Lp, startD, K, temperature, pat, x, prob):
+    lib().orc_softmax_forward(F, Lp, startD, K, C.c_float(temperature), cptr(pat), fptr(x), fptr(prob))
+
+
+def softmax_error(F, Lt, startDOut, K, cap, pat, target, prob):
+    return float(lib().orc_softmax_error(F, Lt, startDOut, K, C.c_long(cap), cptr(pat), fptr(target), fptr(prob)))
+
+
+def softmax_backward(F, Lp, Lt, startD, startDOut, K, pat, target, prob, errors):
+    lib().orc_softmax_backward(F, Lp, Lt, startD, startDOut, K, cptr(pat), fptr(target), fptr(prob), fptr(errors))

@@ -201,3 +201,95 @@ def run_sse_case(D, lengths, seed):
     # elementwise subtraction and masking are exact
     assert np.array_equal(err_d.cpu().numpy(), err_o)
     return abs(float(res.item()) - e_o) / max(abs(e_o), 1e-30)
+
+
+def run_mdn_mixture_case(lengths, M, D, extra, seed, var_floor=0.0, maxT=None):
+    """Mixture unit at column `extra` of the feeding layer; returns worst error over parameters,
+    log-likelihoods, loss and gradients.  Padding handling (exact zeros, the index collision) is part of
+    the gradient comparison because the oracle reproduces the reference's sequential outcome."""
+    import torch
+
+    capi = pkg().capi
+    S, T = len(lengths), max(lengths)
+    maxT = maxT or T
+    F = T * S
+    Lp = extra + M + 2 * M * D
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((F, Lp)).astype(np.float32)
+    x[:, extra + M + M * D:] *= 0.5
+    tgt = rng.standard_normal((F, D)).astype(np.float32)
+    pat = make_pat_types(lengths, T)
+    para_o = np.zeros(F * M * (1 + 2 * D), dtype=np.float32)
+    tmp_o = np.zeros(F * M + F, dtype=np.float32)
+    err_o = np.zeros(maxT * S * Lp, dtype=np.float32)
+    O.mdn_mixture_forward(F, Lp, extra, M, D, var_floor, pat, x.reshape(-1), para_o)
+    nll_o = O.mdn_mixture_error(F, D, 0, M, D, pat, tgt.reshape(-1), para_o, tmp_o)
+    O.mdn_mixture_backward(F, Lp, D, extra, 0, M, D, var_floor, pat, tgt.reshape(-1), para_o, tmp_o, err_o)
+
+    layer = capi.Mdn(Lp, D, S, maxT, [1, extra, Lp, 0, D, M])
+    layer.set_var_floor(0, var_floor)
+    pd, xd, td = dev(pat), dev(x.reshape(-1)), dev(tgt.reshape(-1))
+    res = torch.zeros(1, dtype=torch.float32, device="cuda")
+    err_d = torch.full((maxT * S * Lp,), 9.0, dtype=torch.float32, device="cuda")
+    layer.load_sequences(pd, T)
+    layer.forward(xd)
+    layer.calculate_error(td, res)
+    layer.backward(td, err_d)
+    torch.cuda.synchronize()
+    valid = np.repeat(pat != 0, 1)
+    para_d = layer.unit_buffer(0, 0).cpu().numpy()
+    tmp_d = layer.unit_buffer(0, 1).cpu().numpy()
+    worst = 0.0
+    # weights and std: all frames (padding frames hold the skip marker in both); means: valid frames only
+    worst = max(worst, relerr(para_d[:F * M], para_o[:F * M]))
+    worst = max(worst, relerr(para_d[F * M * (1 + D):], para_o[F * M * (1 + D):]))
+    worst = max(worst, relerr(para_d[F * M:F * M * (1 + D)].reshape(F, -1)[valid], para_o[F * M:F * M * (1 + D)].reshape(F, -1)[valid]))
+    worst = max(worst, relerr(tmp_d[:F * M], tmp_o[:F * M]))
+    worst = max(worst, relerr(tmp_d[F * M:][valid], tmp_o[F * M:][valid]))
+    worst = max(worst, abs(float(res.item()) - nll_o) / abs(nll_o))
+    got = err_d.cpu().numpy()
+    worst = max(worst, relerr(got, err_o))
+    # exact zeros wherever the oracle has exact zeros (padding frames, collisions, untouched columns, tail)
+    # (a gradient that underflows may flush to zero on the GPU only: allowed below 1e-30)
+    assert np.all(got[err_o == 0.0] == 0.0), "a structural zero of the gradient is not zero"
+    assert np.all(np.abs(err_o[got == 0.0]) < 1e-30), "the gradient has a zero where the oracle has a value"
+    layer.close()
+    return worst
+
+
+def run_softmax_case(lengths, K, extra, seed):
+    import torch
+
+    capi = pkg().capi
+    S, T = len(lengths), max(lengths)
+    F = T * S
+    Lp = extra + K
+    rng = np.random.default_rng(seed)
+    x = (2 * rng.standard_normal((F, Lp))).astype(np.float32)
+    tgt = rng.integers(0, K, size=F).astype(np.float32)
+    pat = make_pat_types(lengths, T)
+    prob_o = np.zeros(F * K, dtype=np.float32)
+    err_o = np.zeros(F * Lp, dtype=np.float32)
+    O.softmax_forward(F, Lp, extra, K, 1.0, pat, x.reshape(-1), prob_o)
+    nll_o = O.softmax_error(F, 1, 0, K, F * K, pat, tgt, prob_o)
+    O.softmax_backward(F, Lp, 1, extra, 0, K, pat, tgt, prob_o, err_o)
+
+    layer = capi.Mdn(Lp, 1, S, T, [1, extra, Lp, 0, 1, -1])
+    res = torch.zeros(1, dtype=torch.float32, device="cuda")
+    err_d = torch.full((F * Lp,), 9.0, dtype=torch.float32, device="cuda")
+    pd, xd, td = dev(pat), dev(x.reshape(-1)), dev(tgt)
+    layer.load_sequences(pd, T)
+    layer.forward(xd)
+    layer.calculate_error(td, res)
+    layer.backward(td, err_d)
+    torch.cuda.synchronize()
+    worst = relerr(layer.unit_buffer(0, 0).cpu().numpy(), prob_o)
+    worst = max(worst, abs(float(res.item()) - nll_o) / abs(nll_o))
+    got = err_d.cpu().numpy()
+    worst = max(worst, relerr(got, err_o))
+    assert np.all(got[err_o == 0.0] == 0.0) and np.all(np.abs(err_o[got == 0.0]) < 1e-30)
+    # the one-hot position is an index property: the entry below zero sits exactly at the target class
+    gv = got.reshape(F, Lp)[pat != 0][:, extra:]
+    assert np.array_equal(np.argmin(gv, axis=1), tgt[pat != 0].astype(np.int64))
+    layer.close()
+    return worst
