@@ -78,6 +78,32 @@ float orc_softmax_error(int F, int Lt, int startDOut, int K, long prob_capacity,
 void orc_softmax_backward(int F, int Lp, int Lt, int startD, int startDOut, int K, const char *pat,
                           const float *target, const float *prob, float *errors);
 
+/* WaveNet building blocks (CNNLayer.cu 1-D path, wavNetCore.cu, GatedActLayer.cu, SkipAddLayer.cu).
+   N = T*S slots.  CNN filter d has half width half_width[d] (2*hw+1 weight columns) and tap interval
+   interval[d]; weights = [P x Lw column-major | D bias], Lw = sum(2*hw+1). */
+int orc_cnn_total_width(int D, const int *half_width);
+void orc_cnn_forward(int P, int D, int S, int T, int causal, int output_tanh, float bias, const int *half_width,
+                     const int *interval, const char *pat, const float *weights, const float *x, float *conbuf,
+                     float *out);
+void orc_cnn_backward(int P, int D, int S, int T, int causal, int output_tanh, float bias, const int *half_width,
+                      const int *interval, const char *pat, const float *weights, const float *x, const float *out,
+                      float *err, float *conbuf, float *ex, float *dW);
+void orc_wavnetc_load_context(int C, int S, int N, int max_feature_length, int resolution_one, const float *source,
+                              const float *frame_index, const float *mean_std, const char *pat, float *ctx);
+void orc_wavnetc_forward(int D, int C, int N, const char *pat, const float *weights, const float *ctx,
+                         const float *conv, float *core, float *ctx_tanh, float *out);
+void orc_wavnetc_backward(int D, int C, int N, const char *pat, const float *weights, const float *ctx,
+                          const float *core, float *ctx_tanh, const float *err, float *prev_err, float *dW,
+                          float *ctx_grad);
+void orc_wavnetc_sum_context_grad(int C, int S, int resolution, int n_frames_slots, int N, const char *pat_frames,
+                                  const char *pat, const float *ctx_grad, float *frame_grad);
+void orc_gated_forward(int D, int N, const char *pat, const float *pre, float *out);
+void orc_gated_backward(int D, int N, const char *pat, const float *pre, const float *err, float *prev_err);
+void orc_skipadd_forward(long count, int n_in, const float *const *inputs, float *out, float *errors,
+                         float *errors_from_skip);
+void orc_skipadd_backward(long count, float *errors, const float *errors_from_skip, int n_pre, float *const *targets,
+                          const int *target_is_skip);
+
 #ifdef __cplusplus
 }
 #endif

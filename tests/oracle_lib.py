@@ -137,3 +137,68 @@ def softmax_error(F, Lt, startDOut, K, cap, pat, target, prob):
 
 def softmax_backward(F, Lp, Lt, startD, startDOut, K, pat, target, prob, errors):
     lib().orc_softmax_backward(F, Lp, Lt, startD, startDOut, K, cptr(pat), fptr(target), fptr(prob), fptr(errors))
+
+
+IP = C.POINTER(C.c_int)
+
+
+def iptr(a):
+    assert a.dtype == np.int32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(IP)
+
+
+def cnn_total_width(hw):
+    return int(lib().orc_cnn_total_width(len(hw), iptr(hw)))
+
+
+def cnn_forward(P, D, S, T, causal, out_tanh, bias, hw, inter, pat, W, x, conbuf, out):
+    lib().orc_cnn_forward(P, D, S, T, causal, out_tanh, C.c_float(bias), iptr(hw), iptr(inter), cptr(pat), fptr(W),
+                          fptr(x), fptr(conbuf), fptr(out))
+
+
+def cnn_backward(P, D, S, T, causal, out_tanh, bias, hw, inter, pat, W, x, out, err, conbuf, ex, dW):
+    lib().orc_cnn_backward(P, D, S, T, causal, out_tanh, C.c_float(bias), iptr(hw), iptr(inter), cptr(pat), fptr(W),
+                           fptr(x), fptr(out), fptr(err), fptr(conbuf), fptr(ex), fptr(dW))
+
+
+def wavnetc_load_context(Cdim, S, N, max_len, res_one, source, frame_index, mean_std, pat, ctx):
+    lib().orc_wavnetc_load_context(Cdim, S, N, max_len, int(res_one), fptr(source), fptr(frame_index),
+                                   fptr(mean_std), cptr(pat), fptr(ctx))
+
+
+def wavnetc_forward(D, Cdim, N, pat, W, ctx, conv, core, ctx_tanh, out):
+    lib().orc_wavnetc_forward(D, Cdim, N, cptr(pat), fptr(W), fptr(ctx), fptr(conv), fptr(core), fptr(ctx_tanh),
+                              fptr(out))
+
+
+def wavnetc_backward(D, Cdim, N, pat, W, ctx, core, ctx_tanh, err, prev_err, dW, ctx_grad):
+    lib().orc_wavnetc_backward(D, Cdim, N, cptr(pat), fptr(W), fptr(ctx), fptr(core), fptr(ctx_tanh), fptr(err),
+                               fptr(prev_err), fptr(dW), fptr(ctx_grad))
+
+
+def wavnetc_sum_context_grad(Cdim, S, resolution, n_frame_slots, N, pat_frames, pat, ctx_grad, frame_grad):
+    lib().orc_wavnetc_sum_context_grad(Cdim, S, resolution, n_frame_slots, N, cptr(pat_frames), cptr(pat),
+                                       fptr(ctx_grad), fptr(frame_grad))
+
+
+def gated_forward(D, N, pat, pre, out):
+    lib().orc_gated_forward(D, N, cptr(pat), fptr(pre), fptr(out))
+
+
+def gated_backward(D, N, pat, pre, err, prev_err):
+    lib().orc_gated_backward(D, N, cptr(pat), fptr(pre), fptr(err), fptr(prev_err))
+
+
+def _fpp(arrs):
+    return (FP * len(arrs))(*[fptr(a) for a in arrs])
+
+
+def skipadd_forward(inputs, out, errors, errors_from_skip):
+    lib().orc_skipadd_forward(C.c_long(out.size), len(inputs), _fpp(inputs), fptr(out), fptr(errors),
+                              fptr(errors_from_skip))
+
+
+def skipadd_backward(errors, errors_from_skip, targets, is_skip):
+    flags = (C.c_int * len(is_skip))(*[int(v) for v in is_skip])
+    lib().orc_skipadd_backward(C.c_long(errors.size), fptr(errors), fptr(errors_from_skip), len(targets),
+                               _fpp(targets), flags)
