@@ -150,6 +150,79 @@ int cnt_mdn_backward(cnt_mdn *h, void *stream, const float *targets, float *prev
  * number of floats in use for the current fraction. */
 float *cnt_mdn_unit_buffer(cnt_mdn *h, int unit, int which, long *count);
 
+/* ---- 1-D (dilated, optionally causal) convolution layer -------------------------------------------
+ * CNNLayer<TDevice>, 1-D path (layers/CNNLayer.cu).  Filter d has half width half_width[d]
+ * ("window_width", 2*hw+1 weight columns, the columns after the centre are dead when causal) and tap
+ * interval interval[d] ("window_tap_interval").  weights = [P x Lw column-major | D bias] with
+ * Lw = sum(2*hw+1): the layout the reference stores under "internal" (:971-978).  The 2-D
+ * (window_height) path and repeat_padding are not built; at most 8 live taps per filter. */
+typedef struct cnt_cnn cnt_cnn;
+typedef struct {
+    int P;            /* preceding layer size                   */
+    int D;            /* number of filters = layer size         */
+    int S;            /* parallel sequences                     */
+    int maxT;         /* maxSeqLength                           */
+    int causal;       /* "causal"                               */
+    int output_tanh;  /* "tanhoutput" (default 1 in the reference, layers/CNNLayer.cu:932) */
+    float bias;       /* the layer's constant bias input        */
+} cnt_cnn_desc;
+int cnt_cnn_create(const cnt_cnn_desc *desc, const int *half_width, const int *interval, cnt_cnn **out);
+int cnt_cnn_destroy(cnt_cnn *h);
+long cnt_cnn_weight_count(const cnt_cnn *h);
+/* CNNLayer::computeForwardPass (layers/CNNLayer.cu:1099-1224): outputs (D x T*S); padding slots are left
+ * untouched, as in the reference. */
+int cnt_cnn_forward(cnt_cnn *h, void *stream, const char *patTypes, int curT, const float *weights,
+                    const float *x, float *outputs);
+/* CNNLayer::computeBackwardPass (layers/CNNLayer.cu:1409-1597): output_errors becomes tanh'(y)*err in
+ * place when output_tanh is set; prev_errors is the preceding layer's whole error buffer
+ * (P x maxT*S, cleared beyond the current slots, may be NULL); weight_updates is overwritten. */
+int cnt_cnn_backward(cnt_cnn *h, void *stream, const char *patTypes, int curT, const float *weights,
+                     const float *x, const float *outputs, float *output_errors, float *prev_errors,
+                     float *weight_updates);
+
+/* ---- gated activation, conditioned ("wavnetc") and plain ("gatedact") ------------------------------
+ * WavNetCore<TDevice> (layers/wavNetCore.cu) and GatedActLayer<TDevice> (layers/GatedActLayer.cu).
+ * D = layer size, the preceding layer has 2D units; C = contextDim; N = T*S slots.
+ * The caller owns the buffers the reference keeps as members: core_buf (m_coreBuf, 2D x N),
+ * ctx_tanh (m_contextTanhBuf, 2D x N), ctx (the first core's m_contextBuf, C x N). */
+/* loadLinguisticFeature (layers/wavNetCore.cu:143-190, driver :455-492): ctx[slot] = source frame
+ * frame_index[slot] of the slot's sequence (or slot itself when resolution_one), optionally
+ * (x - mean) / std with mean_std = [C means | C std]; 0 on padding slots. */
+int cnt_wavnetc_load_context(void *stream, int C, int S, int N, int max_feature_length, int resolution_one,
+                             const float *source, const float *frame_index, const float *mean_std,
+                             const char *patTypes, float *ctx);
+/* WavNetCore::computeForwardPass (layers/wavNetCore.cu:629-711). weights is C x 2D column-major.
+ * ctx_tanh may be NULL outside training.  C == 0: unconditioned. */
+int cnt_wavnetc_forward(void *stream, int D, int C, int N, const char *patTypes, const float *weights,
+                        const float *ctx, const float *conv_outputs, float *core_buf, float *ctx_tanh,
+                        float *outputs);
+/* WavNetCore::computeBackwardPass (layers/wavNetCore.cu:801-916): prev_errors (2D x N) is overwritten;
+ * ctx_tanh is overwritten with the gradient w.r.t. W^T ctx; weight_updates (C x 2D) is overwritten;
+ * if ctx_grad (C x N, the first core's m_contextGraBuf) is given, W * gradient is added to it. */
+int cnt_wavnetc_backward(void *stream, int D, int C, int N, const char *patTypes, const float *weights,
+                         const float *ctx, const float *core_buf, float *ctx_tanh, const float *output_errors,
+                         float *prev_errors, float *weight_updates, float *ctx_grad);
+/* SumGradientsForExternalInput (layers/wavNetCore.cu:237-270, driver :895-913): frame_grad (C x
+ * n_frame_slots) = sum of ctx_grad over the `resolution` samples of each frame. */
+int cnt_wavnetc_sum_context_grad(void *stream, int C, int S, int resolution, int n_frame_slots, int N,
+                                 const char *pat_frames, const char *patTypes, const float *ctx_grad,
+                                 float *frame_grad);
+/* GatedActLayer::computeForwardPass / computeBackwardPass (layers/GatedActLayer.cu:177-263). */
+int cnt_gatedact_forward(void *stream, int D, int N, const char *patTypes, const float *pre, float *outputs);
+int cnt_gatedact_backward(void *stream, int D, int N, const char *patTypes, const float *pre,
+                          const float *output_errors, float *prev_errors);
+
+/* ---- skip-add ---------------------------------------------------------------------------------------
+ * SkipAddLayer<TDevice> (layers/SkipAddLayer.cu).  `inputs` / `targets` are HOST arrays of device
+ * pointers (at most 8).  Forward (:186-240): outputs = sum of inputs, errors and errors_from_skip
+ * (SkipLayer::outputErrorsFromSkipLayer) are cleared.  Backward (:305-346): errors += errors_from_skip;
+ * predecessors in reverse order: a skip layer's errors_from_skip buffer (target_is_skip = 1) is added
+ * to, any other layer's error buffer is overwritten. */
+int cnt_skipadd_forward(void *stream, long count, int n_in, const float *const *inputs, float *outputs,
+                        float *errors, float *errors_from_skip);
+int cnt_skipadd_backward(void *stream, long count, float *errors, const float *errors_from_skip, int n_pre,
+                         float *const *targets, const int *target_is_skip);
+
 #ifdef __cplusplus
 }
 #endif

@@ -17,6 +17,11 @@ class MdnDesc(C.Structure):
     _fields_ = [("Lp", C.c_int), ("Lt", C.c_int), ("S", C.c_int), ("maxT", C.c_int), ("tie_variance", C.c_int)]
 
 
+class CnnDesc(C.Structure):
+    _fields_ = [("P", C.c_int), ("D", C.c_int), ("S", C.c_int), ("maxT", C.c_int), ("causal", C.c_int),
+                ("output_tanh", C.c_int), ("bias", C.c_float)]
+
+
 class LstmDesc(C.Structure):
     _fields_ = [("P", C.c_int), ("L", C.c_int), ("bidir", C.c_int), ("S", C.c_int), ("maxT", C.c_int),
                 ("bias", C.c_float)]
@@ -54,6 +59,19 @@ _SIGNATURES = {
     "cnt_mdn_calculate_error": (I, [VP, VP, VP, VP]),
     "cnt_mdn_backward": (I, [VP, VP, VP, VP]),
     "cnt_mdn_unit_buffer": (VP, [VP, I, I, C.POINTER(C.c_long)]),
+    "cnt_cnn_create": (I, [C.POINTER(CnnDesc), C.POINTER(I), C.POINTER(I), C.POINTER(VP)]),
+    "cnt_cnn_destroy": (I, [VP]),
+    "cnt_cnn_weight_count": (C.c_long, [VP]),
+    "cnt_cnn_forward": (I, [VP, VP, VP, I, VP, VP, VP]),
+    "cnt_cnn_backward": (I, [VP, VP, VP, I, VP, VP, VP, VP, VP, VP]),
+    "cnt_wavnetc_load_context": (I, [VP, I, I, I, I, I, VP, VP, VP, VP, VP]),
+    "cnt_wavnetc_forward": (I, [VP, I, I, I, VP, VP, VP, VP, VP, VP, VP]),
+    "cnt_wavnetc_backward": (I, [VP, I, I, I, VP, VP, VP, VP, VP, VP, VP, VP, VP]),
+    "cnt_wavnetc_sum_context_grad": (I, [VP, I, I, I, I, I, VP, VP, VP, VP]),
+    "cnt_gatedact_forward": (I, [VP, I, I, VP, VP, VP]),
+    "cnt_gatedact_backward": (I, [VP, I, I, VP, VP, VP, VP]),
+    "cnt_skipadd_forward": (I, [VP, C.c_long, I, C.POINTER(VP), VP, VP, VP]),
+    "cnt_skipadd_backward": (I, [VP, C.c_long, VP, VP, I, C.POINTER(VP), C.POINTER(I)]),
 }
 
 
@@ -182,6 +200,81 @@ class Lstm:
         n = self.H * self.T * self.S
         torch.cuda.synchronize()
         return torch.as_tensor(_DeviceArray(p, n), device="cuda").clone()
+
+
+class Cnn:
+    """Thin owner of a cnt_cnn handle (1-D convolution layer)."""
+
+    def __init__(self, P, half_width, interval, S, maxT, causal, output_tanh, bias=1.0):
+        D = len(half_width)
+        self.P, self.D, self.S, self.maxT = P, D, S, maxT
+        self.handle = VP()
+        desc = CnnDesc(P, D, S, maxT, int(causal), int(output_tanh), bias)
+        hw = (I * D)(*[int(v) for v in half_width])
+        it = (I * D)(*[int(v) for v in interval])
+        check(lib().cnt_cnn_create(C.byref(desc), hw, it, C.byref(self.handle)))
+        self.weight_count = int(lib().cnt_cnn_weight_count(self.handle))
+
+    def close(self):
+        if self.handle:
+            lib().cnt_cnn_destroy(self.handle)
+            self.handle = VP()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def forward(self, pat, T, W, x, out, stream=None):
+        check(lib().cnt_cnn_forward(self.handle, stream_ptr(stream), ptr(pat), T, ptr(W), ptr(x), ptr(out)))
+
+    def backward(self, pat, T, W, x, out, err, prev_err, dW, stream=None):
+        check(lib().cnt_cnn_backward(self.handle, stream_ptr(stream), ptr(pat), T, ptr(W), ptr(x), ptr(out), ptr(err),
+                                     ptr(prev_err), ptr(dW)))
+
+
+def wavnetc_load_context(Cdim, S, N, max_len, res_one, source, frame_index, mean_std, pat, ctx, stream=None):
+    check(lib().cnt_wavnetc_load_context(stream_ptr(stream), Cdim, S, N, max_len, int(res_one), ptr(source),
+                                         ptr(frame_index), ptr(mean_std), ptr(pat), ptr(ctx)))
+
+
+def wavnetc_forward(D, Cdim, N, pat, W, ctx, conv, core, ctx_tanh, out, stream=None):
+    check(lib().cnt_wavnetc_forward(stream_ptr(stream), D, Cdim, N, ptr(pat), ptr(W), ptr(ctx), ptr(conv), ptr(core),
+                                    ptr(ctx_tanh), ptr(out)))
+
+
+def wavnetc_backward(D, Cdim, N, pat, W, ctx, core, ctx_tanh, err, prev_err, dW, ctx_grad, stream=None):
+    check(lib().cnt_wavnetc_backward(stream_ptr(stream), D, Cdim, N, ptr(pat), ptr(W), ptr(ctx), ptr(core),
+                                     ptr(ctx_tanh), ptr(err), ptr(prev_err), ptr(dW), ptr(ctx_grad)))
+
+
+def wavnetc_sum_context_grad(Cdim, S, resolution, n_frame_slots, N, pat_frames, pat, ctx_grad, frame_grad, stream=None):
+    check(lib().cnt_wavnetc_sum_context_grad(stream_ptr(stream), Cdim, S, resolution, n_frame_slots, N,
+                                             ptr(pat_frames), ptr(pat), ptr(ctx_grad), ptr(frame_grad)))
+
+
+def gatedact_forward(D, N, pat, pre, out, stream=None):
+    check(lib().cnt_gatedact_forward(stream_ptr(stream), D, N, ptr(pat), ptr(pre), ptr(out)))
+
+
+def gatedact_backward(D, N, pat, pre, err, prev_err, stream=None):
+    check(lib().cnt_gatedact_backward(stream_ptr(stream), D, N, ptr(pat), ptr(pre), ptr(err), ptr(prev_err)))
+
+
+def _ptr_array(tensors):
+    return (VP * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def skipadd_forward(inputs, out, errors, errors_from_skip, stream=None):
+    check(lib().cnt_skipadd_forward(stream_ptr(stream), out.numel(), len(inputs), _ptr_array(inputs), ptr(out),
+                                    ptr(errors), ptr(errors_from_skip)))
+
+
+def skipadd_backward(errors, errors_from_skip, targets, is_skip, stream=None):
+    flags = (I * len(is_skip))(*[int(v) for v in is_skip])
+    check(lib().cnt_skipadd_backward(stream_ptr(stream), errors.numel(), ptr(errors), ptr(errors_from_skip),
+                                     len(targets), _ptr_array(targets), flags))
 
 
 class Mdn:

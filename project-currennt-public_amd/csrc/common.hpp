@@ -112,15 +112,30 @@ struct ProfileScope {
 constexpr int kGemmMaxSeg = 8;
 constexpr int kGemmMaxProb = 8;
 
-enum GemmEpilogue { EPI_STORE = 0, EPI_ADD = 1, EPI_ATOMIC = 2, EPI_BIAS_ACT = 3 };
+enum GemmEpilogue {
+    EPI_STORE = 0,          // C = acc
+    EPI_ADD = 1,            // C += acc
+    EPI_ATOMIC = 2,         // atomicAdd(C, acc)   (split-K; C zeroed by the caller)
+    EPI_BIAS_ACT = 3,       // C = act(acc + bias_scale * bias_vec[row])
+    EPI_BIAS_ACT_SKIP = 4,  // as above, but columns whose pattern type is "none" are left untouched
+    EPI_CONTEXT = 5         // th = tanh(acc); aux_out = th; C = aux_in + th; both 0 on "none" columns
+};
 
 struct GemmProblem {
     const float *A[kGemmMaxSeg];
     const float *B[kGemmMaxSeg];
+    int b_shift[kGemmMaxSeg];  // masked mode: time-slot shift of the B operand per operand pair
     float *C;
-    const float *bias_vec;  // EPI_BIAS_ACT: C = act(acc + bias_scale * bias_vec[row])
+    const float *bias_vec;
+    const float *aux_in;  // EPI_CONTEXT, same layout as C
+    float *aux_out;       // EPI_CONTEXT, may be NULL
 };
 
+// Masked mode (dilated convolutions without a materialised column buffer): one index of the B operand is a
+// time slot u -- its row index (b_time_on_k = 0) or its k index (b_time_on_k = 1).  The element is read from
+// slot u + b_shift and counts only if pat[u] != 0, 0 <= u + b_shift < n_slots and pat[u + b_shift] != 0;
+// otherwise it is 0.  This is exactly the set of entries the reference scatters into its column buffer
+// (layers/CNNLayer.cu:182-237).
 struct GemmArgs {
     int m, n, k;
     int lda, ldb, ldc;
@@ -128,6 +143,8 @@ struct GemmArgs {
     int nseg, nprob, splitk;
     int epilogue, act;
     float bias_scale;
+    int masked, b_time_on_k, n_slots;
+    const char *pat;  // masked mode and the *_SKIP / CONTEXT epilogues
     GemmProblem prob[kGemmMaxProb];
     const char *label;  // name under which the launch is timed when profiling is on (may be NULL)
 };

@@ -37,8 +37,11 @@ struct TileStage {
     static constexpr int NLOAD = (128 * BK) / (NTHREADS * VEC);
     typename VecT<VEC>::type r[NLOAD];
 
+    // shift / pat / n_slots: masked mode (pat == nullptr switches it off); time_on_k selects which index is
+    // the time slot
     __device__ __forceinline__ void load(const float *__restrict__ base, int ld, int row0, int k0,
-                                         int rows_total, int k_total, int tid) {
+                                         int rows_total, int k_total, int tid, const char *__restrict__ pat = nullptr,
+                                         int shift = 0, int n_slots = 0, bool time_on_k = false) {
         if (KCONTIG) {
             constexpr int TPR = BK / VEC;        // threads per row
             constexpr int RPP = NTHREADS / TPR;  // rows per pass
@@ -48,8 +51,24 @@ struct TileStage {
             for (int p = 0; p < NLOAD; ++p) {
                 const int row = row0 + rr + p * RPP;
                 typename VecT<VEC>::type v = {};
-                if (row < rows_total && (k0 + kq) < k_total)
-                    v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)row * ld + k0 + kq);
+                if (row < rows_total && (k0 + kq) < k_total) {
+                    if (!pat) {
+                        v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)row * ld + k0 + kq);
+                    } else if (!time_on_k) {
+                        const int src = row + shift;
+                        if (pat[row] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
+                            v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)src * ld + k0 + kq);
+                    } else {
+                        // vector along k = consecutive time slots: element-wise masking
+                        float *e = reinterpret_cast<float *>(&v);
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) {
+                            const int u = k0 + kq + j, src = u + shift;
+                            if (pat[u] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
+                                e[j] = base[(size_t)row * ld + src];
+                        }
+                    }
+                }
                 r[p] = v;
             }
         } else {
@@ -61,8 +80,23 @@ struct TileStage {
             for (int p = 0; p < NLOAD; ++p) {
                 const int k = k0 + kk + p * KPP;
                 typename VecT<VEC>::type v = {};
-                if (k < k_total && (row0 + rq) < rows_total)
-                    v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)k * ld + row0 + rq);
+                if (k < k_total && (row0 + rq) < rows_total) {
+                    if (!pat) {
+                        v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)k * ld + row0 + rq);
+                    } else if (time_on_k) {
+                        const int src = k + shift;
+                        if (pat[k] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
+                            v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)src * ld + row0 + rq);
+                    } else {
+                        float *e = reinterpret_cast<float *>(&v);
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) {
+                            const int u = row0 + rq + j, src = u + shift;
+                            if (pat[u] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
+                                e[j] = base[(size_t)k * ld + src];
+                        }
+                    }
+                }
                 r[p] = v;
             }
         }
@@ -126,12 +160,14 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
 
     TileStage<VA, AK> sa;
     TileStage<VB, BK_> sb;
+    const char *mask_pat = args.masked ? args.pat : nullptr;
 
     {
         const int seg = it_begin / kt_per_seg;
         const int k0 = (it_begin % kt_per_seg) * BK;
         sa.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
-        sb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid);
+        sb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid, mask_pat, pb.b_shift[seg], args.n_slots,
+                args.b_time_on_k != 0);
         sa.store(lds_a[0], tid);
         sb.store(lds_b[0], tid);
     }
@@ -147,7 +183,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
             const int seg = (it + 1) / kt_per_seg;
             const int k0 = ((it + 1) % kt_per_seg) * BK;
             sa.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
-            sb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid);
+            sb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid, mask_pat, pb.b_shift[seg], args.n_slots,
+                    args.b_time_on_k != 0);
         }
 
         float4 fa[2][2], fb[2][2];
@@ -188,20 +225,31 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
         const int m = m0 + wm * 64 + i * 32 + frag_row;
         if (m >= args.m) continue;
         float bterm = 0.0f;
-        if (args.epilogue == EPI_BIAS_ACT) bterm = args.bias_scale * pb.bias_vec[m];
+        if (args.epilogue == EPI_BIAS_ACT || args.epilogue == EPI_BIAS_ACT_SKIP)
+            bterm = args.bias_scale * pb.bias_vec[m];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int n = n0 + wn * 64 + j * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
                 if (n >= args.n) continue;
-                float *dst = C + (size_t)n * args.ldc + m;
+                const size_t idx = (size_t)n * args.ldc + m;
+                float *dst = C + idx;
                 const float v = acc[i][j][r];
                 switch (args.epilogue) {
                     case EPI_STORE: *dst = v; break;
                     case EPI_ADD: *dst = *dst + v; break;
                     case EPI_ATOMIC: atomicAdd(dst, v); break;
-                    default: *dst = act_fn(args.act, v + bterm); break;
+                    case EPI_BIAS_ACT: *dst = act_fn(args.act, v + bterm); break;
+                    case EPI_BIAS_ACT_SKIP:
+                        if (args.pat[n] != 0) *dst = act_fn(args.act, v + bterm);
+                        break;
+                    default: {  // EPI_CONTEXT
+                        const bool valid = args.pat[n] != 0;
+                        const float th = valid ? tanh_act(v) : 0.0f;
+                        if (pb.aux_out) pb.aux_out[idx] = th;
+                        *dst = valid ? pb.aux_in[idx] + th : 0.0f;
+                    } break;
                 }
             }
         }

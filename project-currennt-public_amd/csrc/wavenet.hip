@@ -1,0 +1,504 @@
+// WaveNet building blocks for gfx950: 1-D dilated (causal) convolution layer, conditioned gated
+// activation ("wavnetc"), its unconditioned twin ("gatedact"), and the skip-add fan-in / fan-out.
+//
+// Reference behaviour: layers/CNNLayer.cu (functors :78-246, forward :1099-1224, backward :1409-1597),
+// layers/wavNetCore.cu (functors :69-270, forward :629-711, backward :801-916),
+// layers/GatedActLayer.cu (:64-121, :177-263), layers/SkipAddLayer.cu (:186-240, :305-346).
+//
+// The reference materialises a (sum of window widths) x (T*S) column buffer per layer, zero-fills it
+// and scatters the deltas into it before two matrix products.  Here the column buffer never exists:
+// every window tap is one operand pair of the MFMA GEMM whose B-side loader applies the tap's time
+// shift and the padding mask while staging the tile, so the deltas are read straight from the error
+// buffer.  The dead "future" tap of a causal window is never computed; its gradient columns are the
+// zeros of the weight-update clear.  The elementwise parts are fused streaming kernels.
+#include "common.hpp"
+
+#include <cstring>
+#include <new>
+#include <vector>
+
+namespace cnt {
+namespace {
+
+inline int stream_blocks(size_t count) {
+    size_t b = (count + 255) / 256;
+    if (b > 8192) b = 8192;
+    if (b < 1) b = 1;
+    return (int)b;
+}
+
+__global__ void tanh_delta_kernel(float *__restrict__ err, const float *__restrict__ y, size_t count) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) err[i] = tanh_deriv(y[i]) * err[i];
+}
+
+// conditioning frame of every slot (wavNetCore.cu:143-190)
+__global__ void load_context_kernel(int C, int S, size_t count, int max_feature_length, int resolution_one,
+                                    const float *__restrict__ source, const float *__restrict__ frame_index,
+                                    const float *__restrict__ mean_std, const char *__restrict__ pat,
+                                    float *__restrict__ ctx) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const int t = (int)(i / C), c = (int)(i % C);
+        float v = 0.0f;
+        if (pat[t] != 0) {
+            const float fi = frame_index[t];
+            const int feat = resolution_one ? t : (int)(fi * S + (t % S));
+            if (fi >= max_feature_length) {
+                v = 0.0f;
+            } else if (mean_std) {
+                const float sd = mean_std[c + C];
+                v = (float)((source[(size_t)feat * C + c] - mean_std[c]) / (sd < 1e-5f ? 1.0 : (double)sd));
+            } else {
+                v = source[(size_t)feat * C + c];
+            }
+        }
+        ctx[i] = v;
+    }
+}
+
+// z = tanh(y1) * sigmoid(y2), 0 on padding slots; pre is 2D x N
+__global__ void gated_forward_kernel(int D, size_t count, const char *__restrict__ pat, const float *__restrict__ pre,
+                                     float *__restrict__ out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const size_t t = i / D, d = i % D;
+        out[i] = (pat[t] == 0) ? 0.0f : tanh_act(pre[t * 2 * D + d]) * logistic(pre[t * 2 * D + D + d]);
+    }
+}
+
+// unconditioned core: core = conv (0 on padding), ctx_tanh = 0
+__global__ void core_copy_kernel(int D2, size_t count, const char *__restrict__ pat, const float *__restrict__ conv,
+                                 float *__restrict__ core, float *__restrict__ ctx_tanh) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        core[i] = (pat[i / D2] == 0) ? 0.0f : conv[i] + 0.0f;
+        if (ctx_tanh) ctx_tanh[i] = 0.0f;
+    }
+}
+
+// One thread per (slot, d): both halves of the gate gradient from the same three loads, and -- when the
+// core is conditioned -- the gradient through tanh(X_c) written over ctx_tanh in the same pass.
+__global__ void gated_backward_kernel(int D, size_t count, const char *__restrict__ pat, const float *__restrict__ pre,
+                                      const float *__restrict__ err, float *__restrict__ prev_err,
+                                      float *__restrict__ ctx_tanh) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const size_t t = i / D, d = i % D;
+        const size_t i1 = t * 2 * D + d, i2 = i1 + D;
+        float g1 = 0.0f, g2 = 0.0f;
+        if (pat[t] != 0) {
+            const float th = tanh_act(pre[i1]);
+            const float sg = logistic(pre[i2]);
+            const float e = err[i];
+            g1 = (1.0f - th * th) * sg * e;
+            g2 = th * (sg * (1.0f - sg)) * e;
+        }
+        prev_err[i1] = g1;
+        prev_err[i2] = g2;
+        if (ctx_tanh) {
+            ctx_tanh[i1] = tanh_deriv(ctx_tanh[i1]) * g1;
+            ctx_tanh[i2] = tanh_deriv(ctx_tanh[i2]) * g2;
+        }
+    }
+}
+
+__global__ void sum_context_grad_kernel(int C, int S, int resolution, size_t count, int N,
+                                        const char *__restrict__ pat_frames, const char *__restrict__ pat,
+                                        const float *__restrict__ ctx_grad, float *__restrict__ frame_grad) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const int f = (int)(i / C), c = (int)(i % C);
+        float acc = 0.0f;
+        if (pat_frames[f] != 0) {
+            const int rel = f / S, s = f % S;
+            for (int k = 0; k < resolution; ++k) {
+                const int idx = (rel * resolution + k) * S + s;
+                if (idx < N && pat[idx] != 0) acc += ctx_grad[(size_t)idx * C + c];
+            }
+        }
+        frame_grad[i] = acc;
+    }
+}
+
+constexpr int kSkipMaxFan = 8;
+struct SkipPtrs {
+    const float *in[kSkipMaxFan];
+    float *target[kSkipMaxFan];
+    int is_skip[kSkipMaxFan];
+    int n;
+};
+
+__global__ void skipadd_forward_kernel(size_t count, SkipPtrs p, float *__restrict__ out, float *__restrict__ errors,
+                                       float *__restrict__ errors_from_skip) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        float acc = 0.0f;
+        for (int k = 0; k < p.n; ++k) acc += p.in[k][i];
+        out[i] = acc;
+        if (errors) errors[i] = 0.0f;
+        if (errors_from_skip) errors_from_skip[i] = 0.0f;
+    }
+}
+
+__global__ void skipadd_backward_kernel(size_t count, SkipPtrs p, float *__restrict__ errors,
+                                        const float *__restrict__ errors_from_skip) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const float e = errors_from_skip[i] + errors[i];
+        errors[i] = e;
+        for (int k = p.n - 1; k >= 0; --k) {
+            if (p.is_skip[k]) p.target[k][i] = e + p.target[k][i];
+            else p.target[k][i] = e;
+        }
+    }
+}
+
+}  // namespace
+}  // namespace cnt
+
+// ---------------------------------------------------------------------------------------------------
+// CNN layer handle: filters grouped into runs of equal half width and tap interval
+// ---------------------------------------------------------------------------------------------------
+struct cnt_cnn_group {
+    int d0, d1;   // filter range
+    int hw, dil;  // half width, tap interval
+    int col0;     // first weight column of the run
+};
+
+struct cnt_cnn {
+    cnt_cnn_desc desc;
+    int Lw;
+    std::vector<cnt_cnn_group> groups;
+};
+
+extern "C" {
+
+int cnt_cnn_create(const cnt_cnn_desc *desc, const int *half_width, const int *interval, cnt_cnn **out) {
+    using namespace cnt;
+    CNT_REQUIRE(desc && half_width && interval && out, "cnn_create: null argument");
+    CNT_REQUIRE(desc->P > 0 && desc->D > 0 && desc->S > 0 && desc->maxT > 0, "cnn_create: non-positive size");
+    cnt_cnn *h = new (std::nothrow) cnt_cnn();
+    CNT_REQUIRE(h != nullptr, "cnn_create: out of host memory");
+    h->desc = *desc;
+    int col = 0;
+    for (int d = 0; d < desc->D; ++d) {
+        const int hw = half_width[d], dil = interval[d];
+        const int taps = desc->causal > 0 ? hw + 1 : 2 * hw + 1;
+        if (hw < 0 || dil < 1 || taps > kGemmMaxSeg) {
+            set_error("cnn_create: filter %d has half width %d, tap interval %d; supported: interval >= 1 and at most %d "
+                      "live taps per filter", d, hw, dil, kGemmMaxSeg);
+            delete h;
+            return CNT_ERR_ARG;
+        }
+        if (h->groups.empty() || h->groups.back().hw != hw || h->groups.back().dil != dil) {
+            cnt_cnn_group g = {d, d + 1, hw, dil, col};
+            h->groups.push_back(g);
+        } else {
+            h->groups.back().d1 = d + 1;
+        }
+        col += 2 * hw + 1;
+    }
+    h->Lw = col;
+    *out = h;
+    return CNT_OK;
+}
+
+int cnt_cnn_destroy(cnt_cnn *h) {
+    delete h;
+    return CNT_OK;
+}
+
+long cnt_cnn_weight_count(const cnt_cnn *h) { return h ? (long)h->desc.P * h->Lw + h->desc.D : 0; }
+
+int cnt_cnn_forward(cnt_cnn *h, void *stream_, const char *patTypes, int curT, const float *weights, const float *x,
+                    float *outputs) {
+    using namespace cnt;
+    CNT_REQUIRE(h && patTypes && weights && x && outputs, "cnn_forward: null argument");
+    CNT_REQUIRE(curT >= 1 && curT <= h->desc.maxT, "cnn_forward: curT %d outside 1..%d", curT, h->desc.maxT);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const cnt_cnn_desc &d = h->desc;
+    const int P = d.P, D = d.D, S = d.S, N = curT * S;
+    for (const cnt_cnn_group &g : h->groups) {
+        GemmArgs ga = {};
+        ga.m = g.d1 - g.d0; ga.n = N; ga.k = P;
+        ga.a_kcontig = 1; ga.lda = (2 * g.hw + 1) * P;  // filter d, tap column c: weights[(col0 + (d-d0)*(2hw+1) + c) * P + p]
+        ga.b_kcontig = 1; ga.ldb = P;
+        ga.ldc = D;
+        ga.nprob = 1; ga.splitk = 1;
+        ga.epilogue = EPI_BIAS_ACT_SKIP; ga.act = d.output_tanh ? ACT_TANH : ACT_IDENTITY; ga.bias_scale = d.bias;
+        ga.masked = 1; ga.b_time_on_k = 0; ga.n_slots = N; ga.pat = patTypes;
+        int seg = 0;
+        for (int shift = -g.hw; shift <= (d.causal > 0 ? 0 : g.hw); ++shift, ++seg) {
+            ga.prob[0].A[seg] = weights + (size_t)(g.col0 + g.hw + shift) * P;
+            ga.prob[0].B[seg] = x;
+            ga.prob[0].b_shift[seg] = shift * g.dil * S;
+        }
+        ga.nseg = seg;
+        ga.prob[0].C = outputs + g.d0;
+        ga.prob[0].bias_vec = weights + (size_t)P * h->Lw + g.d0;
+        ga.label = "gemm:cnn_forward";
+        CNT_TRY(gemm_launch(stream, ga));
+    }
+    return CNT_OK;
+}
+
+int cnt_cnn_backward(cnt_cnn *h, void *stream_, const char *patTypes, int curT, const float *weights, const float *x,
+                     const float *outputs, float *output_errors, float *prev_errors, float *weight_updates) {
+    using namespace cnt;
+    CNT_REQUIRE(h && patTypes && weights && x && outputs && output_errors && weight_updates,
+                "cnn_backward: null argument");
+    CNT_REQUIRE(curT >= 1 && curT <= h->desc.maxT, "cnn_backward: curT %d outside 1..%d", curT, h->desc.maxT);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const cnt_cnn_desc &d = h->desc;
+    const int P = d.P, D = d.D, S = d.S, N = curT * S;
+    const size_t count = (size_t)D * N;
+
+    if (d.output_tanh) {
+        ProfileScope prof(stream, "cnn_tanh_delta");
+        hipLaunchKernelGGL(tanh_delta_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, output_errors, outputs,
+                           count);
+        CNT_HIP(hipGetLastError());
+    }
+
+    if (prev_errors) {
+        // the reference clears the whole preceding error buffer, then overwrites the current slots
+        const size_t used = (size_t)P * N, cap = (size_t)P * d.maxT * S;
+        if (cap > used) CNT_TRY(fill_zero(stream, prev_errors + used, cap - used));
+        bool first = true;
+        for (const cnt_cnn_group &g : h->groups) {
+            GemmArgs ga = {};
+            ga.m = P; ga.n = N; ga.k = g.d1 - g.d0;
+            ga.a_kcontig = 0; ga.lda = (2 * g.hw + 1) * P;
+            ga.b_kcontig = 1; ga.ldb = D;
+            ga.ldc = P;
+            ga.nprob = 1; ga.splitk = 1;
+            ga.epilogue = first ? EPI_STORE : EPI_ADD;
+            ga.masked = 1; ga.b_time_on_k = 0; ga.n_slots = N; ga.pat = patTypes;
+            int seg = 0;
+            for (int shift = -g.hw; shift <= (d.causal > 0 ? 0 : g.hw); ++shift, ++seg) {
+                ga.prob[0].A[seg] = weights + (size_t)(g.col0 + g.hw + shift) * P;
+                ga.prob[0].B[seg] = output_errors + g.d0;
+                // column (slot u, tap shift) of the reference's buffer holds the delta of slot u - shift*dil*S
+                ga.prob[0].b_shift[seg] = -shift * g.dil * S;
+            }
+            ga.nseg = seg;
+            ga.prob[0].C = prev_errors;
+            ga.label = "gemm:cnn_prev_errors";
+            CNT_TRY(gemm_launch(stream, ga));
+            first = false;
+        }
+    }
+
+    CNT_TRY(fill_zero(stream, weight_updates, (size_t)P * h->Lw + D));
+    for (const cnt_cnn_group &g : h->groups) {
+        GemmArgs ga = {};
+        ga.m = P; ga.n = g.d1 - g.d0; ga.k = N;
+        ga.a_kcontig = 0; ga.lda = P;
+        ga.b_kcontig = 0; ga.ldb = D;
+        ga.ldc = (2 * g.hw + 1) * P;
+        ga.nseg = 1;
+        ga.epilogue = EPI_ATOMIC;
+        ga.masked = 1; ga.b_time_on_k = 1; ga.n_slots = N; ga.pat = patTypes;
+        int pr = 0;
+        for (int shift = -g.hw; shift <= (d.causal > 0 ? 0 : g.hw); ++shift, ++pr) {
+            ga.prob[pr].A[0] = x;
+            ga.prob[pr].B[0] = output_errors + g.d0;
+            ga.prob[pr].b_shift[0] = -shift * g.dil * S;
+            ga.prob[pr].C = weight_updates + (size_t)(g.col0 + g.hw + shift) * P;
+        }
+        ga.nprob = pr;
+        const int tiles = ((P + 127) / 128) * ((ga.n + 127) / 128) * pr;
+        int s = (512 + tiles - 1) / tiles;
+        const int kt = (N + 15) / 16;
+        ga.splitk = s > kt ? kt : s;
+        ga.label = "gemm:cnn_dW";
+        CNT_TRY(gemm_launch(stream, ga));
+    }
+    // bias gradient over every slot, padding included, as the reference's ones-vector product does
+    return column_sum(stream, output_errors, D, N, d.bias, weight_updates + (size_t)P * h->Lw);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Conditioned / unconditioned gated activation
+// ---------------------------------------------------------------------------------------------------
+int cnt_wavnetc_load_context(void *stream_, int C, int S, int N, int max_feature_length, int resolution_one,
+                             const float *source, const float *frame_index, const float *mean_std,
+                             const char *patTypes, float *ctx) {
+    using namespace cnt;
+    CNT_REQUIRE(source && frame_index && patTypes && ctx, "wavnetc_load_context: null argument");
+    CNT_REQUIRE(C > 0 && S > 0 && N > 0, "wavnetc_load_context: non-positive size");
+    const size_t count = (size_t)C * N;
+    hipLaunchKernelGGL(load_context_kernel, dim3(stream_blocks(count)), dim3(256), 0, static_cast<hipStream_t>(stream_),
+                       C, S, count, max_feature_length, resolution_one, source, frame_index, mean_std, patTypes, ctx);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+int cnt_gatedact_forward(void *stream_, int D, int N, const char *patTypes, const float *pre, float *outputs) {
+    using namespace cnt;
+    CNT_REQUIRE(patTypes && pre && outputs, "gatedact_forward: null argument");
+    CNT_REQUIRE(D > 0 && N > 0, "gatedact_forward: non-positive size");
+    const size_t count = (size_t)D * N;
+    ProfileScope prof(static_cast<hipStream_t>(stream_), "gated_forward");
+    hipLaunchKernelGGL(gated_forward_kernel, dim3(stream_blocks(count)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream_), D, count, patTypes, pre, outputs);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+int cnt_gatedact_backward(void *stream_, int D, int N, const char *patTypes, const float *pre, const float *output_errors,
+                          float *prev_errors) {
+    using namespace cnt;
+    CNT_REQUIRE(patTypes && pre && output_errors && prev_errors, "gatedact_backward: null argument");
+    CNT_REQUIRE(D > 0 && N > 0, "gatedact_backward: non-positive size");
+    const size_t count = (size_t)D * N;
+    ProfileScope prof(static_cast<hipStream_t>(stream_), "gated_backward");
+    hipLaunchKernelGGL(gated_backward_kernel, dim3(stream_blocks(count)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream_), D, count, patTypes, pre, output_errors, prev_errors,
+                       static_cast<float *>(nullptr));
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+int cnt_wavnetc_forward(void *stream_, int D, int C, int N, const char *patTypes, const float *weights, const float *ctx,
+                        const float *conv_outputs, float *core_buf, float *ctx_tanh, float *outputs) {
+    using namespace cnt;
+    CNT_REQUIRE(patTypes && conv_outputs && core_buf && outputs, "wavnetc_forward: null argument");
+    CNT_REQUIRE(D > 0 && N > 0 && C >= 0, "wavnetc_forward: bad size");
+    CNT_REQUIRE(C == 0 || (weights && ctx), "wavnetc_forward: conditioning needs weights and context");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const size_t count2 = (size_t)2 * D * N;
+    if (C == 0) {
+        hipLaunchKernelGGL(core_copy_kernel, dim3(stream_blocks(count2)), dim3(256), 0, stream, 2 * D, count2, patTypes,
+                           conv_outputs, core_buf, ctx_tanh);
+        CNT_HIP(hipGetLastError());
+    } else {
+        // X_c = W^T ctx with the tanh, the sum with the convolution output and the padding mask in the epilogue
+        GemmArgs ga = {};
+        ga.m = 2 * D; ga.n = N; ga.k = C;
+        ga.a_kcontig = 1; ga.lda = C;
+        ga.b_kcontig = 1; ga.ldb = C;
+        ga.ldc = 2 * D;
+        ga.nseg = 1; ga.nprob = 1; ga.splitk = 1;
+        ga.epilogue = EPI_CONTEXT; ga.pat = patTypes;
+        ga.prob[0].A[0] = weights; ga.prob[0].B[0] = ctx; ga.prob[0].C = core_buf;
+        ga.prob[0].aux_in = conv_outputs; ga.prob[0].aux_out = ctx_tanh;
+        ga.label = "gemm:wavnetc_context";
+        CNT_TRY(gemm_launch(stream, ga));
+    }
+    return cnt_gatedact_forward(stream_, D, N, patTypes, core_buf, outputs);
+}
+
+int cnt_wavnetc_backward(void *stream_, int D, int C, int N, const char *patTypes, const float *weights, const float *ctx,
+                         const float *core_buf, float *ctx_tanh, const float *output_errors, float *prev_errors,
+                         float *weight_updates, float *ctx_grad) {
+    using namespace cnt;
+    CNT_REQUIRE(patTypes && core_buf && output_errors && prev_errors, "wavnetc_backward: null argument");
+    CNT_REQUIRE(D > 0 && N > 0 && C >= 0, "wavnetc_backward: bad size");
+    CNT_REQUIRE(C == 0 || (weights && ctx && ctx_tanh && weight_updates),
+                "wavnetc_backward: conditioning needs weights, context, tanh buffer and weight updates");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const size_t count = (size_t)D * N;
+    {
+        ProfileScope prof(stream, "gated_backward");
+        hipLaunchKernelGGL(gated_backward_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, D, count, patTypes,
+                           core_buf, output_errors, prev_errors, C > 0 ? ctx_tanh : static_cast<float *>(nullptr));
+        CNT_HIP(hipGetLastError());
+    }
+    if (C == 0) return CNT_OK;
+    CNT_TRY(fill_zero(stream, weight_updates, (size_t)C * 2 * D));
+    {
+        GemmArgs ga = {};
+        ga.m = C; ga.n = 2 * D; ga.k = N;
+        ga.a_kcontig = 0; ga.lda = C;
+        ga.b_kcontig = 0; ga.ldb = 2 * D;
+        ga.ldc = C;
+        ga.nseg = 1; ga.nprob = 1; ga.epilogue = EPI_ATOMIC;
+        const int tiles = ((C + 127) / 128) * ((2 * D + 127) / 128);
+        int s = (512 + tiles - 1) / tiles;
+        const int kt = (N + 15) / 16;
+        ga.splitk = s > kt ? kt : s;
+        ga.prob[0].A[0] = ctx; ga.prob[0].B[0] = ctx_tanh; ga.prob[0].C = weight_updates;
+        ga.label = "gemm:wavnetc_dW";
+        CNT_TRY(gemm_launch(stream, ga));
+    }
+    if (ctx_grad) {
+        GemmArgs ga = {};
+        ga.m = C; ga.n = N; ga.k = 2 * D;
+        ga.a_kcontig = 0; ga.lda = C;
+        ga.b_kcontig = 1; ga.ldb = 2 * D;
+        ga.ldc = C;
+        ga.nseg = 1; ga.nprob = 1; ga.splitk = 1; ga.epilogue = EPI_ADD;
+        ga.prob[0].A[0] = weights; ga.prob[0].B[0] = ctx_tanh; ga.prob[0].C = ctx_grad;
+        ga.label = "gemm:wavnetc_ctx_grad";
+        CNT_TRY(gemm_launch(stream, ga));
+    }
+    return CNT_OK;
+}
+
+int cnt_wavnetc_sum_context_grad(void *stream_, int C, int S, int resolution, int n_frame_slots, int N,
+                                 const char *pat_frames, const char *patTypes, const float *ctx_grad,
+                                 float *frame_grad) {
+    using namespace cnt;
+    CNT_REQUIRE(pat_frames && patTypes && ctx_grad && frame_grad, "wavnetc_sum_context_grad: null argument");
+    CNT_REQUIRE(C > 0 && S > 0 && resolution > 0 && n_frame_slots > 0 && N > 0, "wavnetc_sum_context_grad: bad size");
+    const size_t count = (size_t)C * n_frame_slots;
+    hipLaunchKernelGGL(sum_context_grad_kernel, dim3(stream_blocks(count)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream_), C, S, resolution, count, N, pat_frames, patTypes, ctx_grad,
+                       frame_grad);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Skip-add
+// ---------------------------------------------------------------------------------------------------
+int cnt_skipadd_forward(void *stream_, long count, int n_in, const float *const *inputs, float *outputs,
+                        float *errors, float *errors_from_skip) {
+    using namespace cnt;
+    CNT_REQUIRE(inputs && outputs, "skipadd_forward: null argument");
+    CNT_REQUIRE(count > 0 && n_in >= 1 && n_in <= kSkipMaxFan, "skipadd_forward: %d inputs, supported 1..%d", n_in,
+                kSkipMaxFan);
+    SkipPtrs p = {};
+    p.n = n_in;
+    for (int k = 0; k < n_in; ++k) {
+        CNT_REQUIRE(inputs[k], "skipadd_forward: null input %d", k);
+        p.in[k] = inputs[k];
+    }
+    ProfileScope prof(static_cast<hipStream_t>(stream_), "skipadd_forward");
+    hipLaunchKernelGGL(skipadd_forward_kernel, dim3(stream_blocks((size_t)count)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream_), (size_t)count, p, outputs, errors, errors_from_skip);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+int cnt_skipadd_backward(void *stream_, long count, float *errors, const float *errors_from_skip, int n_pre,
+                         float *const *targets, const int *target_is_skip) {
+    using namespace cnt;
+    CNT_REQUIRE(errors && errors_from_skip && targets && target_is_skip, "skipadd_backward: null argument");
+    CNT_REQUIRE(count > 0 && n_pre >= 1 && n_pre <= kSkipMaxFan, "skipadd_backward: %d predecessors, supported 1..%d",
+                n_pre, kSkipMaxFan);
+    SkipPtrs p = {};
+    p.n = n_pre;
+    for (int k = 0; k < n_pre; ++k) {
+        CNT_REQUIRE(targets[k], "skipadd_backward: null target %d", k);
+        p.target[k] = targets[k];
+        p.is_skip[k] = target_is_skip[k];
+    }
+    ProfileScope prof(static_cast<hipStream_t>(stream_), "skipadd_backward");
+    hipLaunchKernelGGL(skipadd_backward_kernel, dim3(stream_blocks((size_t)count)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream_), (size_t)count, p, errors, errors_from_skip);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+}  // extern "C"

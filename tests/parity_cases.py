@@ -293,3 +293,180 @@ def run_softmax_case(lengths, K, extra, seed):
     assert np.array_equal(np.argmin(gv, axis=1), tgt[pat != 0].astype(np.int64))
     layer.close()
     return worst
+
+
+def run_cnn_case(P, half_width, interval, lengths, causal, out_tanh, seed, bias=1.0, maxT=None):
+    """1-D convolution layer forward + backward against the oracle (which scatters into a real column buffer)."""
+    import torch
+
+    capi = pkg().capi
+    hw = np.asarray(half_width, dtype=np.int32)
+    it = np.asarray(interval, dtype=np.int32)
+    D = len(hw)
+    S, T = len(lengths), max(lengths)
+    maxT = maxT or T
+    N = T * S
+    rng = np.random.default_rng(seed)
+    Lw = O.cnn_total_width(hw)
+    W = rng.uniform(-0.1, 0.1, P * Lw + D).astype(np.float32)
+    x = rng.standard_normal((T, S, P)).astype(np.float32)
+    err = rng.standard_normal((T, S, D)).astype(np.float32)
+    pat = make_pat_types(lengths, T)
+    stale = rng.standard_normal(D * N).astype(np.float32)  # outputs keep their old content on padding slots
+    con = np.zeros(Lw * N, dtype=np.float32)
+    out_o = stale.copy()
+    O.cnn_forward(P, D, S, T, causal, out_tanh, bias, hw, it, pat, W, x.reshape(-1), con, out_o)
+    err_o = err.reshape(-1).copy()
+    ex_o = np.zeros(P * maxT * S, dtype=np.float32)
+    dW_o = np.zeros_like(W)
+    O.cnn_backward(P, D, S, T, causal, out_tanh, bias, hw, it, pat, W, x.reshape(-1), out_o, err_o, con, ex_o[:P * N], dW_o)
+
+    layer = capi.Cnn(P, hw, it, S, maxT, causal, out_tanh, bias)
+    assert layer.weight_count == len(W)
+    pd, Wd, xd = dev(pat), dev(W), dev(x.reshape(-1))
+    out_d = dev(stale)
+    layer.forward(pd, T, Wd, xd, out_d)
+    err_d = dev(err.reshape(-1))
+    ex_d = torch.full((P * maxT * S,), 4.0, dtype=torch.float32, device="cuda")
+    dW_d = torch.full((len(W),), 4.0, dtype=torch.float32, device="cuda")
+    layer.backward(pd, T, Wd, xd, out_d, err_d, ex_d, dW_d)
+    torch.cuda.synchronize()
+    worst = 0.0
+    got_out = out_d.cpu().numpy()
+    worst = max(worst, relerr(got_out, out_o))
+    dummy = (pat == 0)
+    if dummy.any():  # untouched means bit-identical to what was there
+        assert np.array_equal(got_out.reshape(N, D)[dummy], stale.reshape(N, D)[dummy])
+    worst = max(worst, relerr(err_d.cpu().numpy(), err_o))
+    got_ex = ex_d.cpu().numpy()
+    worst = max(worst, relerr(got_ex, ex_o))
+    assert not got_ex[P * N:].any()
+    if dummy.any():
+        assert not got_ex[:P * N].reshape(N, P)[dummy].any()
+    got_dW = dW_d.cpu().numpy()
+    worst = max(worst, relerr(got_dW[:P * Lw], dW_o[:P * Lw]))
+    worst = max(worst, relerr(got_dW[P * Lw:], dW_o[P * Lw:]))
+    # dilation / tap indexing: weight columns that get no signal are exactly zero in both
+    cols_g = got_dW[:P * Lw].reshape(Lw, P)
+    cols_o = dW_o[:P * Lw].reshape(Lw, P)
+    assert np.array_equal(np.abs(cols_g).sum(1) == 0, np.abs(cols_o).sum(1) == 0)
+    layer.close()
+    return worst
+
+
+def run_wavnetc_case(D, Cdim, lengths, seed, with_ctx_grad=True):
+    import torch
+
+    capi = pkg().capi
+    S, T = len(lengths), max(lengths)
+    N = S * T
+    rng = np.random.default_rng(seed)
+    pat = make_pat_types(lengths, T)
+    W = rng.uniform(-0.3, 0.3, max(Cdim, 1) * 2 * D).astype(np.float32)
+    ctx = rng.standard_normal((N, max(Cdim, 1))).astype(np.float32)
+    ctx[pat == 0] = 0
+    conv = rng.standard_normal((N, 2 * D)).astype(np.float32)
+    err = rng.standard_normal((N, D)).astype(np.float32)
+    core_o = np.zeros(2 * D * N, dtype=np.float32)
+    cth_o = np.zeros_like(core_o)
+    out_o = np.zeros(D * N, dtype=np.float32)
+    O.wavnetc_forward(D, Cdim, N, pat, W, ctx.reshape(-1), conv.reshape(-1), core_o, cth_o, out_o)
+    prev_o = np.zeros_like(core_o)
+    dW_o = np.zeros_like(W)
+    cg0 = rng.standard_normal(max(Cdim, 1) * N).astype(np.float32)
+    cg_o = cg0.copy()
+    core_keep = core_o.copy()
+    O.wavnetc_backward(D, Cdim, N, pat, W, ctx.reshape(-1), core_o, cth_o, err.reshape(-1), prev_o, dW_o,
+                       cg_o if with_ctx_grad else None)
+
+    pd, Wd, cd, cvd = dev(pat), dev(W), dev(ctx.reshape(-1)), dev(conv.reshape(-1))
+    core_d = torch.full((2 * D * N,), 3.0, dtype=torch.float32, device="cuda")
+    cth_d = torch.full((2 * D * N,), 3.0, dtype=torch.float32, device="cuda")
+    out_d = torch.full((D * N,), 3.0, dtype=torch.float32, device="cuda")
+    capi.wavnetc_forward(D, Cdim, N, pd, Wd, cd, cvd, core_d, cth_d, out_d)
+    torch.cuda.synchronize()
+    worst = relerr(core_d.cpu().numpy(), core_keep)
+    worst = max(worst, relerr(out_d.cpu().numpy(), out_o))
+    prev_d = torch.full((2 * D * N,), 3.0, dtype=torch.float32, device="cuda")
+    dW_d = torch.full((len(W),), 3.0, dtype=torch.float32, device="cuda")
+    cg_d = dev(cg0)
+    capi.wavnetc_backward(D, Cdim, N, pd, Wd, cd, core_d, cth_d, dev(err.reshape(-1)), prev_d, dW_d,
+                          cg_d if with_ctx_grad else None)
+    torch.cuda.synchronize()
+    worst = max(worst, relerr(prev_d.cpu().numpy(), prev_o))
+    dummy = (pat == 0)
+    if dummy.any():
+        assert not prev_d.cpu().numpy().reshape(N, 2 * D)[dummy].any()
+        assert not out_d.cpu().numpy().reshape(N, D)[dummy].any()
+    if Cdim > 0:
+        worst = max(worst, relerr(cth_d.cpu().numpy(), cth_o))
+        worst = max(worst, relerr(dW_d.cpu().numpy(), dW_o))
+        if with_ctx_grad:
+            worst = max(worst, relerr(cg_d.cpu().numpy(), cg_o))
+    # the unconditioned layer type on the same pre-activations
+    out2 = torch.zeros(D * N, dtype=torch.float32, device="cuda")
+    prev2 = torch.zeros(2 * D * N, dtype=torch.float32, device="cuda")
+    capi.gatedact_forward(D, N, pd, core_d, out2)
+    capi.gatedact_backward(D, N, pd, core_d, dev(err.reshape(-1)), prev2)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out_d) and torch.equal(prev2, prev_d)
+    return worst
+
+
+def run_context_case(Cdim, res, lengths, seed, use_mean_std):
+    import torch
+
+    capi = pkg().capi
+    S, T = len(lengths), max(lengths)
+    N = T * S
+    pat = make_pat_types(lengths, T)
+    nfr = [-(-n // res) for n in lengths]
+    Tf = max(nfr)
+    rng = np.random.default_rng(seed)
+    src = rng.standard_normal(Tf * S * Cdim).astype(np.float32)
+    fidx = np.array([[t // res for s in range(S)] for t in range(T)], dtype=np.float32).reshape(-1)
+    mv = np.concatenate([rng.standard_normal(Cdim), rng.uniform(0.5, 2.0, Cdim)]).astype(np.float32)
+    mv[-1] = 1e-7
+    ctx_o = np.zeros(Cdim * N, dtype=np.float32)
+    O.wavnetc_load_context(Cdim, S, N, Tf, False, src, fidx, mv if use_mean_std else None, pat, ctx_o)
+    ctx_d = torch.full((Cdim * N,), 2.0, dtype=torch.float32, device="cuda")
+    capi.wavnetc_load_context(Cdim, S, N, Tf, False, dev(src), dev(fidx), dev(mv) if use_mean_std else None, dev(pat), ctx_d)
+    g = rng.standard_normal(Cdim * N).astype(np.float32)
+    pat_f = make_pat_types(nfr, Tf)
+    fg_o = np.zeros(Tf * S * Cdim, dtype=np.float32)
+    O.wavnetc_sum_context_grad(Cdim, S, res, Tf * S, N, pat_f, pat, g, fg_o)
+    fg_d = torch.full((Tf * S * Cdim,), 2.0, dtype=torch.float32, device="cuda")
+    capi.wavnetc_sum_context_grad(Cdim, S, res, Tf * S, N, dev(pat_f), dev(pat), dev(g), fg_d)
+    torch.cuda.synchronize()
+    if not use_mean_std:  # a pure gather: bit-exact
+        assert np.array_equal(ctx_d.cpu().numpy(), ctx_o)
+    return max(relerr(ctx_d.cpu().numpy(), ctx_o), relerr(fg_d.cpu().numpy(), fg_o))
+
+
+def run_skipadd_case(n, seed):
+    import torch
+
+    capi = pkg().capi
+    rng = np.random.default_rng(seed)
+    ins = [rng.standard_normal(n).astype(np.float32) for _ in range(3)]
+    out_o, e_o, es_o = np.zeros(n, np.float32), np.ones(n, np.float32), np.ones(n, np.float32)
+    O.skipadd_forward(ins, out_o, e_o, es_o)
+    out_d = torch.ones(n, device="cuda")
+    e_d = torch.ones(n, device="cuda")
+    es_d = torch.ones(n, device="cuda")
+    capi.skipadd_forward([dev(a) for a in ins], out_d, e_d, es_d)
+    torch.cuda.synchronize()
+    assert np.array_equal(out_d.cpu().numpy(), out_o) and not e_d.any() and not es_d.any()
+    e = rng.standard_normal(n).astype(np.float32)
+    es = rng.standard_normal(n).astype(np.float32)
+    tg = [rng.standard_normal(n).astype(np.float32) for _ in range(3)]
+    flags = [1, 0, 1]
+    e_o, tg_o = e.copy(), [t.copy() for t in tg]
+    O.skipadd_backward(e_o, es, tg_o, flags)
+    e_d, tg_d = dev(e), [dev(t) for t in tg]
+    capi.skipadd_backward(e_d, dev(es), tg_d, flags)
+    torch.cuda.synchronize()
+    assert np.array_equal(e_d.cpu().numpy(), e_o)
+    for a, b in zip(tg_d, tg_o):
+        assert np.array_equal(a.cpu().numpy(), b)
+    return 0.0
