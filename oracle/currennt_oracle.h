@@ -104,6 +104,15 @@ void orc_skipadd_forward(long count, int n_in, const float *const *inputs, float
 void orc_skipadd_backward(long count, float *errors, const float *errors_from_skip, int n_pre, float *const *targets,
                           const int *target_is_skip);
 
+/* DFT log-amplitude loss (helpers/FFTMat.cu, layers/DFTErrorPostoutputLayer.cu); transforms follow cuFFT's
+   R2C / C2R conventions (unnormalised, n/2+1 bins, imaginary parts of DC and Nyquist ignored by C2R). */
+int orc_dft_frame_count(int signal_length, int frame_length, int frame_shift);
+void orc_dft_r2c(int n, const float *in, float *out);
+void orc_dft_c2r(int n, const float *in, float *out);
+float orc_dft_logamp_loss(int fft_length, int frame_length, int frame_shift, int window_type, int max_length,
+                          int length, float gamma, float log_floor, const float *source, const float *target,
+                          float *grad);
+
 #ifdef __cplusplus
 }
 #endif

@@ -68,6 +68,7 @@ def lib():
         L.orc_sse_error.restype = C.c_float
         L.orc_mdn_mixture_error.restype = C.c_float
         L.orc_softmax_error.restype = C.c_float
+        L.orc_dft_logamp_loss.restype = C.c_float
         _lib = L
     return _lib
 
@@ -202,3 +203,28 @@ def skipadd_backward(errors, errors_from_skip, targets, is_skip):
     flags = (C.c_int * len(is_skip))(*[int(v) for v in is_skip])
     lib().orc_skipadd_backward(C.c_long(errors.size), fptr(errors), fptr(errors_from_skip), len(targets),
                                _fpp(targets), flags)
+
+
+def dft_frame_count(n, frame_length, frame_shift):
+    return int(lib().orc_dft_frame_count(n, frame_length, frame_shift))
+
+
+def dft_r2c(x):
+    n = len(x)
+    out = np.zeros(2 * (n // 2 + 1), dtype=np.float32)
+    lib().orc_dft_r2c(n, fptr(x), fptr(out))
+    return out[0::2] + 1j * out[1::2]
+
+
+def dft_c2r(X, n):
+    buf = np.zeros(2 * (n // 2 + 1), dtype=np.float32)
+    buf[0::2] = X.real
+    buf[1::2] = X.imag
+    out = np.zeros(n, dtype=np.float32)
+    lib().orc_dft_c2r(n, fptr(buf), fptr(out))
+    return out
+
+
+def dft_logamp_loss(N, Nw, Hs, window_type, max_len, length, gamma, floor, src, tgt, grad):
+    return float(lib().orc_dft_logamp_loss(N, Nw, Hs, window_type, max_len, length, C.c_float(gamma), C.c_float(floor),
+                                           fptr(src), fptr(tgt), fptr(grad)))

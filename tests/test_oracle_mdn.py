@@ -45,7 +45,7 @@ def torch_mixture_nll(x, tgt, valid, startD, M, D):
     logp = logw - 0.5 * (z * z).sum(2) - ls.sum(2) - D * math.log(2 * PI_REF) / 2
     nll = -(torch.logsumexp(logp, dim=1) * torch.tensor(valid, dtype=torch.float64)).sum()
     nll.backward()
-    return float(nll), xt.grad.numpy()
+    return float(nll.detach()), xt.grad.numpy()
 
 
 def test_mixture_matches_closed_form_all_valid():
