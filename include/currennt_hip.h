@@ -223,6 +223,36 @@ int cnt_skipadd_forward(void *stream, long count, int n_in, const float *const *
 int cnt_skipadd_backward(void *stream, long count, float *errors, const float *errors_from_skip, int n_pre,
                          float *const *targets, const int *target_is_skip);
 
+/* ---- DFT (multi-resolution STFT log-amplitude) loss -------------------------------------------------
+ * DFTPostoutputLayer<TDevice> with helpers::FFTMat (layers/DFTErrorPostoutputLayer.cu, helpers/FFTMat.cu)
+ * for specDisType 0 and up to three resolutions ("fftLength/frameLength/frameShift" with suffix "", "2",
+ * "3", layers/DFTErrorPostoutputLayer.cu:752-845).  The layer has size 1; a waveform occupies max_length
+ * consecutive floats.  The reference handles one waveform per fraction; here n_waves waveforms with their
+ * own lengths can be processed by one call (waveform w at offset w*max_length).  FFT lengths must be
+ * powers of two in 32..4096. */
+typedef struct cnt_dft cnt_dft;
+typedef struct {
+    int n_res;
+    int fft_length[3], frame_length[3], frame_shift[3];
+    int window_type[3];  /* 0 Hann (the reference's default), 1 square */
+    float gamma;         /* "gamma": weight of the spectral amplitude loss            */
+    float log_floor;     /* "logSpecAmpFloor", 1e-5 by default (helpers/FFTMat.hpp:53) */
+    int spec_dis_type;   /* "specDisType"; only 0 is built                            */
+    int max_length;      /* maxSeqLength in samples                                   */
+    int max_waves;       /* waveforms per call, 1..32                                 */
+} cnt_dft_desc;
+int cnt_dft_create(const cnt_dft_desc *desc, cnt_dft **out);
+int cnt_dft_destroy(cnt_dft *h);
+/* DFTPostoutputLayer::computeForwardPass in training mode (layers/DFTErrorPostoutputLayer.cu:1782-1839,
+ * :1186-1244): computes the loss of every waveform and resolution into errors_dev[w*n_res + r] (device
+ * memory) AND the gradient w.r.t. the source samples, which is kept inside the handle, as the reference
+ * keeps it in m_fftDiffData.  lengths is a host array.  Samples at or beyond a waveform's length count as 0. */
+int cnt_dft_forward(cnt_dft *h, void *stream, int n_waves, const int *lengths, const float *source,
+                    const float *target, float *errors_dev);
+/* DFTPostoutputLayer::computeBackwardPass (layers/DFTErrorPostoutputLayer.cu:1849-1885, :1699-1714):
+ * prev_errors (n_waves x max_length) = sum over resolutions of the stored gradients, 0 beyond each length. */
+int cnt_dft_backward(cnt_dft *h, void *stream, float *prev_errors);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,6 +22,12 @@ class CnnDesc(C.Structure):
                 ("output_tanh", C.c_int), ("bias", C.c_float)]
 
 
+class DftDesc(C.Structure):
+    _fields_ = [("n_res", C.c_int), ("fft_length", C.c_int * 3), ("frame_length", C.c_int * 3),
+                ("frame_shift", C.c_int * 3), ("window_type", C.c_int * 3), ("gamma", C.c_float),
+                ("log_floor", C.c_float), ("spec_dis_type", C.c_int), ("max_length", C.c_int), ("max_waves", C.c_int)]
+
+
 class LstmDesc(C.Structure):
     _fields_ = [("P", C.c_int), ("L", C.c_int), ("bidir", C.c_int), ("S", C.c_int), ("maxT", C.c_int),
                 ("bias", C.c_float)]
@@ -59,6 +65,10 @@ _SIGNATURES = {
     "cnt_mdn_calculate_error": (I, [VP, VP, VP, VP]),
     "cnt_mdn_backward": (I, [VP, VP, VP, VP]),
     "cnt_mdn_unit_buffer": (VP, [VP, I, I, C.POINTER(C.c_long)]),
+    "cnt_dft_create": (I, [C.POINTER(DftDesc), C.POINTER(VP)]),
+    "cnt_dft_destroy": (I, [VP]),
+    "cnt_dft_forward": (I, [VP, VP, I, C.POINTER(I), VP, VP, VP]),
+    "cnt_dft_backward": (I, [VP, VP, VP]),
     "cnt_cnn_create": (I, [C.POINTER(CnnDesc), C.POINTER(I), C.POINTER(I), C.POINTER(VP)]),
     "cnt_cnn_destroy": (I, [VP]),
     "cnt_cnn_weight_count": (C.c_long, [VP]),
@@ -275,6 +285,40 @@ def skipadd_backward(errors, errors_from_skip, targets, is_skip, stream=None):
     flags = (I * len(is_skip))(*[int(v) for v in is_skip])
     check(lib().cnt_skipadd_backward(stream_ptr(stream), errors.numel(), ptr(errors), ptr(errors_from_skip),
                                      len(targets), _ptr_array(targets), flags))
+
+
+class Dft:
+    """Thin owner of a cnt_dft handle.  resolutions: list of (fftLength, frameLength, frameShift)."""
+
+    def __init__(self, resolutions, max_length, max_waves, gamma=1.0, log_floor=1e-5, window_type=0, spec_dis_type=0):
+        d = DftDesc()
+        d.n_res = len(resolutions)
+        for r, (n, nw, hs) in enumerate(resolutions[:3]):
+            d.fft_length[r], d.frame_length[r], d.frame_shift[r], d.window_type[r] = n, nw, hs, window_type
+        d.gamma, d.log_floor, d.spec_dis_type = gamma, log_floor, spec_dis_type
+        d.max_length, d.max_waves = max_length, max_waves
+        self.n_res = d.n_res
+        self.handle = VP()
+        check(lib().cnt_dft_create(C.byref(d), C.byref(self.handle)))
+
+    def close(self):
+        if self.handle:
+            lib().cnt_dft_destroy(self.handle)
+            self.handle = VP()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def forward(self, lengths, source, target, errors, stream=None):
+        arr = (I * len(lengths))(*[int(v) for v in lengths])
+        check(lib().cnt_dft_forward(self.handle, stream_ptr(stream), len(lengths), arr, ptr(source), ptr(target),
+                                    ptr(errors)))
+
+    def backward(self, prev_errors, stream=None):
+        check(lib().cnt_dft_backward(self.handle, stream_ptr(stream), ptr(prev_errors)))
 
 
 class Mdn:

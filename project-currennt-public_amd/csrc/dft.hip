@@ -1,0 +1,318 @@
+// Multi-resolution STFT log-amplitude loss and its gradient for gfx950, with an in-house radix-2 FFT.
+//
+// Reference behaviour: helpers/FFTMat.cu (FrameSignal :282-312, distance :473-496, gradient :760-782,
+// cleanDummyGradients :456-471, collectGrad :965-1006, drivers :1246-1274, :1350-1475, :1637-1770,
+// :1833-1886) and layers/DFTErrorPostoutputLayer.cu (:1186-1244, :1699-1714, :1782-1885).  The reference
+// runs about a dozen launches and three cuFFT calls per resolution and waveform, with every intermediate
+// (framed signals, spectra, per-bin differences, framed gradients) in device memory.
+//
+// Here one workgroup owns one frame end to end and nothing but the waveforms and the gradient touches HBM:
+//   frame + window source and target  ->  ONE complex FFT of z = source + i*target in LDS (both real
+//   spectra are recovered from Z[b] and Z[N-b])  ->  per-bin log-amplitude difference, loss partial and
+//   gradient spectrum, written back as its Hermitian extension  ->  inverse FFT in LDS  ->  windowed
+//   overlap-add straight into the per-sample gradient with float atomics.
+// The forward transform is decimation-in-frequency (natural order in, bit-reversed out), the per-bin stage
+// addresses bins through the bit-reversal, and the inverse is decimation-in-time (bit-reversed in, natural
+// out), so no reordering pass exists.  Twiddles and the window (with the reference's constant 3.141215) are
+// tabulated in double on the host.  Transform conventions are cuFFT's: unnormalised, N/2+1 bins, the
+// imaginary parts of the DC and Nyquist bins do not enter the inverse.
+#include "common.hpp"
+
+#include <cmath>
+#include <cstring>
+#include <new>
+#include <vector>
+
+namespace cnt {
+namespace {
+
+constexpr int kMaxRes = 3;
+constexpr int kMaxWavesPerLaunch = 32;
+
+struct DftParams {
+    int N, Nw, Hs;       // fft length, frame length, frame shift
+    int max_length;      // samples per waveform buffer
+    int n_waves, n_res, res;
+    int lengths[kMaxWavesPerLaunch];
+    float gamma, log_floor;
+    const float2 *twiddle;  // N/2 entries exp(-2*pi*i*k/N)
+    const float *window;    // Nw entries
+    const float *source, *target;
+    float *grad;    // n_waves x max_length, accumulated over resolutions
+    float *errors;  // n_waves x n_res
+};
+
+__host__ __device__ inline int frame_count(int length, int Nw, int Hs) {
+    return length < Nw ? 1 : 1 + (length - Nw) / Hs;
+}
+
+template <int LOGN>
+__global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
+    constexpr int N = 1 << LOGN;
+    constexpr int HALF = N / 2;
+    constexpr int TPF = HALF < 256 ? HALF : 256;  // threads per frame
+    constexpr int FPB = 256 / TPF;                // frames per block
+    __shared__ float2 z[FPB][N];
+    __shared__ float2 tw[HALF];
+    __shared__ float err_part[4];
+
+    const int tid = threadIdx.x;
+    const int fl = tid / TPF, ft = tid % TPF;  // frame slot in the block, thread within the frame
+    const int wave_id = blockIdx.y;
+    const int length = p.lengths[wave_id];
+    const int Kvalid = frame_count(length, p.Nw, p.Hs);
+    const int k = blockIdx.x * FPB + fl;
+    const bool active = k < Kvalid;  // every thread stays for the barriers
+    const float *src = p.source + (size_t)wave_id * p.max_length;
+    const float *tgt = p.target + (size_t)wave_id * p.max_length;
+
+    for (int i = tid; i < HALF; i += 256) tw[i] = p.twiddle[i];
+    for (int j = ft; j < N; j += TPF) {
+        float2 v = make_float2(0.0f, 0.0f);
+        const int pos = k * p.Hs + j;
+        if (active && j < p.Nw && pos < length) {
+            const float w = p.window[j];
+            v = make_float2(src[pos] * w, tgt[pos] * w);
+        }
+        z[fl][j] = v;
+    }
+    __syncthreads();
+
+    // forward: decimation in frequency
+#pragma unroll 1
+    for (int s = LOGN - 1; s >= 0; --s) {
+        const int half = 1 << s;
+        for (int i = ft; i < HALF; i += TPF) {
+            const int pos = i & (half - 1);
+            const int a = ((i >> s) << (s + 1)) + pos, b = a + half;
+            const float2 u = z[fl][a], v = z[fl][b];
+            const float2 w = tw[pos << (LOGN - 1 - s)];
+            const float dx = u.x - v.x, dy = u.y - v.y;
+            z[fl][a] = make_float2(u.x + v.x, u.y + v.y);
+            z[fl][b] = make_float2(dx * w.x - dy * w.y, dx * w.y + dy * w.x);
+        }
+        __syncthreads();
+    }
+
+    // per-bin stage on the pairs (b, N-b); bin b lives at position bitrev(b)
+    float err = 0.0f;
+    for (int b = ft; b <= HALF; b += TPF) {
+        const int nb = (N - b) & (N - 1);
+        const int pb = (int)(__brev((unsigned)b) >> (32 - LOGN));
+        const int pnb = (int)(__brev((unsigned)nb) >> (32 - LOGN));
+        const float2 zb = z[fl][pb], zn = z[fl][pnb];
+        // S = (Z[b] + conj(Z[N-b])) / 2,  T = (Z[b] - conj(Z[N-b])) / (2i)
+        const float sx = 0.5f * (zb.x + zn.x), sy = 0.5f * (zb.y - zn.y);
+        const float tx = 0.5f * (zb.y + zn.y), ty = -0.5f * (zb.x - zn.x);
+        const float spec = sx * sx + sy * sy + p.log_floor;
+        const float d = safe_log(spec) - safe_log(tx * tx + ty * ty + p.log_floor);
+        if (active) err += d * d;
+        const float gx = d * sx / spec, gy = d * sy / spec;
+        if (b == 0 || b == HALF) {
+            z[fl][pb] = make_float2(gx, 0.0f);
+        } else {
+            z[fl][pb] = make_float2(gx, gy);
+            z[fl][pnb] = make_float2(gx, -gy);
+        }
+    }
+    __syncthreads();
+
+    // inverse: decimation in time with conjugated twiddles, unnormalised
+#pragma unroll 1
+    for (int s = 0; s < LOGN; ++s) {
+        const int half = 1 << s;
+        for (int i = ft; i < HALF; i += TPF) {
+            const int pos = i & (half - 1);
+            const int a = ((i >> s) << (s + 1)) + pos, b = a + half;
+            const float2 u = z[fl][a], x = z[fl][b];
+            const float2 w = tw[pos << (LOGN - 1 - s)];
+            const float vx = x.x * w.x + x.y * w.y, vy = x.y * w.x - x.x * w.y;
+            z[fl][a] = make_float2(u.x + vx, u.y + vy);
+            z[fl][b] = make_float2(u.x - vx, u.y - vy);
+        }
+        __syncthreads();
+    }
+
+    // windowed overlap-add; frames at or beyond Kvalid contribute nothing
+    const float inv = 1.0f / (float)((HALF + 1) * Kvalid);
+    if (active) {
+        const float scale = p.gamma * inv;
+        float *g = p.grad + (size_t)wave_id * p.max_length;
+        for (int j = ft; j < p.Nw; j += TPF) {
+            const int pos = k * p.Hs + j;
+            if (pos < length) atomicAdd(&g[pos], scale * z[fl][j].x * p.window[j]);
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) err += __shfl_xor(err, o);
+    if ((tid & 63) == 0) err_part[tid >> 6] = err;
+    __syncthreads();
+    if (tid == 0) {
+        const float e = (err_part[0] + err_part[1] + err_part[2] + err_part[3]) * inv;
+        if (e != 0.0f) atomicAdd(&p.errors[wave_id * p.n_res + p.res], e);
+    }
+}
+
+__global__ void dft_backward_kernel(int max_length, int n_waves, DftParams p, float *__restrict__ prev_errors) {
+    const size_t count = (size_t)max_length * n_waves;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const int w = (int)(i / max_length), t = (int)(i % max_length);
+        prev_errors[i] = t < p.lengths[w] ? p.grad[i] : 0.0f;
+    }
+}
+
+typedef void (*dft_kernel_t)(const DftParams);
+dft_kernel_t pick_dft_kernel(int logn) {
+    switch (logn) {
+        case 5: return dft_loss_kernel<5>;
+        case 6: return dft_loss_kernel<6>;
+        case 7: return dft_loss_kernel<7>;
+        case 8: return dft_loss_kernel<8>;
+        case 9: return dft_loss_kernel<9>;
+        case 10: return dft_loss_kernel<10>;
+        case 11: return dft_loss_kernel<11>;
+        case 12: return dft_loss_kernel<12>;
+        default: return nullptr;
+    }
+}
+
+}  // namespace
+}  // namespace cnt
+
+struct cnt_dft {
+    cnt_dft_desc desc;
+    int logn[cnt::kMaxRes];
+    float2 *twiddle[cnt::kMaxRes];
+    float *window[cnt::kMaxRes];
+    float *grad;  // max_waves x max_length
+    int lengths[cnt::kMaxWavesPerLaunch];
+    int n_waves;  // of the last forward
+};
+
+extern "C" {
+
+int cnt_dft_destroy(cnt_dft *h) {
+    if (!h) return CNT_OK;
+    for (int r = 0; r < cnt::kMaxRes; ++r) {
+        if (h->twiddle[r]) (void)hipFree(h->twiddle[r]);
+        if (h->window[r]) (void)hipFree(h->window[r]);
+    }
+    if (h->grad) (void)hipFree(h->grad);
+    delete h;
+    return CNT_OK;
+}
+
+int cnt_dft_create(const cnt_dft_desc *desc, cnt_dft **out) {
+    using namespace cnt;
+    CNT_REQUIRE(desc && out, "dft_create: null argument");
+    CNT_REQUIRE(desc->n_res >= 1 && desc->n_res <= kMaxRes, "dft_create: %d resolutions, supported 1..%d", desc->n_res,
+                kMaxRes);
+    CNT_REQUIRE(desc->max_length > 0 && desc->max_waves >= 1 && desc->max_waves <= kMaxWavesPerLaunch,
+                "dft_create: max_length must be positive and max_waves in 1..%d", kMaxWavesPerLaunch);
+    // the reference implements the Hann window (default) and the square window; other distances than the
+    // log-amplitude MSE (specDisType 0) are not built
+    CNT_REQUIRE(desc->spec_dis_type == 0, "dft_create: only specDisType 0 (log-amplitude MSE) is built");
+    cnt_dft *h = new (std::nothrow) cnt_dft();
+    CNT_REQUIRE(h != nullptr, "dft_create: out of host memory");
+    std::memset(h, 0, sizeof(*h));
+    h->desc = *desc;
+    hipError_t err = hipSuccess;
+    for (int r = 0; r < desc->n_res && err == hipSuccess; ++r) {
+        const int N = desc->fft_length[r], Nw = desc->frame_length[r], Hs = desc->frame_shift[r];
+        int logn = 0;
+        while ((1 << logn) < N) ++logn;
+        if ((1 << logn) != N || !pick_dft_kernel(logn) || Nw < 2 || Nw > N || Hs < 1) {
+            set_error("dft_create: resolution %d has fftLength %d, frameLength %d, frameShift %d; supported: fftLength a "
+                      "power of two in 32..4096, 2 <= frameLength <= fftLength, frameShift >= 1", r, N, Nw, Hs);
+            cnt_dft_destroy(h);
+            return CNT_ERR_ARG;
+        }
+        h->logn[r] = logn;
+        std::vector<float2> tw((size_t)N / 2);
+        for (int k2 = 0; k2 < N / 2; ++k2) {
+            const double a = -2.0 * 3.14159265358979323846 * k2 / N;
+            tw[(size_t)k2] = make_float2((float)std::cos(a), (float)std::sin(a));
+        }
+        std::vector<float> win((size_t)Nw);
+        for (int j = 0; j < Nw; ++j)
+            win[(size_t)j] = desc->window_type[r] == 1 ? 1.0f
+                                                       : (float)(0.5 * (1 - std::cos(2.0 * 3.141215 * j / (Nw - 1))));
+        err = hipMalloc(reinterpret_cast<void **>(&h->twiddle[r]), tw.size() * sizeof(float2));
+        if (err == hipSuccess) err = hipMemcpy(h->twiddle[r], tw.data(), tw.size() * sizeof(float2), hipMemcpyHostToDevice);
+        if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->window[r]), win.size() * sizeof(float));
+        if (err == hipSuccess) err = hipMemcpy(h->window[r], win.data(), win.size() * sizeof(float), hipMemcpyHostToDevice);
+    }
+    if (err == hipSuccess)
+        err = hipMalloc(reinterpret_cast<void **>(&h->grad), (size_t)desc->max_waves * desc->max_length * sizeof(float));
+    if (err != hipSuccess) {
+        set_error("dft_create: %s", hipGetErrorString(err));
+        cnt_dft_destroy(h);
+        return CNT_ERR_HIP;
+    }
+    *out = h;
+    return CNT_OK;
+}
+
+static void fill_params(const cnt_dft *h, cnt::DftParams &p) {
+    std::memset(&p, 0, sizeof(p));
+    p.max_length = h->desc.max_length;
+    p.n_waves = h->n_waves;
+    p.n_res = h->desc.n_res;
+    for (int w = 0; w < h->n_waves; ++w) p.lengths[w] = h->lengths[w];
+    p.gamma = h->desc.gamma;
+    p.log_floor = h->desc.log_floor;
+    p.grad = h->grad;
+}
+
+int cnt_dft_forward(cnt_dft *h, void *stream_, int n_waves, const int *lengths, const float *source,
+                    const float *target, float *errors_dev) {
+    using namespace cnt;
+    CNT_REQUIRE(h && lengths && source && target && errors_dev, "dft_forward: null argument");
+    CNT_REQUIRE(n_waves >= 1 && n_waves <= h->desc.max_waves, "dft_forward: %d waveforms, handle allows 1..%d", n_waves,
+                h->desc.max_waves);
+    for (int w = 0; w < n_waves; ++w)
+        CNT_REQUIRE(lengths[w] >= 1 && lengths[w] <= h->desc.max_length, "dft_forward: length %d of waveform %d outside 1..%d",
+                    lengths[w], w, h->desc.max_length);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    h->n_waves = n_waves;
+    for (int w = 0; w < n_waves; ++w) h->lengths[w] = lengths[w];
+    CNT_TRY(fill_zero(stream, h->grad, (size_t)n_waves * h->desc.max_length));
+    CNT_TRY(fill_zero(stream, errors_dev, (size_t)n_waves * h->desc.n_res));
+    int max_len = 0;
+    for (int w = 0; w < n_waves; ++w) max_len = lengths[w] > max_len ? lengths[w] : max_len;
+    for (int r = 0; r < h->desc.n_res; ++r) {
+        DftParams p;
+        fill_params(h, p);
+        p.N = h->desc.fft_length[r]; p.Nw = h->desc.frame_length[r]; p.Hs = h->desc.frame_shift[r];
+        p.res = r;
+        p.twiddle = h->twiddle[r]; p.window = h->window[r];
+        p.source = source; p.target = target; p.errors = errors_dev;
+        const int half = p.N / 2;
+        const int fpb = half < 256 ? 256 / half : 1;
+        const int kmax = frame_count(max_len, p.Nw, p.Hs);
+        dim3 grid((kmax + fpb - 1) / fpb, n_waves);
+        ProfileScope prof(stream, "dft_loss");
+        hipLaunchKernelGGL(pick_dft_kernel(h->logn[r]), grid, dim3(256), 0, stream, p);
+        CNT_HIP(hipGetLastError());
+    }
+    return CNT_OK;
+}
+
+int cnt_dft_backward(cnt_dft *h, void *stream_, float *prev_errors) {
+    using namespace cnt;
+    CNT_REQUIRE(h && prev_errors, "dft_backward: null argument");
+    CNT_REQUIRE(h->n_waves > 0, "dft_backward: forward has not been called");
+    DftParams p;
+    fill_params(h, p);
+    const size_t count = (size_t)h->desc.max_length * h->n_waves;
+    size_t blocks = (count + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    ProfileScope prof(static_cast<hipStream_t>(stream_), "dft_backward");
+    hipLaunchKernelGGL(dft_backward_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream_),
+                       h->desc.max_length, h->n_waves, p, prev_errors);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+}  // extern "C"

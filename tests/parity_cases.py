@@ -470,3 +470,35 @@ def run_skipadd_case(n, seed):
     for a, b in zip(tg_d, tg_o):
         assert np.array_equal(a.cpu().numpy(), b)
     return 0.0
+
+
+def run_dft_case(resolutions, max_len, lengths, seed, gamma=1.0):
+    """Multi-resolution DFT loss: per-resolution losses and the summed gradient against the oracle."""
+    import torch
+
+    capi = pkg().capi
+    rng = np.random.default_rng(seed)
+    W = len(lengths)
+    src = (0.3 * rng.standard_normal((W, max_len))).astype(np.float32)
+    tgt = (0.3 * rng.standard_normal((W, max_len))).astype(np.float32)
+    err_o = np.zeros((W, len(resolutions)))
+    grad_o = np.zeros((W, max_len), dtype=np.float64)
+    for w in range(W):
+        for r, (N, Nw, Hs) in enumerate(resolutions):
+            g = np.zeros(max_len, dtype=np.float32)
+            err_o[w, r] = O.dft_logamp_loss(N, Nw, Hs, 0, max_len, lengths[w], gamma, 1e-5, src[w].copy(), tgt[w].copy(), g)
+            g[lengths[w]:] = 0  # the layer only passes on the first `length` samples
+            grad_o[w] += g
+    layer = capi.Dft(resolutions, max_len, W, gamma=gamma)
+    err_d = torch.full((W * len(resolutions),), 7.0, dtype=torch.float32, device="cuda")
+    prev_d = torch.full((W * max_len,), 7.0, dtype=torch.float32, device="cuda")
+    layer.forward(lengths, dev(src.reshape(-1)), dev(tgt.reshape(-1)), err_d)
+    layer.backward(prev_d)
+    torch.cuda.synchronize()
+    got_g = prev_d.cpu().numpy().reshape(W, max_len)
+    worst = relerr(err_d.cpu().numpy(), err_o)
+    for w in range(W):
+        worst = max(worst, relerr(got_g[w], grad_o[w]))
+        assert not got_g[w, lengths[w]:].any()
+    layer.close()
+    return worst
