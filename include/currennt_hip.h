@@ -57,6 +57,15 @@ int cnt_dense_backward(void *stream, int P, int D, int N, int act, float bias, c
                        const float *x, const float *y, float *err, float *prev_err,
                        float *weight_updates);
 
+/* The two halves of cnt_dense_backward, for callers that schedule them on different streams: the error
+ * half (delta in place, prev_err) is what the next layer's backward waits for; the weight half
+ * (weight_updates from x and the deltas) has no consumer before the optimizer.  The reference has no such
+ * split; calling both in this order on one stream is cnt_dense_backward. */
+int cnt_dense_backward_errors(void *stream, int P, int D, int N, int act, const float *weights, const float *y,
+                              float *err, float *prev_err);
+int cnt_dense_backward_weights(void *stream, int P, int D, int N, float bias, const float *x, const float *err,
+                               float *weight_updates);
+
 /* ---- SSE post-output layer ---------------------------------------------------------------------
  * SsePostOutputLayer::computeBackwardPass (layers/SsePostOutputLayer.cu:224-267):
  * err = y - target, exactly 0 on padding slots. */
@@ -101,6 +110,11 @@ int cnt_lstm_forward(cnt_lstm *h, void *stream, const float *weights, const floa
 int cnt_lstm_backward(cnt_lstm *h, void *stream, const float *weights, const float *x,
                       const float *outputs, float *output_errors, float *prev_errors,
                       float *weight_updates);
+/* The two halves of cnt_lstm_backward (layers/LstmLayer.cu:2066-2334 and :2337-2375), for callers that put
+ * the weight gradients on another stream: the second half only reads x and the handle's state. */
+int cnt_lstm_backward_errors(cnt_lstm *h, void *stream, const float *weights, float *output_errors,
+                             float *prev_errors);
+int cnt_lstm_backward_weights(cnt_lstm *h, void *stream, const float *x, float *weight_updates);
 /* Device pointer to one internal buffer.  dir: 0 forward, 1 backward states.  which:
  * 0 niActs 1 igActs 2 fgActs 3 ogActs 4 cellStates 5 tmpOutputs 6 tmpOutputErrors
  * 7 niDeltas 8 igDeltas 9 fgDeltas 10 ogDeltas 11 cellStateErrors.  NULL if out of range. */

@@ -47,6 +47,8 @@ _SIGNATURES = {
     "cnt_matrix_product": (I, [VP, VP, I, I, I, VP, I, VP, I, I]),
     "cnt_dense_forward": (I, [VP, I, I, I, I, F, VP, VP, VP]),
     "cnt_dense_backward": (I, [VP, I, I, I, I, F, VP, VP, VP, VP, VP, VP]),
+    "cnt_dense_backward_errors": (I, [VP, I, I, I, I, VP, VP, VP, VP]),
+    "cnt_dense_backward_weights": (I, [VP, I, I, I, F, VP, VP, VP]),
     "cnt_sse_backward": (I, [VP, I, I, VP, VP, VP, VP]),
     "cnt_sse_error": (I, [VP, I, I, VP, VP, VP, VP]),
     "cnt_lstm_create": (I, [C.POINTER(LstmDesc), C.POINTER(VP)]),
@@ -54,6 +56,8 @@ _SIGNATURES = {
     "cnt_lstm_load_sequences": (I, [VP, VP, VP, I, I]),
     "cnt_lstm_forward": (I, [VP, VP, VP, VP, VP]),
     "cnt_lstm_backward": (I, [VP, VP, VP, VP, VP, VP, VP, VP]),
+    "cnt_lstm_backward_errors": (I, [VP, VP, VP, VP, VP]),
+    "cnt_lstm_backward_weights": (I, [VP, VP, VP, VP]),
     "cnt_lstm_state": (VP, [VP, I, I]),
     "cnt_lstm_weight_count": (C.c_long, [I, I, I]),
     "cnt_lstm_check": (I, [VP, VP]),
@@ -155,6 +159,14 @@ def dense_backward(P, D, N, act, bias, W, x, y, err, prev_err, dW, stream=None):
                                    ptr(prev_err), ptr(dW)))
 
 
+def dense_backward_errors(P, D, N, act, W, y, err, prev_err, stream=None):
+    check(lib().cnt_dense_backward_errors(stream_ptr(stream), P, D, N, act, ptr(W), ptr(y), ptr(err), ptr(prev_err)))
+
+
+def dense_backward_weights(P, D, N, bias, x, err, dW, stream=None):
+    check(lib().cnt_dense_backward_weights(stream_ptr(stream), P, D, N, bias, ptr(x), ptr(err), ptr(dW)))
+
+
 def sse_backward(D, N, pat, y, tgt, err, stream=None):
     check(lib().cnt_sse_backward(stream_ptr(stream), D, N, ptr(pat), ptr(y), ptr(tgt), ptr(err)))
 
@@ -196,6 +208,12 @@ class Lstm:
     def backward(self, W, x, out, outerr, prev_err, dW, stream=None):
         check(lib().cnt_lstm_backward(self.handle, stream_ptr(stream), ptr(W), ptr(x), ptr(out), ptr(outerr),
                                       ptr(prev_err), ptr(dW)))
+
+    def backward_errors(self, W, outerr, prev_err, stream=None):
+        check(lib().cnt_lstm_backward_errors(self.handle, stream_ptr(stream), ptr(W), ptr(outerr), ptr(prev_err)))
+
+    def backward_weights(self, x, dW, stream=None):
+        check(lib().cnt_lstm_backward_weights(self.handle, stream_ptr(stream), ptr(x), ptr(dW)))
 
     def check(self, stream=None):
         check(lib().cnt_lstm_check(self.handle, stream_ptr(stream)))

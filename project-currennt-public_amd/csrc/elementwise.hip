@@ -102,15 +102,16 @@ int cnt_dense_forward(void *stream_, int P, int D, int N, int act, float bias, c
     return gemm_launch(static_cast<hipStream_t>(stream_), ga);
 }
 
-int cnt_dense_backward(void *stream_, int P, int D, int N, int act, float bias, const float *weights, const float *x,
-                       const float *y, float *err, float *prev_err, float *weight_updates) {
+int cnt_dense_backward_errors(void *stream_, int P, int D, int N, int act, const float *weights, const float *y,
+                              float *err, float *prev_err) {
     using namespace cnt;
-    CNT_REQUIRE(weights && x && y && err && weight_updates, "dense_backward: null argument");
-    CNT_REQUIRE(P > 0 && D > 0 && N > 0, "dense_backward: non-positive size");
-    CNT_REQUIRE(act >= 0 && act <= 3, "dense_backward: unknown activation %d", act);
+    CNT_REQUIRE(weights && y && err, "dense_backward_errors: null argument");
+    CNT_REQUIRE(P > 0 && D > 0 && N > 0, "dense_backward_errors: non-positive size");
+    CNT_REQUIRE(act >= 0 && act <= 3, "dense_backward_errors: unknown activation %d", act);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const size_t count = (size_t)D * N;
     if (act != ACT_IDENTITY) {
+        ProfileScope prof(stream, "dense_delta");
         hipLaunchKernelGGL(dense_delta_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, err, y, count, act);
         CNT_HIP(hipGetLastError());
     }
@@ -125,6 +126,15 @@ int cnt_dense_backward(void *stream_, int P, int D, int N, int act, float bias, 
         ga.label = "gemm:dense_prev_errors";
         CNT_TRY(gemm_launch(stream, ga));
     }
+    return CNT_OK;
+}
+
+int cnt_dense_backward_weights(void *stream_, int P, int D, int N, float bias, const float *x, const float *err,
+                               float *weight_updates) {
+    using namespace cnt;
+    CNT_REQUIRE(x && err && weight_updates, "dense_backward_weights: null argument");
+    CNT_REQUIRE(P > 0 && D > 0 && N > 0, "dense_backward_weights: non-positive size");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
     CNT_TRY(fill_zero(stream, weight_updates, (size_t)P * D + D));
     {
         GemmArgs ga = {};
@@ -142,6 +152,14 @@ int cnt_dense_backward(void *stream_, int P, int D, int N, int act, float bias, 
         CNT_TRY(gemm_launch(stream, ga));
     }
     return column_sum(stream, err, D, N, bias, weight_updates + (size_t)P * D);
+}
+
+int cnt_dense_backward(void *stream, int P, int D, int N, int act, float bias, const float *weights, const float *x,
+                       const float *y, float *err, float *prev_err, float *weight_updates) {
+    using namespace cnt;
+    CNT_REQUIRE(x && weight_updates, "dense_backward: null argument");
+    CNT_TRY(cnt_dense_backward_errors(stream, P, D, N, act, weights, y, err, prev_err));
+    return cnt_dense_backward_weights(stream, P, D, N, bias, x, err, weight_updates);
 }
 
 int cnt_sse_backward(void *stream_, int D, int N, const char *patTypes, const float *y, const float *target,

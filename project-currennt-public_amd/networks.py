@@ -105,6 +105,34 @@ class StackedNetwork:
             else:
                 L["handle"].backward(L["weights"], x, L["outputs"], L["errors"], prev_err, L["updates"])
 
+    def backward_overlapped(self, side_stream):
+        """Same result as backward(); the weight-gradient halves run on `side_stream` while the main stream goes
+        on with the next layer's error recursion (nothing reads weight updates before the optimizer).  The caller
+        joins the two streams (torch.cuda.synchronize() or an event) before reading `updates`."""
+        N = self.T * self.S
+        main = torch.cuda.current_stream()
+        for i in range(len(self.layers) - 1, -1, -1):
+            L = self.layers[i]
+            t = L["type"]
+            x = self.layers[i - 1]["outputs"] if i > 0 else self.inputs
+            prev_err = self.layers[i - 1]["errors"] if i > 0 else self.input_errors
+            if t == "sse":
+                capi.sse_backward(L["size"], N, self.pat, self.layers[i - 1]["outputs"], L["outputs"], prev_err)
+                continue
+            if t in _FF_ACT:
+                capi.dense_backward_errors(L["prev"], L["size"], N, _FF_ACT[t], L["weights"], L["outputs"], L["errors"],
+                                           prev_err)
+            else:
+                L["handle"].backward_errors(L["weights"], L["errors"], prev_err)
+            ev = torch.cuda.Event()
+            ev.record(main)
+            side_stream.wait_event(ev)
+            if t in _FF_ACT:
+                capi.dense_backward_weights(L["prev"], L["size"], N, L["bias"], x, L["errors"], L["updates"],
+                                            stream=side_stream)
+            else:
+                L["handle"].backward_weights(x, L["updates"], stream=side_stream)
+
     def check(self):
         for L in self.layers:
             if "handle" in L:

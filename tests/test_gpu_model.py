@@ -49,6 +49,16 @@ def test_acoustic_model_forward_backward():
     net.backward()
     net.check()
     torch.cuda.synchronize()
+    plain_updates = [L["updates"].clone() for L in net.layers if "updates" in L]
+    # second pass with the weight-gradient halves on a side stream: same results
+    side = torch.cuda.Stream()
+    net.load_sequences(pat_d, T, min(lengths))
+    net.backward_overlapped(side)
+    torch.cuda.current_stream().wait_stream(side)
+    net.check()
+    torch.cuda.synchronize()
+    for a, L in zip(plain_updates, [L for L in net.layers if "updates" in L]):
+        assert PC.relerr(L["updates"].cpu().numpy(), a.cpu().numpy()) < 1e-5
 
     assert abs(loss - ref_loss) <= 1e-4 * abs(ref_loss)
     N = T * S
