@@ -94,6 +94,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--cpu-sample-T", type=int, default=160)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--workload", default="acoustic", choices=["acoustic", "lstm_c1", "mdn_c3", "dft_c5", "wavenet_c4"],
+                    help="acoustic = BASELINE configs[1] (the headline metric); the others are the remaining configs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no multi-GPU part); "
@@ -109,6 +111,12 @@ def main():
         sys.exit(3)
     pkg = load_package()
     capi, networks = pkg.capi, pkg.networks
+    if args.workload != "acoustic":
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        import bench_workloads
+
+        print(json.dumps(bench_workloads.run(args.workload, args, pkg)))
+        return
 
     S, Tmax, seed = 10, 600, 20240
     input_size, specs = networks.acoustic_model_spec()

@@ -1,0 +1,105 @@
+"""BASELINE config 4 as a benchmark workload: backward pass of the 30-block WaveNet-style stack,
+2 waveforms x 16000 samples.  A backward pass consumes state that only the forward pass rebuilds (the skip
+layers' cleared error buffers, the tanh(context) buffer that the gated layer overwrites with its gradient), so
+every timed backward is preceded by an untimed restore of exactly that state; the backward itself is timed with
+events on the launch stream."""
+import os
+import time
+
+import numpy as np
+
+import oracle_models as OM
+import wavenet_data as WD
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def flops_per_sample(nb, Q, R, K, C):
+    block = 2 * (2 * R * 2 * R) * 2 + 2 * C * 2 * R + 4 * R * R + 4 * R * K  # cnn dX+dW (2 live taps), cond dW, out, skip 1x1
+    return nb * block + 4 * K * K + 4 * K * Q + 2 * Q * R
+
+
+def run(args, pkg):
+    import torch
+
+    import bench_workloads as BW
+
+    capi, networks = pkg.capi, pkg.networks
+    nb, Q, R, K, C = 30, 1024, 64, 128, 80
+    lengths = [16000, 16000]
+    S, T = 2, 16000
+    pat, onehot, ctx, target, N = WD.make(lengths, Q, C, upsample=80, seed=4)
+    net = networks.WaveNet(networks.HipBackend(), nb, S, T, Q=Q, R=R, K=K, C=C, cnn_tanh=1)
+    shapes = {k: len(net.buf[k]["W"]) for k in net.weight_names()}
+    for k, w in WD.init_weights(shapes, seed=5).items():
+        net.buf[k]["W"].copy_(torch.from_numpy(w))
+    net.set_inputs(BW._dev(pat), BW._dev(onehot), BW._dev(ctx), BW._dev(target))
+    net.forward()
+    net.calculate_error()
+    saved = {k: v["cth"].clone() for k, v in net.buf.items() if "cth" in v}
+
+    def restore():
+        net.reset_skip_errors()
+        for k, v in saved.items():
+            net.buf[k]["cth"].copy_(v)
+
+    def timed_backward(n):
+        total = 0.0
+        for _ in range(n):
+            restore()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            net.backward()
+            e1.record()
+            torch.cuda.synchronize()
+            total += e0.elapsed_time(e1) * 1e-3
+        return total / n
+
+    timed_backward(args.warmup)
+    sec = timed_backward(args.steps)
+    capi.profile_enable(True)
+    restore()
+    net.backward()
+    torch.cuda.synchronize()
+    prof = capi.profile_read()
+    capi.profile_enable(False)
+    kernels = {k: {"launches": n, "avg_ms": ms / max(n, 1), "ms_per_step": ms} for k, (n, ms) in prof.items()}
+    dom = max(kernels, key=lambda k: kernels[k]["ms_per_step"])
+    step_flops = flops_per_sample(nb, Q, R, K, C) * N
+    roof = {"bound": "hbm", "kernel": dom, "traffic": None, "peak": PEAK_HBM_GBS, "unit": "GB/s"}
+    if dom == "gemm:cnn_dW":
+        # per launch: read x (R) and the deltas (2R) for each of the two live taps, write nothing of size N
+        nbytes = 2 * (R + 2 * R) * 4.0 * N
+    elif dom == "gemm:cnn_prev_errors":
+        nbytes = (2 * 2 * R + R) * 4.0 * N
+    else:
+        nbytes = 155e3 * N / max(1, sum(v["launches"] for v in kernels.values()))
+    roof["achieved"] = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
+    roof["frac"] = roof["achieved"] / PEAK_HBM_GBS
+    extra = {"roofline": roof, "kernels": kernels,
+             "step_roofline": {"bound": "hbm", "achieved": 155e3 * N / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                               "frac": 155e3 * N / sec / 1e9 / PEAK_HBM_GBS, "bytes_per_sample": 155e3,
+                               "mfma_tflops": step_flops / sec / 1e12}}
+    if not args.no_cpu:
+        # one block-sized slice of the same stack on the oracle: 2 blocks, 2 x 600 samples, scaled per sample and block
+        nb_s, T_s = 2, 600
+        p2, o2, c2, t2, N2 = WD.make([T_s, T_s], Q, C, upsample=80, seed=4)
+        ref = networks.WaveNet(OM.OracleBackend(), nb_s, S, T_s, Q=Q, R=R, K=K, C=C, cnn_tanh=1)
+        sh = {k: len(ref.buf[k]["W"]) for k in ref.weight_names()}
+        for k, w in WD.init_weights(sh, seed=5).items():
+            ref.buf[k]["W"][:] = w
+        ref.set_inputs(p2, o2, c2, t2)
+        ref.forward()
+        t0 = time.perf_counter()
+        ref.backward()
+        dt = time.perf_counter() - t0
+        # cost model: per-sample cost = a*blocks + b; measured with 2 blocks; the block-independent part (softmax
+        # layers) is included once, so scaling the whole by 30/2 overstates the CPU's speed: say so
+        extra["cpu_baseline"] = {"value": N2 / dt * nb_s / nb, "unit": "samples/s", "cores": 1, "kind": "port",
+                                 "sample": "CPU oracle on the same topology with 2 of the 30 blocks and 2 x 600 samples "
+                                           "(%.1f s), scaled by 2/30 per sample; host has %d cores" % (dt, os.cpu_count() or 0)}
+    net.close()
+    return BW._base(args, N / sec, "samples/s", sec,
+                    "configs[3]: WaveNet-style stack backward, 30 blocks (dilations 1..512 x3), 64 residual / 128 skip "
+                    "channels, 80-dim conditioning, 1024-way softmax, 2 x 16000 samples", extra)

@@ -1,0 +1,210 @@
+"""Secondary benchmark workloads (BASELINE configs 1, 3, 4, 5), reached through `bench.py --workload ...`.
+Each returns the same JSON fields as the headline workload: value in the config's unit, a roofline entry for
+the dominant kernel (duration from the library's HIP-event hooks) and a cpu_baseline (the oracle, one core)."""
+import os
+import time
+
+import numpy as np
+
+import oracle_lib as O
+from torch_models import make_pat_types
+
+METRIC = "BLSTM backward frames/sec at 1 MI355X; % HBM/MFMA roofline vs host CPU"
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def _timed(step, steps, warmup):
+    import torch
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def _profile(capi, step, steps):
+    import torch
+
+    capi.profile_enable(True)
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    prof = capi.profile_read()
+    capi.profile_enable(False)
+    return {k: {"launches": n, "avg_ms": ms / max(n, 1), "ms_per_step": ms / steps} for k, (n, ms) in prof.items()}
+
+
+def _base(args, value, unit, sec, workload, extra):
+    out = {"metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": 1e3 * sec, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+           "data": "synthetic", "config": {"workload": workload}}
+    out.update(extra)
+    return out
+
+
+def _dev(a):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def lstm_c1(args, pkg):
+    import torch
+
+    capi = pkg.capi
+    P, H, S, lengths = 382, 256, 4, [200, 200, 200, 150]
+    T, N = 200, 800
+    rng = np.random.default_rng(1)
+    nW = O.lib().orc_lstm_weight_count(P, H, 0)
+    W = rng.uniform(-0.1, 0.1, nW).astype(np.float32)
+    x = rng.standard_normal((T, S, P)).astype(np.float32)
+    err = (0.1 * rng.standard_normal((T, S, H))).astype(np.float32)
+    x[150:, 3] = 0
+    err[150:, 3] = 0
+    pat = make_pat_types(lengths, T)
+    layer = capi.Lstm(P, H, False, S, T, 1.0)
+    Wd, xd, pd = _dev(W), _dev(x.reshape(-1)), _dev(pat)
+    out = torch.zeros(H * N, device="cuda")
+    ex = torch.zeros(P * N, device="cuda")
+    dW = torch.zeros(nW, device="cuda")
+    err0 = _dev(err.reshape(-1))
+    errd = err0.clone()
+    layer.load_sequences(pd, T, 150)
+    layer.forward(Wd, xd, out)
+
+    def step():
+        errd.copy_(err0)  # the unidirectional backward adds the recurrent terms in place
+        layer.load_sequences(pd, T, 150)
+        layer.backward(Wd, xd, out, errd, ex, dW)
+
+    sec = _timed(step, args.steps, args.warmup)
+    layer.check()
+    kernels = _profile(capi, step, args.steps)
+    frames = sum(lengths)
+    dom = "lstm_backward_chain"
+    flops = 8.0 * H * H * N
+    ach = flops / (kernels[dom]["avg_ms"] * 1e-3) / 1e12
+    roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_FP32_MFMA_TFLOPS,
+            "traffic": None, "kernel": dom, "note": "latency-bound recursion (T sequential steps)"}
+    extra = {"roofline": roof, "kernels": kernels}
+    if not args.no_cpu:
+        desc = O.LstmDesc(P, H, 0, S, T, 150, 1.0)
+        fw = O.LstmState(H, N)
+        o = np.zeros(H * N, dtype=np.float32)
+        O.lstm_forward(desc, W, pat, x.reshape(-1), fw, None, o)
+        exo, dWo = np.zeros(P * N, dtype=np.float32), np.zeros_like(W)
+        t0 = time.perf_counter()
+        O.lstm_backward(desc, W, pat, x.reshape(-1), err.reshape(-1), fw, None, exo, dWo)
+        dt = time.perf_counter() - t0
+        extra["cpu_baseline"] = {"value": frames / dt, "unit": "frames/s", "cores": 1, "kind": "port",
+                                 "sample": "the full config-1 backward once (%.1f s), CPU oracle, host has %d cores" % (dt, os.cpu_count() or 0)}
+    layer.close()
+    return _base(args, frames / sec, "frames/s", sec,
+                 "configs[0]: unidirectional LSTM P=382 H=256 T=200 S=4 (one sequence of 150), full BPTT backward", extra)
+
+
+def mdn_c3(args, pkg):
+    import torch
+
+    capi = pkg.capi
+    M, D, S, T = 16, 60, 10, 600
+    F, Lp = S * T, 16 + 2 * 16 * 60
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((F, Lp)).astype(np.float32)
+    x[:, M + M * D:] *= 0.5
+    tgt = rng.standard_normal((F, D)).astype(np.float32)
+    pat = make_pat_types([T] * S, T)
+    layer = capi.Mdn(Lp, D, S, T, [1, 0, Lp, 0, D, M])
+    pd, xd, td = _dev(pat), _dev(x.reshape(-1)), _dev(tgt.reshape(-1))
+    res = torch.zeros(1, device="cuda")
+    err = torch.zeros(F * Lp, device="cuda")
+    layer.load_sequences(pd, T)
+    layer.forward(xd)
+    layer.calculate_error(td, res)
+
+    def step():
+        layer.backward(td, err)
+
+    sec = _timed(step, args.steps, args.warmup)
+    kernels = _profile(capi, step, args.steps)
+    dom = "mdn_mixture_backward"
+    nbytes = F * (Lp * 4 + (M + 1) * 4 + D * 4 + Lp * 4)
+    ach = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
+    roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None,
+            "kernel": dom}
+
+    def full():
+        layer.forward(xd)
+        layer.calculate_error(td, res)
+        layer.backward(td, err)
+
+    sec_full = _timed(full, args.steps, 1)
+    extra = {"roofline": roof, "kernels": kernels, "forward_error_backward_ms": 1e3 * sec_full}
+    if not args.no_cpu:
+        para = np.zeros(F * M * (1 + 2 * D), dtype=np.float32)
+        tmp = np.zeros(F * M + F, dtype=np.float32)
+        eo = np.zeros(F * Lp, dtype=np.float32)
+        O.mdn_mixture_forward(F, Lp, 0, M, D, 0.0, pat, x.reshape(-1), para)
+        O.mdn_mixture_error(F, D, 0, M, D, pat, tgt.reshape(-1), para, tmp)
+        t0 = time.perf_counter()
+        for _ in range(20):
+            O.mdn_mixture_backward(F, Lp, D, 0, 0, M, D, 0.0, pat, tgt.reshape(-1), para, tmp, eo)
+        dt = (time.perf_counter() - t0) / 20
+        extra["cpu_baseline"] = {"value": F / dt, "unit": "frames/s", "cores": 1, "kind": "port",
+                                 "sample": "the full config-3 gradient, 20 repetitions (%.2f s each), CPU oracle, host has %d cores" % (dt, os.cpu_count() or 0)}
+    layer.close()
+    return _base(args, F / sec, "frames/s", sec,
+                 "configs[2]: mixture density layer backward, 16 mixtures x 60 dims, T=600 S=10 (6000 frames)", extra)
+
+
+def dft_c5(args, pkg):
+    import torch
+
+    capi = pkg.capi
+    res = [(512, 512, 80), (128, 128, 40), (2048, 2048, 640)]
+    W, n = 8, 16000
+    rng = np.random.default_rng(5)
+    src = (0.3 * rng.standard_normal((W, n))).astype(np.float32)
+    tgt = (0.3 * rng.standard_normal((W, n))).astype(np.float32)
+    layer = capi.Dft(res, n, W)
+    sd, td = _dev(src.reshape(-1)), _dev(tgt.reshape(-1))
+    errs = torch.zeros(W * 3, device="cuda")
+    grad = torch.zeros(W * n, device="cuda")
+
+    def step():
+        layer.forward([n] * W, sd, td, errs)
+        layer.backward(grad)
+
+    sec = _timed(step, args.steps, args.warmup)
+    kernels = _profile(capi, step, args.steps)
+    dom = "dft_loss"
+    nbytes = 12.0 * W * n  # per launch = one resolution: read source + target, write gradient
+    ach = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
+    roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None,
+            "kernel": dom, "note": "4.6 MB and 0.17 GFLOP in total: launch- and latency-bound, far from either roof"}
+    extra = {"roofline": roof, "kernels": kernels}
+    if not args.no_cpu:
+        g = np.zeros(n, dtype=np.float32)
+        t0 = time.perf_counter()
+        for (N, Nw, Hs) in res:
+            O.dft_logamp_loss(N, Nw, Hs, 0, n, n, 1.0, 1e-5, src[0].copy(), tgt[0].copy(), g)
+        dt = time.perf_counter() - t0
+        extra["cpu_baseline"] = {"value": n / dt, "unit": "samples/s", "cores": 1, "kind": "port",
+                                 "sample": "one of the 8 waveforms, all three resolutions (%.2f s); the reference has no host FFT, "
+                                           "the oracle's own double-precision radix-2 FFT is used; host has %d cores" % (dt, os.cpu_count() or 0)}
+    layer.close()
+    return _base(args, W * n / sec, "samples/s", sec,
+                 "configs[4]: DFT multi-resolution log-amplitude loss, forward (loss + gradient) and backward, 8 x 16000 samples", extra)
+
+
+def run(name, args, pkg):
+    if name == "wavenet_c4":
+        import bench_wavenet
+
+        return bench_wavenet.run(args, pkg)
+    return {"lstm_c1": lstm_c1, "mdn_c3": mdn_c3, "dft_c5": dft_c5}[name](args, pkg)

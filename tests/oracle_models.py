@@ -83,3 +83,71 @@ class OracleNetwork:
             else:
                 O.lstm_backward(L["desc"], L["weights"], self.pat, x, L["errors"], L["fw"], L["bw"], prev_err,
                                 L["updates"])
+
+
+class OracleSoftmax:
+    """Softmax MDN unit on the oracle with the interface the WaveNet graph walk expects."""
+
+    def __init__(self, Lp, S, T):
+        self.Lp, self.S, self.T = Lp, S, T
+        self.prob = np.zeros(Lp * S * T, dtype=np.float32)
+
+    def load_sequences(self, pat, T):
+        self.pat = pat
+
+    def forward(self, x):
+        O.softmax_forward(self.S * self.T, self.Lp, 0, self.Lp, 1.0, self.pat, x, self.prob)
+
+    def calculate_error(self, target, loss):
+        loss[0] = O.softmax_error(self.S * self.T, 1, 0, self.Lp, len(self.prob), self.pat, target, self.prob)
+
+    def backward(self, target, err):
+        err[:] = 0
+        O.softmax_backward(self.S * self.T, self.Lp, 1, 0, 0, self.Lp, self.pat, target, self.prob, err)
+
+    def close(self):
+        pass
+
+
+class OracleBackend:
+    """Layer primitives on the CPU oracle; buffers are numpy arrays."""
+
+    def zeros(self, n):
+        return np.zeros(n, dtype=np.float32)
+
+    def upload(self, a):
+        return np.ascontiguousarray(a)
+
+    def dense_forward(self, P, D, N, act, W, x, y):
+        O.dense_forward(P, D, N, act, 1.0, W, x, y)
+
+    def dense_backward(self, P, D, N, act, W, x, y, err, prev_err, dW):
+        O.dense_backward(P, D, N, act, 1.0, W, x, y, err, prev_err, dW)
+
+    def cnn_forward(self, key, P, D, S, T, dil, out_tanh, pat, W, x, out):
+        hw, it = np.ones(D, dtype=np.int32), np.full(D, dil, dtype=np.int32)
+        con = np.zeros(3 * D * S * T, dtype=np.float32)
+        O.cnn_forward(P, D, S, T, 1, out_tanh, 1.0, hw, it, pat, W, x, con, out)
+
+    def cnn_backward(self, key, P, D, S, T, dil, out_tanh, pat, W, x, out, err, prev_err, dW):
+        hw, it = np.ones(D, dtype=np.int32), np.full(D, dil, dtype=np.int32)
+        con = np.zeros(3 * D * S * T, dtype=np.float32)
+        O.cnn_backward(P, D, S, T, 1, out_tanh, 1.0, hw, it, pat, W, x, out, err, con, prev_err, dW)
+
+    def wavnetc_forward(self, D, C, N, pat, W, ctx, conv, core, cth, out):
+        O.wavnetc_forward(D, C, N, pat, W, ctx, conv, core, cth, out)
+
+    def wavnetc_backward(self, D, C, N, pat, W, ctx, core, cth, err, prev_err, dW):
+        O.wavnetc_backward(D, C, N, pat, W, ctx, core, cth, err, prev_err, dW, None)
+
+    def skipadd_forward(self, inputs, out, errors, errors_from_skip):
+        O.skipadd_forward(inputs, out, errors, errors_from_skip)
+
+    def skipadd_backward(self, errors, errors_from_skip, targets, is_skip, zero):
+        O.skipadd_backward(errors, errors_from_skip, targets, is_skip)
+
+    def softmax_make(self, Lp, S, T):
+        return OracleSoftmax(Lp, S, T)
+
+    def close(self):
+        pass
