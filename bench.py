@@ -96,6 +96,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--workload", default="acoustic", choices=["acoustic", "lstm_c1", "mdn_c3", "dft_c5", "wavenet_c4"],
                     help="acoustic = BASELINE configs[1] (the headline metric); the others are the remaining configs")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (a kernel of known traffic, to scale rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no multi-GPU part); "
@@ -111,6 +114,13 @@ def main():
         sys.exit(3)
     pkg = load_package()
     capi, networks = pkg.capi, pkg.networks
+    if args.calibrate_copy:
+        a = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
     if args.workload != "acoustic":
         sys.path.insert(0, os.path.join(ROOT, "tests"))
         import bench_workloads
