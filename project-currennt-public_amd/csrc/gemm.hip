@@ -6,9 +6,12 @@
 // products of a BLSTM become one pass), several independent problems per launch, split-K for the
 // long-K weight-gradient shapes, and a fused bias + activation epilogue for the dense forward.
 //
-// Tiling: 128 x 128 x 16 per workgroup, four 64-lane waves in a 2 x 2 arrangement, each wave owning
-// a 64 x 64 block as 2 x 2 tiles of v_mfma_f32_32x32x2_f32.  Both operand tiles sit in LDS as
-// [row][k] with a 20-float row pitch so that the 16-byte fragment reads are bank-conflict free.
+// Tiling: 128 x 128 x 32 per workgroup, four 64-lane waves in a 2 x 2 arrangement, each wave owning
+// a 64 x 64 block as 2 x 2 tiles of v_mfma_f32_32x32x2_f32.  An operand tile sits in LDS in the
+// orientation it has in memory, so that staging never transposes: k-contiguous operands as [row][k] with
+// a (BK+4)-float pitch (16-byte fragment reads, conflict free), row-contiguous operands as [k][row]
+// (4-byte fragment reads along consecutive rows).  A transposing store of the latter into [row][k]
+// costs a 16-way LDS bank conflict.
 // The MFMA operands are swapped (the B tile feeds the instruction's A port) so that lane%32 walks
 // along the column-major output's contiguous dimension and every store is a 128-byte segment.
 #include "common.hpp"
@@ -102,6 +105,22 @@ struct TileStage {
         }
     }
 
+    // k values [k_first, k_first + BK/2) of tile row `row`, in MFMA issue order
+    static __device__ __forceinline__ void fragment(const float *__restrict__ lds, int row, int k_first,
+                                                    float (&f)[BK / 2]) {
+        if (KCONTIG) {
+            const float *p = lds + row * PITCH + k_first;
+#pragma unroll
+            for (int q = 0; q < BK / 8; ++q) {
+                const float4 v = *reinterpret_cast<const float4 *>(p + 4 * q);
+                f[4 * q] = v.x; f[4 * q + 1] = v.y; f[4 * q + 2] = v.z; f[4 * q + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < BK / 2; ++q) f[q] = lds[(k_first + q) * 128 + row];
+        }
+    }
+
     __device__ __forceinline__ void store(float *__restrict__ lds, int tid) const {
         if (KCONTIG) {
             constexpr int TPR = BK / VEC;
@@ -117,11 +136,8 @@ struct TileStage {
             const int rq = (tid % TPK) * VEC;
             const int kk = tid / TPK;
 #pragma unroll
-            for (int p = 0; p < NLOAD; ++p) {
-                const float *e = reinterpret_cast<const float *>(&r[p]);
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) lds[(rq + j) * PITCH + kk + p * KPP] = e[j];
-            }
+            for (int p = 0; p < NLOAD; ++p)
+                *reinterpret_cast<typename VecT<VEC>::type *>(lds + (kk + p * KPP) * 128 + rq) = r[p];
         }
     }
 };
@@ -174,7 +190,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     __syncthreads();
 
     const int frag_row = lane & 31;
-    const int frag_k = (lane >> 5) * 8;
+    constexpr int FK = BK / 2;  // k values per half-wave and tile
+    const int frag_k = (lane >> 5) * FK;
 
     for (int it = it_begin; it < it_end; ++it) {
         const int cur = (it - it_begin) & 1;
@@ -187,26 +204,19 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
                     args.b_time_on_k != 0);
         }
 
-        float4 fa[2][2], fb[2][2];
+        float fa[2][FK], fb[2][FK];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const float *pa = &lds_a[cur][(wm * 64 + i * 32 + frag_row) * PITCH + frag_k];
-            fa[i][0] = *reinterpret_cast<const float4 *>(pa);
-            fa[i][1] = *reinterpret_cast<const float4 *>(pa + 4);
-            const float *pbq = &lds_b[cur][(wn * 64 + i * 32 + frag_row) * PITCH + frag_k];
-            fb[i][0] = *reinterpret_cast<const float4 *>(pbq);
-            fb[i][1] = *reinterpret_cast<const float4 *>(pbq + 4);
+            TileStage<VA, AK>::fragment(lds_a[cur], wm * 64 + i * 32 + frag_row, frag_k, fa[i]);
+            TileStage<VB, BK_>::fragment(lds_b[cur], wn * 64 + i * 32 + frag_row, frag_k, fb[i]);
         }
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
+        for (int kk = 0; kk < FK; ++kk) {
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                const float av = reinterpret_cast<const float *>(&fa[i][0])[kk];
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const float bv = reinterpret_cast<const float *>(&fb[j][0])[kk];
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv, av, acc[i][j], 0, 0, 0);
-                }
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][kk], fa[i][kk], acc[i][j], 0, 0, 0);
             }
         }
 
