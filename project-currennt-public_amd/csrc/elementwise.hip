@@ -13,6 +13,12 @@ __global__ void fill_zero_kernel(float *__restrict__ p, size_t count) {
     for (; i < count; i += stride) p[i] = 0.0f;
 }
 
+__global__ void fill_words_kernel(unsigned *__restrict__ p, size_t count, unsigned word) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) p[i] = word;
+}
+
 // delta = act'(y) * err in place, on every slot (the reference does not mask padding here)
 __global__ void dense_delta_kernel(float *__restrict__ err, const float *__restrict__ y, size_t count, int act) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -67,6 +73,13 @@ inline int stream_blocks(size_t count) {
 int fill_zero(hipStream_t stream, float *p, size_t count) {
     if (count == 0) return CNT_OK;
     hipLaunchKernelGGL(fill_zero_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, p, count);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+int fill_words(hipStream_t stream, unsigned *p, size_t count, unsigned word) {
+    if (count == 0) return CNT_OK;
+    hipLaunchKernelGGL(fill_words_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, p, count, word);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }

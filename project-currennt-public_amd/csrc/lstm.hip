@@ -45,7 +45,8 @@ struct DirPtrs {
     const float *w_int;    // gate 0 block of this direction; gate g at + g*L*H
     const float *b[4];     // bias weights per gate
     const float *peep[3];  // ig, fg, og peepholes
-    u64 *mailbox;          // 2 slots
+    u64 *mailbox;          // forward: 2 slots of tagged words
+    float *bmail;          // backward: 3 slots of plain words
 };
 
 struct ChainParams {
@@ -287,18 +288,71 @@ __global__ __launch_bounds__(kThreads) void lstm_forward_chain(const ChainParams
 
 // ---------------------------------------------------------------------------------------------------
 // Backward (error) recursion.
+//
+// The partial output errors travel through a mailbox of plain 4-byte words, laid out
+// [slot][receiving workgroup][sending workgroup][sequence][cell of the receiver]:
+//   * a word that holds kEmpty (an all-ones NaN pattern no product can yield) has not been written yet;
+//     a sender stores the JB values of one (receiver, sequence) pair as 16-byte vectors, a receiver polls
+//     its contiguous G*S*JB words with 16-byte loads and validates every word on its own;
+//   * after reading, the receiver puts kEmpty back.  Three slots rotate (step % 3): the reset of a slot is
+//     issued in step k+1, the receiver's next wait (step k+2) drains all of its outstanding stores before
+//     it can finish, and the sender writes the slot again only in step k+3, after it has seen what the
+//     receiver published at the end of step k+2 -- so the reset is always ordered before the rewrite.
+// The host fills the mailbox with kEmpty before every launch.
 // ---------------------------------------------------------------------------------------------------
+constexpr unsigned kEmpty = 0xFFFFFFFFu;
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+// s_waitcnt vmcnt(0) (expcnt and lgkmcnt left at their maxima) as a builtin, so that the compiler's own wait
+// insertion sees that nothing is outstanding afterwards and adds no waits of its own for older loads.
+__device__ __forceinline__ void wait_all_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// N 16-byte loads that bypass the non-coherent caches (device scope), all in flight together, then one wait.
+// Inline assembly because the polled words change under the compiler's feet: the loads may neither be
+// hoisted out of the polling loop nor merged.
+template <int N>
+__device__ __forceinline__ void poll_load(const float *base, unsigned byte_off, unsigned q_stride_bytes,
+                                          u32x4 (&w)[N]) {
+#pragma unroll
+    for (int q = 0; q < N; ++q) {
+        const float *bq = reinterpret_cast<const float *>(reinterpret_cast<const char *>(base) +
+                                                          (size_t)q * q_stride_bytes);
+        asm volatile("global_load_dwordx4 %0, %1, %2 sc1" : "=v"(w[q]) : "v"(byte_off), "s"(bq) : "memory");
+    }
+    wait_all_vmem();
+#pragma unroll
+    for (int q = 0; q < N; ++q) asm volatile("" : "+v"(w[q]));  // consumers stay behind the wait
+}
+
+// 16-byte store written through to the device-coherent level (cache policy bit 4 = sc1).  A compiler builtin,
+// unlike the loads above, so that the compiler's own wait counting knows the store is in flight.
+__device__ __forceinline__ void store128_device(__amdgpu_buffer_rsrc_t rsrc, unsigned byte_off, u32x4 v) {
+    __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (int)byte_off, 0, 16);
+}
+
+// Workgroup layout: four "main" waves carry the recursion (poll, reduce, cell update, product, publish); a
+// fifth "memory" wave owns every other global access of the step.  One step ahead it loads what the cell
+// update needs, folds everything that does not depend on the recursion into five coefficients per cell and
+// leaves them in LDS; one step behind it writes the results of the cell update to the state arrays.  The main
+// waves therefore never have an ordinary global load or store in flight: the only memory operations they wait
+// for are their own mailbox polls, and the compiler has no reason to insert waits into the loop.
+constexpr int kBwdThreads = kThreads + 64;
+
 template <int HT, int JB, int NT>
-__global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParams p) {
+__global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainParams p) {
     constexpr int H = 64 * HT;
     constexpr int G = H / JB;
     constexpr int NS = 16 * NT;
     constexpr int MT = H / 64;  // 16-row tiles of receiving cells per wave (each wave covers H/4)
     constexpr int KS = JB;      // k = (gate, own cell): 4*JB values, 4 per MFMA
     constexpr int EL = JB * NS; // (cell, sequence) pairs of this workgroup, padded
-    constexpr int NPART = kThreads / EL;
-    constexpr int NPOLL = G / NPART;
-    static_assert(kThreads % EL == 0 && G % NPART == 0, "mailbox polling layout");
+    constexpr int JV = JB / 4;  // 16-byte vectors per (sender, sequence) pair
+    constexpr int PG = kThreads / NS;   // sender groups polled side by side
+    constexpr int NPOLL = G / PG;       // senders per polling lane
+    constexpr int PITCH = EL + 4;
+    constexpr int EIT = (EL + 63) / 64; // elements per lane of the memory wave
+    static_assert(G % PG == 0 && NPOLL >= 1 && JB % 4 == 0 && EL <= kThreads, "mailbox polling layout");
+    enum { C_OG = 0, C_CE, C_NI, C_FG, C_IG, C_E, C_DOG, C_FGACT, C_DUMMY, NCOEF };
 
     int dir, me;
     if (!map_block(p, G, dir, me)) return;
@@ -308,12 +362,90 @@ __global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParam
     const int j0 = me * JB;
     const int n = S * H;
 
-    __shared__ float psum[NPART][JB][NS + 1];
+    __shared__ __attribute__((aligned(16))) float psum[PG][PITCH];
     __shared__ float dl[4 * JB][NS + 1];
+    __shared__ float coef[NCOEF][EL];
+    __shared__ float res[2][EL];  // summed output error, cell error
     __shared__ int wait_failed;
     if (threadIdx.x == 0) wait_failed = 0;
-    lds_barrier();
 
+    auto slot_of = [&](int step) { return dir ? step : (T - 1 - step); };
+
+    if (wave == kWaves) {
+        // ------------------------------------------------------------------ memory wave
+        struct StepIn { float e, ni, ig, fg, og, dog_old, c, c_earlier; char pat; };
+        int cs[EIT], cj[EIT];
+        bool valid[EIT];
+#pragma unroll
+        for (int it = 0; it < EIT; ++it) {
+            const int id = it * 64 + lane;
+            cs[it] = id / JB; cj[it] = id % JB;
+            valid[it] = id < EL && cs[it] < S;
+        }
+        auto load_step = [&](int step, StepIn (&v)[EIT]) {
+            const int t = slot_of(step);
+#pragma unroll
+            for (int it = 0; it < EIT; ++it) {
+                v[it] = StepIn{0, 0, 0, 0, 0, 0, 0, 0, 1};
+                if (!valid[it]) continue;
+                const size_t gi = (size_t)t * n + (size_t)cs[it] * H + j0 + cj[it];
+                v[it].e = p.outerr[((size_t)t * S + cs[it]) * p.L + dir * H + j0 + cj[it]];
+                v[it].ni = D.ni[gi]; v[it].ig = D.ig[gi]; v[it].fg = D.fg[gi]; v[it].og = D.og[gi];
+                v[it].dog_old = D.dog[gi];
+                v[it].c = D.c[gi];
+                if (step + 1 < T)
+                    v[it].c_earlier = D.c[(size_t)slot_of(step + 1) * n + (size_t)cs[it] * H + j0 + cj[it]];
+                v[it].pat = p.pat[t * S + cs[it]];
+            }
+        };
+        auto put_coef = [&](int step, const StepIn (&v)[EIT]) {
+            const int t = slot_of(step);
+#pragma unroll
+            for (int it = 0; it < EIT; ++it) {
+                const int id = it * 64 + lane;
+                if (id >= EL) continue;
+                const StepIn &x = v[it];
+                const float tc = tanh_act(x.c);
+                coef[C_OG][id] = logistic_deriv(x.og) * tc;         // d_og = this * e + dog_old
+                coef[C_CE][id] = x.og * tanh_deriv(tc);             // ce   = this * e + ...
+                coef[C_NI][id] = x.ig * tanh_deriv(x.ni);           // d_ni = this * ce
+                coef[C_FG][id] = logistic_deriv(x.fg) * x.c_earlier;  // d_fg = this * ce
+                coef[C_IG][id] = logistic_deriv(x.ig) * x.ni;       // d_ig = this * ce
+                coef[C_E][id] = x.e;
+                coef[C_DOG][id] = x.dog_old;
+                coef[C_FGACT][id] = x.fg;
+                coef[C_DUMMY][id] = ((t >= p.Tmin) && (x.pat == 0)) ? 1.0f : 0.0f;
+            }
+        };
+        StepIn in[EIT];
+        load_step(0, in);
+        put_coef(0, in);
+        lds_barrier();  // start of the recursion
+        for (int step = 0; step < T; ++step) {
+            const int t = slot_of(step);
+            if (step > 0) {
+                lds_barrier();  // A: partial sums are in LDS
+                if (wait_failed) return;
+            }
+            if (step + 1 < T) load_step(step + 1, in);
+            lds_barrier();  // B: results of this step are in LDS
+#pragma unroll
+            for (int it = 0; it < EIT; ++it) {
+                if (!valid[it]) continue;
+                const int id = it * 64 + lane;
+                const size_t gi = (size_t)t * n + (size_t)cs[it] * H + j0 + cj[it];
+                D.dni[gi] = dl[0 * JB + cj[it]][cs[it]]; D.dig[gi] = dl[1 * JB + cj[it]][cs[it]];
+                D.dfg[gi] = dl[2 * JB + cj[it]][cs[it]]; D.dog[gi] = dl[3 * JB + cj[it]][cs[it]];
+                D.cerr[gi] = res[1][id];
+                if (p.herr_out) p.herr_out[gi] = res[0][id];
+                else D.herr[gi] = res[0][id];
+            }
+            if (step + 1 < T) put_coef(step + 1, in);
+        }
+        return;
+    }
+
+    // ---------------------------------------------------------------------- main waves
     // recurrent weights as MFMA A operands: row = receiving ("from") cell, k = (gate, own cell)
     float wA[MT][KS];
     {
@@ -327,10 +459,18 @@ __global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParam
         }
     }
 
-    // polling role: element (cell pj, sequence ps), sources part, part+NPART, ...
-    const int pe = tid % EL, part = tid / EL;
-    const int pj = pe / NS, ps = pe % NS;
-    // cell-phase role: jj fastest so that global accesses of neighbouring lanes touch one segment
+    // mailbox geometry, in floats
+    const unsigned pair_words = (unsigned)S * JB;           // one (receiver, sender) pair
+    const unsigned recv_words = (unsigned)G * pair_words;   // everything one receiver gets in a step
+    const size_t slot_words = (size_t)G * recv_words;
+    const size_t mail_bytes = 3 * slot_words * sizeof(float);
+    const __amdgpu_buffer_rsrc_t mail = __builtin_amdgcn_make_buffer_rsrc(D.bmail, 0, (int)mail_bytes, 0x00020000);
+    // polling role: sequence ps, senders pg, pg + PG, ...
+    const int ps = tid % NS, pg = tid / NS;
+    const bool polls = ps < S;
+    const unsigned poll_off = ((unsigned)(pg * S + ps) * JB) * 4u;  // bytes inside the receiver's block
+    const unsigned poll_stride = (unsigned)PG * pair_words * 4u;
+    // cell-update role: element tid = (sequence cs, cell cj), cell fastest
     const bool cell_thread = tid < EL;
     const int cs = tid / JB, cj = tid % JB;
     const bool cell_valid = cell_thread && cs < S;
@@ -342,58 +482,51 @@ __global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParam
     const bool timing = p.phase_ticks != nullptr;
     const long long tk_begin = timing ? wall_clock64() : 0;
 
-    // Everything the cell update reads besides the recursion is requested one step ahead (cell states
-    // two steps ahead, because a step also needs the cell state of the slot processed next), right
-    // after the wait of the current step; see the forward kernel.
-    struct StepIn { float e, ni, ig, fg, og, dog_old; char pat; };
-    auto slot_of = [&](int step) { return dir ? step : (T - 1 - step); };
-    auto load_step = [&](int step) {
-        StepIn v = {0, 0, 0, 0, 0, 0, 1};
-        if (cell_valid) {
-            const int t = slot_of(step);
-            const size_t gi = (size_t)t * n + (size_t)cs * H + j0 + cj;
-            v.e = p.outerr[((size_t)t * S + cs) * p.L + dir * H + j0 + cj];
-            v.ni = D.ni[gi]; v.ig = D.ig[gi]; v.fg = D.fg[gi]; v.og = D.og[gi];
-            v.dog_old = D.dog[gi];
-            v.pat = p.pat[t * S + cs];
-        }
-        return v;
-    };
-    auto load_c = [&](int step) {
-        if (!cell_valid || step >= T) return 0.0f;
-        return D.c[(size_t)slot_of(step) * n + (size_t)cs * H + j0 + cj];
-    };
-    StepIn cur = load_step(0);
-    float c_cur = load_c(0), c_next = load_c(1);
+    // weights and peepholes are in registers before the recursion starts
+    wait_all_vmem();
+    lds_barrier();  // start of the recursion: coefficients of step 0 are in LDS
 
     for (int step = 0; step < T; ++step) {
         const long long tk0 = timing ? wall_clock64() : 0;
-        const int t = slot_of(step);
         const bool first = (step == 0), last = (step == T - 1);
-        const size_t gi = (size_t)t * n + (size_t)cs * H + j0 + cj;
-        float e = cur.e;
-        const float ni = cur.ni, ig = cur.ig, fg = cur.fg, og = cur.og, dog_old = cur.dog_old;
-        const float c = c_cur, c_earlier = c_next;
-        const bool dummy = (t >= p.Tmin) && (cur.pat == 0);
 
         if (!first) {
-            const unsigned tag = p.tag_base + (unsigned)step;
-            const u64 *slot = D.mailbox + (size_t)((step - 1) & 1) * G * G * EL;
-            float part_sum = 0.0f;
+            const float *mine = D.bmail + (size_t)((step - 1) % 3) * slot_words + (size_t)me * recv_words;
             bool ok = true;
-            if (ps < S) {
-                const u64 *addr[NPOLL];
-                float v[NPOLL];
+            if (polls) {
+                u32x4 w[JV][NPOLL];
+                unsigned spins = 0;
+                for (;;) {
+                    unsigned worst = 0;
 #pragma unroll
-                for (int q = 0; q < NPOLL; ++q)
-                    addr[q] = slot + ((size_t)(me * G + part + NPART * q) * JB + pj) * NS + ps;
-                ok = mb_wait<NPOLL>(addr, v, tag, p.spin_limit, p.abort_flag);
+                    for (int jv = 0; jv < JV; ++jv) {
+                        poll_load<NPOLL>(mine, poll_off + 16u * jv, poll_stride, w[jv]);
 #pragma unroll
-                for (int q = 0; q < NPOLL; ++q) part_sum += v[q];
+                        for (int q = 0; q < NPOLL; ++q)
+                            worst = max(max(worst, w[jv][q].x), max(max(w[jv][q].y, w[jv][q].z), w[jv][q].w));
+                    }
+                    if (worst != kEmpty) break;
+                    if (++spins > p.spin_limit) { ok = false; break; }
+                    if ((spins & 255u) == 0u &&
+                        __hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+                        ok = false;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+#pragma unroll
+                for (int jv = 0; jv < JV; ++jv) {
+                    f32x4 sum = {0, 0, 0, 0};
+#pragma unroll
+                    for (int q = 0; q < NPOLL; ++q) sum += __builtin_bit_cast(f32x4, w[jv][q]);
+                    *reinterpret_cast<f32x4 *>(&psum[pg][ps * JB + 4 * jv]) = sum;
+                }
             }
-            psum[part][pj][ps] = part_sum;
+            // polling lanes have drained their memory operations; stated for all lanes so that the compiler
+            // knows nothing is outstanding here
+            wait_all_vmem();
             if (!ok) wait_failed = 1;
-            lds_barrier();
+            lds_barrier();  // A
             if (wait_failed) {
                 if (tid == 0) __hip_atomic_store(p.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 return;
@@ -401,39 +534,34 @@ __global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParam
         }
 
         const long long tk1 = timing ? wall_clock64() : 0;
-        if (!last) cur = load_step(step + 1);
-        c_cur = c_next;
-        c_next = load_c(step + 2);
         if (cell_valid) {
+            float e = coef[C_E][tid];
             if (!first) {
 #pragma unroll
-                for (int q = 0; q < NPART; ++q) e += psum[q][cj][cs];
+                for (int q = 0; q < PG; ++q) e += psum[q][tid];
             }
+            const float fg = coef[C_FGACT][tid];
             float s_ni = 0, s_ig = 0, s_fg = 0, s_og = 0, ce = 0;
-            if (!dummy) {
-                const float tc = tanh_act(c);
-                const float d_og = (logistic_deriv(og) * tc * e) + dog_old;
-                ce = og * tanh_deriv(tc) * e + p_og * d_og;
+            if (coef[C_DUMMY][tid] == 0.0f) {
+                const float d_og = (coef[C_OG][tid] * e) + coef[C_DOG][tid];
+                ce = coef[C_CE][tid] * e + p_og * d_og;
                 if (!first) ce += (fg_later * cerr_later + p_ig * dig_later + p_fg * dfg_later);
-                const float d_ni = ig * tanh_deriv(ni) * ce;
-                const float d_fg = last ? 0.0f : logistic_deriv(fg) * c_earlier * ce;
-                const float d_ig = logistic_deriv(ig) * ni * ce;
+                const float d_ni = coef[C_NI][tid] * ce;
+                const float d_fg = last ? 0.0f : coef[C_FG][tid] * ce;
+                const float d_ig = coef[C_IG][tid] * ce;
                 s_ni = clip1(d_ni); s_ig = clip1(d_ig); s_fg = clip1(d_fg); s_og = clip1(d_og);
             }
-            D.dni[gi] = s_ni; D.dig[gi] = s_ig; D.dfg[gi] = s_fg; D.dog[gi] = s_og; D.cerr[gi] = ce;
-            if (p.herr_out) p.herr_out[gi] = e;
-            else D.herr[gi] = e;
             dl[0 * JB + cj][cs] = s_ni; dl[1 * JB + cj][cs] = s_ig;
             dl[2 * JB + cj][cs] = s_fg; dl[3 * JB + cj][cs] = s_og;
+            res[0][tid] = e; res[1][tid] = ce;
             fg_later = fg; cerr_later = ce; dig_later = s_ig; dfg_later = s_fg;
         }
-        lds_barrier();
+        lds_barrier();  // B
         const long long tk2 = timing ? wall_clock64() : 0;
 
         if (!last) {
             // partial output errors of every receiving cell from this workgroup's deltas
-            const unsigned tag = p.tag_base + (unsigned)step + 1u;
-            u64 *slot = D.mailbox + (size_t)(step & 1) * G * G * EL;
+            const unsigned slot_off = (unsigned)((size_t)(step % 3) * slot_words * 4u);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const int s = nt * 16 + (lane & 15);
@@ -449,17 +577,31 @@ __global__ __launch_bounds__(kThreads) void lstm_backward_chain(const ChainParam
                 }
                 if (s < S) {
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            const int from = wave * (H / 4) + mt * 16 + 4 * (lane >> 4) + r;
-                            const int dst = from / JB, jd = from % JB;
-                            mb_store(slot + ((size_t)(dst * G + me) * JB + jd) * NS + s, acc[mt][r], tag);
-                        }
+                    for (int mt = 0; mt < MT; ++mt) {
+                        // the four accumulator rows of a lane are four neighbouring receiving cells
+                        const int from = wave * (H / 4) + mt * 16 + 4 * (lane >> 4);
+                        const int dst = from / JB, jd = from % JB;
+                        u32x4 v = __builtin_bit_cast(u32x4, acc[mt]);
+                        // a NaN that happens to look like the empty marker is sent as the default NaN
+                        v.x = v.x == kEmpty ? 0x7FC00000u : v.x; v.y = v.y == kEmpty ? 0x7FC00000u : v.y;
+                        v.z = v.z == kEmpty ? 0x7FC00000u : v.z; v.w = v.w == kEmpty ? 0x7FC00000u : v.w;
+                        store128_device(mail, slot_off + ((unsigned)dst * recv_words + (unsigned)(me * S + s) * JB + jd) * 4u, v);
+                    }
                 }
             }
         }
-        // `dl` and `psum` are rewritten only after the next step's barrier
+        if (!first && polls) {
+            // hand the words consumed in this step back as empty (off the critical path; the next wait drains
+            // these stores before it can complete)
+            const u32x4 empty = {kEmpty, kEmpty, kEmpty, kEmpty};
+            const unsigned mine_off = (unsigned)(((size_t)((step - 1) % 3) * slot_words + (size_t)me * recv_words) * 4u);
+#pragma unroll
+            for (int jv = 0; jv < JV; ++jv)
+#pragma unroll
+                for (int q = 0; q < NPOLL; ++q)
+                    store128_device(mail, mine_off + poll_off + 16u * jv + (unsigned)q * poll_stride, empty);
+        }
+        // `dl`, `res` and `psum` are rewritten only after the next step's barrier A
         if (timing) {
             const long long tk3 = wall_clock64();
             ph0 += tk1 - tk0; ph1 += tk2 - tk1; ph2 += tk3 - tk2;
@@ -525,8 +667,10 @@ struct cnt_lstm {
     int T, Tmin;  // current fraction
     const char *pat;
     float *state[2][12];
-    cnt::u64 *mailbox[2];
+    cnt::u64 *mailbox[2];  // forward recursion
     size_t mailbox_bytes;
+    float *bmail[2];       // backward recursion
+    size_t bmail_words;
     int *abort_flag;
     unsigned epoch;
     int device;
@@ -583,6 +727,7 @@ void fill_chain_params(const cnt_lstm *h, const float *weights, ChainParams &p) 
         for (int g = 0; g < 4; ++g) D.b[g] = weights + off_bias + (size_t)g * L + dir * H;
         for (int k = 0; k < 3; ++k) D.peep[k] = weights + off_peep + (size_t)k * L + dir * H;
         D.mailbox = h->mailbox[dir];
+        D.bmail = h->bmail[dir];
     }
     p.spin_limit = h->spin_limit;
     p.abort_flag = h->abort_flag;
@@ -606,11 +751,17 @@ int next_epoch(cnt_lstm *h, hipStream_t stream, unsigned &tag_base) {
 int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     chain_kernel_t k = pick_kernel(fwd, h->H, h->JB, h->NT);
     CNT_REQUIRE(k != nullptr, "lstm: no recursion kernel for H=%d JB=%d S=%d", h->H, h->JB, h->desc.S);
-    CNT_TRY(next_epoch(h, stream, p.tag_base));
+    if (fwd) {
+        CNT_TRY(next_epoch(h, stream, p.tag_base));
+    } else {
+        // every word of the backward mailbox starts out empty
+        for (int dir = 0; dir < h->ndir; ++dir)
+            CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->bmail[dir]), h->bmail_words, kEmpty));
+    }
     const int G = h->H / h->JB;
     const int blocks = h->xcd_pack ? 8 * G : h->ndir * G;
     ProfileScope prof(stream, fwd ? "lstm_forward_chain" : "lstm_backward_chain");
-    hipLaunchKernelGGL(k, dim3(blocks), dim3(kThreads), 0, stream, p);
+    hipLaunchKernelGGL(k, dim3(blocks), dim3(fwd ? kThreads : kBwdThreads), 0, stream, p);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
@@ -649,8 +800,9 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     hipError_t err = hipGetDevice(&h->device);
     const size_t nstate = (size_t)H * desc->maxT * desc->S;
     const int G = H / JB, NS = 16 * NT;
-    // forward needs H*NS words per slot, backward G*G*JB*NS = H*G*NS
-    h->mailbox_bytes = (size_t)2 * H * G * NS * sizeof(u64);
+    // forward: 2 slots of H*NS tagged words; backward: 3 slots of G*G*JB*S plain words
+    h->mailbox_bytes = (size_t)2 * H * NS * sizeof(u64);
+    h->bmail_words = (size_t)3 * G * H * desc->S;
     for (int dir = 0; dir < ndir && err == hipSuccess; ++dir) {
         for (int w = 0; w < 12 && err == hipSuccess; ++w) {
             err = hipMalloc(reinterpret_cast<void **>(&h->state[dir][w]), nstate * sizeof(float));
@@ -658,6 +810,7 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
         }
         if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->mailbox[dir]), h->mailbox_bytes);
         if (err == hipSuccess) err = hipMemset(h->mailbox[dir], 0, h->mailbox_bytes);
+        if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->bmail[dir]), h->bmail_words * sizeof(float));
     }
     if (err == hipSuccess && std::getenv("CNT_LSTM_TIMING"))
         err = hipMalloc(reinterpret_cast<void **>(&h->phase_ticks), 8 * 512 * 4 * sizeof(long long));
@@ -678,6 +831,7 @@ int cnt_lstm_destroy(cnt_lstm *h) {
         for (int w = 0; w < 12; ++w)
             if (h->state[dir][w]) (void)hipFree(h->state[dir][w]);
         if (h->mailbox[dir]) (void)hipFree(h->mailbox[dir]);
+        if (h->bmail[dir]) (void)hipFree(h->bmail[dir]);
     }
     if (h->abort_flag) (void)hipFree(h->abort_flag);
     if (h->phase_ticks) (void)hipFree(h->phase_ticks);
