@@ -429,6 +429,8 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
             }
             if (step + 1 < T) load_step(step + 1, in);
             lds_barrier();  // B: results of this step are in LDS
+            // coefficients first: the main waves need them at the next barrier A, the state stores can trail
+            if (step + 1 < T) put_coef(step + 1, in);
 #pragma unroll
             for (int it = 0; it < EIT; ++it) {
                 if (!valid[it]) continue;
@@ -440,7 +442,6 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
                 if (p.herr_out) p.herr_out[gi] = res[0][id];
                 else D.herr[gi] = res[0][id];
             }
-            if (step + 1 < T) put_coef(step + 1, in);
         }
         return;
     }
