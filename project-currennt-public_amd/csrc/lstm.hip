@@ -46,7 +46,7 @@ struct DirPtrs {
     const float *b[4];     // bias weights per gate
     const float *peep[3];  // ig, fg, og peepholes
     u64 *mailbox;          // forward: 2 slots of tagged words
-    float *bmail;          // backward: 3 slots of plain words
+    float *bmail;          // backward: kMailSlots slots of plain words
 };
 
 struct ChainParams {
@@ -61,7 +61,8 @@ struct ChainParams {
     unsigned spin_limit;
     int *abort_flag;
     int xcd_pack;
-    long long *phase_ticks;  // optional diagnostic: per workgroup 4 accumulated phase durations (100 MHz ticks)
+    long long *phase_ticks;  // optional diagnostic: per workgroup accumulated phase durations (100 MHz ticks)
+    int poll_delay, poll_gap;  // s_sleep units before the first poll of a step / between polls
 };
 
 __device__ __forceinline__ u64 mb_load(const u64 *p) {
@@ -329,21 +330,30 @@ __device__ __forceinline__ void poll_load(const float *base, unsigned byte_off, 
 __device__ __forceinline__ void store128_device(__amdgpu_buffer_rsrc_t rsrc, unsigned byte_off, u32x4 v) {
     __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (int)byte_off, 0, 16);
 }
-
-// Workgroup layout: four "main" waves carry the recursion (poll, reduce, cell update, product, publish); a
-// fifth "memory" wave owns every other global access of the step.  One step ahead it loads what the cell
-// update needs, folds everything that does not depend on the recursion into five coefficients per cell and
-// leaves them in LDS; one step behind it writes the results of the cell update to the state arrays.  The main
-// waves therefore never have an ordinary global load or store in flight: the only memory operations they wait
-// for are their own mailbox polls, and the compiler has no reason to insert waits into the loop.
-constexpr int kBwdThreads = kThreads + 64;
+// Workgroup layout, nine waves in three roles that meet at two workgroup barriers per step:
+//   receive waves (4)  poll the mailbox, reduce the partial errors through LDS (barrier A), run the cell update
+//                      and leave the gate deltas in LDS (barrier B).  They issue no stores at all, so the only
+//                      memory operations their wait counter ever covers are their own polls.
+//   product waves (4)  hold the recurrent weight slice as MFMA operands; after barrier B they multiply it with
+//                      the deltas and publish the partial errors.  They never wait for a store.
+//   memory wave (1)    owns every other global access: two steps ahead it loads what the cell update needs,
+//                      one step ahead it folds everything that does not depend on the recursion into five
+//                      coefficients per cell (LDS), one step behind it writes the cell update's results to the
+//                      state arrays.
+// Mailbox slots rotate over four steps.  The product waves also hand the words their workgroup consumed in a
+// step back as empty, and drain all of their stores once per step (right after barrier A, when only stores of
+// the previous step can still be in flight), so the reset of the words consumed in step k is complete before
+// this workgroup publishes in step k+1; a sender rewrites those words only in step k+3, after it has seen
+// that publication.
+constexpr int kBwdThreads = 2 * kThreads + 64;
+constexpr int kMailSlots = 4;
 
 template <int HT, int JB, int NT>
 __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainParams p) {
     constexpr int H = 64 * HT;
     constexpr int G = H / JB;
     constexpr int NS = 16 * NT;
-    constexpr int MT = H / 64;  // 16-row tiles of receiving cells per wave (each wave covers H/4)
+    constexpr int MT = H / 64;  // 16-row tiles of receiving cells per product wave (each covers H/4)
     constexpr int KS = JB;      // k = (gate, own cell): 4*JB values, 4 per MFMA
     constexpr int EL = JB * NS; // (cell, sequence) pairs of this workgroup, padded
     constexpr int JV = JB / 4;  // 16-byte vectors per (sender, sequence) pair
@@ -370,8 +380,14 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
     if (threadIdx.x == 0) wait_failed = 0;
 
     auto slot_of = [&](int step) { return dir ? step : (T - 1 - step); };
+    // mailbox geometry, in floats
+    const unsigned pair_words = (unsigned)S * JB;           // one (receiver, sender) pair
+    const unsigned recv_words = (unsigned)G * pair_words;   // everything one receiver gets in a step
+    const size_t slot_words = (size_t)G * recv_words;
+    const size_t mail_bytes = kMailSlots * slot_words * sizeof(float);
+    const __amdgpu_buffer_rsrc_t mail = __builtin_amdgcn_make_buffer_rsrc(D.bmail, 0, (int)mail_bytes, 0x00020000);
 
-    if (wave == kWaves) {
+    if (wave == 2 * kWaves) {
         // ------------------------------------------------------------------ memory wave
         struct StepIn { float e, ni, ig, fg, og, dog_old, c, c_earlier; char pat; };
         int cs[EIT], cj[EIT];
@@ -387,7 +403,7 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
 #pragma unroll
             for (int it = 0; it < EIT; ++it) {
                 v[it] = StepIn{0, 0, 0, 0, 0, 0, 0, 0, 1};
-                if (!valid[it]) continue;
+                if (!valid[it] || step >= T) continue;
                 const size_t gi = (size_t)t * n + (size_t)cs[it] * H + j0 + cj[it];
                 v[it].e = p.outerr[((size_t)t * S + cs[it]) * p.L + dir * H + j0 + cj[it]];
                 v[it].ni = D.ni[gi]; v[it].ig = D.ig[gi]; v[it].fg = D.fg[gi]; v[it].og = D.og[gi];
@@ -417,20 +433,23 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
                 coef[C_DUMMY][id] = ((t >= p.Tmin) && (x.pat == 0)) ? 1.0f : 0.0f;
             }
         };
-        StepIn in[EIT];
-        load_step(0, in);
-        put_coef(0, in);
-        lds_barrier();  // start of the recursion
-        for (int step = 0; step < T; ++step) {
+        const bool mtiming = p.phase_ticks != nullptr;
+        long long mbusy = 0;
+        // one step of the memory wave; `far` receives the inputs of step+2, `near` holds those of step+1
+        auto run_step = [&](const int step, StepIn (&far)[EIT], const StepIn (&near)[EIT]) __attribute__((always_inline)) -> bool {
             const int t = slot_of(step);
             if (step > 0) {
                 lds_barrier();  // A: partial sums are in LDS
-                if (wait_failed) return;
+                if (wait_failed) return false;
             }
-            if (step + 1 < T) load_step(step + 1, in);
+            // everything still in flight is at least a step old: state stores and mailbox resets of the
+            // previous step, inputs requested a step ago
+            wait_all_vmem();
+            load_step(step + 2, far);
             lds_barrier();  // B: results of this step are in LDS
-            // coefficients first: the main waves need them at the next barrier A, the state stores can trail
-            if (step + 1 < T) put_coef(step + 1, in);
+            const long long tm0 = mtiming ? wall_clock64() : 0;
+            // coefficients first: the receive waves need them at the next barrier A, the stores can trail
+            if (step + 1 < T) put_coef(step + 1, near);
 #pragma unroll
             for (int it = 0; it < EIT; ++it) {
                 if (!valid[it]) continue;
@@ -442,30 +461,112 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
                 if (p.herr_out) p.herr_out[gi] = res[0][id];
                 else D.herr[gi] = res[0][id];
             }
+            if (mtiming) mbusy += wall_clock64() - tm0;
+            return true;
+        };
+        StepIn in_a[EIT], in_b[EIT];
+        load_step(0, in_a);
+        load_step(1, in_b);
+        put_coef(0, in_a);
+        lds_barrier();  // start of the recursion
+        for (int step = 0; step < T; step += 2) {
+            if (!run_step(step, in_a, in_b)) return;
+            if (step + 1 < T && !run_step(step + 1, in_b, in_a)) return;
         }
+        if (mtiming && lane == 0) p.phase_ticks[(size_t)blockIdx.x * 6 + 5] = mbusy;
         return;
     }
 
-    // ---------------------------------------------------------------------- main waves
-    // recurrent weights as MFMA A operands: row = receiving ("from") cell, k = (gate, own cell)
-    float wA[MT][KS];
-    {
-        const int i = lane & 15, kq = lane >> 4;
+    if (wave >= kWaves) {
+        // ------------------------------------------------------------------ product waves
+        const int pw = wave - kWaves;
+        // recurrent weights as MFMA A operands: row = receiving ("from") cell, k = (gate, own cell)
+        float wA[MT][KS];
+        {
+            const int i = lane & 15, kq = lane >> 4;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const int k = 4 * ks + kq, g = k / JB, jj = k % JB;
-            const float *wg = D.w_int + (size_t)g * p.L * H + (size_t)(j0 + jj) * H;
+            for (int ks = 0; ks < KS; ++ks) {
+                const int k = 4 * ks + kq, g = k / JB, jj = k % JB;
+                const float *wg = D.w_int + (size_t)g * p.L * H + (size_t)(j0 + jj) * H;
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) wA[mt][ks] = wg[wave * (H / 4) + mt * 16 + i];
+                for (int mt = 0; mt < MT; ++mt) wA[mt][ks] = wg[pw * (H / 4) + mt * 16 + i];
+            }
         }
+        // reset role: the same words this workgroup's receive waves poll (sequence ps, senders pg, pg + PG, ...)
+        const int ptid = tid - kThreads;
+        const int ps = ptid % NS, pg = ptid / NS;
+        const unsigned poll_off = ((unsigned)(pg * S + ps) * JB) * 4u;
+        const unsigned poll_stride = (unsigned)PG * pair_words * 4u;
+        wait_all_vmem();
+        lds_barrier();  // start of the recursion
+        const bool timing = p.phase_ticks != nullptr;
+        long long busy = 0;
+        for (int step = 0; step < T; ++step) {
+            if (step > 0) {
+                lds_barrier();  // A
+                if (wait_failed) return;
+                // everything this wave stored in the previous step (partial errors, resets) is complete
+                // before it publishes again; the wait hides behind the cell update of the receive waves
+                wait_all_vmem();
+            }
+            lds_barrier();  // B: the deltas of this step are in LDS
+            const long long tp0 = timing ? wall_clock64() : 0;
+            if (step < T - 1) {
+                // partial output errors of every receiving cell from this workgroup's deltas
+                const unsigned slot_off = (unsigned)((size_t)(step % kMailSlots) * slot_words * 4u);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const int s = nt * 16 + (lane & 15);
+                    float bv[KS];
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) bv[ks] = dl[4 * ks + (lane >> 4)][s];
+                    // two tiles at a time: two independent accumulation chains keep the matrix pipe busy, and
+                    // the first partial errors leave while the later tiles are still computed
+#pragma unroll
+                    for (int m0 = 0; m0 < MT; m0 += 2) {
+                        f32x4 acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                            for (int u = 0; u < 2; ++u)
+                                if (m0 + u < MT)
+                                    acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(wA[m0 + u][ks], bv[ks], acc[u], 0, 0, 0);
+                        if (s < S) {
+#pragma unroll
+                            for (int u = 0; u < 2; ++u) {
+                                if (m0 + u >= MT) continue;
+                                // the four accumulator rows of a lane are four neighbouring receiving cells
+                                const int from = pw * (H / 4) + (m0 + u) * 16 + 4 * (lane >> 4);
+                                const int dst = from / JB, jd = from % JB;
+                                u32x4 v = __builtin_bit_cast(u32x4, acc[u]);
+                                // a NaN that happens to look like the empty marker is sent as the default NaN
+                                v.x = v.x == kEmpty ? 0x7FC00000u : v.x; v.y = v.y == kEmpty ? 0x7FC00000u : v.y;
+                                v.z = v.z == kEmpty ? 0x7FC00000u : v.z; v.w = v.w == kEmpty ? 0x7FC00000u : v.w;
+                                store128_device(mail, slot_off + ((unsigned)dst * recv_words + (unsigned)(me * S + s) * JB + jd) * 4u, v);
+                            }
+                        }
+                    }
+                }
+            }
+            if (step > 0 && ps < S) {
+                // the words the receive waves consumed in this step (before barrier A) are empty again
+                const u32x4 empty = {kEmpty, kEmpty, kEmpty, kEmpty};
+                const unsigned mine_off =
+                    (unsigned)(((size_t)((step - 1) % kMailSlots) * slot_words + (size_t)me * recv_words) * 4u);
+#pragma unroll
+                for (int jv = 0; jv < JV; ++jv)
+#pragma unroll
+                    for (int q = 0; q < NPOLL; ++q)
+                        store128_device(mail, mine_off + poll_off + 16u * jv + (unsigned)q * poll_stride, empty);
+            }
+            // `dl` is rewritten only after the next barrier A, which this wave reaches after its LDS reads
+            if (timing) busy += wall_clock64() - tp0;
+        }
+        if (timing && tid == kThreads) p.phase_ticks[(size_t)blockIdx.x * 6 + 2] = busy;
+        return;
     }
 
-    // mailbox geometry, in floats
-    const unsigned pair_words = (unsigned)S * JB;           // one (receiver, sender) pair
-    const unsigned recv_words = (unsigned)G * pair_words;   // everything one receiver gets in a step
-    const size_t slot_words = (size_t)G * recv_words;
-    const size_t mail_bytes = 3 * slot_words * sizeof(float);
-    const __amdgpu_buffer_rsrc_t mail = __builtin_amdgcn_make_buffer_rsrc(D.bmail, 0, (int)mail_bytes, 0x00020000);
+    // ---------------------------------------------------------------------- receive waves
     // polling role: sequence ps, senders pg, pg + PG, ...
     const int ps = tid % NS, pg = tid / NS;
     const bool polls = ps < S;
@@ -479,24 +580,26 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
     if (cell_valid) { p_ig = D.peep[0][j0 + cj]; p_fg = D.peep[1][j0 + cj]; p_og = D.peep[2][j0 + cj]; }
     // this cell's values at the slot processed in the previous iteration
     float fg_later = 0, cerr_later = 0, dig_later = 0, dfg_later = 0;
-    long long ph0 = 0, ph1 = 0, ph2 = 0, ph3 = 0;
+    long long ph0 = 0, ph1 = 0, ph3 = 0, poll_rounds = 0;
     const bool timing = p.phase_ticks != nullptr;
     const long long tk_begin = timing ? wall_clock64() : 0;
 
-    // weights and peepholes are in registers before the recursion starts
-    wait_all_vmem();
-    lds_barrier();  // start of the recursion: coefficients of step 0 are in LDS
+    wait_all_vmem();  // peepholes are in registers before the recursion starts
+    lds_barrier();    // start of the recursion: coefficients of step 0 are in LDS
 
     for (int step = 0; step < T; ++step) {
         const long long tk0 = timing ? wall_clock64() : 0;
         const bool first = (step == 0), last = (step == T - 1);
 
         if (!first) {
-            const float *mine = D.bmail + (size_t)((step - 1) % 3) * slot_words + (size_t)me * recv_words;
+            const float *mine = D.bmail + (size_t)((step - 1) % kMailSlots) * slot_words + (size_t)me * recv_words;
             bool ok = true;
             if (polls) {
                 u32x4 w[JV][NPOLL];
                 unsigned spins = 0;
+                // the partial errors cannot be there before the senders' products are done: a poll that comes back
+                // incomplete costs a whole memory round trip, a poll that starts a little late only the delay
+                for (int d = 0; d < p.poll_delay; ++d) __builtin_amdgcn_s_sleep(1);
                 for (;;) {
                     unsigned worst = 0;
 #pragma unroll
@@ -506,6 +609,7 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
                         for (int q = 0; q < NPOLL; ++q)
                             worst = max(max(worst, w[jv][q].x), max(max(w[jv][q].y, w[jv][q].z), w[jv][q].w));
                     }
+                    if (timing) ++poll_rounds;
                     if (worst != kEmpty) break;
                     if (++spins > p.spin_limit) { ok = false; break; }
                     if ((spins & 255u) == 0u &&
@@ -513,7 +617,7 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
                         ok = false;
                         break;
                     }
-                    __builtin_amdgcn_s_sleep(1);
+                    for (int d = 0; d < p.poll_gap; ++d) __builtin_amdgcn_s_sleep(1);
                 }
 #pragma unroll
                 for (int jv = 0; jv < JV; ++jv) {
@@ -523,8 +627,8 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
                     *reinterpret_cast<f32x4 *>(&psum[pg][ps * JB + 4 * jv]) = sum;
                 }
             }
-            // polling lanes have drained their memory operations; stated for all lanes so that the compiler
-            // knows nothing is outstanding here
+            // polling lanes have drained their loads; stated for all lanes so that the compiler knows nothing
+            // is outstanding here
             wait_all_vmem();
             if (!ok) wait_failed = 1;
             lds_barrier();  // A
@@ -558,60 +662,16 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
             fg_later = fg; cerr_later = ce; dig_later = s_ig; dfg_later = s_fg;
         }
         lds_barrier();  // B
-        const long long tk2 = timing ? wall_clock64() : 0;
-
-        if (!last) {
-            // partial output errors of every receiving cell from this workgroup's deltas
-            const unsigned slot_off = (unsigned)((size_t)(step % 3) * slot_words * 4u);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const int s = nt * 16 + (lane & 15);
-                f32x4 acc[MT];
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0, 0, 0, 0};
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const float bv = dl[4 * ks + (lane >> 4)][s];
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wA[mt][ks], bv, acc[mt], 0, 0, 0);
-                }
-                if (s < S) {
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) {
-                        // the four accumulator rows of a lane are four neighbouring receiving cells
-                        const int from = wave * (H / 4) + mt * 16 + 4 * (lane >> 4);
-                        const int dst = from / JB, jd = from % JB;
-                        u32x4 v = __builtin_bit_cast(u32x4, acc[mt]);
-                        // a NaN that happens to look like the empty marker is sent as the default NaN
-                        v.x = v.x == kEmpty ? 0x7FC00000u : v.x; v.y = v.y == kEmpty ? 0x7FC00000u : v.y;
-                        v.z = v.z == kEmpty ? 0x7FC00000u : v.z; v.w = v.w == kEmpty ? 0x7FC00000u : v.w;
-                        store128_device(mail, slot_off + ((unsigned)dst * recv_words + (unsigned)(me * S + s) * JB + jd) * 4u, v);
-                    }
-                }
-            }
-        }
-        if (!first && polls) {
-            // hand the words consumed in this step back as empty (off the critical path; the next wait drains
-            // these stores before it can complete)
-            const u32x4 empty = {kEmpty, kEmpty, kEmpty, kEmpty};
-            const unsigned mine_off = (unsigned)(((size_t)((step - 1) % 3) * slot_words + (size_t)me * recv_words) * 4u);
-#pragma unroll
-            for (int jv = 0; jv < JV; ++jv)
-#pragma unroll
-                for (int q = 0; q < NPOLL; ++q)
-                    store128_device(mail, mine_off + poll_off + 16u * jv + (unsigned)q * poll_stride, empty);
-        }
-        // `dl`, `res` and `psum` are rewritten only after the next step's barrier A
+        // `dl`, `res`, `coef` and `psum` change only between the barriers of later steps
         if (timing) {
-            const long long tk3 = wall_clock64();
-            ph0 += tk1 - tk0; ph1 += tk2 - tk1; ph2 += tk3 - tk2;
+            const long long tk2 = wall_clock64();
+            ph0 += tk1 - tk0; ph1 += tk2 - tk1;
         }
     }
     if (timing) ph3 = wall_clock64() - tk_begin;
     if (timing && tid == 0) {
-        long long *o = p.phase_ticks + (size_t)blockIdx.x * 4;
-        o[0] = ph0; o[1] = ph1; o[2] = ph2; o[3] = ph3;
+        long long *o = p.phase_ticks + (size_t)blockIdx.x * 6;
+        o[0] = ph0; o[1] = ph1; o[3] = ph3; o[4] = poll_rounds;
     }
 }
 
@@ -677,8 +737,9 @@ struct cnt_lstm {
     int device;
     int JB, NT;
     unsigned spin_limit;
-    int xcd_pack;
+    int xcd_pack;   // forward recursion: one direction per XCD
     long long *phase_ticks;  // diagnostic buffer, allocated when CNT_LSTM_TIMING is set
+    int poll_delay, poll_gap;
 };
 
 namespace cnt {
@@ -732,8 +793,8 @@ void fill_chain_params(const cnt_lstm *h, const float *weights, ChainParams &p) 
     }
     p.spin_limit = h->spin_limit;
     p.abort_flag = h->abort_flag;
-    p.xcd_pack = h->xcd_pack;
     p.phase_ticks = h->phase_ticks;
+    p.poll_delay = h->poll_delay; p.poll_gap = h->poll_gap;
 }
 
 int next_epoch(cnt_lstm *h, hipStream_t stream, unsigned &tag_base) {
@@ -760,7 +821,8 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
             CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->bmail[dir]), h->bmail_words, kEmpty));
     }
     const int G = h->H / h->JB;
-    const int blocks = h->xcd_pack ? 8 * G : h->ndir * G;
+    p.xcd_pack = fwd ? h->xcd_pack : 0;
+    const int blocks = p.xcd_pack ? 8 * G : h->ndir * G;
     ProfileScope prof(stream, fwd ? "lstm_forward_chain" : "lstm_backward_chain");
     hipLaunchKernelGGL(k, dim3(blocks), dim3(fwd ? kThreads : kBwdThreads), 0, stream, p);
     CNT_HIP(hipGetLastError());
@@ -798,12 +860,18 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     if (const char *e = std::getenv("CNT_LSTM_SPIN_LIMIT")) h->spin_limit = (unsigned)std::strtoul(e, nullptr, 10);
     h->xcd_pack = 0;
     if (const char *e = std::getenv("CNT_LSTM_XCD_PACK")) h->xcd_pack = std::atoi(e) != 0;
+    // Backward recursion: pause before the first poll of a step, in units of 64 clocks -- roughly the time the
+    // senders need for their products (32 clocks per MFMA, (H/64)*JB*NT of them per wave) plus the time a store
+    // takes to become visible.  Measured optimum on MI355X for H=256, JB=4, S=10: 28.
+    h->poll_delay = 20 + (H / 64) * JB * NT / 2;
+    if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY")) h->poll_delay = std::atoi(e);
+    if (const char *e = std::getenv("CNT_LSTM_POLL_GAP")) h->poll_gap = std::atoi(e);
     hipError_t err = hipGetDevice(&h->device);
     const size_t nstate = (size_t)H * desc->maxT * desc->S;
     const int G = H / JB, NS = 16 * NT;
-    // forward: 2 slots of H*NS tagged words; backward: 3 slots of G*G*JB*S plain words
+    // forward: 2 slots of H*NS tagged words; backward: kMailSlots slots of G*G*JB*S plain words
     h->mailbox_bytes = (size_t)2 * H * NS * sizeof(u64);
-    h->bmail_words = (size_t)3 * G * H * desc->S;
+    h->bmail_words = (size_t)kMailSlots * G * H * desc->S;
     for (int dir = 0; dir < ndir && err == hipSuccess; ++dir) {
         for (int w = 0; w < 12 && err == hipSuccess; ++w) {
             err = hipMalloc(reinterpret_cast<void **>(&h->state[dir][w]), nstate * sizeof(float));
@@ -814,7 +882,7 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
         if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->bmail[dir]), h->bmail_words * sizeof(float));
     }
     if (err == hipSuccess && std::getenv("CNT_LSTM_TIMING"))
-        err = hipMalloc(reinterpret_cast<void **>(&h->phase_ticks), 8 * 512 * 4 * sizeof(long long));
+        err = hipMalloc(reinterpret_cast<void **>(&h->phase_ticks), 8 * 512 * 6 * sizeof(long long));
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->abort_flag), sizeof(int));
     if (err == hipSuccess) err = hipMemset(h->abort_flag, 0, sizeof(int));
     if (err != hipSuccess) {
@@ -865,15 +933,22 @@ int cnt_lstm_check(cnt_lstm *h, void *stream) {
     CNT_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     CNT_HIP(hipMemcpy(&flag, h->abort_flag, sizeof(int), hipMemcpyDeviceToHost));
     if (h->phase_ticks) {
-        // diagnostic: mean phase durations of the last backward recursion, in 10 ns ticks
+        // diagnostic: mean phase durations of the last backward recursion over the workgroups that took part
         const int blocks = h->ndir * (h->H / h->JB);
-        std::vector<long long> t((size_t)blocks * 4);
+        std::vector<long long> t((size_t)blocks * 6);
         CNT_HIP(hipMemcpy(t.data(), h->phase_ticks, t.size() * sizeof(long long), hipMemcpyDeviceToHost));
-        double m[4] = {0, 0, 0, 0};
-        for (int b = 0; b < blocks; ++b)
-            for (int q = 0; q < 4; ++q) m[q] += (double)t[(size_t)b * 4 + q] / blocks;
-        std::fprintf(stderr, "lstm backward phases per step [us]: wait %.3f cell %.3f product+publish %.3f loop %.3f (T=%d)\n",
-                     m[0] * 0.01 / h->T, m[1] * 0.01 / h->T, m[2] * 0.01 / h->T, m[3] * 0.01 / h->T, h->T);
+        CNT_HIP(hipMemset(h->phase_ticks, 0, t.size() * sizeof(long long)));
+        double m[6] = {0, 0, 0, 0, 0, 0};
+        int active = 0;
+        for (int b = 0; b < blocks; ++b) {
+            if (t[(size_t)b * 6 + 3] == 0) continue;
+            ++active;
+            for (int q = 0; q < 6; ++q) m[q] += (double)t[(size_t)b * 6 + q];
+        }
+        const double us = active ? 0.01 / active / h->T : 0.0;
+        std::fprintf(stderr, "lstm backward per step [us]: receive waves wait %.3f cell %.3f loop %.3f poll rounds %.2f | "
+                     "product waves busy %.3f | memory wave busy after B %.3f (T=%d, %d workgroups)\n",
+                     m[0] * us, m[1] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, m[2] * us, m[5] * us, h->T, active);
     }
     if (flag != 0) {
         CNT_HIP(hipMemset(h->abort_flag, 0, sizeof(int)));
