@@ -28,6 +28,11 @@ sys.path.insert(0, ROOT)
 
 import numpy as np  # noqa: E402
 
+# HBM bytes one launch of lstm_backward_chain moves on this workload (T=588, S=10, H=256, two directions), from
+# two rocprofv3 --pmc runs scaled by a copy of known size: 1071 MiB read + 1605 MiB written
+# (profiles/acoustic_backward_hbm_traffic.md).  Algorithmic bytes of the same launch: 120 MB.
+CHAIN_TRAFFIC_BYTES = int((1071.4 + 1605.3) * 2 ** 20)
+
 METRIC = "BLSTM backward frames/sec at 1 MI355X; % HBM/MFMA roofline vs host CPU"
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
@@ -199,10 +204,12 @@ def main():
         # recursion is the recurrent product, 8*H^2 flops per slot and direction
         flops = 2 * 8.0 * H * H * slots
         roof = {"bound": "mfma", "achieved": flops / dom_avg_s / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "traffic": None,
+                "unit": "TFLOP/s", "traffic": CHAIN_TRAFFIC_BYTES,
                 "kernel": dom,
                 "note": "latency-bound recursion: T sequential steps, each a 256x1024x%d product spread over "
-                        "32 workgroups per direction plus one mailbox round trip" % S}
+                        "64 workgroups per direction plus one mailbox round trip; traffic = HBM bytes per launch "
+                        "from rocprofv3 FETCH_SIZE/WRITE_SIZE (profiles/acoustic_backward_hbm_traffic.md), mostly "
+                        "mailbox write-through and polls" % S}
     elif dom.startswith("gemm"):
         flops = backward_flops_per_slot(input_size, specs) * slots / max(1, len([k for k in kernels if k.startswith("gemm")]))
         roof = {"bound": "mfma", "achieved": flops / dom_avg_s / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS,
