@@ -25,6 +25,13 @@ constexpr int NTHREADS = 256;
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+// workgroup barrier that orders LDS traffic only; global loads issued before it stay in flight
+__device__ __forceinline__ void lds_only_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 template <int V>
 struct VecT;
 template <>
@@ -54,10 +61,16 @@ struct TileStage {
             for (int p = 0; p < NLOAD; ++p) {
                 const int row = row0 + rr + p * RPP;
                 typename VecT<VEC>::type v = {};
-                if (row < rows_total && (k0 + kq) < k_total) {
-                    if (!pat) {
-                        v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)row * ld + k0 + kq);
-                    } else if (!time_on_k) {
+                if (!pat) {
+                    // branch-free: the load always executes (on a clamped address) and is zeroed afterwards, so
+                    // that the number of loads in flight is the same on every path and the compiler can wait for
+                    // the tile of the next iteration while the one after it stays in flight
+                    const bool inside = row < rows_total && (k0 + kq) < k_total;
+                    const int rc = min(row, rows_total - 1), kc = (k0 + kq) < k_total ? k0 + kq : 0;
+                    v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)rc * ld + kc);
+                    if (!inside) v = typename VecT<VEC>::type{};
+                } else if (row < rows_total && (k0 + kq) < k_total) {
+                    if (!time_on_k) {
                         const int src = row + shift;
                         if (pat[row] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
                             v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)src * ld + k0 + kq);
@@ -83,10 +96,13 @@ struct TileStage {
             for (int p = 0; p < NLOAD; ++p) {
                 const int k = k0 + kk + p * KPP;
                 typename VecT<VEC>::type v = {};
-                if (k < k_total && (row0 + rq) < rows_total) {
-                    if (!pat) {
-                        v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)k * ld + row0 + rq);
-                    } else if (time_on_k) {
+                if (!pat) {
+                    const bool inside = k < k_total && (row0 + rq) < rows_total;
+                    const int kc = min(k, k_total - 1), rc = (row0 + rq) < rows_total ? row0 + rq : 0;
+                    v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)kc * ld + rc);
+                    if (!inside) v = typename VecT<VEC>::type{};
+                } else if (k < k_total && (row0 + rq) < rows_total) {
+                    if (time_on_k) {
                         const int src = k + shift;
                         if (pat[k] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
                             v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)src * ld + row0 + rq);
@@ -142,7 +158,10 @@ struct TileStage {
     }
 };
 
-template <int VA, bool AK, int VB, bool BK_>
+// MASKED selects the time-shifted, padding-masked B loader at compile time: its per-element predication is a lot
+// of code, and four copies of it (two prologue fetches, two in the unrolled loop) inside the plain kernels would
+// push their hot loop out of the instruction cache.
+template <int VA, bool AK, int VB, bool BK_, bool MASKED>
 __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args) {
     __shared__ __attribute__((aligned(16))) float lds_a[2][BM * PITCH];
     __shared__ __attribute__((aligned(16))) float lds_b[2][BN * PITCH];
@@ -174,35 +193,39 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    TileStage<VA, AK> sa;
-    TileStage<VB, BK_> sb;
-    const char *mask_pat = args.masked ? args.pat : nullptr;
-
-    {
-        const int seg = it_begin / kt_per_seg;
-        const int k0 = (it_begin % kt_per_seg) * BK;
-        sa.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
-        sb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid, mask_pat, pb.b_shift[seg], args.n_slots,
+    // Two register sets per operand: tile it+1 waits in one of them while tile it+2 is being fetched into the
+    // other, so that a global load has two k-iterations of MFMA work (about 4000 clocks) to arrive in; with one
+    // workgroup per compute unit, which is what the benchmark's shapes give, nothing else hides that latency.
+    // The loop is unrolled by two so that the sets swap roles without register copies, and its barrier orders
+    // LDS only (__syncthreads() would also drain the loads in flight).
+    TileStage<VA, AK> sa0, sa1;
+    TileStage<VB, BK_> sb0, sb1;
+    const char *mask_pat = MASKED ? args.pat : nullptr;
+    auto fetch = [&](int it, TileStage<VA, AK> &ra, TileStage<VB, BK_> &rb) __attribute__((always_inline)) {
+        const int seg = it / kt_per_seg;
+        const int k0 = (it % kt_per_seg) * BK;
+        ra.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
+        rb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid, mask_pat, pb.b_shift[seg], args.n_slots,
                 args.b_time_on_k != 0);
-        sa.store(lds_a[0], tid);
-        sb.store(lds_b[0], tid);
-    }
-    __syncthreads();
+    };
+
+    fetch(it_begin, sa0, sb0);
+    fetch(min(it_begin + 1, it_end - 1), sa1, sb1);
+    sa0.store(lds_a[0], tid);
+    sb0.store(lds_b[0], tid);
+    lds_only_barrier();
 
     const int frag_row = lane & 31;
     constexpr int FK = BK / 2;  // k values per half-wave and tile
     const int frag_k = (lane >> 5) * FK;
 
-    for (int it = it_begin; it < it_end; ++it) {
-        const int cur = (it - it_begin) & 1;
-        const bool has_next = (it + 1) < it_end;
-        if (has_next) {
-            const int seg = (it + 1) / kt_per_seg;
-            const int k0 = ((it + 1) % kt_per_seg) * BK;
-            sa.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
-            sb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid, mask_pat, pb.b_shift[seg], args.n_slots,
-                    args.b_time_on_k != 0);
-        }
+    // one k-iteration on LDS buffer `cur`; `held` carries tile it+1, `recv` receives tile it+2
+    auto iterate = [&](int it, int cur, TileStage<VA, AK> &held_a, TileStage<VB, BK_> &held_b,
+                       TileStage<VA, AK> &recv_a, TileStage<VB, BK_> &recv_b) __attribute__((always_inline)) {
+        // always issued (the last iterations refetch the final tile) so that the count of loads in flight is
+        // the same on every path
+        fetch(min(it + 2, it_end - 1), recv_a, recv_b);
+        __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMA block: the scheduler would sink them
 
         float fa[2][FK], fb[2][FK];
 #pragma unroll
@@ -220,11 +243,15 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
             }
         }
 
-        if (has_next) {
-            sa.store(lds_a[cur ^ 1], tid);
-            sb.store(lds_b[cur ^ 1], tid);
+        if (it + 1 < it_end) {
+            held_a.store(lds_a[cur ^ 1], tid);
+            held_b.store(lds_b[cur ^ 1], tid);
         }
-        __syncthreads();
+        lds_only_barrier();
+    };
+    for (int it = it_begin; it < it_end; it += 2) {
+        iterate(it, 0, sa1, sb1, sa0, sb0);
+        if (it + 1 < it_end) iterate(it + 1, 1, sa0, sb0, sa1, sb1);
     }
 
     // epilogue: lane%32 runs along m (contiguous), the 16 accumulators along n
@@ -284,10 +311,15 @@ inline int pick_vec(const GemmArgs &a, bool for_a) {
     return v;
 }
 
+template <int VA, bool AK, int VB, bool BK_>
+void launch_m(const GemmArgs &a, dim3 grid, hipStream_t s) {
+    if (a.masked) hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, true>), grid, dim3(NTHREADS), 0, s, a);
+    else hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, false>), grid, dim3(NTHREADS), 0, s, a);
+}
 template <int VA, bool AK, int VB>
 void launch_b(const GemmArgs &a, dim3 grid, hipStream_t s, bool bk) {
-    if (bk) hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, true>), grid, dim3(NTHREADS), 0, s, a);
-    else hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, false>), grid, dim3(NTHREADS), 0, s, a);
+    if (bk) launch_m<VA, AK, VB, true>(a, grid, s);
+    else launch_m<VA, AK, VB, false>(a, grid, s);
 }
 template <int VA, bool AK>
 void launch_vb(const GemmArgs &a, dim3 grid, hipStream_t s, int vb, bool bk) {
