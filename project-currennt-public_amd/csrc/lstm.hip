@@ -13,10 +13,12 @@
 //   backward: each workgroup multiplies its own 4*JB gate deltas with its weight slice and
 //             scatters partial output errors to the owners of the receiving cells (H x S words per
 //             workgroup instead of the 4H x S a gather of the deltas would need).
-// Mailbox words are 8 bytes, (value, tag), written and polled with relaxed agent-scope atomics; the
-// tag carries launch epoch and step, so a word validates itself and no fence sits on the critical
-// path.  Two mailbox slots alternate by step parity.  Every poll loop is bounded: when the bound is
-// hit the workgroup raises a device flag and every workgroup drains out.
+// Mailbox words are plain 4-byte floats; a reserved NaN pattern means "not written yet", so a word validates
+// itself and neither tags nor fences sit on the critical path.  Words are moved 16 bytes at a time, polled with
+// loads that bypass the non-coherent caches, and handed back as empty after use; four slots rotate.  Every
+// poll loop is bounded: when the bound is hit the workgroup raises a device flag and every workgroup drains
+// out.  Inside a workgroup, waves specialise (polling waves that never store, product / cell waves that never
+// wait for a store, one memory wave for all ordinary loads and stores), see the kernels' comments.
 //
 // The dense work that does not sit on the recursion is batched over all time steps on the MFMA
 // GEMM: input projections (8 problems, one launch), the error to the preceding layer
@@ -37,7 +39,6 @@ typedef unsigned long long u64;
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-constexpr unsigned kStepBits = 20;  // tag = epoch << 20 | (step + 1)
 
 struct DirPtrs {
     float *ni, *ig, *fg, *og, *c, *h;
@@ -45,7 +46,7 @@ struct DirPtrs {
     const float *w_int;    // gate 0 block of this direction; gate g at + g*L*H
     const float *b[4];     // bias weights per gate
     const float *peep[3];  // ig, fg, og peepholes
-    u64 *mailbox;          // forward: 2 slots of tagged words
+    float *fmail;          // forward: kMailSlots slots of H*S plain words
     float *bmail;          // backward: kMailSlots slots of plain words
 };
 
@@ -57,47 +58,13 @@ struct ChainParams {
     float *out;           // forward: L x (T*S) layer outputs (NULL when it aliases d[0].h)
     const float *outerr;  // backward: L x (T*S) output errors
     float *herr_out;      // backward, unidirectional: where the summed error is written back
-    unsigned tag_base;
     unsigned spin_limit;
     int *abort_flag;
     int xcd_pack;
     long long *phase_ticks;  // optional diagnostic: per workgroup accumulated phase durations (100 MHz ticks)
     int poll_delay, poll_gap;  // s_sleep units before the first poll of a step / between polls
+    int poll_delay_fwd;
 };
-
-__device__ __forceinline__ u64 mb_load(const u64 *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void mb_store(u64 *p, float v, unsigned tag) {
-    const u64 w = ((u64)tag << 32) | (u64)__float_as_uint(v);
-    __hip_atomic_store(p, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Polls N mailbox words until each carries `tag`.  Every retry round re-issues all N loads back to back, so a
-// round costs one memory round trip however many words are still missing (re-polling word by word would
-// serialise up to N round trips).  Returns false when the spin bound is hit or another workgroup has raised
-// the abort flag.
-template <int N>
-__device__ __forceinline__ bool mb_wait(const u64 *const (&addr)[N], float (&val)[N], unsigned tag,
-                                        unsigned spin_limit, const int *abort_flag) {
-    unsigned spins = 0;
-    for (;;) {
-        u64 w[N];
-#pragma unroll
-        for (int q = 0; q < N; ++q) w[q] = mb_load(addr[q]);
-        bool all = true;
-#pragma unroll
-        for (int q = 0; q < N; ++q) {
-            all = all && ((unsigned)(w[q] >> 32) == tag);
-            val[q] = __uint_as_float((unsigned)w[q]);
-        }
-        if (all) return true;
-        if (++spins > spin_limit) return false;
-        if ((spins & 255u) == 0u && __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
-            return false;
-        __builtin_amdgcn_s_sleep(1);
-    }
-}
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
 // global load and store of the wave, which would put the HBM latency of the look-ahead loads and the
@@ -125,169 +92,6 @@ __device__ __forceinline__ bool map_block(const ChainParams &p, int G, int &dir,
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Forward recursion.  HT = H/64, JB = cells per workgroup, NT = ceil(S/16).
-// ---------------------------------------------------------------------------------------------------
-template <int HT, int JB, int NT>
-__global__ __launch_bounds__(kThreads) void lstm_forward_chain(const ChainParams p) {
-    constexpr int H = 64 * HT;
-    constexpr int G = H / JB;
-    constexpr int NS = 16 * NT;
-    constexpr int MT = (4 * JB) / 16;  // output tiles: rows are (gate, cell)
-    constexpr int KS = H / 16;         // k-steps of 4 per wave (each wave covers H/4 source cells)
-    static_assert((4 * JB) % 16 == 0, "JB must be a multiple of 4");
-    static_assert(JB * NS <= kThreads, "cell phase needs one thread per (cell, sequence)");
-
-    int dir, me;
-    if (!map_block(p, G, dir, me)) return;
-    const DirPtrs &D = p.d[dir];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int S = p.S, T = p.T;
-    const int j0 = me * JB;
-    const int n = S * H;
-
-    __shared__ float red[kWaves][4 * JB][NS + 1];
-    __shared__ int wait_failed;
-    if (threadIdx.x == 0) wait_failed = 0;
-    lds_barrier();
-
-    // recurrent weights as MFMA A operands: row (gate, cell), k = source cell
-    float wA[MT][KS];
-    {
-        const int i = lane & 15, kq = lane >> 4;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int o = mt * 16 + i, g = o / JB, jj = o % JB;
-            const float *wg = D.w_int + (size_t)g * p.L * H + (size_t)(j0 + jj) * H;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) wA[mt][ks] = wg[wave * (H / 4) + 4 * ks + kq];
-        }
-    }
-
-    // cell phase thread: one (sequence, cell) pair
-    const bool cell_thread = tid < JB * NS;
-    const int cs = tid / JB, cj = tid % JB;
-    const bool cell_valid = cell_thread && cs < S;
-    float b_ni = 0, b_ig = 0, b_fg = 0, b_og = 0, p_ig = 0, p_fg = 0, p_og = 0;
-    if (cell_valid) {
-        b_ni = p.bias * D.b[0][j0 + cj]; b_ig = p.bias * D.b[1][j0 + cj];
-        b_fg = p.bias * D.b[2][j0 + cj]; b_og = p.bias * D.b[3][j0 + cj];
-        p_ig = D.peep[0][j0 + cj]; p_fg = D.peep[1][j0 + cj]; p_og = D.peep[2][j0 + cj];
-    }
-    float c_prev = 0.0f;
-
-    // Pre-activations of the input projection do not depend on the recursion: they are requested one
-    // step ahead, right after the wait of the current step, so that their HBM latency is hidden
-    // behind the cell update and the next wait instead of stacking up in front of the mailbox polls.
-    struct StepIn { float a_ni, a_ig, a_fg, a_og; char pat; };  // pat is compared at use, not at load
-    auto load_step = [&](int step) {
-        StepIn v = {0, 0, 0, 0, 1};
-        if (cell_valid) {
-            const int t = dir ? (T - 1 - step) : step;
-            const size_t gi = (size_t)t * n + (size_t)cs * H + j0 + cj;
-            v.a_ni = D.ni[gi]; v.a_ig = D.ig[gi]; v.a_fg = D.fg[gi]; v.a_og = D.og[gi];
-            v.pat = p.pat[t * S + cs];
-        }
-        return v;
-    };
-    StepIn cur = load_step(0);
-
-    for (int step = 0; step < T; ++step) {
-        const int t = dir ? (T - 1 - step) : step;
-        const bool first = (step == 0);
-        const size_t gi = (size_t)t * n + (size_t)cs * H + j0 + cj;
-        float a_ni = cur.a_ni, a_ig = cur.a_ig, a_fg = cur.a_fg, a_og = cur.a_og;
-        const bool dummy = (t >= p.Tmin) && (cur.pat == 0);
-
-        if (!first) {
-            // gather h of the previous step straight into MFMA B operands
-            const unsigned tag = p.tag_base + (unsigned)step;  // published at the end of step-1
-            const u64 *slot = D.mailbox + (size_t)((step - 1) & 1) * H * NS;
-            f32x4 acc[MT][NT];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0, 0, 0, 0};
-            bool ok = true;
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const int s = nt * 16 + (lane & 15);
-                float hv[KS];
-                if (s < S) {
-                    const u64 *addr[KS];
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks)
-                        addr[ks] = slot + ((size_t)(wave * KS + ks) * NS + s) * 4 + (lane >> 4);
-                    ok = mb_wait<KS>(addr, hv, tag, p.spin_limit, p.abort_flag) && ok;
-                } else {
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) hv[ks] = 0.0f;
-                }
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wA[mt][ks], hv[ks], acc[mt][nt], 0, 0, 0);
-            }
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        red[wave][mt * 16 + 4 * (lane >> 4) + r][nt * 16 + (lane & 15)] = acc[mt][nt][r];
-            if (!ok) wait_failed = 1;
-            lds_barrier();
-            if (wait_failed) {
-                if (tid == 0) __hip_atomic_store(p.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                return;
-            }
-        }
-
-        if (step + 1 < T) cur = load_step(step + 1);
-
-        if (cell_valid) {
-            if (!first) {
-#pragma unroll
-                for (int w = 0; w < kWaves; ++w) {
-                    a_ni += red[w][0 * JB + cj][cs];
-                    a_ig += red[w][1 * JB + cj][cs];
-                    a_fg += red[w][2 * JB + cj][cs];
-                    a_og += red[w][3 * JB + cj][cs];
-                }
-            }
-            float hval = 0.0f;
-            if (dummy) {
-                // the reference leaves the summed pre-activations in place on padding slots, clears the
-                // cell only in the time-reversed direction and emits a zero output
-                if (!first) { D.ni[gi] = a_ni; D.ig[gi] = a_ig; D.fg[gi] = a_fg; D.og[gi] = a_og; }
-                if (dir) { D.c[gi] = 0.0f; c_prev = 0.0f; }
-                else c_prev = D.c[gi];
-            } else {
-                float x_ni = a_ni + b_ni, x_ig = a_ig + b_ig, x_fg = a_fg + b_fg, x_og = a_og + b_og;
-                if (!first) { x_ig += c_prev * p_ig; x_fg += c_prev * p_fg; }
-                const float ni = tanh_act(x_ni), ig = logistic(x_ig), fg = logistic(x_fg);
-                float c = ni * ig;
-                if (!first) c += c_prev * fg;
-                x_og += c * p_og;
-                const float og = logistic(x_og);
-                hval = tanh_act(c) * og;
-                D.ni[gi] = ni; D.ig[gi] = ig; D.fg[gi] = fg; D.og[gi] = og; D.c[gi] = c;
-                c_prev = c;
-            }
-            if (step + 1 < T) {
-                const int from = j0 + cj;
-                u64 *slot = D.mailbox + (size_t)(step & 1) * H * NS;
-                mb_store(slot + ((size_t)(from >> 2) * NS + cs) * 4 + (from & 3), hval,
-                         p.tag_base + (unsigned)step + 1u);
-            }
-            D.h[gi] = hval;
-            if (p.out) p.out[((size_t)t * S + cs) * p.L + dir * H + j0 + cj] = hval;
-        }
-        lds_barrier();  // `red` is rewritten in the next step
-    }
-}
-
-// ---------------------------------------------------------------------------------------------------
 // Backward (error) recursion.
 //
 // The partial output errors travel through a mailbox of plain 4-byte words, laid out
@@ -302,6 +106,7 @@ __global__ __launch_bounds__(kThreads) void lstm_forward_chain(const ChainParams
 // The host fills the mailbox with kEmpty before every launch.
 // ---------------------------------------------------------------------------------------------------
 constexpr unsigned kEmpty = 0xFFFFFFFFu;
+constexpr int kMailSlots = 4;
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 // s_waitcnt vmcnt(0) (expcnt and lgkmcnt left at their maxima) as a builtin, so that the compiler's own wait
@@ -330,6 +135,305 @@ __device__ __forceinline__ void poll_load(const float *base, unsigned byte_off, 
 __device__ __forceinline__ void store128_device(__amdgpu_buffer_rsrc_t rsrc, unsigned byte_off, u32x4 v) {
     __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (int)byte_off, 0, 16);
 }
+// ---------------------------------------------------------------------------------------------------
+// Forward recursion.  HT = H/64, JB = cells per workgroup, NT = ceil(S/16).
+//
+// Every workgroup needs the block outputs h[t-1] of ALL cells.  They travel through a mailbox of plain
+// 4-byte words laid out [slot][cell / 4][sequence][cell % 4]; a word that holds kEmpty has not been written.
+// Four slots rotate.  The producer of a word empties it again two steps after writing it -- by then every
+// workgroup has consumed it, because a workgroup can only publish h[t] after it has seen h[t-1] of all others
+// -- and drains its stores before it publishes again, so a reader that has seen h[t-1] can never find the
+// value of four steps earlier in the slot of h[t].  The host fills the mailbox with kEmpty before each launch.
+//
+// Waves and their roles (one LDS-only barrier per step):
+//   gather waves (4)   wait, poll h[t-1] straight into MFMA B operands (each wave a quarter of the source
+//                      cells), multiply with their register-resident weight slice, leave the partial
+//                      pre-activations in LDS.  They issue no stores.
+//   cell waves (CW)    after the barrier: add the four partials to the input projection, run the gate / cell
+//                      update of JB x S elements, publish h[t], empty the slot of h[t-2], leave the step's
+//                      results in LDS.
+//   memory wave (1)    loads the input projections two steps ahead and hands them over through LDS one step
+//                      ahead; writes the results of the finished step to the state arrays and the layer output.
+// ---------------------------------------------------------------------------------------------------
+constexpr int fwd_cell_waves(int JB, int NT) { return (JB * 16 * NT + 63) / 64; }
+constexpr int fwd_threads(int JB, int NT) { return kThreads + 64 * fwd_cell_waves(JB, NT) + 64; }
+
+template <int HT, int JB, int NT>
+__global__ __launch_bounds__(fwd_threads(JB, NT)) void lstm_forward_chain(const ChainParams p) {
+    constexpr int H = 64 * HT;
+    constexpr int G = H / JB;
+    constexpr int NS = 16 * NT;
+    constexpr int MT = (4 * JB) / 16;  // output tiles: rows are (gate, cell)
+    constexpr int KS = H / 16;         // k-steps of 4 per gather wave (each covers H/4 source cells)
+    constexpr int KV = KS / 4;         // 16-byte vectors (4 source cells) per lane and column tile
+    constexpr int EL = JB * NS;        // (cell, sequence) elements, padded
+    constexpr int CW = fwd_cell_waves(JB, NT);
+    constexpr int EPAD = 64 * CW;
+    static_assert((4 * JB) % 16 == 0 && KS % 4 == 0, "JB must be a multiple of 4, H of 64");
+    enum { R_NI = 0, R_IG, R_FG, R_OG, R_C, R_H, NRES };
+
+    int dir, me;
+    if (!map_block(p, G, dir, me)) return;
+    const DirPtrs &D = p.d[dir];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int S = p.S, T = p.T;
+    const int j0 = me * JB;
+    const int n = S * H;
+
+    __shared__ float red[2][kWaves][4 * JB][NS + 1];  // partial pre-activations, by step parity
+    __shared__ float pre[2][4][EPAD];                 // input projections of the step, by step parity
+    __shared__ int pre_dummy[2][EPAD];
+    __shared__ float res[2][NRES][EPAD];              // results of the step, by step parity
+    __shared__ int res_flags[2][EPAD];                // bit 0: gate activations to store, bit 1: cell state to store
+    __shared__ int wait_failed;
+    if (threadIdx.x == 0) wait_failed = 0;
+
+    auto slot_of = [&](int step) { return dir ? (T - 1 - step) : step; };
+    const unsigned slot_words = (unsigned)H * S;
+    const __amdgpu_buffer_rsrc_t mail =
+        __builtin_amdgcn_make_buffer_rsrc(D.fmail, 0, (int)(kMailSlots * slot_words * sizeof(float)), 0x00020000);
+
+    if (wave == kWaves + CW) {
+        // ------------------------------------------------------------------ memory wave
+        constexpr int EIT = CW;
+        struct StepIn { float a[4]; char pat; };
+        int cs[EIT], cj[EIT];
+        bool valid[EIT];
+#pragma unroll
+        for (int it = 0; it < EIT; ++it) {
+            const int id = it * 64 + lane;
+            cs[it] = id / JB; cj[it] = id % JB;
+            valid[it] = id < EL && cs[it] < S;
+        }
+        auto load_step = [&](int step, StepIn (&v)[EIT]) {
+            const int t = slot_of(step);
+#pragma unroll
+            for (int it = 0; it < EIT; ++it) {
+                v[it] = StepIn{{0, 0, 0, 0}, 1};
+                if (!valid[it] || step >= T) continue;
+                const size_t gi = (size_t)t * n + (size_t)cs[it] * H + j0 + cj[it];
+                v[it].a[0] = D.ni[gi]; v[it].a[1] = D.ig[gi]; v[it].a[2] = D.fg[gi]; v[it].a[3] = D.og[gi];
+                v[it].pat = p.pat[t * S + cs[it]];
+            }
+        };
+        auto put_pre = [&](int step, const StepIn (&v)[EIT]) {
+            const int t = slot_of(step);
+#pragma unroll
+            for (int it = 0; it < EIT; ++it) {
+                const int id = it * 64 + lane;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) pre[step & 1][g][id] = v[it].a[g];
+                pre_dummy[step & 1][id] = ((t >= p.Tmin) && (v[it].pat == 0)) ? 1 : 0;
+            }
+        };
+        auto store_results = [&](int step) {
+            const int t = slot_of(step), b = step & 1;
+#pragma unroll
+            for (int it = 0; it < EIT; ++it) {
+                if (!valid[it]) continue;
+                const int id = it * 64 + lane;
+                const size_t gi = (size_t)t * n + (size_t)cs[it] * H + j0 + cj[it];
+                const int flags = res_flags[b][id];
+                if (flags & 1) {
+                    D.ni[gi] = res[b][R_NI][id]; D.ig[gi] = res[b][R_IG][id];
+                    D.fg[gi] = res[b][R_FG][id]; D.og[gi] = res[b][R_OG][id];
+                }
+                if (flags & 2) D.c[gi] = res[b][R_C][id];
+                const float hval = res[b][R_H][id];
+                D.h[gi] = hval;
+                if (p.out) p.out[((size_t)t * S + cs[it]) * p.L + dir * H + j0 + cj[it]] = hval;
+            }
+        };
+        auto run_step = [&](const int step, StepIn (&far)[EIT], const StepIn (&near)[EIT]) __attribute__((always_inline)) -> bool {
+            lds_barrier();  // results of step-1 and partial sums of this step are in LDS
+            if (wait_failed) return false;
+            wait_all_vmem();  // whatever is still in flight was issued a step ago
+            load_step(step + 2, far);
+            if (step + 1 < T) put_pre(step + 1, near);
+            if (step > 0) store_results(step - 1);
+            return true;
+        };
+        StepIn in_a[EIT], in_b[EIT];
+        load_step(0, in_a);
+        load_step(1, in_b);
+        put_pre(0, in_a);
+        lds_barrier();  // start of the recursion
+        for (int step = 0; step < T; step += 2) {
+            if (!run_step(step, in_a, in_b)) return;
+            if (step + 1 < T && !run_step(step + 1, in_b, in_a)) return;
+        }
+        lds_barrier();  // results of the last step
+        if (wait_failed) return;
+        store_results(T - 1);
+        return;
+    }
+
+    if (wave >= kWaves) {
+        // ------------------------------------------------------------------ cell waves
+        const int id = tid - kThreads;
+        const int cs = id / JB, cj = id % JB;
+        const bool cell_valid = id < EL && cs < S;
+        float b_ni = 0, b_ig = 0, b_fg = 0, b_og = 0, p_ig = 0, p_fg = 0, p_og = 0;
+        if (cell_valid) {
+            b_ni = p.bias * D.b[0][j0 + cj]; b_ig = p.bias * D.b[1][j0 + cj];
+            b_fg = p.bias * D.b[2][j0 + cj]; b_og = p.bias * D.b[3][j0 + cj];
+            p_ig = D.peep[0][j0 + cj]; p_fg = D.peep[1][j0 + cj]; p_og = D.peep[2][j0 + cj];
+        }
+        // word of this element inside a mailbox slot: [cell / 4][sequence][cell % 4]
+        const unsigned my_word = ((unsigned)((j0 + cj) >> 2) * S + cs) * 4u + ((j0 + cj) & 3);
+        float c_prev = 0.0f;
+        wait_all_vmem();
+        lds_barrier();  // start of the recursion
+        for (int step = 0; step < T; ++step) {
+            const bool first = (step == 0);
+            const int b = step & 1;
+            lds_barrier();
+            if (wait_failed) return;
+            // stores of the previous step (publication, reset) are complete before this step publishes
+            wait_all_vmem();
+            if (!cell_valid) continue;
+            float a_ni = pre[b][0][id], a_ig = pre[b][1][id], a_fg = pre[b][2][id], a_og = pre[b][3][id];
+            if (!first) {
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) {
+                    a_ni += red[b][w][0 * JB + cj][cs];
+                    a_ig += red[b][w][1 * JB + cj][cs];
+                    a_fg += red[b][w][2 * JB + cj][cs];
+                    a_og += red[b][w][3 * JB + cj][cs];
+                }
+            }
+            float hval = 0.0f;
+            int flags;
+            if (pre_dummy[b][id]) {
+                // the reference leaves the summed pre-activations in place on padding slots, clears the
+                // cell only in the time-reversed direction and emits a zero output
+                res[b][R_NI][id] = a_ni; res[b][R_IG][id] = a_ig; res[b][R_FG][id] = a_fg; res[b][R_OG][id] = a_og;
+                res[b][R_C][id] = 0.0f;
+                flags = (first ? 0 : 1) | (dir ? 2 : 0);
+                if (dir) c_prev = 0.0f;
+            } else {
+                float x_ni = a_ni + b_ni, x_ig = a_ig + b_ig, x_fg = a_fg + b_fg, x_og = a_og + b_og;
+                if (!first) { x_ig += c_prev * p_ig; x_fg += c_prev * p_fg; }
+                const float ni = tanh_act(x_ni), ig = logistic(x_ig), fg = logistic(x_fg);
+                float c = ni * ig;
+                if (!first) c += c_prev * fg;
+                x_og += c * p_og;
+                const float og = logistic(x_og);
+                hval = tanh_act(c) * og;
+                res[b][R_NI][id] = ni; res[b][R_IG][id] = ig; res[b][R_FG][id] = fg; res[b][R_OG][id] = og;
+                res[b][R_C][id] = c;
+                flags = 3;
+                c_prev = c;
+            }
+            if (step + 1 < T) {
+                unsigned bits = __float_as_uint(hval);
+                if (bits == kEmpty) bits = 0x7FC00000u;
+                __builtin_amdgcn_raw_buffer_store_b32(bits, mail, (int)(((unsigned)(step % kMailSlots) * slot_words + my_word) * 4u), 0, 16);
+            }
+            if (step >= 2 && step + 2 < T)
+                __builtin_amdgcn_raw_buffer_store_b32(kEmpty, mail, (int)(((unsigned)((step + 2) % kMailSlots) * slot_words + my_word) * 4u), 0, 16);
+            res[b][R_H][id] = hval;
+            res_flags[b][id] = flags;
+        }
+        lds_barrier();  // results of the last step are in LDS
+        return;
+    }
+
+    // ---------------------------------------------------------------------- gather waves
+    // Recurrent weights as MFMA A operands: row (gate, cell); the k order is free as long as both operands
+    // agree, and it is chosen so that the four k values of a lane and k-step group are the four cells of one
+    // 16-byte mailbox vector: k-step (j, c) of lane group kq is source cell  wave*H/4 + 4*(kq + 4*j) + c.
+    float wA[MT][KS];
+    {
+        const int i = lane & 15, kq = lane >> 4;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int o = mt * 16 + i, g = o / JB, jj = o % JB;
+            const float *wg = D.w_int + (size_t)g * p.L * H + (size_t)(j0 + jj) * H;
+#pragma unroll
+            for (int j = 0; j < KV; ++j)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) wA[mt][4 * j + c] = wg[wave * (H / 4) + 4 * (kq + 4 * j) + c];
+        }
+    }
+    long long ph0 = 0, ph3 = 0, poll_rounds = 0;
+    const bool timing = p.phase_ticks != nullptr;
+    const long long tk_begin = timing ? wall_clock64() : 0;
+    const int kq = lane >> 4;
+    wait_all_vmem();
+    lds_barrier();  // start of the recursion
+    lds_barrier();  // step 0 has nothing to gather
+
+    for (int step = 1; step < T; ++step) {
+        const long long tk0 = timing ? wall_clock64() : 0;
+        const float *slot = D.fmail + (size_t)((step - 1) % kMailSlots) * slot_words;
+        bool ok = true;
+        f32x4 acc[MT][NT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0, 0, 0, 0};
+        // h[t-1] cannot be there before the cell waves of the other workgroups are done; see the backward kernel
+        for (int d = 0; d < p.poll_delay_fwd; ++d) __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int s = nt * 16 + (lane & 15);
+            u32x4 w[KV];
+#pragma unroll
+            for (int j = 0; j < KV; ++j) w[j] = u32x4{0, 0, 0, 0};
+            if (s < S) {
+                // vector j of this lane: cells 4*quad .. 4*quad+3 with quad = wave*H/16 + kq + 4*j
+                const unsigned off = (((unsigned)(wave * (H / 16) + kq)) * S + s) * 16u;
+                unsigned spins = 0;
+                for (;;) {
+                    poll_load<KV>(slot, off, 4u * (unsigned)S * 16u, w);
+                    unsigned worst = 0;
+#pragma unroll
+                    for (int j = 0; j < KV; ++j) worst = max(max(worst, w[j].x), max(max(w[j].y, w[j].z), w[j].w));
+                    if (timing) ++poll_rounds;
+                    if (worst != kEmpty) break;
+                    if (++spins > p.spin_limit) { ok = false; break; }
+                    if ((spins & 255u) == 0u &&
+                        __hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+                        ok = false;
+                        break;
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < KV; ++j) {
+                const f32x4 hv = __builtin_bit_cast(f32x4, w[j]);
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wA[mt][4 * j + c], hv[c], acc[mt][nt], 0, 0, 0);
+            }
+        }
+        wait_all_vmem();
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    red[step & 1][wave][mt * 16 + 4 * (lane >> 4) + r][nt * 16 + (lane & 15)] = acc[mt][nt][r];
+        if (!ok) wait_failed = 1;
+        lds_barrier();
+        if (wait_failed) {
+            if (tid == 0) __hip_atomic_store(p.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+        if (timing) ph0 += wall_clock64() - tk0;
+    }
+    lds_barrier();  // results of the last step
+    if (timing) ph3 = wall_clock64() - tk_begin;
+    if (timing && tid == 0) {
+        long long *o = p.phase_ticks + (size_t)blockIdx.x * 6;
+        o[0] = ph0; o[1] = 0; o[3] = ph3; o[4] = poll_rounds;
+    }
+}
+
 // Workgroup layout, nine waves in three roles that meet at two workgroup barriers per step:
 //   receive waves (4)  poll the mailbox, reduce the partial errors through LDS (barrier A), run the cell update
 //                      and leave the gate deltas in LDS (barrier B).  They issue no stores at all, so the only
@@ -346,7 +450,6 @@ __device__ __forceinline__ void store128_device(__amdgpu_buffer_rsrc_t rsrc, uns
 // this workgroup publishes in step k+1; a sender rewrites those words only in step k+3, after it has seen
 // that publication.
 constexpr int kBwdThreads = 2 * kThreads + 64;
-constexpr int kMailSlots = 4;
 
 template <int HT, int JB, int NT>
 __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainParams p) {
@@ -728,18 +831,18 @@ struct cnt_lstm {
     int T, Tmin;  // current fraction
     const char *pat;
     float *state[2][12];
-    cnt::u64 *mailbox[2];  // forward recursion
-    size_t mailbox_bytes;
+    float *fmail[2];       // forward recursion
+    size_t fmail_words;
     float *bmail[2];       // backward recursion
     size_t bmail_words;
     int *abort_flag;
-    unsigned epoch;
     int device;
     int JB, NT;
     unsigned spin_limit;
     int xcd_pack;   // forward recursion: one direction per XCD
     long long *phase_ticks;  // diagnostic buffer, allocated when CNT_LSTM_TIMING is set
-    int poll_delay, poll_gap;
+    int poll_delay, poll_gap, poll_delay_fwd;
+    int last_was_forward;  // which recursion the diagnostic buffer describes
 };
 
 namespace cnt {
@@ -788,43 +891,29 @@ void fill_chain_params(const cnt_lstm *h, const float *weights, ChainParams &p) 
         D.w_int = weights + off_int + (size_t)dir * H * H;
         for (int g = 0; g < 4; ++g) D.b[g] = weights + off_bias + (size_t)g * L + dir * H;
         for (int k = 0; k < 3; ++k) D.peep[k] = weights + off_peep + (size_t)k * L + dir * H;
-        D.mailbox = h->mailbox[dir];
+        D.fmail = h->fmail[dir];
         D.bmail = h->bmail[dir];
     }
     p.spin_limit = h->spin_limit;
     p.abort_flag = h->abort_flag;
     p.phase_ticks = h->phase_ticks;
-    p.poll_delay = h->poll_delay; p.poll_gap = h->poll_gap;
-}
-
-int next_epoch(cnt_lstm *h, hipStream_t stream, unsigned &tag_base) {
-    // tags are epoch << 20 | step+1; when the 12-bit epoch wraps the mailboxes are wiped so that a
-    // word of an old launch can never validate
-    h->epoch += 1;
-    if (h->epoch >= (1u << (32 - kStepBits))) {
-        for (int dir = 0; dir < h->ndir; ++dir)
-            CNT_TRY(fill_zero(stream, reinterpret_cast<float *>(h->mailbox[dir]), h->mailbox_bytes / 4));
-        h->epoch = 1;
-    }
-    tag_base = h->epoch << kStepBits;
-    return CNT_OK;
+    p.poll_delay = h->poll_delay; p.poll_gap = h->poll_gap; p.poll_delay_fwd = h->poll_delay_fwd;
 }
 
 int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     chain_kernel_t k = pick_kernel(fwd, h->H, h->JB, h->NT);
     CNT_REQUIRE(k != nullptr, "lstm: no recursion kernel for H=%d JB=%d S=%d", h->H, h->JB, h->desc.S);
-    if (fwd) {
-        CNT_TRY(next_epoch(h, stream, p.tag_base));
-    } else {
-        // every word of the backward mailbox starts out empty
-        for (int dir = 0; dir < h->ndir; ++dir)
-            CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->bmail[dir]), h->bmail_words, kEmpty));
+    // every word of the mailbox starts out empty
+    for (int dir = 0; dir < h->ndir; ++dir) {
+        if (fwd) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->fmail[dir]), h->fmail_words, kEmpty));
+        else CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->bmail[dir]), h->bmail_words, kEmpty));
     }
     const int G = h->H / h->JB;
     p.xcd_pack = fwd ? h->xcd_pack : 0;
     const int blocks = p.xcd_pack ? 8 * G : h->ndir * G;
+    h->last_was_forward = fwd ? 1 : 0;
     ProfileScope prof(stream, fwd ? "lstm_forward_chain" : "lstm_backward_chain");
-    hipLaunchKernelGGL(k, dim3(blocks), dim3(fwd ? kThreads : kBwdThreads), 0, stream, p);
+    hipLaunchKernelGGL(k, dim3(blocks), dim3(fwd ? kThreads + 64 * ((h->JB * 16 * h->NT + 63) / 64) + 64 : kBwdThreads), 0, stream, p);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
@@ -844,7 +933,6 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     CNT_REQUIRE(!desc->bidir || desc->L % 2 == 0, "Cannot create a bidirectional layer with an odd layer size");
     const int ndir = desc->bidir ? 2 : 1;
     const int H = desc->L / ndir;
-    CNT_REQUIRE(desc->maxT < (1 << kStepBits) - 2, "lstm_create: maxT %d too long", desc->maxT);
     const int NT = (desc->S + 15) / 16;
     int JB = default_jb(H);
     if (const char *e = std::getenv("CNT_LSTM_JB")) JB = std::atoi(e);
@@ -865,20 +953,22 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     // takes to become visible.  Measured optimum on MI355X for H=256, JB=4, S=10: 28.
     h->poll_delay = 20 + (H / 64) * JB * NT / 2;
     if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY")) h->poll_delay = std::atoi(e);
+    // forward recursion: the senders' cell update (a few hundred clocks) plus store visibility
+    h->poll_delay_fwd = 34;  // measured optimum on MI355X at H=256, S=10
+    if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY_FWD")) h->poll_delay_fwd = std::atoi(e);
     if (const char *e = std::getenv("CNT_LSTM_POLL_GAP")) h->poll_gap = std::atoi(e);
     hipError_t err = hipGetDevice(&h->device);
     const size_t nstate = (size_t)H * desc->maxT * desc->S;
-    const int G = H / JB, NS = 16 * NT;
-    // forward: 2 slots of H*NS tagged words; backward: kMailSlots slots of G*G*JB*S plain words
-    h->mailbox_bytes = (size_t)2 * H * NS * sizeof(u64);
+    const int G = H / JB;
+    // mailboxes, kMailSlots slots each: forward H*S words, backward G*G*JB*S words
+    h->fmail_words = (size_t)kMailSlots * H * desc->S;
     h->bmail_words = (size_t)kMailSlots * G * H * desc->S;
     for (int dir = 0; dir < ndir && err == hipSuccess; ++dir) {
         for (int w = 0; w < 12 && err == hipSuccess; ++w) {
             err = hipMalloc(reinterpret_cast<void **>(&h->state[dir][w]), nstate * sizeof(float));
             if (err == hipSuccess) err = hipMemset(h->state[dir][w], 0, nstate * sizeof(float));
         }
-        if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->mailbox[dir]), h->mailbox_bytes);
-        if (err == hipSuccess) err = hipMemset(h->mailbox[dir], 0, h->mailbox_bytes);
+        if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->fmail[dir]), h->fmail_words * sizeof(float));
         if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->bmail[dir]), h->bmail_words * sizeof(float));
     }
     if (err == hipSuccess && std::getenv("CNT_LSTM_TIMING"))
@@ -899,7 +989,7 @@ int cnt_lstm_destroy(cnt_lstm *h) {
     for (int dir = 0; dir < 2; ++dir) {
         for (int w = 0; w < 12; ++w)
             if (h->state[dir][w]) (void)hipFree(h->state[dir][w]);
-        if (h->mailbox[dir]) (void)hipFree(h->mailbox[dir]);
+        if (h->fmail[dir]) (void)hipFree(h->fmail[dir]);
         if (h->bmail[dir]) (void)hipFree(h->bmail[dir]);
     }
     if (h->abort_flag) (void)hipFree(h->abort_flag);
@@ -946,9 +1036,13 @@ int cnt_lstm_check(cnt_lstm *h, void *stream) {
             for (int q = 0; q < 6; ++q) m[q] += (double)t[(size_t)b * 6 + q];
         }
         const double us = active ? 0.01 / active / h->T : 0.0;
-        std::fprintf(stderr, "lstm backward per step [us]: receive waves wait %.3f cell %.3f loop %.3f poll rounds %.2f | "
-                     "product waves busy %.3f | memory wave busy after B %.3f (T=%d, %d workgroups)\n",
-                     m[0] * us, m[1] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, m[2] * us, m[5] * us, h->T, active);
+        if (h->last_was_forward)
+            std::fprintf(stderr, "lstm forward per step [us]: gather waves wait+product %.3f loop %.3f poll rounds %.2f "
+                         "(T=%d, %d workgroups)\n", m[0] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, h->T, active);
+        else
+            std::fprintf(stderr, "lstm backward per step [us]: receive waves wait %.3f cell %.3f loop %.3f poll rounds %.2f | "
+                         "product waves busy %.3f | memory wave busy after B %.3f (T=%d, %d workgroups)\n",
+                         m[0] * us, m[1] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, m[2] * us, m[5] * us, h->T, active);
     }
     if (flag != 0) {
         CNT_HIP(hipMemset(h->abort_flag, 0, sizeof(int)));
