@@ -267,6 +267,35 @@ int cnt_dft_forward(cnt_dft *h, void *stream, int n_waves, const int *lengths, c
  * prev_errors (n_waves x max_length) = sum over resolutions of the stored gradients, 0 beyond each length. */
 int cnt_dft_backward(cnt_dft *h, void *stream, float *prev_errors);
 
+/* ---- weight update of the training loop (SURVEY "next": optimizer step on device) -----------------
+ * optimizer option numbers are the reference's (MacroDefine.hpp:33-37): 0 plain SGD, 1 AdaGrad,
+ * 2 gradient averaged over the fraction, 3 stochastic AdaGrad (statistics only), 4 SGD with decaying
+ * learning rate (the decay is host logic; treated as 0 here), 5 Adam.  `stats` holds one float per weight
+ * for AdaGrad (the reference initialises it to 1e-6, optimizers/Optimizer.cu:427-433) and interleaved
+ * (m, v) pairs for Adam (zero-initialised, :443-447).  `mask` is the optional weight mask (NULL = none).
+ *
+ * cnt_opt_accumulate: per-fraction copy (add = 0) or accumulation (add != 0) of a layer's weightUpdates()
+ * into the optimizer's current weight updates (optimizers/Optimizer.cu:186-198). */
+int cnt_opt_accumulate(void *stream, long n, const float *layer_updates, float *cur_updates, int add);
+/* The gradient adjustment SteepestDescentOptimizer::_updateWeights applies before the update
+ * (optimizers/SteepestDescentOptimizer.cu:312-405; functors :119-203).  frac_length is the fraction's
+ * fracTimeLength(); beta?_accum are m_adamBeta?Accum AFTER this call's multiplication by beta
+ * (cnt_opt_next_beta_accum reproduces that float-times-double product, :345-349). */
+int cnt_opt_adjust_gradient(void *stream, int option, long n, float *cur_updates, float *stats, const float *mask,
+                            float frac_length, float beta1_accum, float beta2_accum);
+/* UpdateWeightFn / UpdateWeightFn_withMask (optimizers/SteepestDescentOptimizer.cu:41-98, :408-436):
+ * NaN / Inf gradients are zeroed in place, delta = momentum*delta - lr*g, w = (w + delta) [* mask].
+ * A negative learning rate skips the update, as the reference does (:283-285). */
+int cnt_opt_update_weights(void *stream, long n, float *weights, float *cur_updates, float *weight_deltas,
+                           const float *mask, float learning_rate, float momentum);
+/* The three calls above (copy, adjust, update) for one layer in a single pass over its weights; same
+ * results, a third of the memory traffic.  For the hybrid online/batch mode, where the reference updates
+ * after every fraction (optimizers/Optimizer.cu:229-231). */
+int cnt_opt_step(void *stream, int option, long n, float *weights, const float *layer_updates, float *cur_updates,
+                 float *stats, float *weight_deltas, const float *mask, float frac_length, float beta1_accum,
+                 float beta2_accum, float learning_rate, float momentum);
+float cnt_opt_next_beta_accum(float accum, int which);
+
 #ifdef __cplusplus
 }
 #endif

@@ -113,6 +113,14 @@ float orc_dft_logamp_loss(int fft_length, int frame_length, int frame_shift, int
                           int length, float gamma, float log_floor, const float *source, const float *target,
                           float *grad);
 
+/* weight update of the training loop (optimizers/Optimizer.cu:186-198, optimizers/SteepestDescentOptimizer.cu) */
+void orc_opt_accumulate(long n, const float *layer_updates, float *cur_updates, int add);
+void orc_opt_adjust_gradient(int option, long n, float *g, float *stats, const float *mask, float frac_length,
+                             float beta1_accum, float beta2_accum);
+void orc_opt_update_weights(long n, float *weights, float *g, float *deltas, const float *mask, float learning_rate,
+                            float momentum);
+float orc_opt_next_beta_accum(float accum, int which);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,9 +22,15 @@ FLAGS = [
 ]
 
 
+# Per-file additions.  The weight update is specified operation by operation (every product and sum rounded
+# on its own, as the reference's host and device code do), so its file is compiled without contraction into
+# fused multiply-adds; HIP's __fmul_rn / __fadd_rn are plain operators and do not prevent it.
+EXTRA_FLAGS = {"optimizer.hip": ["-ffp-contract=off"]}
+
+
 def _compile(src):
     obj = os.path.join(OBJ, os.path.basename(src) + ".o")
-    cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
+    cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(os.path.basename(src), []) + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     return src, obj, r.returncode, r.stdout + r.stderr
 

@@ -51,6 +51,11 @@ _SIGNATURES = {
     "cnt_dense_backward_weights": (I, [VP, I, I, I, F, VP, VP, VP]),
     "cnt_sse_backward": (I, [VP, I, I, VP, VP, VP, VP]),
     "cnt_sse_error": (I, [VP, I, I, VP, VP, VP, VP]),
+    "cnt_opt_accumulate": (I, [VP, C.c_long, VP, VP, I]),
+    "cnt_opt_adjust_gradient": (I, [VP, I, C.c_long, VP, VP, VP, F, F, F]),
+    "cnt_opt_update_weights": (I, [VP, C.c_long, VP, VP, VP, VP, F, F]),
+    "cnt_opt_step": (I, [VP, I, C.c_long, VP, VP, VP, VP, VP, VP, F, F, F, F, F]),
+    "cnt_opt_next_beta_accum": (F, [F, I]),
     "cnt_lstm_create": (I, [C.POINTER(LstmDesc), C.POINTER(VP)]),
     "cnt_lstm_destroy": (I, [VP]),
     "cnt_lstm_load_sequences": (I, [VP, VP, VP, I, I]),
@@ -173,6 +178,34 @@ def sse_backward(D, N, pat, y, tgt, err, stream=None):
 
 def sse_error(D, N, pat, y, tgt, result, stream=None):
     check(lib().cnt_sse_error(stream_ptr(stream), D, N, ptr(pat), ptr(y), ptr(tgt), ptr(result)))
+
+
+OPT_SGD, OPT_ADAGRAD, OPT_AVEGRAD, OPT_STOCHASTIC_ADAGRAD, OPT_SGD_DECAY, OPT_ADAM = 0, 1, 2, 3, 4, 5
+
+
+def opt_accumulate(layer_updates, cur_updates, add, stream=None):
+    check(lib().cnt_opt_accumulate(stream_ptr(stream), layer_updates.numel(), ptr(layer_updates), ptr(cur_updates), int(add)))
+
+
+def opt_adjust_gradient(option, cur_updates, stats, mask, frac_length, beta1_accum=0.0, beta2_accum=0.0, stream=None):
+    check(lib().cnt_opt_adjust_gradient(stream_ptr(stream), option, cur_updates.numel(), ptr(cur_updates), ptr(stats),
+                                        ptr(mask), frac_length, beta1_accum, beta2_accum))
+
+
+def opt_update_weights(weights, cur_updates, deltas, mask, learning_rate, momentum, stream=None):
+    check(lib().cnt_opt_update_weights(stream_ptr(stream), weights.numel(), ptr(weights), ptr(cur_updates), ptr(deltas),
+                                       ptr(mask), learning_rate, momentum))
+
+
+def opt_step(option, weights, layer_updates, cur_updates, stats, deltas, mask, frac_length, beta1_accum, beta2_accum,
+             learning_rate, momentum, stream=None):
+    check(lib().cnt_opt_step(stream_ptr(stream), option, weights.numel(), ptr(weights), ptr(layer_updates),
+                             ptr(cur_updates), ptr(stats), ptr(deltas), ptr(mask), frac_length, beta1_accum,
+                             beta2_accum, learning_rate, momentum))
+
+
+def opt_next_beta_accum(accum, which):
+    return float(lib().cnt_opt_next_beta_accum(accum, which))
 
 
 class Lstm:

@@ -202,9 +202,57 @@ def dft_c5(args, pkg):
                  "configs[4]: DFT multi-resolution log-amplitude loss, forward (loss + gradient) and backward, 8 x 16000 samples", extra)
 
 
+def opt_step(args, pkg):
+    """Adam step (copy + adjust + update in one pass) over the acoustic model's 3.7 M weights, one launch per layer."""
+    import torch
+
+    capi = pkg.capi
+    sizes = [382 * 512 + 512, 512 * 512 + 512, 1576448, 1576448, 512 * 187 + 187]
+    rng = np.random.default_rng(5)
+    layers = []
+    for n in sizes:
+        layers.append({"w": _dev(rng.standard_normal(n).astype(np.float32)),
+                       "g": _dev(rng.standard_normal(n).astype(np.float32)),
+                       "cur": torch.zeros(n, device="cuda"), "stats": torch.zeros(2 * n, device="cuda"),
+                       "deltas": torch.zeros(n, device="cuda")})
+    state = {"b1": 1.0, "b2": 1.0}
+
+    def step():
+        state["b1"] = capi.opt_next_beta_accum(state["b1"], 1)
+        state["b2"] = capi.opt_next_beta_accum(state["b2"], 2)
+        for L in layers:
+            capi.opt_step(capi.OPT_ADAM, L["w"], L["g"], L["cur"], L["stats"], L["deltas"], None, 4904.0,
+                          state["b1"], state["b2"], 1e-4, 0.0)
+
+    sec = _timed(step, args.steps, args.warmup)
+    kernels = _profile(capi, step, args.steps)
+    total = sum(sizes)
+    nbytes = total * 40.0  # per weight: read g, m, v, delta, w; write cur, m, v, delta, w
+    ach = nbytes / (kernels["opt_step"]["ms_per_step"] * 1e-3) / 1e9
+    roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
+            "traffic": None, "kernel": "opt_step",
+            "note": "5 launches of 0.2-1.6 M weights each; 40 B per weight"}
+    extra = {"roofline": roof, "kernels": kernels}
+    if not args.no_cpu:
+        hw = [np.zeros(n, np.float32) for n in sizes]
+        t0 = time.perf_counter()
+        reps = 5
+        for _ in range(reps):
+            for n, w in zip(sizes, hw):
+                g = np.ones(n, np.float32); cur = np.empty(n, np.float32)
+                O.opt_accumulate(g, cur, False)
+                O.opt_adjust_gradient(5, cur, np.zeros(2 * n, np.float32), None, 4904.0, 0.9, 0.999)
+                O.opt_update_weights(w, cur, np.zeros(n, np.float32), None, 1e-4, 0.0)
+        dt = (time.perf_counter() - t0) / reps
+        extra["cpu_baseline"] = {"value": total / dt, "unit": "weights/s", "cores": 1, "kind": "port",
+                                 "sample": "the same 3.7 M weights, %d repetitions, CPU oracle (three passes as in the reference)" % reps}
+    return _base(args, total / sec, "weights/s", sec,
+                 "next row f3: Adam weight update of the acoustic model (3.7 M weights in 5 layers), one fused pass per layer", extra)
+
+
 def run(name, args, pkg):
     if name == "wavenet_c4":
         import bench_wavenet
 
         return bench_wavenet.run(args, pkg)
-    return {"lstm_c1": lstm_c1, "mdn_c3": mdn_c3, "dft_c5": dft_c5}[name](args, pkg)
+    return {"lstm_c1": lstm_c1, "mdn_c3": mdn_c3, "dft_c5": dft_c5, "opt_step": opt_step}[name](args, pkg)

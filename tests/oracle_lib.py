@@ -69,6 +69,8 @@ def lib():
         L.orc_mdn_mixture_error.restype = C.c_float
         L.orc_softmax_error.restype = C.c_float
         L.orc_dft_logamp_loss.restype = C.c_float
+        L.orc_opt_next_beta_accum.restype = C.c_float
+        L.orc_opt_next_beta_accum.argtypes = [C.c_float, C.c_int]
         _lib = L
     return _lib
 
@@ -228,3 +230,23 @@ def dft_c2r(X, n):
 def dft_logamp_loss(N, Nw, Hs, window_type, max_len, length, gamma, floor, src, tgt, grad):
     return float(lib().orc_dft_logamp_loss(N, Nw, Hs, window_type, max_len, length, C.c_float(gamma), C.c_float(floor),
                                            fptr(src), fptr(tgt), fptr(grad)))
+
+
+def opt_accumulate(layer_updates, cur_updates, add):
+    lib().orc_opt_accumulate(C.c_long(cur_updates.size), fptr(layer_updates), fptr(cur_updates), int(add))
+
+
+def opt_adjust_gradient(option, g, stats, mask, frac_length, beta1_accum=0.0, beta2_accum=0.0):
+    lib().orc_opt_adjust_gradient(int(option), C.c_long(g.size), fptr(g), fptr(stats) if stats is not None else None,
+                                  fptr(mask) if mask is not None else None, C.c_float(frac_length),
+                                  C.c_float(beta1_accum), C.c_float(beta2_accum))
+
+
+def opt_update_weights(weights, g, deltas, mask, learning_rate, momentum):
+    lib().orc_opt_update_weights(C.c_long(g.size), fptr(weights), fptr(g), fptr(deltas),
+                                 fptr(mask) if mask is not None else None, C.c_float(learning_rate),
+                                 C.c_float(momentum))
+
+
+def opt_next_beta_accum(accum, which):
+    return float(lib().orc_opt_next_beta_accum(accum, which))
