@@ -99,7 +99,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--cpu-sample-T", type=int, default=160)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
-    ap.add_argument("--workload", default="acoustic", choices=["acoustic", "lstm_c1", "mdn_c3", "dft_c5", "wavenet_c4", "opt_step"],
+    ap.add_argument("--workload", default="acoustic", choices=["acoustic", "lstm_c1", "mdn_c3", "dft_c5", "wavenet_c4", "opt_step", "nc_fraction"],
                     help="acoustic = BASELINE configs[1] (the headline metric); the others are the remaining configs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, to scale rocprofv3's "

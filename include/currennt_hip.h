@@ -296,6 +296,38 @@ int cnt_opt_step(void *stream, int option, long n, float *weights, const float *
                  float beta2_accum, float learning_rate, float momentum);
 float cnt_opt_next_beta_accum(float accum, int which);
 
+/* ---- the .nc data path (SURVEY "next": NetCDF reader and fraction builder; host memory only) --------
+ * data_sets::DataSet's constructor for ONE .nc file (data_sets/DataSet.cpp:1376-1907): reads the
+ * dimensions and seqLengths / seqTags, keeps the first max(1, int(numSeqs * fraction)) sequences, cuts a
+ * sequence longer than 1.5 * truncate_seq into segments of truncate_seq (0 = off), and in training mode
+ * sorts the segments by ascending length (stable here; the reference's std::sort leaves ties unspecified).
+ * Classic (CDF-1) and 64-bit-offset (CDF-2) files are read without libnetcdf. */
+typedef struct cnt_dataset cnt_dataset;
+typedef struct {
+    int parallel_sequences; /* S: sequences per fraction                         */
+    int training_mode;      /* != 0: sort by length (Configuration::trainingMode) */
+    int truncate_seq;       /* --truncate_seq, 0 = off                             */
+    float fraction;         /* --train_fraction etc., in (0, 1]                    */
+} cnt_dataset_desc;
+int cnt_dataset_open(const char *nc_path, const cnt_dataset_desc *desc, cnt_dataset **out);
+int cnt_dataset_close(cnt_dataset *d);
+/* DataSet::totalSequences / inputPatternSize / outputPatternSize / isClassificationData / totalTimesteps /
+ * minSeqLength / maxSeqLength (data_sets/DataSet.hpp); any pointer may be NULL. */
+int cnt_dataset_info(cnt_dataset *d, int *num_sequences, int *input_size, int *output_size, int *is_classification,
+                     long *total_timesteps, int *min_len, int *max_len);
+/* one entry of the (sorted) segment list: length, index of the segment inside its utterance, tag */
+int cnt_dataset_sequence(cnt_dataset *d, int index, int *length, int *original_seq_idx, char *tag, int tag_cap);
+/* DataSet::_makeFractionTask(firstSeqIdx) (data_sets/DataSet.cpp:642-1022) in two steps.  _shape gives
+ * numSequences, maxSeqLength, minSeqLength and fracTimeLength of the fraction that starts at first_seq;
+ * _fill writes, into host buffers the caller sized from it, patTypes[maxLen*S] (0 none, 1 first, 2 normal,
+ * 3 last), inputs[maxLen*S*inputSize] and targets[maxLen*S*outputSize] (regression) or
+ * target_classes[maxLen*S] (classification, -1 on padding): slot t*S+i holds time step t of the i-th
+ * sequence, padding slots are zero. */
+int cnt_dataset_fraction_shape(cnt_dataset *d, int first_seq, int *num_seqs, int *max_len, int *min_len,
+                               int *total_length);
+int cnt_dataset_fraction_fill(cnt_dataset *d, int first_seq, char *patTypes, float *inputs, float *targets,
+                              int *target_classes);
+
 #ifdef __cplusplus
 }
 #endif

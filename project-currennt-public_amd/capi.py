@@ -28,6 +28,11 @@ class DftDesc(C.Structure):
                 ("log_floor", C.c_float), ("spec_dis_type", C.c_int), ("max_length", C.c_int), ("max_waves", C.c_int)]
 
 
+class DatasetDesc(C.Structure):
+    _fields_ = [("parallel_sequences", C.c_int), ("training_mode", C.c_int), ("truncate_seq", C.c_int),
+                ("fraction", C.c_float)]
+
+
 class LstmDesc(C.Structure):
     _fields_ = [("P", C.c_int), ("L", C.c_int), ("bidir", C.c_int), ("S", C.c_int), ("maxT", C.c_int),
                 ("bias", C.c_float)]
@@ -51,6 +56,13 @@ _SIGNATURES = {
     "cnt_dense_backward_weights": (I, [VP, I, I, I, F, VP, VP, VP]),
     "cnt_sse_backward": (I, [VP, I, I, VP, VP, VP, VP]),
     "cnt_sse_error": (I, [VP, I, I, VP, VP, VP, VP]),
+    "cnt_dataset_open": (I, [C.c_char_p, C.POINTER(DatasetDesc), C.POINTER(VP)]),
+    "cnt_dataset_close": (I, [VP]),
+    "cnt_dataset_info": (I, [VP, C.POINTER(I), C.POINTER(I), C.POINTER(I), C.POINTER(I), C.POINTER(C.c_long),
+                             C.POINTER(I), C.POINTER(I)]),
+    "cnt_dataset_sequence": (I, [VP, I, C.POINTER(I), C.POINTER(I), C.c_char_p, I]),
+    "cnt_dataset_fraction_shape": (I, [VP, I, C.POINTER(I), C.POINTER(I), C.POINTER(I), C.POINTER(I)]),
+    "cnt_dataset_fraction_fill": (I, [VP, I, VP, VP, VP, VP]),
     "cnt_opt_accumulate": (I, [VP, C.c_long, VP, VP, I]),
     "cnt_opt_adjust_gradient": (I, [VP, I, C.c_long, VP, VP, VP, F, F, F]),
     "cnt_opt_update_weights": (I, [VP, C.c_long, VP, VP, VP, VP, F, F]),
@@ -178,6 +190,49 @@ def sse_backward(D, N, pat, y, tgt, err, stream=None):
 
 def sse_error(D, N, pat, y, tgt, result, stream=None):
     check(lib().cnt_sse_error(stream_ptr(stream), D, N, ptr(pat), ptr(y), ptr(tgt), ptr(result)))
+
+
+class Dataset:
+    """One .nc file as the reference's data_sets::DataSet sees it; fractions come back as numpy arrays."""
+
+    def __init__(self, path, parallel_sequences, training_mode=True, truncate_seq=0, fraction=1.0):
+        self.handle = VP()
+        self.S = parallel_sequences
+        desc = DatasetDesc(parallel_sequences, int(training_mode), truncate_seq, fraction)
+        check(lib().cnt_dataset_open(path.encode(), C.byref(desc), C.byref(self.handle)))
+        n, p, q, cls, mn, mx = I(), I(), I(), I(), I(), I()
+        tot = C.c_long()
+        check(lib().cnt_dataset_info(self.handle, C.byref(n), C.byref(p), C.byref(q), C.byref(cls), C.byref(tot),
+                                     C.byref(mn), C.byref(mx)))
+        self.num_sequences, self.input_size, self.output_size = n.value, p.value, q.value
+        self.is_classification, self.total_timesteps = bool(cls.value), tot.value
+        self.min_len, self.max_len = mn.value, mx.value
+
+    def sequence(self, index):
+        length, orig = I(), I()
+        tag = C.create_string_buffer(512)
+        check(lib().cnt_dataset_sequence(self.handle, index, C.byref(length), C.byref(orig), tag, 512))
+        return length.value, orig.value, tag.value.decode()
+
+    def fraction(self, first_seq):
+        import numpy as np
+
+        n, mx, mn, tot = I(), I(), I(), I()
+        check(lib().cnt_dataset_fraction_shape(self.handle, first_seq, C.byref(n), C.byref(mx), C.byref(mn), C.byref(tot)))
+        slots = mx.value * self.S
+        pat = np.zeros(slots, np.int8)
+        x = np.zeros(slots * self.input_size, np.float32)
+        tgt = np.zeros(slots * self.output_size, np.float32) if not self.is_classification else None
+        cls = np.zeros(slots, np.int32) if self.is_classification else None
+        as_ptr = lambda a: a.ctypes.data_as(VP) if a is not None else None
+        check(lib().cnt_dataset_fraction_fill(self.handle, first_seq, as_ptr(pat), as_ptr(x), as_ptr(tgt), as_ptr(cls)))
+        return {"num_seqs": n.value, "max_len": mx.value, "min_len": mn.value, "total_length": tot.value,
+                "patTypes": pat, "inputs": x, "targets": tgt, "target_classes": cls}
+
+    def close(self):
+        if self.handle:
+            lib().cnt_dataset_close(self.handle)
+            self.handle = VP()
 
 
 OPT_SGD, OPT_ADAGRAD, OPT_AVEGRAD, OPT_STOCHASTIC_ADAGRAD, OPT_SGD_DECAY, OPT_ADAM = 0, 1, 2, 3, 4, 5

@@ -250,9 +250,67 @@ def opt_step(args, pkg):
                  "next row f3: Adam weight update of the acoustic model (3.7 M weights in 5 layers), one fused pass per layer", extra)
 
 
+def nc_fraction(args, pkg):
+    """Host-side: build the C2-shaped fraction (10 sequences of 300..600 frames, 382 inputs, 187 targets) from a
+    .nc file.  No kernel runs; the figure is frames per second of the reader + interleaver on one host core."""
+    import importlib.util
+    import tempfile
+
+    from scipy.io import netcdf_file
+
+    capi = pkg.capi
+    rng = np.random.default_rng(9)
+    lengths = [int(v) for v in rng.integers(300, 601, 10)]
+    total, P, Q, S = sum(lengths), 382, 187, 10
+    tmp = tempfile.mkdtemp(prefix="cnt_nc_")
+    path = os.path.join(tmp, "c2.nc")
+    f = netcdf_file(path, "w", version=2)
+    for name, n in (("numSeqs", S), ("numTimesteps", total), ("inputPattSize", P), ("targetPattSize", Q), ("maxSeqTagLength", 8)):
+        f.createDimension(name, n)
+    tags = f.createVariable("seqTags", "c", ("numSeqs", "maxSeqTagLength"))
+    for i in range(S):
+        tags[i] = np.frombuffer(("u%02d" % i).encode().ljust(8, b"\0"), dtype="S1")
+    f.createVariable("seqLengths", "i", ("numSeqs",))[:] = np.asarray(lengths, np.int32)
+    f.createVariable("inputs", "f", ("numTimesteps", "inputPattSize"))[:] = rng.standard_normal((total, P)).astype(np.float32)
+    f.createVariable("targetPatterns", "f", ("numTimesteps", "targetPattSize"))[:] = rng.standard_normal((total, Q)).astype(np.float32)
+    f.close()
+    ds = capi.Dataset(path, S, True, 0, 1.0)
+
+    def step():
+        ds.fraction(0)
+
+    for _ in range(args.warmup):
+        step()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    sec = (time.perf_counter() - t0) / args.steps
+    nbytes = total * (P + Q) * 4.0
+    extra = {"roofline": {"bound": "hbm", "achieved": nbytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                          "frac": nbytes / sec / 1e9 / PEAK_HBM_GBS, "traffic": None, "kernel": "none (host code)",
+                          "note": "host-side reader: the figure is file bytes delivered per second by one CPU core; the "
+                                  "HBM peak is listed only because the field is mandatory"}}
+    if not args.no_cpu:
+        spec = importlib.util.spec_from_file_location("nc_fraction", os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "nc_fraction.py"))
+        NF = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(NF)
+        segs = NF.segments(path)
+        t0 = time.perf_counter()
+        NF.make_fraction(path, segs, 0, S)
+        dt = time.perf_counter() - t0
+        extra["cpu_baseline"] = {"value": total / dt, "unit": "frames/s", "cores": 1, "kind": "port",
+                                 "sample": "the same fraction once, numpy oracle with scipy's NetCDF reader (%.2f s)" % dt}
+    ds.close()
+    os.remove(path)
+    os.rmdir(tmp)
+    return _base(args, total / sec, "frames/s", sec,
+                 "next row f2: one C2-shaped fraction (%d frames, 382 inputs + 187 targets, S=10) from a 64-bit-offset .nc file, host code" % total,
+                 extra)
+
+
 def run(name, args, pkg):
     if name == "wavenet_c4":
         import bench_wavenet
 
         return bench_wavenet.run(args, pkg)
-    return {"lstm_c1": lstm_c1, "mdn_c3": mdn_c3, "dft_c5": dft_c5, "opt_step": opt_step}[name](args, pkg)
+    return {"lstm_c1": lstm_c1, "mdn_c3": mdn_c3, "dft_c5": dft_c5, "opt_step": opt_step, "nc_fraction": nc_fraction}[name](args, pkg)

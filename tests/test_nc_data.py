@@ -1,0 +1,144 @@
+"""CPU-only: the .nc data path (NetCDF-3 reader + fraction builder) behind the C ABI against the numpy oracle,
+which is itself pinned by a hand-computed case.  Files are written with scipy.io.netcdf_file, the writer the
+reference's own tooling uses, in both the classic and the 64-bit-offset variant.  All comparisons are exact."""
+import importlib.util
+import os
+
+import numpy as np
+import pytest
+from scipy.io import netcdf_file
+
+from __graft_entry__ import ROOT, load_package
+
+_spec = importlib.util.spec_from_file_location("nc_fraction", os.path.join(ROOT, "oracle", "nc_fraction.py"))
+NF = importlib.util.module_from_spec(_spec)
+_spec.loader.exec_module(NF)
+
+
+def write_nc(path, lengths, P, Q, version, classes=0, seed=0, extra_attr=True):
+    rng = np.random.default_rng(seed)
+    total = int(sum(lengths))
+    f = netcdf_file(path, "w", version=version)
+    if extra_attr:
+        f.history = "written by the test"
+    f.createDimension("numSeqs", len(lengths))
+    f.createDimension("numTimesteps", total)
+    f.createDimension("inputPattSize", P)
+    f.createDimension("maxSeqTagLength", 12)
+    tags = f.createVariable("seqTags", "c", ("numSeqs", "maxSeqTagLength"))
+    for i in range(len(lengths)):
+        t = ("utt%03d" % i).encode().ljust(12, b"\0")
+        tags[i] = np.frombuffer(t, dtype="S1")
+    ln = f.createVariable("seqLengths", "i", ("numSeqs",))
+    ln[:] = np.asarray(lengths, np.int32)
+    x = f.createVariable("inputs", "f", ("numTimesteps", "inputPattSize"))
+    x.units = "none"
+    x[:] = rng.standard_normal((total, P)).astype(np.float32)
+    if classes:
+        f.createDimension("numLabels", classes)
+        c = f.createVariable("targetClasses", "i", ("numTimesteps",))
+        c[:] = rng.integers(0, classes, total).astype(np.int32)
+    else:
+        f.createDimension("targetPattSize", Q)
+        y = f.createVariable("targetPatterns", "f", ("numTimesteps", "targetPattSize"))
+        y[:] = rng.standard_normal((total, Q)).astype(np.float32)
+    f.close()
+
+
+def test_oracle_fraction_hand_computed(tmp_path):
+    # two sequences of lengths 3 and 1, one input, one target: inputs are 10,11,12 | 20
+    p = str(tmp_path / "tiny.nc")
+    f = netcdf_file(p, "w")
+    for name, n in (("numSeqs", 2), ("numTimesteps", 4), ("inputPattSize", 1), ("targetPattSize", 1), ("maxSeqTagLength", 2)):
+        f.createDimension(name, n)
+    f.createVariable("seqTags", "c", ("numSeqs", "maxSeqTagLength"))[:] = np.array([[b"a", b"\0"], [b"b", b"\0"]])
+    f.createVariable("seqLengths", "i", ("numSeqs",))[:] = np.array([3, 1], np.int32)
+    f.createVariable("inputs", "f", ("numTimesteps", "inputPattSize"))[:] = np.array([[10], [11], [12], [20]], np.float32)
+    f.createVariable("targetPatterns", "f", ("numTimesteps", "targetPattSize"))[:] = np.array([[1], [2], [3], [4]], np.float32)
+    f.close()
+    segs = NF.segments(p, training_mode=True)
+    assert [(s["length"], s["tag"]) for s in segs] == [(1, "b"), (3, "a")]   # sorted by ascending length
+    fr = NF.make_fraction(p, segs, 0, 2)
+    # slot t*S+i: i=0 is "b" (length 1), i=1 is "a" (length 3)
+    assert fr["max_len"] == 3 and fr["min_len"] == 1 and fr["total_length"] == 4
+    assert fr["inputs"].tolist() == [20, 10, 0, 11, 0, 12]
+    assert fr["targets"].tolist() == [4, 1, 0, 2, 0, 3]
+    assert fr["patTypes"].tolist() == [1, 1, 0, 2, 0, 3]     # a length-1 sequence is FIRST, not LAST
+    # truncation cuts only while more than 1.5 segments remain: 3 steps at truncate 2 stay whole (3 > 3 is false),
+    # at truncate 1 they become 1 + 1 + 1
+    segs = NF.segments(p, truncate_seq=2, training_mode=False)
+    assert [s["length"] for s in segs] == [3, 1]
+    segs = NF.segments(p, truncate_seq=1, training_mode=False)
+    assert [s["length"] for s in segs] == [1, 1, 1, 1] and [s["original_seq_idx"] for s in segs] == [0, 1, 2, 0]
+    assert [s["begin"] for s in segs] == [0, 1, 2, 3]
+
+
+@pytest.mark.parametrize("version,classes,S,trunc,frac,train", [
+    (1, 0, 4, 0, 1.0, True), (2, 0, 3, 0, 1.0, False), (2, 0, 5, 7, 1.0, True), (1, 5, 2, 0, 1.0, True),
+    (1, 2, 4, 0, 0.5, True), (2, 0, 1, 0, 0.01, True),
+])
+def test_reader_matches_oracle(tmp_path, version, classes, S, trunc, frac, train):
+    capi = load_package().capi
+    lengths = [17, 5, 23, 9, 31, 12, 1, 40, 8]
+    P, Q = 7, 3
+    p = str(tmp_path / "data.nc")
+    write_nc(p, lengths, P, Q, version, classes, seed=version + classes + S)
+    segs = NF.segments(p, frac, trunc, train)
+    ds = capi.Dataset(p, S, train, trunc, frac)
+    try:
+        assert ds.num_sequences == len(segs)
+        assert ds.input_size == P and ds.output_size == ((1 if classes == 2 else classes) if classes else Q)
+        assert ds.is_classification == bool(classes)
+        take = max(int(len(lengths) * frac), 1)
+        assert ds.total_timesteps == sum(lengths[:take])
+        assert ds.min_len == min(s["length"] for s in segs) and ds.max_len == max(s["length"] for s in segs)
+        got = [ds.sequence(i) for i in range(ds.num_sequences)]
+        assert got == [(s["length"], s["original_seq_idx"], s["tag"]) for s in segs]
+        for first in range(0, len(segs), S):
+            a, b = ds.fraction(first), NF.make_fraction(p, segs, first, S)
+            for key in ("num_seqs", "max_len", "min_len", "total_length"):
+                assert a[key] == b[key], key
+            for key in ("patTypes", "inputs", "targets", "target_classes"):
+                if b[key] is None:
+                    assert a[key] is None
+                else:
+                    assert np.array_equal(a[key], b[key]), (key, first)
+    finally:
+        ds.close()
+
+
+def test_reader_errors(tmp_path):
+    capi = load_package().capi
+    with pytest.raises(RuntimeError, match="Could not open"):
+        capi.Dataset(str(tmp_path / "missing.nc"), 2)
+    bad = tmp_path / "bad.nc"
+    bad.write_bytes(b"\x89HDF\r\n\x1a\n" + b"\0" * 64)      # a NetCDF-4 (HDF5) file is not the classic format
+    with pytest.raises(RuntimeError, match="CDF magic"):
+        capi.Dataset(str(bad), 2)
+    p = str(tmp_path / "ok.nc")
+    write_nc(p, [4, 6], 2, 2, 1)
+    with pytest.raises(RuntimeError, match="Invalid fraction"):
+        capi.Dataset(p, 2, fraction=0.0)
+    # a file without targets of either kind
+    q = str(tmp_path / "notargets.nc")
+    f = netcdf_file(q, "w")
+    for name, n in (("numSeqs", 1), ("numTimesteps", 2), ("inputPattSize", 1), ("maxSeqTagLength", 2)):
+        f.createDimension(name, n)
+    f.createVariable("seqLengths", "i", ("numSeqs",))[:] = np.array([2], np.int32)
+    f.close()
+    with pytest.raises(RuntimeError, match="targetPattSize"):
+        capi.Dataset(q, 1)
+    # an unlimited (record) dimension is refused, not misread
+    r = str(tmp_path / "record.nc")
+    f = netcdf_file(r, "w")
+    f.createDimension("numTimesteps", None); f.createDimension("numSeqs", 1); f.createDimension("inputPattSize", 1)
+    f.createDimension("targetPattSize", 1); f.createDimension("maxSeqTagLength", 2)
+    f.createVariable("seqTags", "c", ("numSeqs", "maxSeqTagLength"))[:] = np.array([[b"a", b"\0"]])
+    f.createVariable("seqLengths", "i", ("numSeqs",))[:] = np.array([2], np.int32)
+    f.createVariable("inputs", "f", ("numTimesteps", "inputPattSize"))[0:2] = np.zeros((2, 1), np.float32)
+    f.createVariable("targetPatterns", "f", ("numTimesteps", "targetPattSize"))[0:2] = np.zeros((2, 1), np.float32)
+    f.close()
+    ds = capi.Dataset(r, 1)
+    with pytest.raises(RuntimeError, match="unlimited"):
+        ds.fraction(0)
+    ds.close()
