@@ -144,6 +144,128 @@ class StackedNetwork:
                 L["handle"].close()
 
 
+# ---------------------------------------------------------------------------------------------------------
+# Network files.  The reference keeps a network as JSON: "layers" is the ordered list of
+# {"name", "type", "size", "bias", ...} objects (Layer::exportLayer, layers/Layer.cu:308-329, and
+# TrainableLayer::exportLayer, layers/TrainableLayer.cu:483-492); "weights" maps a layer name to its
+# "input" / "bias" / "internal" arrays, which are consecutive sections of the layer's flat weight vector
+# (TrainableLayer::exportWeights, layers/TrainableLayer.cu:441-480; read back in the constructor, :100-170).
+# ---------------------------------------------------------------------------------------------------------
+def load_network_json(path):
+    """Returns (input_size, layer specs without the input layer, per-layer flat weight arrays or None)."""
+    import json
+
+    import numpy as np
+
+    with open(path) as f:
+        doc = json.load(f)
+    layers = doc.get("layers")
+    if not isinstance(layers, list) or len(layers) < 3:
+        raise ValueError("%s: a network needs an input layer, a hidden or output layer and a post-output layer" % path)
+    if layers[0].get("type") != "input":
+        raise ValueError("%s: the first layer must be of type 'input'" % path)
+    input_size = int(layers[0]["size"])
+    specs, weights = [], []
+    have_weights = isinstance(doc.get("weights"), dict)
+    prev = input_size
+    for obj in layers[1:]:
+        t = obj.get("type")
+        if t not in _FF_ACT and t not in ("lstm", "blstm", "sse"):
+            raise ValueError("%s: layer '%s' has type '%s', which this path does not cover" % (path, obj.get("name"), t))
+        spec = {"name": obj.get("name", t), "type": t, "size": int(obj["size"])}
+        if "bias" in obj:
+            spec["bias"] = float(obj["bias"])
+        specs.append(spec)
+        nW = layer_weight_count(spec, prev)
+        if nW and have_weights:
+            sec = doc["weights"].get(spec["name"])
+            if sec is None:
+                raise ValueError("%s: no weights for layer '%s'" % (path, spec["name"]))
+            w = np.concatenate([np.asarray(sec.get(k, []), dtype=np.float32) for k in ("input", "bias", "internal")])
+            if w.size != nW:
+                raise ValueError("%s: layer '%s' has %d weights, expected %d" % (path, spec["name"], w.size, nW))
+            weights.append(w)
+        prev = spec["size"]
+    if specs[-1]["type"] != "sse":
+        raise ValueError("%s: the last layer must be the sse post-output layer" % path)
+    return input_size, specs, (weights if have_weights else None)
+
+
+def weight_sections(spec, prev_size):
+    """Lengths of the "input", "bias" and "internal" sections of a layer's weight vector."""
+    D = spec["size"]
+    if spec["type"] in _FF_ACT:
+        return prev_size * D, D, 0
+    if spec["type"] in ("lstm", "blstm"):
+        H = D // (2 if spec["type"] == "blstm" else 1)
+        return 4 * prev_size * D, 4 * D, 4 * D * H + 3 * D
+    return 0, 0, 0
+
+
+def save_network_json(path, net):
+    """Writes layers and weights of a StackedNetwork in the reference's structure (the autosave's network part)."""
+    import json
+
+    layers = [{"size": net.input_size, "name": "input", "type": "input"}]
+    weights = {}
+    for i, L in enumerate(net.layers):
+        spec = L["spec"]
+        obj = {"size": L["size"], "name": spec.get("name", "%s_%d" % (L["type"], i)), "type": L["type"]}
+        if "weights" in L:
+            obj["bias"] = L["bias"]
+            w = L["weights"].detach().cpu().numpy()
+            n_in, n_bias, n_int = weight_sections(spec, L["prev"])
+            weights[obj["name"]] = {"input": [float(v) for v in w[:n_in]],
+                                    "bias": [float(v) for v in w[n_in:n_in + n_bias]],
+                                    "internal": [float(v) for v in w[n_in + n_bias:]]}
+        layers.append(obj)
+    with open(path, "w") as f:
+        json.dump({"layers": layers, "weights": weights}, f)
+
+
+class Trainer:
+    """One training step per fraction, as Optimizer::_processDataSet does in hybrid online/batch mode
+    (optimizers/Optimizer.cu:95-237): load the fraction, forward, error, backward, then for every trainable layer
+    the copy / gradient adjustment / momentum update of SteepestDescentOptimizer::_updateWeights in one fused
+    pass.  `option` is the reference's optimizer option number (0 SGD, 1 AdaGrad, 2 averaged gradient, 5 Adam)."""
+
+    def __init__(self, net, learning_rate, momentum=0.0, option=0):
+        self.net, self.lr, self.momentum, self.option = net, learning_rate, momentum, option
+        self.beta1 = self.beta2 = 1.0
+        self.side = torch.cuda.Stream()
+        for L in net.layers:
+            if "weights" in L:
+                n = L["weights"].numel()
+                L["cur_updates"] = torch.zeros(n, dtype=torch.float32, device="cuda")
+                L["deltas"] = torch.zeros(n, dtype=torch.float32, device="cuda")
+                if option in (capi.OPT_ADAGRAD, capi.OPT_STOCHASTIC_ADAGRAD):
+                    L["stats"] = torch.full((n,), 1e-6, dtype=torch.float32, device="cuda")
+                elif option == capi.OPT_ADAM:
+                    L["stats"] = torch.zeros(2 * n, dtype=torch.float32, device="cuda")
+                else:
+                    L["stats"] = None
+
+    def train_fraction(self, fraction):
+        """`fraction`: dict from capi.Dataset.fraction().  Returns the fraction's training error (a device tensor)."""
+        net = self.net
+        T = fraction["max_len"]
+        pat = torch.from_numpy(fraction["patTypes"]).cuda()
+        net.load_sequences(pat, T, fraction["min_len"], torch.from_numpy(fraction["inputs"]).cuda(),
+                           torch.from_numpy(fraction["targets"]).cuda())
+        net.forward()
+        loss = net.calculate_error().clone()
+        net.backward_overlapped(self.side)
+        torch.cuda.current_stream().wait_stream(self.side)
+        if self.option == capi.OPT_ADAM:
+            self.beta1 = capi.opt_next_beta_accum(self.beta1, 1)
+            self.beta2 = capi.opt_next_beta_accum(self.beta2, 2)
+        for L in net.layers:
+            if "weights" in L:
+                capi.opt_step(self.option, L["weights"], L["updates"], L["cur_updates"], L["stats"], L["deltas"], None,
+                              float(fraction["total_length"]), self.beta1, self.beta2, self.lr, self.momentum)
+        return loss
+
+
 def acoustic_model_spec():
     """BASELINE config 2: 382 -> 2 x feedforward_tanh 512 -> 2 x blstm 512 -> feedforward_identity 187 -> sse."""
     return 382, [
