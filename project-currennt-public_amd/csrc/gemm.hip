@@ -6,8 +6,8 @@
 // products of a BLSTM become one pass), several independent problems per launch, split-K for the
 // long-K weight-gradient shapes, and a fused bias + activation epilogue for the dense forward.
 //
-// Tiling: 128 x 128 x 32 per workgroup, four 64-lane waves in a 2 x 2 arrangement, each wave owning
-// a 64 x 64 block as 2 x 2 tiles of v_mfma_f32_32x32x2_f32.  An operand tile sits in LDS in the
+// Tiling: T x T x 16 per workgroup with T = 128 or 64, four 64-lane waves in a 2 x 2 arrangement, each wave
+// owning a T/2 x T/2 block as tiles of v_mfma_f32_32x32x2_f32.  An operand tile sits in LDS in the
 // orientation it has in memory, so that staging never transposes: k-contiguous operands as [row][k] with
 // a (BK+4)-float pitch (16-byte fragment reads, conflict free), row-contiguous operands as [k][row]
 // (4-byte fragment reads along consecutive rows).  A transposing store of the latter into [row][k]
@@ -16,10 +16,12 @@
 // along the column-major output's contiguous dimension and every store is a 128-byte segment.
 #include "common.hpp"
 
+#include <cstdlib>
+
 namespace cnt {
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 16;
+constexpr int BK = 16;  // the tile edge (rows of A = columns of B per workgroup) is a template parameter: 128 or 64
 constexpr int PITCH = BK + 4;
 constexpr int NTHREADS = 256;
 
@@ -41,10 +43,11 @@ struct VecT<2> { typedef float2 type; };
 template <>
 struct VecT<4> { typedef float4 type; };
 
-// Stages one 128-row x 16-k operand tile: global -> registers -> LDS [row][k].
-template <int VEC, bool KCONTIG>
+// Stages one ROWS-row x 16-k operand tile: global -> registers -> LDS.
+template <int VEC, bool KCONTIG, int ROWS>
 struct TileStage {
-    static constexpr int NLOAD = (128 * BK) / (NTHREADS * VEC);
+    static constexpr int NLOAD = (ROWS * BK) / (NTHREADS * VEC);
+    static_assert(NLOAD >= 1, "tile too small for this vector width");
     typename VecT<VEC>::type r[NLOAD];
 
     // shift / pat / n_slots: masked mode (pat == nullptr switches it off); time_on_k selects which index is
@@ -88,7 +91,7 @@ struct TileStage {
                 r[p] = v;
             }
         } else {
-            constexpr int TPK = 128 / VEC;       // threads per k line
+            constexpr int TPK = ROWS / VEC;      // threads per k line
             constexpr int KPP = NTHREADS / TPK;  // k lines per pass
             const int rq = (tid % TPK) * VEC;
             const int kk = tid / TPK;
@@ -133,7 +136,7 @@ struct TileStage {
             }
         } else {
 #pragma unroll
-            for (int q = 0; q < BK / 2; ++q) f[q] = lds[(k_first + q) * 128 + row];
+            for (int q = 0; q < BK / 2; ++q) f[q] = lds[(k_first + q) * ROWS + row];
         }
     }
 
@@ -147,13 +150,13 @@ struct TileStage {
             for (int p = 0; p < NLOAD; ++p)
                 *reinterpret_cast<typename VecT<VEC>::type *>(lds + (rr + p * RPP) * PITCH + kq) = r[p];
         } else {
-            constexpr int TPK = 128 / VEC;
+            constexpr int TPK = ROWS / VEC;
             constexpr int KPP = NTHREADS / TPK;
             const int rq = (tid % TPK) * VEC;
             const int kk = tid / TPK;
 #pragma unroll
             for (int p = 0; p < NLOAD; ++p)
-                *reinterpret_cast<typename VecT<VEC>::type *>(lds + (kk + p * KPP) * 128 + rq) = r[p];
+                *reinterpret_cast<typename VecT<VEC>::type *>(lds + (kk + p * KPP) * ROWS + rq) = r[p];
         }
     }
 };
@@ -161,8 +164,11 @@ struct TileStage {
 // MASKED selects the time-shifted, padding-masked B loader at compile time: its per-element predication is a lot
 // of code, and four copies of it (two prologue fetches, two in the unrolled loop) inside the plain kernels would
 // push their hot loop out of the instruction cache.
-template <int VA, bool AK, int VB, bool BK_, bool MASKED>
+template <int VA, bool AK, int VB, bool BK_, bool MASKED, int TILE>
 __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args) {
+    constexpr int BM = TILE, BN = TILE;
+    constexpr int WT = TILE / 2;   // edge of a wave's block (waves are arranged 2 x 2)
+    constexpr int NB = WT / 32;    // 32 x 32 MFMA tiles per wave and dimension
     __shared__ __attribute__((aligned(16))) float lds_a[2][BM * PITCH];
     __shared__ __attribute__((aligned(16))) float lds_b[2][BN * PITCH];
 
@@ -185,11 +191,11 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     const int it_end = min(total_it, it_begin + per_split);
     if (it_begin >= it_end) return;
 
-    f32x16 acc[2][2];
+    f32x16 acc[NB][NB];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NB; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
@@ -198,10 +204,10 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     // workgroup per compute unit, which is what the benchmark's shapes give, nothing else hides that latency.
     // The loop is unrolled by two so that the sets swap roles without register copies, and its barrier orders
     // LDS only (__syncthreads() would also drain the loads in flight).
-    TileStage<VA, AK> sa0, sa1;
-    TileStage<VB, BK_> sb0, sb1;
+    TileStage<VA, AK, TILE> sa0, sa1;
+    TileStage<VB, BK_, TILE> sb0, sb1;
     const char *mask_pat = MASKED ? args.pat : nullptr;
-    auto fetch = [&](int it, TileStage<VA, AK> &ra, TileStage<VB, BK_> &rb) __attribute__((always_inline)) {
+    auto fetch = [&](int it, TileStage<VA, AK, TILE> &ra, TileStage<VB, BK_, TILE> &rb) __attribute__((always_inline)) {
         const int seg = it / kt_per_seg;
         const int k0 = (it % kt_per_seg) * BK;
         ra.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
@@ -220,25 +226,25 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     const int frag_k = (lane >> 5) * FK;
 
     // one k-iteration on LDS buffer `cur`; `held` carries tile it+1, `recv` receives tile it+2
-    auto iterate = [&](int it, int cur, TileStage<VA, AK> &held_a, TileStage<VB, BK_> &held_b,
-                       TileStage<VA, AK> &recv_a, TileStage<VB, BK_> &recv_b) __attribute__((always_inline)) {
+    auto iterate = [&](int it, int cur, TileStage<VA, AK, TILE> &held_a, TileStage<VB, BK_, TILE> &held_b,
+                       TileStage<VA, AK, TILE> &recv_a, TileStage<VB, BK_, TILE> &recv_b) __attribute__((always_inline)) {
         // always issued (the last iterations refetch the final tile) so that the count of loads in flight is
         // the same on every path
         fetch(min(it + 2, it_end - 1), recv_a, recv_b);
         __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMA block: the scheduler would sink them
 
-        float fa[2][FK], fb[2][FK];
+        float fa[NB][FK], fb[NB][FK];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            TileStage<VA, AK>::fragment(lds_a[cur], wm * 64 + i * 32 + frag_row, frag_k, fa[i]);
-            TileStage<VB, BK_>::fragment(lds_b[cur], wn * 64 + i * 32 + frag_row, frag_k, fb[i]);
+        for (int i = 0; i < NB; ++i) {
+            TileStage<VA, AK, TILE>::fragment(lds_a[cur], wm * WT + i * 32 + frag_row, frag_k, fa[i]);
+            TileStage<VB, BK_, TILE>::fragment(lds_b[cur], wn * WT + i * 32 + frag_row, frag_k, fb[i]);
         }
 #pragma unroll
         for (int kk = 0; kk < FK; ++kk) {
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < NB; ++i) {
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < NB; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][kk], fa[i][kk], acc[i][j], 0, 0, 0);
             }
         }
@@ -258,17 +264,17 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     float *__restrict__ C = pb.C;
     const int half = lane >> 5;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int m = m0 + wm * 64 + i * 32 + frag_row;
+    for (int i = 0; i < NB; ++i) {
+        const int m = m0 + wm * WT + i * 32 + frag_row;
         if (m >= args.m) continue;
         float bterm = 0.0f;
         if (args.epilogue == EPI_BIAS_ACT || args.epilogue == EPI_BIAS_ACT_SKIP)
             bterm = args.bias_scale * pb.bias_vec[m];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < NB; ++j) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int n = n0 + wn * 64 + j * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                const int n = n0 + wn * WT + j * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
                 if (n >= args.n) continue;
                 const size_t idx = (size_t)n * args.ldc + m;
                 float *dst = C + idx;
@@ -311,26 +317,44 @@ inline int pick_vec(const GemmArgs &a, bool for_a) {
     return v;
 }
 
-template <int VA, bool AK, int VB, bool BK_>
+// Tile edge.  128 x 128 tiles give the most MFMA work per byte staged, but a launch that yields only a few of
+// them per compute unit leaves the machine waiting on memory latency (one or two workgroups of four waves per
+// CU) and on the last, partly filled round of workgroups.  Measured on MI355X, 64 x 64 tiles -- four times as
+// many workgroups -- are faster for every product of the benchmark networks (the acoustic model's 512 x 5880
+// error products by 1.4x, the WaveNet layers' K = 64..384 products over 32 000 slots by 2x); the large tile is
+// kept for launches that fill the machine many times over anyway.
+int pick_tile(const GemmArgs &a) {
+    static const int forced = [] { const char *e = std::getenv("CNT_GEMM_TILE"); return e ? std::atoi(e) : 0; }();
+    if (forced == 64 || forced == 128) return forced;
+    const long t128 = (long)((a.m + 127) / 128) * ((a.n + 127) / 128) * a.splitk * a.nprob;
+    return t128 < 2048 ? 64 : 128;
+}
+
+template <int VA, bool AK, int VB, bool BK_, int TILE>
 void launch_m(const GemmArgs &a, dim3 grid, hipStream_t s) {
-    if (a.masked) hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, true>), grid, dim3(NTHREADS), 0, s, a);
-    else hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, false>), grid, dim3(NTHREADS), 0, s, a);
+    if (a.masked) hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, true, TILE>), grid, dim3(NTHREADS), 0, s, a);
+    else hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, false, TILE>), grid, dim3(NTHREADS), 0, s, a);
+}
+template <int VA, bool AK, int VB, bool BK_>
+void launch_t(const GemmArgs &a, dim3 grid, hipStream_t s, int tile) {
+    if (tile == 64) launch_m<VA, AK, VB, BK_, 64>(a, grid, s);
+    else launch_m<VA, AK, VB, BK_, 128>(a, grid, s);
 }
 template <int VA, bool AK, int VB>
-void launch_b(const GemmArgs &a, dim3 grid, hipStream_t s, bool bk) {
-    if (bk) launch_m<VA, AK, VB, true>(a, grid, s);
-    else launch_m<VA, AK, VB, false>(a, grid, s);
+void launch_b(const GemmArgs &a, dim3 grid, hipStream_t s, bool bk, int tile) {
+    if (bk) launch_t<VA, AK, VB, true>(a, grid, s, tile);
+    else launch_t<VA, AK, VB, false>(a, grid, s, tile);
 }
 template <int VA, bool AK>
-void launch_vb(const GemmArgs &a, dim3 grid, hipStream_t s, int vb, bool bk) {
-    if (vb == 4) launch_b<VA, AK, 4>(a, grid, s, bk);
-    else if (vb == 2) launch_b<VA, AK, 2>(a, grid, s, bk);
-    else launch_b<VA, AK, 1>(a, grid, s, bk);
+void launch_vb(const GemmArgs &a, dim3 grid, hipStream_t s, int vb, bool bk, int tile) {
+    if (vb == 4) launch_b<VA, AK, 4>(a, grid, s, bk, tile);
+    else if (vb == 2) launch_b<VA, AK, 2>(a, grid, s, bk, tile);
+    else launch_b<VA, AK, 1>(a, grid, s, bk, tile);
 }
 template <int VA>
-void launch_ak(const GemmArgs &a, dim3 grid, hipStream_t s, bool ak, int vb, bool bk) {
-    if (ak) launch_vb<VA, true>(a, grid, s, vb, bk);
-    else launch_vb<VA, false>(a, grid, s, vb, bk);
+void launch_ak(const GemmArgs &a, dim3 grid, hipStream_t s, bool ak, int vb, bool bk, int tile) {
+    if (ak) launch_vb<VA, true>(a, grid, s, vb, bk, tile);
+    else launch_vb<VA, false>(a, grid, s, vb, bk, tile);
 }
 
 }  // namespace
@@ -350,12 +374,13 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args) {
             CNT_REQUIRE(args.prob[p].A[s] && args.prob[p].B[s], "gemm: null operand");
     }
     const int va = pick_vec(args, true), vb = pick_vec(args, false);
-    const int tiles = ((args.m + BM - 1) / BM) * ((args.n + BN - 1) / BN);
+    const int tile = pick_tile(args);
+    const int tiles = ((args.m + tile - 1) / tile) * ((args.n + tile - 1) / tile);
     dim3 grid(tiles, args.splitk, args.nprob);
     ProfileScope prof(stream, args.label ? args.label : "gemm");
-    if (va == 4) launch_ak<4>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig);
-    else if (va == 2) launch_ak<2>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig);
-    else launch_ak<1>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig);
+    if (va == 4) launch_ak<4>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
+    else if (va == 2) launch_ak<2>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
+    else launch_ak<1>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
