@@ -4,6 +4,8 @@
 // :1060-1101 forward) and layers/SsePostOutputLayer.cu (:94-136, :166-267).
 #include "common.hpp"
 
+#include <algorithm>
+
 namespace cnt {
 namespace {
 
@@ -26,15 +28,31 @@ __global__ void dense_delta_kernel(float *__restrict__ err, const float *__restr
     for (; i < count; i += stride) err[i] = act_deriv(act, y[i]) * err[i];
 }
 
-// out[d] += scale * sum_i v[d + i*D] over a chunk of columns; out is zeroed by the caller
-__global__ void column_sum_kernel(const float *__restrict__ v, int D, int N, int chunk, float scale,
-                                  float *__restrict__ out) {
-    const int d = blockIdx.x * blockDim.x + threadIdx.x;
-    if (d >= D) return;
-    const int i0 = blockIdx.y * chunk, i1 = min(N, i0 + chunk);
-    float acc = 0.0f;
-    for (int i = i0; i < i1; ++i) acc += scale * v[(size_t)i * D + d];
-    atomicAdd(out + d, acc);
+// out[d] += scale * sum_i v[d + i*D]; out is zeroed by the caller.  A block is 64 rows x 4 column lanes (one
+// wave per lane, 256-byte row segments); every lane strides over the columns with eight loads in flight, the
+// four partial sums meet in LDS and leave as one atomic per row and block.  The number of blocks is kept near
+// 512: atomics to one address serialise, and with thousands of blocks they, not the reads, set the run time.
+__global__ __launch_bounds__(256) void column_sum_kernel(const float *__restrict__ v, int D, int N, float scale,
+                                                         float *__restrict__ out) {
+    __shared__ float part[4][64];
+    const int tx = threadIdx.x, ty = threadIdx.y;
+    const int d = blockIdx.x * 64 + tx;
+    const int stride = 4 * gridDim.y;
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+    if (d < D) {
+        int i = blockIdx.y * 4 + ty;
+        for (; i + 7 * stride < N; i += 8 * stride) {
+            float x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) x[u] = v[(size_t)(i + u * stride) * D + d];
+            a0 += scale * x[0]; a1 += scale * x[1]; a2 += scale * x[2]; a3 += scale * x[3];
+            a0 += scale * x[4]; a1 += scale * x[5]; a2 += scale * x[6]; a3 += scale * x[7];
+        }
+        for (; i < N; i += stride) a0 += scale * v[(size_t)i * D + d];
+    }
+    part[ty][tx] = (a0 + a1) + (a2 + a3);
+    __syncthreads();
+    if (ty == 0 && d < D) atomicAdd(out + d, (part[0][tx] + part[1][tx]) + (part[2][tx] + part[3][tx]));
 }
 
 __global__ void sse_backward_kernel(int D, size_t count, const char *__restrict__ pat, const float *__restrict__ y,
@@ -85,9 +103,11 @@ int fill_words(hipStream_t stream, unsigned *p, size_t count, unsigned word) {
 }
 
 int column_sum(hipStream_t stream, const float *v, int D, int N, float scale, float *out) {
-    const int chunk = 64;
-    dim3 grid((D + 255) / 256, (N + chunk - 1) / chunk);
-    hipLaunchKernelGGL(column_sum_kernel, grid, dim3(256), 0, stream, v, D, N, chunk, scale, out);
+    const int gx = (D + 63) / 64;
+    int gy = (N + 31) / 32;  // at least eight columns per lane
+    gy = std::min(gy, std::max(1, 512 / gx));
+    gy = std::max(gy, 1);
+    hipLaunchKernelGGL(column_sum_kernel, dim3(gx, gy), dim3(64, 4), 0, stream, v, D, N, scale, out);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
@@ -156,10 +176,7 @@ int cnt_dense_backward_weights(void *stream_, int P, int D, int N, float bias, c
         ga.b_kcontig = 0; ga.ldb = D;
         ga.ldc = P;
         ga.nseg = 1; ga.nprob = 1; ga.epilogue = EPI_ATOMIC;
-        const int tiles = ((P + 127) / 128) * ((D + 127) / 128);
-        int s = (512 + tiles - 1) / tiles;
-        const int kt = (N + 15) / 16;
-        ga.splitk = s > kt ? kt : s;
+        ga.splitk = 0;  // chosen by the launcher
         ga.prob[0].A[0] = x; ga.prob[0].B[0] = err; ga.prob[0].C = weight_updates;
         ga.label = "gemm:dense_dW";
         CNT_TRY(gemm_launch(stream, ga));

@@ -16,6 +16,7 @@
 // along the column-major output's contiguous dimension and every store is a 128-byte segment.
 #include "common.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 
 namespace cnt {
@@ -359,14 +360,15 @@ void launch_ak(const GemmArgs &a, dim3 grid, hipStream_t s, bool ak, int vb, boo
 
 }  // namespace
 
-int gemm_launch(hipStream_t stream, const GemmArgs &args) {
+int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
+    GemmArgs args = args_in;
     CNT_REQUIRE(args.m > 0 && args.n > 0 && args.k > 0, "gemm: empty problem %d x %d x %d", args.m, args.n,
                 args.k);
     CNT_REQUIRE(args.nseg >= 1 && args.nseg <= kGemmMaxSeg, "gemm: %d operand pairs, supported 1..%d",
                 args.nseg, kGemmMaxSeg);
     CNT_REQUIRE(args.nprob >= 1 && args.nprob <= kGemmMaxProb, "gemm: %d problems, supported 1..%d",
                 args.nprob, kGemmMaxProb);
-    CNT_REQUIRE(args.splitk >= 1 && (args.splitk == 1 || args.epilogue == EPI_ATOMIC),
+    CNT_REQUIRE(args.splitk >= 0 && (args.splitk == 1 || args.epilogue == EPI_ATOMIC),
                 "gemm: split-K needs the atomic epilogue");
     for (int p = 0; p < args.nprob; ++p) {
         CNT_REQUIRE(args.prob[p].C != nullptr, "gemm: null output");
@@ -374,6 +376,17 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args) {
             CNT_REQUIRE(args.prob[p].A[s] && args.prob[p].B[s], "gemm: null operand");
     }
     const int va = pick_vec(args, true), vb = pick_vec(args, false);
+    if (args.splitk == 0) {
+        // Long-K products with a small output (weight gradients): cut K so that the launch has about
+        // `target` workgroups of 64 x 64 tiles, but leave every workgroup at least eight k-iterations -- each
+        // one ends with an atomic add of its whole tile, and those, not the products, dominate short ranges.
+        static const int target = [] { const char *e = std::getenv("CNT_GEMM_SPLIT_TARGET"); return e ? std::atoi(e) : 512; }();
+        const long tiles = (long)((args.m + 63) / 64) * ((args.n + 63) / 64) * args.nprob;
+        const long kt = ((long)args.k + BK - 1) / BK * args.nseg;
+        long s = (target + tiles - 1) / tiles;
+        s = std::min(s, std::max(1L, kt / 8));
+        args.splitk = (int)std::max(1L, s);
+    }
     const int tile = pick_tile(args);
     const int tiles = ((args.m + tile - 1) / tile) * ((args.n + tile - 1) / tile);
     dim3 grid(tiles, args.splitk, args.nprob);

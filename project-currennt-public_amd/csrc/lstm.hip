@@ -1134,13 +1134,6 @@ int cnt_lstm_backward_weights(cnt_lstm *h, void *stream_, const float *x, float 
     CNT_TRY(fill_zero(stream, weight_updates, nW));
     const size_t off_bias = (size_t)4 * P * L, off_int = off_bias + (size_t)4 * L;
     const size_t off_peep = off_int + (size_t)4 * L * H;
-    auto split_for = [](int tiles, int k) {
-        int s = (512 + tiles - 1) / tiles;
-        const int kt = (k + 15) / 16;
-        if (s > kt) s = kt;
-        if (s < 1) s = 1;
-        return s;
-    };
     {
         // input weights: dW_in[g,dir] (P x H) = x (P x N) * delta^T
         GemmArgs ga = {};
@@ -1149,7 +1142,7 @@ int cnt_lstm_backward_weights(cnt_lstm *h, void *stream_, const float *x, float 
         ga.b_kcontig = 0; ga.ldb = H;
         ga.ldc = P;
         ga.nseg = 1; ga.nprob = 4 * h->ndir; ga.epilogue = EPI_ATOMIC;
-        ga.splitk = split_for(((P + 127) / 128) * ((H + 127) / 128) * ga.nprob, N);
+        ga.splitk = 0;  // chosen by the launcher
         for (int dir = 0; dir < h->ndir; ++dir)
             for (int g = 0; g < 4; ++g) {
                 GemmProblem &pb = ga.prob[dir * 4 + g];
@@ -1168,7 +1161,7 @@ int cnt_lstm_backward_weights(cnt_lstm *h, void *stream_, const float *x, float 
         ga.b_kcontig = 0; ga.ldb = H;
         ga.ldc = H;
         ga.nseg = 1; ga.nprob = 4 * h->ndir; ga.epilogue = EPI_ATOMIC;
-        ga.splitk = split_for(((H + 127) / 128) * ((H + 127) / 128) * ga.nprob, N - S);
+        ga.splitk = 0;  // chosen by the launcher
         for (int dir = 0; dir < h->ndir; ++dir)
             for (int g = 0; g < 4; ++g) {
                 GemmProblem &pb = ga.prob[dir * 4 + g];

@@ -316,10 +316,7 @@ int cnt_cnn_backward(cnt_cnn *h, void *stream_, const char *patTypes, int curT, 
             ga.prob[pr].C = weight_updates + (size_t)(g.col0 + g.hw + shift) * P;
         }
         ga.nprob = pr;
-        const int tiles = ((P + 127) / 128) * ((ga.n + 127) / 128) * pr;
-        int s = (512 + tiles - 1) / tiles;
-        const int kt = (N + 15) / 16;
-        ga.splitk = s > kt ? kt : s;
+        ga.splitk = 0;  // chosen by the launcher
         ga.label = "gemm:cnn_dW";
         CNT_TRY(gemm_launch(stream, ga));
     }
@@ -423,10 +420,7 @@ int cnt_wavnetc_backward(void *stream_, int D, int C, int N, const char *patType
         ga.b_kcontig = 0; ga.ldb = 2 * D;
         ga.ldc = C;
         ga.nseg = 1; ga.nprob = 1; ga.epilogue = EPI_ATOMIC;
-        const int tiles = ((C + 127) / 128) * ((2 * D + 127) / 128);
-        int s = (512 + tiles - 1) / tiles;
-        const int kt = (N + 15) / 16;
-        ga.splitk = s > kt ? kt : s;
+        ga.splitk = 0;  // chosen by the launcher
         ga.prob[0].A[0] = ctx; ga.prob[0].B[0] = ctx_tanh; ga.prob[0].C = weight_updates;
         ga.label = "gemm:wavnetc_dW";
         CNT_TRY(gemm_launch(stream, ga));
