@@ -48,6 +48,10 @@ def test_sse():
     (48, 512, True, [16, 9, 13, 16, 16, 5, 16, 12, 10, 16]),
     (33, 256, True, [1]),
     (33, 128, False, [6] * 20),
+    (32, 512, False, [8, 8, 5, 8]),        # 512 cells per direction: the largest recursion kernel
+    (32, 1024, True, [7, 5, 7]),
+    (20, 256, False, [5] * 24),            # more than 16 parallel sequences with 256 cells
+    (16, 128, True, [1, 1]),               # a single time step, two sequences
 ])
 def test_lstm(P, L, bidir, lengths):
     print("lstm case", P, L, bidir, lengths, flush=True)
