@@ -14,291 +14,13 @@
 // costs a 16-way LDS bank conflict.
 // The MFMA operands are swapped (the B tile feeds the instruction's A port) so that lane%32 walks
 // along the column-major output's contiguous dimension and every store is a 128-byte segment.
-#include "common.hpp"
+#include "gemm_kernel.hpp"
 
 #include <algorithm>
 #include <cstdlib>
 
 namespace cnt {
 namespace {
-
-constexpr int BK = 16;  // the tile edge (rows of A = columns of B per workgroup) is a template parameter: 128 or 64
-constexpr int PITCH = BK + 4;
-constexpr int NTHREADS = 256;
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-// workgroup barrier that orders LDS traffic only; global loads issued before it stay in flight
-__device__ __forceinline__ void lds_only_barrier() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-template <int V>
-struct VecT;
-template <>
-struct VecT<1> { typedef float type; };
-template <>
-struct VecT<2> { typedef float2 type; };
-template <>
-struct VecT<4> { typedef float4 type; };
-
-// Stages one ROWS-row x 16-k operand tile: global -> registers -> LDS.
-template <int VEC, bool KCONTIG, int ROWS>
-struct TileStage {
-    static constexpr int NLOAD = (ROWS * BK) / (NTHREADS * VEC);
-    static_assert(NLOAD >= 1, "tile too small for this vector width");
-    typename VecT<VEC>::type r[NLOAD];
-
-    // shift / pat / n_slots: masked mode (pat == nullptr switches it off); time_on_k selects which index is
-    // the time slot
-    __device__ __forceinline__ void load(const float *__restrict__ base, int ld, int row0, int k0,
-                                         int rows_total, int k_total, int tid, const char *__restrict__ pat = nullptr,
-                                         int shift = 0, int n_slots = 0, bool time_on_k = false) {
-        if (KCONTIG) {
-            constexpr int TPR = BK / VEC;        // threads per row
-            constexpr int RPP = NTHREADS / TPR;  // rows per pass
-            const int kq = (tid % TPR) * VEC;
-            const int rr = tid / TPR;
-#pragma unroll
-            for (int p = 0; p < NLOAD; ++p) {
-                const int row = row0 + rr + p * RPP;
-                typename VecT<VEC>::type v = {};
-                if (!pat) {
-                    // branch-free: the load always executes (on a clamped address) and is zeroed afterwards, so
-                    // that the number of loads in flight is the same on every path and the compiler can wait for
-                    // the tile of the next iteration while the one after it stays in flight
-                    const bool inside = row < rows_total && (k0 + kq) < k_total;
-                    const int rc = min(row, rows_total - 1), kc = (k0 + kq) < k_total ? k0 + kq : 0;
-                    v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)rc * ld + kc);
-                    if (!inside) v = typename VecT<VEC>::type{};
-                } else if (row < rows_total && (k0 + kq) < k_total) {
-                    if (!time_on_k) {
-                        const int src = row + shift;
-                        if (pat[row] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
-                            v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)src * ld + k0 + kq);
-                    } else {
-                        // vector along k = consecutive time slots: element-wise masking
-                        float *e = reinterpret_cast<float *>(&v);
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) {
-                            const int u = k0 + kq + j, src = u + shift;
-                            if (pat[u] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
-                                e[j] = base[(size_t)row * ld + src];
-                        }
-                    }
-                }
-                r[p] = v;
-            }
-        } else {
-            constexpr int TPK = ROWS / VEC;      // threads per k line
-            constexpr int KPP = NTHREADS / TPK;  // k lines per pass
-            const int rq = (tid % TPK) * VEC;
-            const int kk = tid / TPK;
-#pragma unroll
-            for (int p = 0; p < NLOAD; ++p) {
-                const int k = k0 + kk + p * KPP;
-                typename VecT<VEC>::type v = {};
-                if (!pat) {
-                    const bool inside = k < k_total && (row0 + rq) < rows_total;
-                    const int kc = min(k, k_total - 1), rc = (row0 + rq) < rows_total ? row0 + rq : 0;
-                    v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)kc * ld + rc);
-                    if (!inside) v = typename VecT<VEC>::type{};
-                } else if (k < k_total && (row0 + rq) < rows_total) {
-                    if (time_on_k) {
-                        const int src = k + shift;
-                        if (pat[k] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
-                            v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)src * ld + row0 + rq);
-                    } else {
-                        float *e = reinterpret_cast<float *>(&v);
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) {
-                            const int u = row0 + rq + j, src = u + shift;
-                            if (pat[u] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
-                                e[j] = base[(size_t)k * ld + src];
-                        }
-                    }
-                }
-                r[p] = v;
-            }
-        }
-    }
-
-    // k values [k_first, k_first + BK/2) of tile row `row`, in MFMA issue order
-    static __device__ __forceinline__ void fragment(const float *__restrict__ lds, int row, int k_first,
-                                                    float (&f)[BK / 2]) {
-        if (KCONTIG) {
-            const float *p = lds + row * PITCH + k_first;
-#pragma unroll
-            for (int q = 0; q < BK / 8; ++q) {
-                const float4 v = *reinterpret_cast<const float4 *>(p + 4 * q);
-                f[4 * q] = v.x; f[4 * q + 1] = v.y; f[4 * q + 2] = v.z; f[4 * q + 3] = v.w;
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < BK / 2; ++q) f[q] = lds[(k_first + q) * ROWS + row];
-        }
-    }
-
-    __device__ __forceinline__ void store(float *__restrict__ lds, int tid) const {
-        if (KCONTIG) {
-            constexpr int TPR = BK / VEC;
-            constexpr int RPP = NTHREADS / TPR;
-            const int kq = (tid % TPR) * VEC;
-            const int rr = tid / TPR;
-#pragma unroll
-            for (int p = 0; p < NLOAD; ++p)
-                *reinterpret_cast<typename VecT<VEC>::type *>(lds + (rr + p * RPP) * PITCH + kq) = r[p];
-        } else {
-            constexpr int TPK = ROWS / VEC;
-            constexpr int KPP = NTHREADS / TPK;
-            const int rq = (tid % TPK) * VEC;
-            const int kk = tid / TPK;
-#pragma unroll
-            for (int p = 0; p < NLOAD; ++p)
-                *reinterpret_cast<typename VecT<VEC>::type *>(lds + (kk + p * KPP) * ROWS + rq) = r[p];
-        }
-    }
-};
-
-// MASKED selects the time-shifted, padding-masked B loader at compile time: its per-element predication is a lot
-// of code, and four copies of it (two prologue fetches, two in the unrolled loop) inside the plain kernels would
-// push their hot loop out of the instruction cache.
-template <int VA, bool AK, int VB, bool BK_, bool MASKED, int TILE>
-__global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args) {
-    constexpr int BM = TILE, BN = TILE;
-    constexpr int WT = TILE / 2;   // edge of a wave's block (waves are arranged 2 x 2)
-    constexpr int NB = WT / 32;    // 32 x 32 MFMA tiles per wave and dimension
-    __shared__ __attribute__((aligned(16))) float lds_a[2][BM * PITCH];
-    __shared__ __attribute__((aligned(16))) float lds_b[2][BN * PITCH];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int wm = wave & 1, wn = wave >> 1;
-
-    const int tiles_m = (args.m + BM - 1) / BM;
-    const int tile = blockIdx.x;
-    const int m0 = (tile % tiles_m) * BM;
-    const int n0 = (tile / tiles_m) * BN;
-    const GemmProblem &pb = args.prob[blockIdx.z];
-
-    // iteration space: segments x k-tiles, cut into splitk contiguous ranges
-    const int kt_per_seg = (args.k + BK - 1) / BK;
-    const int total_it = kt_per_seg * args.nseg;
-    const int per_split = (total_it + args.splitk - 1) / args.splitk;
-    const int it_begin = blockIdx.y * per_split;
-    const int it_end = min(total_it, it_begin + per_split);
-    if (it_begin >= it_end) return;
-
-    f32x16 acc[NB][NB];
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < NB; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-    // Two register sets per operand: tile it+1 waits in one of them while tile it+2 is being fetched into the
-    // other, so that a global load has two k-iterations of MFMA work (about 4000 clocks) to arrive in; with one
-    // workgroup per compute unit, which is what the benchmark's shapes give, nothing else hides that latency.
-    // The loop is unrolled by two so that the sets swap roles without register copies, and its barrier orders
-    // LDS only (__syncthreads() would also drain the loads in flight).
-    TileStage<VA, AK, TILE> sa0, sa1;
-    TileStage<VB, BK_, TILE> sb0, sb1;
-    const char *mask_pat = MASKED ? args.pat : nullptr;
-    auto fetch = [&](int it, TileStage<VA, AK, TILE> &ra, TileStage<VB, BK_, TILE> &rb) __attribute__((always_inline)) {
-        const int seg = it / kt_per_seg;
-        const int k0 = (it % kt_per_seg) * BK;
-        ra.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
-        rb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid, mask_pat, pb.b_shift[seg], args.n_slots,
-                args.b_time_on_k != 0);
-    };
-
-    fetch(it_begin, sa0, sb0);
-    fetch(min(it_begin + 1, it_end - 1), sa1, sb1);
-    sa0.store(lds_a[0], tid);
-    sb0.store(lds_b[0], tid);
-    lds_only_barrier();
-
-    const int frag_row = lane & 31;
-    constexpr int FK = BK / 2;  // k values per half-wave and tile
-    const int frag_k = (lane >> 5) * FK;
-
-    // one k-iteration on LDS buffer `cur`; `held` carries tile it+1, `recv` receives tile it+2
-    auto iterate = [&](int it, int cur, TileStage<VA, AK, TILE> &held_a, TileStage<VB, BK_, TILE> &held_b,
-                       TileStage<VA, AK, TILE> &recv_a, TileStage<VB, BK_, TILE> &recv_b) __attribute__((always_inline)) {
-        // always issued (the last iterations refetch the final tile) so that the count of loads in flight is
-        // the same on every path
-        fetch(min(it + 2, it_end - 1), recv_a, recv_b);
-        __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMA block: the scheduler would sink them
-
-        float fa[NB][FK], fb[NB][FK];
-#pragma unroll
-        for (int i = 0; i < NB; ++i) {
-            TileStage<VA, AK, TILE>::fragment(lds_a[cur], wm * WT + i * 32 + frag_row, frag_k, fa[i]);
-            TileStage<VB, BK_, TILE>::fragment(lds_b[cur], wn * WT + i * 32 + frag_row, frag_k, fb[i]);
-        }
-#pragma unroll
-        for (int kk = 0; kk < FK; ++kk) {
-#pragma unroll
-            for (int i = 0; i < NB; ++i) {
-#pragma unroll
-                for (int j = 0; j < NB; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][kk], fa[i][kk], acc[i][j], 0, 0, 0);
-            }
-        }
-
-        if (it + 1 < it_end) {
-            held_a.store(lds_a[cur ^ 1], tid);
-            held_b.store(lds_b[cur ^ 1], tid);
-        }
-        lds_only_barrier();
-    };
-    for (int it = it_begin; it < it_end; it += 2) {
-        iterate(it, 0, sa1, sb1, sa0, sb0);
-        if (it + 1 < it_end) iterate(it + 1, 1, sa0, sb0, sa1, sb1);
-    }
-
-    // epilogue: lane%32 runs along m (contiguous), the 16 accumulators along n
-    float *__restrict__ C = pb.C;
-    const int half = lane >> 5;
-#pragma unroll
-    for (int i = 0; i < NB; ++i) {
-        const int m = m0 + wm * WT + i * 32 + frag_row;
-        if (m >= args.m) continue;
-        float bterm = 0.0f;
-        if (args.epilogue == EPI_BIAS_ACT || args.epilogue == EPI_BIAS_ACT_SKIP)
-            bterm = args.bias_scale * pb.bias_vec[m];
-#pragma unroll
-        for (int j = 0; j < NB; ++j) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int n = n0 + wn * WT + j * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (n >= args.n) continue;
-                const size_t idx = (size_t)n * args.ldc + m;
-                float *dst = C + idx;
-                const float v = acc[i][j][r];
-                switch (args.epilogue) {
-                    case EPI_STORE: *dst = v; break;
-                    case EPI_ADD: *dst = *dst + v; break;
-                    case EPI_ATOMIC: atomicAdd(dst, v); break;
-                    case EPI_BIAS_ACT: *dst = act_fn(args.act, v + bterm); break;
-                    case EPI_BIAS_ACT_SKIP:
-                        if (args.pat[n] != 0) *dst = act_fn(args.act, v + bterm);
-                        break;
-                    default: {  // EPI_CONTEXT
-                        const bool valid = args.pat[n] != 0;
-                        const float th = valid ? tanh_act(v) : 0.0f;
-                        if (pb.aux_out) pb.aux_out[idx] = th;
-                        *dst = valid ? pb.aux_in[idx] + th : 0.0f;
-                    } break;
-                }
-            }
-        }
-    }
-}
 
 inline int pick_vec(const GemmArgs &a, bool for_a) {
     const int ld = for_a ? a.lda : a.ldb;
@@ -329,33 +51,6 @@ int pick_tile(const GemmArgs &a) {
     if (forced == 64 || forced == 128) return forced;
     const long t128 = (long)((a.m + 127) / 128) * ((a.n + 127) / 128) * a.splitk * a.nprob;
     return t128 < 2048 ? 64 : 128;
-}
-
-template <int VA, bool AK, int VB, bool BK_, int TILE>
-void launch_m(const GemmArgs &a, dim3 grid, hipStream_t s) {
-    if (a.masked) hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, true, TILE>), grid, dim3(NTHREADS), 0, s, a);
-    else hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, false, TILE>), grid, dim3(NTHREADS), 0, s, a);
-}
-template <int VA, bool AK, int VB, bool BK_>
-void launch_t(const GemmArgs &a, dim3 grid, hipStream_t s, int tile) {
-    if (tile == 64) launch_m<VA, AK, VB, BK_, 64>(a, grid, s);
-    else launch_m<VA, AK, VB, BK_, 128>(a, grid, s);
-}
-template <int VA, bool AK, int VB>
-void launch_b(const GemmArgs &a, dim3 grid, hipStream_t s, bool bk, int tile) {
-    if (bk) launch_t<VA, AK, VB, true>(a, grid, s, tile);
-    else launch_t<VA, AK, VB, false>(a, grid, s, tile);
-}
-template <int VA, bool AK>
-void launch_vb(const GemmArgs &a, dim3 grid, hipStream_t s, int vb, bool bk, int tile) {
-    if (vb == 4) launch_b<VA, AK, 4>(a, grid, s, bk, tile);
-    else if (vb == 2) launch_b<VA, AK, 2>(a, grid, s, bk, tile);
-    else launch_b<VA, AK, 1>(a, grid, s, bk, tile);
-}
-template <int VA>
-void launch_ak(const GemmArgs &a, dim3 grid, hipStream_t s, bool ak, int vb, bool bk, int tile) {
-    if (ak) launch_vb<VA, true>(a, grid, s, vb, bk, tile);
-    else launch_vb<VA, false>(a, grid, s, vb, bk, tile);
 }
 
 }  // namespace
@@ -391,9 +86,10 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
     const int tiles = ((args.m + tile - 1) / tile) * ((args.n + tile - 1) / tile);
     dim3 grid(tiles, args.splitk, args.nprob);
     ProfileScope prof(stream, args.label ? args.label : "gemm");
-    if (va == 4) launch_ak<4>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
-    else if (va == 2) launch_ak<2>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
-    else launch_ak<1>(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
+    if (va == 4) gemm_dispatch_va4(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
+    else if (va == 2) gemm_dispatch_va2(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
+    else if (args.a_kcontig) gemm_dispatch_va1k(args, grid, stream, vb, args.b_kcontig, tile);
+    else gemm_dispatch_va1r(args, grid, stream, vb, args.b_kcontig, tile);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
