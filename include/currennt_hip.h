@@ -115,9 +115,20 @@ int cnt_lstm_backward(cnt_lstm *h, void *stream, const float *weights, const flo
 int cnt_lstm_backward_errors(cnt_lstm *h, void *stream, const float *weights, float *output_errors,
                              float *prev_errors);
 int cnt_lstm_backward_weights(cnt_lstm *h, void *stream, const float *x, float *weight_updates);
+/* The product at the end of the first half on its own (layers/LstmLayer.cu:2298-2334): prev_errors =
+ * sum over gates and directions of W_in * delta.  cnt_lstm_backward_errors with prev_errors == NULL runs only the
+ * recursion; a caller can then start cnt_lstm_backward_weights on another stream as soon as the recursion is
+ * done and compute the preceding layer's errors meanwhile. */
+int cnt_lstm_backward_prev_errors(cnt_lstm *h, void *stream, const float *weights, float *prev_errors);
 /* Device pointer to one internal buffer.  dir: 0 forward, 1 backward states.  which:
  * 0 niActs 1 igActs 2 fgActs 3 ogActs 4 cellStates 5 tmpOutputs 6 tmpOutputErrors
  * 7 niDeltas 8 igDeltas 9 fgDeltas 10 ogDeltas 11 cellStateErrors.  NULL if out of range. */
+/* Bounds of the recursion kernels' waits (no counterpart in the reference, which has no inter-workgroup waits):
+ * spin_limit = poll rounds a workgroup tries before it gives up and stops the whole recursion (default 2^22;
+ * the failure surfaces at cnt_lstm_check); poll_delay_* = pause before the first poll of a step in units of 64
+ * clocks.  Defaults come from the geometry (and CNT_LSTM_SPIN_LIMIT / CNT_LSTM_POLL_DELAY[_FWD]).  A tiny
+ * spin_limit lets a test exercise the give-up path without any kernel hanging. */
+int cnt_lstm_set_wait_bounds(cnt_lstm *h, unsigned spin_limit, int poll_delay_backward, int poll_delay_forward);
 float *cnt_lstm_state(cnt_lstm *h, int dir, int which);
 long cnt_lstm_weight_count(int P, int L, int bidir);
 /* Waits for the stream and reports whether a recursion kernel of this handle gave up waiting for a

@@ -75,6 +75,8 @@ _SIGNATURES = {
     "cnt_lstm_backward": (I, [VP, VP, VP, VP, VP, VP, VP, VP]),
     "cnt_lstm_backward_errors": (I, [VP, VP, VP, VP, VP]),
     "cnt_lstm_backward_weights": (I, [VP, VP, VP, VP]),
+    "cnt_lstm_backward_prev_errors": (I, [VP, VP, VP, VP]),
+    "cnt_lstm_set_wait_bounds": (I, [VP, C.c_uint, I, I]),
     "cnt_lstm_state": (VP, [VP, I, I]),
     "cnt_lstm_weight_count": (C.c_long, [I, I, I]),
     "cnt_lstm_check": (I, [VP, VP]),
@@ -302,6 +304,12 @@ class Lstm:
 
     def backward_weights(self, x, dW, stream=None):
         check(lib().cnt_lstm_backward_weights(self.handle, stream_ptr(stream), ptr(x), ptr(dW)))
+
+    def set_wait_bounds(self, spin_limit, poll_delay_backward, poll_delay_forward):
+        check(lib().cnt_lstm_set_wait_bounds(self.handle, spin_limit, poll_delay_backward, poll_delay_forward))
+
+    def backward_prev_errors(self, W, prev_err, stream=None):
+        check(lib().cnt_lstm_backward_prev_errors(self.handle, stream_ptr(stream), ptr(W), ptr(prev_err)))
 
     def check(self, stream=None):
         check(lib().cnt_lstm_check(self.handle, stream_ptr(stream)))

@@ -843,6 +843,7 @@ struct cnt_lstm {
     long long *phase_ticks;  // diagnostic buffer, allocated when CNT_LSTM_TIMING is set
     int poll_delay, poll_gap, poll_delay_fwd;
     int last_was_forward;  // which recursion the diagnostic buffer describes
+    int bmail_dirty;       // the backward mailbox may hold words that are not empty
 };
 
 namespace cnt {
@@ -903,11 +904,14 @@ void fill_chain_params(const cnt_lstm *h, const float *weights, ChainParams &p) 
 int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     chain_kernel_t k = pick_kernel(fwd, h->H, h->JB, h->NT);
     CNT_REQUIRE(k != nullptr, "lstm: no recursion kernel for H=%d JB=%d S=%d", h->H, h->JB, h->desc.S);
-    // every word of the mailbox starts out empty
+    // Every word of the mailbox starts out empty.  The forward recursion leaves its last outputs behind; the
+    // backward recursion hands every word back, so its mailbox only needs the fill once and again after a
+    // recursion that gave up (cnt_lstm_check marks it dirty).
     for (int dir = 0; dir < h->ndir; ++dir) {
         if (fwd) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->fmail[dir]), h->fmail_words, kEmpty));
-        else CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->bmail[dir]), h->bmail_words, kEmpty));
+        else if (h->bmail_dirty) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->bmail[dir]), h->bmail_words, kEmpty));
     }
+    if (!fwd) h->bmail_dirty = 0;
     const int G = h->H / h->JB;
     p.xcd_pack = fwd ? h->xcd_pack : 0;
     const int blocks = p.xcd_pack ? 8 * G : h->ndir * G;
@@ -944,6 +948,7 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     CNT_REQUIRE(h != nullptr, "lstm_create: out of host memory");
     std::memset(h, 0, sizeof(*h));
     h->desc = *desc; h->ndir = ndir; h->H = H; h->JB = JB; h->NT = NT;
+    h->bmail_dirty = 1;
     h->spin_limit = 1u << 22;
     if (const char *e = std::getenv("CNT_LSTM_SPIN_LIMIT")) h->spin_limit = (unsigned)std::strtoul(e, nullptr, 10);
     h->xcd_pack = 0;
@@ -1011,6 +1016,17 @@ int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int
     return CNT_OK;
 }
 
+int cnt_lstm_set_wait_bounds(cnt_lstm *h, unsigned spin_limit, int poll_delay_backward, int poll_delay_forward) {
+    using namespace cnt;
+    CNT_REQUIRE(h, "lstm_set_wait_bounds: null handle");
+    CNT_REQUIRE(poll_delay_backward >= 0 && poll_delay_backward <= 4096 && poll_delay_forward >= 0 &&
+                poll_delay_forward <= 4096, "lstm_set_wait_bounds: poll delays must be within 0..4096");
+    h->spin_limit = spin_limit;
+    h->poll_delay = poll_delay_backward;
+    h->poll_delay_fwd = poll_delay_forward;
+    return CNT_OK;
+}
+
 float *cnt_lstm_state(cnt_lstm *h, int dir, int which) {
     if (!h || dir < 0 || dir >= h->ndir || which < 0 || which >= 12) return nullptr;
     return h->state[dir][which];
@@ -1045,6 +1061,7 @@ int cnt_lstm_check(cnt_lstm *h, void *stream) {
                          m[0] * us, m[1] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, m[2] * us, m[5] * us, h->T, active);
     }
     if (flag != 0) {
+        h->bmail_dirty = 1;
         CNT_HIP(hipMemset(h->abort_flag, 0, sizeof(int)));
         set_error("lstm: a recursion kernel gave up waiting for a neighbouring workgroup; results are invalid");
         return CNT_ERR_DEVICE;
@@ -1091,8 +1108,6 @@ int cnt_lstm_backward_errors(cnt_lstm *h, void *stream_, const float *weights, f
     CNT_REQUIRE(h && weights && output_errors, "lstm_backward_errors: null argument");
     CNT_REQUIRE(h->T > 0, "lstm_backward_errors: load_sequences has not been called");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    const cnt_lstm_desc &d = h->desc;
-    const int P = d.P, L = d.L, H = h->H, S = d.S, N = h->T * S;
 
     // 1. error recursion (splits the interleaved output errors on the fly)
     ChainParams p;
@@ -1101,8 +1116,20 @@ int cnt_lstm_backward_errors(cnt_lstm *h, void *stream_, const float *weights, f
     p.herr_out = (h->ndir == 1) ? output_errors : nullptr;
     CNT_TRY(launch_chain(h, stream, false, p));
 
-    // 2. error to the preceding layer: e_x = sum_{dir,g} W_in[g,dir] * delta[g,dir]  (overwrite)
-    if (prev_errors) {
+    // 2. error to the preceding layer
+    if (prev_errors) return cnt_lstm_backward_prev_errors(h, stream_, weights, prev_errors);
+    return CNT_OK;
+}
+
+int cnt_lstm_backward_prev_errors(cnt_lstm *h, void *stream_, const float *weights, float *prev_errors) {
+    using namespace cnt;
+    CNT_REQUIRE(h && weights && prev_errors, "lstm_backward_prev_errors: null argument");
+    CNT_REQUIRE(h->T > 0, "lstm_backward_prev_errors: load_sequences has not been called");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const cnt_lstm_desc &d = h->desc;
+    const int P = d.P, L = d.L, H = h->H, S = d.S, N = h->T * S;
+    // e_x = sum_{dir,g} W_in[g,dir] * delta[g,dir]  (overwrite)
+    {
         GemmArgs ga = {};
         ga.m = P; ga.n = N; ga.k = H;
         ga.a_kcontig = 0; ga.lda = P;

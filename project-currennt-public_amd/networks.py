@@ -124,6 +124,9 @@ class StackedNetwork:
                                            prev_err)
             else:
                 L["handle"].backward_errors(L["weights"], L["errors"], prev_err)
+            # The weight gradients wait for the error product above as well: started right after the recursion
+            # (cnt_lstm_backward_prev_errors allows that) the two products share the machine and the one on the
+            # critical path takes 1.5x as long -- measured slower overall.
             ev = torch.cuda.Event()
             ev.record(main)
             side_stream.wait_event(ev)

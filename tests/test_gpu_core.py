@@ -72,6 +72,52 @@ def test_lstm_config1_unidirectional():
     assert PC.run_lstm_case(382, 256, False, [200, 200, 200, 150], seed=1) < TOL
 
 
+def test_lstm_gives_up_cleanly_and_recovers():
+    """Failure handling, forced from the host: with a spin limit of zero and no pause before the first poll a
+    workgroup gives up the moment a neighbour's data is not there yet; every workgroup then drains, the kernels
+    end normally, cnt_lstm_check reports the failure, and the same handle works again afterwards."""
+    import numpy as np
+    import torch
+
+    print("lstm give-up case", flush=True)
+    capi = PC.pkg().capi
+    P, L, S, T = 24, 512, 6, 40
+    rng = np.random.default_rng(3)
+    W = torch.from_numpy(rng.uniform(-0.1, 0.1, capi.lib().cnt_lstm_weight_count(P, L, 1)).astype(np.float32)).cuda()
+    x = torch.from_numpy(rng.standard_normal(P * T * S).astype(np.float32)).cuda()
+    pat = torch.full((T * S,), 2, dtype=torch.int8, device="cuda")
+    out = torch.zeros(L * T * S, device="cuda"); err = torch.ones(L * T * S, device="cuda") * 0.01
+    ex = torch.zeros(P * T * S, device="cuda"); dW = torch.zeros_like(W)
+    layer = capi.Lstm(P, L, True, S, T)
+    layer.load_sequences(pat, T, T)
+    layer.forward(W, x, out)
+    layer.backward(W, x, out, err.clone(), ex, dW)
+    layer.check()
+    good_out, good_ex, good_dW = out.clone(), ex.clone(), dW.clone()
+    layer.set_wait_bounds(0, 0, 0)
+    failures = 0
+    for _ in range(3):  # an attempt only fails if some poll really comes back incomplete
+        layer.load_sequences(pat, T, T)
+        layer.forward(W, x, out)
+        layer.backward(W, x, out, err.clone(), ex, dW)
+        try:
+            layer.check()
+        except RuntimeError as e:
+            assert "gave up" in str(e)
+            failures += 1
+    assert failures >= 1
+    layer.set_wait_bounds(1 << 22, 28, 34)
+    layer.load_sequences(pat, T, T)
+    layer.forward(W, x, out)
+    layer.backward(W, x, out, err.clone(), ex, dW)
+    layer.check()
+    torch.cuda.synchronize()
+    assert PC.relerr(out.cpu().numpy(), good_out.cpu().numpy()) < 1e-6
+    assert PC.relerr(ex.cpu().numpy(), good_ex.cpu().numpy()) < 1e-6
+    assert PC.relerr(dW.cpu().numpy(), good_dW.cpu().numpy()) < 1e-5   # atomic accumulation order differs
+    layer.close()
+
+
 def test_lstm_unsupported_geometry_is_an_error():
     capi = PC.pkg().capi
     with pytest.raises(RuntimeError):
