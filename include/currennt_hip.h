@@ -137,12 +137,15 @@ long cnt_lstm_weight_count(int P, int L, int bidir);
 int cnt_lstm_check(cnt_lstm *h, void *stream);
 
 /* ---- mixture-density post-output layer ----------------------------------------------------------
- * MDNLayer<TDevice> with MDNUnit_softmax (flat) and MDNUnit_mixture (untied variance) units
+ * MDNLayer<TDevice> with MDNUnit_sigmoid, MDNUnit_softmax (flat) and MDNUnit_mixture (untied variance) units
  * (layers/MDNLayer.cu, layers/MDNUnit.cu).  The handle owns what the units keep between calls: the
  * distribution parameters (m_paraVec) and the per-mixture log-likelihoods and log-sums (m_tmpPat).
  * `config` is the content of the reference's binary mdn config: [n, (startD, endD, startDOut, endDOut,
- * type) x n] as floats (layers/MDNLayer.cu:286-324); type -1 = softmax, > 0 = number of Gaussians
- * (layers/MDNLayer.hpp:35-36).  Other unit types and tied variances are rejected. */
+ * type) x n] as floats (layers/MDNLayer.cu:286-324); type 0 = sigmoid (one target per column), -1 = softmax,
+ * > 0 = number of Gaussians (layers/MDNLayer.hpp:35-36).  Other unit types and tied variances are rejected.
+ * cnt_mdn_calculate_error adds up the units' errors as the reference does: the mixture and softmax units
+ * contribute their summed negative log-likelihood, a sigmoid unit its cross entropy divided by the number
+ * of non-padding frames (layers/MDNUnit.cu:3821). */
 typedef struct cnt_mdn cnt_mdn;
 
 typedef struct {
@@ -151,6 +154,7 @@ typedef struct {
     int S;             /* parallel sequences                                 */
     int maxT;          /* maxSeqLength                                       */
     int tie_variance;  /* --tieVariance; only 0 is supported                 */
+    int sigmoid_continuous; /* sigmoid units: targets are probabilities (the layer's conValSig flag, MDNLayer.cu:466) */
 } cnt_mdn_desc;
 
 /* MDNLayer::MDNLayer (layers/MDNLayer.cu:280-324, 457-545). */

@@ -113,6 +113,13 @@ float orc_dft_logamp_loss(int fft_length, int frame_length, int frame_shift, int
                           int length, float gamma, float log_floor, const float *source, const float *target,
                           float *grad);
 
+/* MDN sigmoid unit (layers/MDNUnit.cu:198-225, 539-676, 3553-3856): K columns, one target per column */
+void orc_sigmoid_forward(int F, int Lp, int startD, int K, const char *pat, const float *x, float *prob);
+float orc_sigmoid_error(int F, int Lt, int startDOut, int K, int continuous, const char *pat, const float *target,
+                        const float *prob);
+void orc_sigmoid_backward(int F, int Lp, int Lt, int startD, int startDOut, int K, int continuous, const char *pat,
+                          const float *target, const float *prob, float *errors);
+
 /* weight update of the training loop (optimizers/Optimizer.cu:186-198, optimizers/SteepestDescentOptimizer.cu) */
 void orc_opt_accumulate(long n, const float *layer_updates, float *cur_updates, int add);
 void orc_opt_adjust_gradient(int option, long n, float *g, float *stats, const float *mask, float frac_length,

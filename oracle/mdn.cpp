@@ -179,4 +179,49 @@ void orc_softmax_backward(int F, int Lp, int Lt, int startD, int startDOut, int 
     }
 }
 
+// ---- sigmoid unit (layers/MDNUnit.cu:198-225 ComputeSigmoid, :563-596 ComputeSigmoidError, :539-551 FrameNum,
+// :634-676 ComputeSigmoidBP, drivers :3553-3588, :3729-3823, :3825-3856).  K = endD - startD columns, one target
+// per column.  The error is the summed binary cross entropy divided by the number of non-padding frames (the
+// gradient is not divided); continuous = the unit's conValSig flag.
+void orc_sigmoid_forward(int F, int Lp, int startD, int K, const char *pat, const float *x, float *prob) {
+    for (int f = 0; f < F; ++f)
+        for (int k = 0; k < K; ++k)
+            prob[(size_t)f * K + k] = pat[f] == orc::PAT_NONE ? 0.0f : orc::logistic(x[(size_t)f * Lp + startD + k]);
+}
+
+float orc_sigmoid_error(int F, int Lt, int startDOut, int K, int continuous, const char *pat, const float *target,
+                        const float *prob) {
+    float likelihood = 0.0f, num = 0.0f;
+    for (int f = 0; f < F; ++f) {
+        if (pat[f] == orc::PAT_NONE) continue;
+        num += 1.0f;
+        for (int k = 0; k < K; ++k) {
+            const float p = prob[(size_t)f * K + k], pr = (float)(1.0 - p);
+            const float d = target[(size_t)f * Lt + startDOut + k];
+            float v;
+            if (continuous) {
+                const float p1 = std::log(p > orc::Lim::kMin ? p : orc::Lim::kMin);
+                const float p2 = std::log(pr > orc::Lim::kMin ? pr : orc::Lim::kMin);
+                v = (float)(-1.0 * d * p1 - (1 - d) * p2);
+            } else {
+                const float b = d > 0 ? p : 1 - p;
+                v = (float)(-1.0 * std::log(b > orc::Lim::kMin ? b : orc::Lim::kMin));
+            }
+            likelihood += v;
+        }
+    }
+    return likelihood / num;
+}
+
+void orc_sigmoid_backward(int F, int Lp, int Lt, int startD, int startDOut, int K, int continuous, const char *pat,
+                          const float *target, const float *prob, float *errors) {
+    for (int f = 0; f < F; ++f)
+        for (int k = 0; k < K; ++k) {
+            float &e = errors[(size_t)f * Lp + startD + k];
+            if (pat[f] == orc::PAT_NONE) { e = 0.0f; continue; }
+            const float p = prob[(size_t)f * K + k], d = target[(size_t)f * Lt + startDOut + k];
+            e = continuous ? p - d : (d > 0 ? -1 + p : p);
+        }
+}
+
 }  // extern "C"

@@ -14,7 +14,8 @@ LSTM_STATE = {"ni": 0, "ig": 1, "fg": 2, "og": 3, "c": 4, "h": 5, "herr": 6, "dn
 
 
 class MdnDesc(C.Structure):
-    _fields_ = [("Lp", C.c_int), ("Lt", C.c_int), ("S", C.c_int), ("maxT", C.c_int), ("tie_variance", C.c_int)]
+    _fields_ = [("Lp", C.c_int), ("Lt", C.c_int), ("S", C.c_int), ("maxT", C.c_int), ("tie_variance", C.c_int),
+                ("sigmoid_continuous", C.c_int)]
 
 
 class CnnDesc(C.Structure):
@@ -438,9 +439,9 @@ class Dft:
 class Mdn:
     """Thin owner of a cnt_mdn handle.  config: flat list [n, (startD, endD, startDOut, endDOut, type) * n]."""
 
-    def __init__(self, Lp, Lt, S, maxT, config, tie_variance=False):
+    def __init__(self, Lp, Lt, S, maxT, config, tie_variance=False, sigmoid_continuous=False):
         self.handle = VP()
-        desc = MdnDesc(Lp, Lt, S, maxT, int(tie_variance))
+        desc = MdnDesc(Lp, Lt, S, maxT, int(tie_variance), int(sigmoid_continuous))
         arr = (F * len(config))(*[float(v) for v in config])
         check(lib().cnt_mdn_create(C.byref(desc), arr, len(config), C.byref(self.handle)))
 

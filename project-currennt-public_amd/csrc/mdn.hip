@@ -18,6 +18,8 @@
 // earlier valid frame reads 0.  The kernels reproduce exactly that outcome without a race.
 #include "common.hpp"
 
+#include <algorithm>
+
 #include <cmath>
 #include <cstring>
 #include <new>
@@ -73,6 +75,70 @@ struct UnitGeom {
     float var_floor, temperature;
     long capacity;  // allocated elements of the unit's parameter buffer
 };
+
+// ---- sigmoid unit (layers/MDNUnit.cu:198-225, 563-596, 634-676): M columns, one target per column -------
+__global__ void sigmoid_forward_kernel(UnitGeom g, const char *__restrict__ pat, const float *__restrict__ x,
+                                       float *__restrict__ prob) {
+    const size_t n = (size_t)g.F * g.M;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t f = i / g.M;
+        const int k = (int)(i % g.M);
+        prob[i] = pat[f] == 0 ? 0.0f : logistic(x[f * g.Lp + g.startD + k]);
+    }
+}
+
+// sums[0] += binary cross entropy of the valid frames, sums[1] += number of valid frames
+__global__ void sigmoid_error_kernel(UnitGeom g, int continuous, const char *__restrict__ pat,
+                                     const float *__restrict__ target, const float *__restrict__ prob,
+                                     float *__restrict__ sums) {
+    const size_t n = (size_t)g.F * g.M;
+    float v = 0.0f, cnt = 0.0f;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t f = i / g.M;
+        const int k = (int)(i % g.M);
+        if (pat[f] == 0) continue;
+        if (k == 0) cnt += 1.0f;
+        const float p = prob[i], pr = (float)(1.0 - p);
+        const float d = target[f * g.Lt + g.startDOut + k];
+        if (continuous) {
+            const float p1 = logf(fmaxf(lim::kMin, p)), p2 = logf(fmaxf(lim::kMin, pr));
+            v += (float)(-1.0 * d * p1 - (1 - d) * p2);
+        } else {
+            const float b = d > 0 ? p : 1 - p;
+            v += -logf(fmaxf(lim::kMin, b));
+        }
+    }
+    v = wave_sum(v);
+    cnt = wave_sum(cnt);
+    if ((threadIdx.x & 63) == 0) {
+        if (v != 0.0f) atomicAdd(sums, v);
+        if (cnt != 0.0f) atomicAdd(sums + 1, cnt);
+    }
+}
+
+// the unit's error is the summed cross entropy divided by the number of valid frames (MDNUnit.cu:3821)
+__global__ void sigmoid_error_finish_kernel(const float *__restrict__ sums, float *__restrict__ result) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *result += sums[0] / sums[1];
+}
+
+__global__ void sigmoid_backward_kernel(UnitGeom g, int continuous, const char *__restrict__ pat,
+                                        const float *__restrict__ target, const float *__restrict__ prob,
+                                        float *__restrict__ errors) {
+    const size_t n = (size_t)g.F * g.M;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t f = i / g.M;
+        const int k = (int)(i % g.M);
+        float e = 0.0f;
+        if (pat[f] != 0) {
+            const float p = prob[i], d = target[f * g.Lt + g.startDOut + k];
+            e = continuous ? p - d : (d > 0 ? -1 + p : p);
+        }
+        errors[f * g.Lp + g.startD + k] = e;
+    }
+}
 
 // ---- softmax unit -----------------------------------------------------------------------------------
 __global__ void softmax_forward_kernel(UnitGeom g, const char *__restrict__ pat, const float *__restrict__ x,
@@ -236,7 +302,7 @@ __global__ void mixture_backward_kernel(UnitGeom g, const char *__restrict__ pat
 // Host side
 // ---------------------------------------------------------------------------------------------------
 struct cnt_mdn_unit {
-    int type;  // >0 mixtures, -1 softmax
+    int type;  // >0 mixtures, -1 softmax, 0 sigmoid
     int startD, endD, startDOut, endDOut;
     int M, D;
     float var_floor;
@@ -291,6 +357,11 @@ int cnt_mdn_create(const cnt_mdn_desc *desc, const float *config, int config_len
             u.para_capacity = maxF * u.M;
             u.tmp_capacity = 0;
             ok = (dims == 1);
+        } else if (ok && u.type == 0) {
+            u.M = cols; u.D = 1;
+            u.para_capacity = maxF * u.M;
+            u.tmp_capacity = 2;  // cross-entropy sum and frame count
+            ok = (dims == cols);
         } else if (ok && u.type > 0) {
             u.M = u.type; u.D = dims;
             ok = !desc->tie_variance && cols == u.M * (1 + 2 * u.D);
@@ -300,8 +371,9 @@ int cnt_mdn_create(const cnt_mdn_desc *desc, const float *config, int config_len
             ok = false;
         }
         if (!ok) {
-            set_error("mdn_create: unit %d (type %d, columns %d..%d, targets %d..%d) is not supported: only flat softmax "
-                      "(-1) and untied-variance mixture units (>0 with columns = M*(1+2*D)) are built",
+            set_error("mdn_create: unit %d (type %d, columns %d..%d, targets %d..%d) is not supported: only sigmoid (0, one "
+                      "target per column), flat softmax (-1) and untied-variance mixture units (>0 with columns = "
+                      "M*(1+2*D)) are built",
                       i, u.type, u.startD, u.endD, u.startDOut, u.endDOut);
             cnt_mdn_destroy(h);
             return CNT_ERR_ARG;
@@ -349,10 +421,10 @@ float *cnt_mdn_unit_buffer(cnt_mdn *h, int unit, int which, long *count) {
     cnt_mdn_unit &u = h->units[(size_t)unit];
     const long F = (long)h->T * h->desc.S;
     if (which == 0) {
-        if (count) *count = u.type == -1 ? F * u.M : F * u.M * (1 + 2 * u.D);
+        if (count) *count = u.type <= 0 ? F * u.M : F * u.M * (1 + 2 * u.D);
         return u.para;
     }
-    if (which == 1 && u.tmp) {
+    if (which == 1 && u.tmp && u.type > 0) {
         if (count) *count = F * (u.M + 1);
         return u.tmp;
     }
@@ -376,7 +448,12 @@ int cnt_mdn_forward(cnt_mdn *h, void *stream_, const float *nn_outputs) {
     for (auto &u : h->units) {
         const UnitGeom g = unit_geom(h, u);
         const dim3 grid((g.F + kFramesPerBlock - 1) / kFramesPerBlock), block(64 * kFramesPerBlock);
-        if (u.type == -1) {
+        if (u.type == 0) {
+            ProfileScope prof(stream, "mdn_sigmoid_forward");
+            const size_t n = (size_t)g.F * g.M;
+            hipLaunchKernelGGL(sigmoid_forward_kernel, dim3((unsigned)std::min<size_t>((n + 255) / 256, 4096)), dim3(256), 0,
+                               stream, g, h->pat, nn_outputs, u.para);
+        } else if (u.type == -1) {
             ProfileScope prof(stream, "mdn_softmax_forward");
             hipLaunchKernelGGL(softmax_forward_kernel, grid, block, 0, stream, g, h->pat, nn_outputs, u.para);
         } else {
@@ -396,7 +473,14 @@ int cnt_mdn_calculate_error(cnt_mdn *h, void *stream_, const float *targets, flo
     CNT_TRY(fill_zero(stream, result_dev, 1));
     for (auto &u : h->units) {
         const UnitGeom g = unit_geom(h, u);
-        if (u.type == -1) {
+        if (u.type == 0) {
+            ProfileScope prof(stream, "mdn_sigmoid_error");
+            const size_t n = (size_t)g.F * g.M;
+            CNT_TRY(fill_zero(stream, u.tmp, 2));
+            hipLaunchKernelGGL(sigmoid_error_kernel, dim3((unsigned)std::min<size_t>((n + 255) / 256, 1024)), dim3(256), 0,
+                               stream, g, h->desc.sigmoid_continuous, h->pat, targets, u.para, u.tmp);
+            hipLaunchKernelGGL(sigmoid_error_finish_kernel, dim3(1), dim3(64), 0, stream, u.tmp, result_dev);
+        } else if (u.type == -1) {
             ProfileScope prof(stream, "mdn_softmax_error");
             hipLaunchKernelGGL(softmax_error_kernel, dim3((g.F + 255) / 256), dim3(256), 0, stream, g, h->pat, targets,
                                u.para, result_dev);
@@ -425,7 +509,12 @@ int cnt_mdn_backward(cnt_mdn *h, void *stream_, const float *targets, float *pre
     for (auto &u : h->units) {
         const UnitGeom g = unit_geom(h, u);
         const dim3 grid((g.F + kFramesPerBlock - 1) / kFramesPerBlock), block(64 * kFramesPerBlock);
-        if (u.type == -1) {
+        if (u.type == 0) {
+            ProfileScope prof(stream, "mdn_sigmoid_backward");
+            const size_t n = (size_t)g.F * g.M;
+            hipLaunchKernelGGL(sigmoid_backward_kernel, dim3((unsigned)std::min<size_t>((n + 255) / 256, 4096)), dim3(256), 0,
+                               stream, g, h->desc.sigmoid_continuous, h->pat, targets, u.para, prev_errors);
+        } else if (u.type == -1) {
             ProfileScope prof(stream, "mdn_softmax_backward");
             hipLaunchKernelGGL(softmax_backward_kernel, grid, block, 0, stream, g, h->pat, targets, u.para,
                                prev_errors);

@@ -68,6 +68,7 @@ def lib():
         L.orc_sse_error.restype = C.c_float
         L.orc_mdn_mixture_error.restype = C.c_float
         L.orc_softmax_error.restype = C.c_float
+        L.orc_sigmoid_error.restype = C.c_float
         L.orc_dft_logamp_loss.restype = C.c_float
         L.orc_opt_next_beta_accum.restype = C.c_float
         L.orc_opt_next_beta_accum.argtypes = [C.c_float, C.c_int]
@@ -250,3 +251,16 @@ def opt_update_weights(weights, g, deltas, mask, learning_rate, momentum):
 
 def opt_next_beta_accum(accum, which):
     return float(lib().orc_opt_next_beta_accum(accum, which))
+
+
+def sigmoid_forward(F, Lp, startD, K, pat, x, prob):
+    lib().orc_sigmoid_forward(F, Lp, startD, K, cptr(pat), fptr(x), fptr(prob))
+
+
+def sigmoid_error(F, Lt, startDOut, K, continuous, pat, target, prob):
+    return float(lib().orc_sigmoid_error(F, Lt, startDOut, K, int(continuous), cptr(pat), fptr(target), fptr(prob)))
+
+
+def sigmoid_backward(F, Lp, Lt, startD, startDOut, K, continuous, pat, target, prob, errors):
+    lib().orc_sigmoid_backward(F, Lp, Lt, startD, startDOut, K, int(continuous), cptr(pat), fptr(target), fptr(prob),
+                               fptr(errors))

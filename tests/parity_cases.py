@@ -295,6 +295,56 @@ def run_softmax_case(lengths, K, extra, seed):
     return worst
 
 
+def run_sigmoid_case(lengths, K, extra, continuous, seed, with_softmax=False):
+    """MDN sigmoid unit (optionally next to a softmax unit in the same layer) against the oracle."""
+    import torch
+
+    capi = pkg().capi
+    S, T = len(lengths), max(lengths)
+    F = T * S
+    Ks = 5 if with_softmax else 0
+    Lp = extra + K + Ks
+    Lt = K + (1 if with_softmax else 0)
+    rng = np.random.default_rng(seed)
+    x = (2 * rng.standard_normal((F, Lp))).astype(np.float32)
+    tgt = np.zeros((F, Lt), dtype=np.float32)
+    tgt[:, :K] = rng.uniform(0, 1, (F, K)) if continuous else (rng.uniform(0, 1, (F, K)) > 0.5)
+    if with_softmax:
+        tgt[:, K] = rng.integers(0, Ks, size=F)
+    pat = make_pat_types(lengths, T)
+    prob_o = np.zeros(F * K, dtype=np.float32)
+    err_o = np.zeros(F * Lp, dtype=np.float32)
+    O.sigmoid_forward(F, Lp, extra, K, pat, x.reshape(-1), prob_o)
+    loss_o = O.sigmoid_error(F, Lt, 0, K, continuous, pat, tgt.reshape(-1), prob_o)
+    O.sigmoid_backward(F, Lp, Lt, extra, 0, K, continuous, pat, tgt.reshape(-1), prob_o, err_o)
+    config = [1, extra, extra + K, 0, K, 0]
+    if with_softmax:
+        sm_o = np.zeros(F * Ks, dtype=np.float32)
+        O.softmax_forward(F, Lp, extra + K, Ks, 1.0, pat, x.reshape(-1), sm_o)
+        loss_o += O.softmax_error(F, Lt, K, Ks, F * Ks, pat, tgt.reshape(-1), sm_o)
+        O.softmax_backward(F, Lp, Lt, extra + K, K, Ks, pat, tgt.reshape(-1), sm_o, err_o)
+        config = [2, extra, extra + K, 0, K, 0, extra + K, Lp, K, K + 1, -1]
+
+    layer = capi.Mdn(Lp, Lt, S, T, config, sigmoid_continuous=continuous)
+    res = torch.zeros(1, dtype=torch.float32, device="cuda")
+    err_d = torch.full((F * Lp,), 9.0, dtype=torch.float32, device="cuda")
+    pd, xd, td = dev(pat), dev(x.reshape(-1)), dev(tgt.reshape(-1))
+    layer.load_sequences(pd, T)
+    layer.forward(xd)
+    layer.calculate_error(td, res)
+    layer.backward(td, err_d)
+    torch.cuda.synchronize()
+    worst = relerr(layer.unit_buffer(0, 0).cpu().numpy(), prob_o)
+    worst = max(worst, abs(float(res.item()) - loss_o) / abs(loss_o))
+    got = err_d.cpu().numpy()
+    worst = max(worst, relerr(got, err_o))
+    # padding frames and the columns no unit owns are exactly zero
+    g2, o2 = got.reshape(F, Lp), err_o.reshape(F, Lp)
+    assert np.all(g2[pat == 0] == 0.0) and np.all(g2[:, :extra] == 0.0) and np.all(o2[:, :extra] == 0.0)
+    layer.close()
+    return worst
+
+
 def run_cnn_case(P, half_width, interval, lengths, causal, out_tanh, seed, bias=1.0, maxT=None):
     """1-D convolution layer forward + backward against the oracle (which scatters into a real column buffer)."""
     import torch

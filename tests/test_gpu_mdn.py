@@ -39,3 +39,12 @@ def test_unsupported_units_are_rejected():
         capi.Mdn(10, 2, 2, 4, [1, 0, 10, 0, 2, 2], tie_variance=True)
     with pytest.raises(RuntimeError):
         capi.Mdn(10, 2, 2, 4, [2, 0, 10, 0, 2, 2])      # length does not match the unit count
+
+
+@pytest.mark.parametrize("lengths,K,extra,continuous,with_softmax", [
+    ([9, 5, 9], 7, 0, False, False), ([12, 12], 3, 4, True, False), ([20, 11, 20, 3], 16, 2, False, True),
+    ([6], 1, 0, True, False),
+])
+def test_sigmoid_unit(lengths, K, extra, continuous, with_softmax):
+    print("mdn sigmoid case", lengths, K, extra, continuous, with_softmax, flush=True)
+    assert PC.run_sigmoid_case(lengths, K, extra, continuous, seed=K + extra, with_softmax=with_softmax) < TOL

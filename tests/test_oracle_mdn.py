@@ -125,3 +125,33 @@ def test_softmax_unit_matches_cross_entropy():
     p = prob.reshape(F, K)
     assert np.all(p[pat == 0] == np.float32(3.4028235e38))  # the reference's skip marker
     assert relerr(p[pat != 0], torch.softmax(xt[valid][:, startD:], 1).detach().numpy()) < 1e-6
+
+
+def test_sigmoid_unit_matches_binary_cross_entropy_autograd():
+    """Forward = logistic, error = BCE summed over elements and divided by the number of non-padding frames,
+    gradient = d(sum BCE)/d(logit) = p - t (not divided): float64 autograd on the unnormalised sum."""
+    import torch
+
+    rng = np.random.default_rng(4)
+    lengths, K, extra = [7, 4, 7], 5, 2
+    S, T = len(lengths), max(lengths)
+    F, Lp = S * T, extra + K
+    pat = make_pat_types(lengths, T)
+    x = rng.standard_normal((F, Lp)).astype(np.float32)
+    for continuous in (False, True):
+        tgt = (rng.uniform(0, 1, (F, K)).astype(np.float32) if continuous
+               else (rng.uniform(0, 1, (F, K)) > 0.4).astype(np.float32))
+        prob = np.zeros(F * K, np.float32); err = np.full(F * Lp, 5.0, np.float32)
+        O.sigmoid_forward(F, Lp, extra, K, pat, x.reshape(-1), prob)
+        loss = O.sigmoid_error(F, K, 0, K, continuous, pat, tgt.reshape(-1), prob)
+        O.sigmoid_backward(F, Lp, K, extra, 0, K, continuous, pat, tgt.reshape(-1), prob, err)
+        xt = torch.tensor(x[:, extra:], dtype=torch.float64, requires_grad=True)
+        valid = torch.tensor(pat != 0)
+        bce = torch.nn.functional.binary_cross_entropy_with_logits(xt, torch.tensor(tgt, dtype=torch.float64), reduction="none")
+        total = (bce * valid[:, None]).sum()
+        total.backward()
+        assert abs(loss - float(total) / int(valid.sum())) < 1e-5 * max(1.0, abs(loss))
+        e = err.reshape(F, Lp)
+        assert np.max(np.abs(e[:, extra:] - xt.grad.numpy())) < 1e-6
+        assert np.all(e[:, :extra] == 5.0)                       # columns outside the unit are not touched
+        assert np.all(e[pat == 0][:, extra:] == 0.0) and np.all(prob.reshape(F, K)[pat == 0] == 0.0)
