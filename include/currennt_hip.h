@@ -252,9 +252,10 @@ int cnt_skipadd_forward(void *stream, long count, int n_in, const float *const *
 int cnt_skipadd_backward(void *stream, long count, float *errors, const float *errors_from_skip, int n_pre,
                          float *const *targets, const int *target_is_skip);
 
-/* ---- DFT (multi-resolution STFT log-amplitude) loss -------------------------------------------------
+/* ---- DFT (multi-resolution STFT spectral) loss ------------------------------------------------------
  * DFTPostoutputLayer<TDevice> with helpers::FFTMat (layers/DFTErrorPostoutputLayer.cu, helpers/FFTMat.cu)
- * for specDisType 0 and up to three resolutions ("fftLength/frameLength/frameShift" with suffix "", "2",
+ * for the amplitude / spectrum distances specDisType 0..6 (helpers/FFTMat.hpp:29-35; distance functors
+ * helpers/FFTMat.cu:473-628, gradients :760-900) and up to three resolutions ("fftLength/frameLength/frameShift" with suffix "", "2",
  * "3", layers/DFTErrorPostoutputLayer.cu:752-845).  The layer has size 1; a waveform occupies max_length
  * consecutive floats.  The reference handles one waveform per fraction; here n_waves waveforms with their
  * own lengths can be processed by one call (waveform w at offset w*max_length).  FFT lengths must be
@@ -266,7 +267,8 @@ typedef struct {
     int window_type[3];  /* 0 Hann (the reference's default), 1 square */
     float gamma;         /* "gamma": weight of the spectral amplitude loss            */
     float log_floor;     /* "logSpecAmpFloor", 1e-5 by default (helpers/FFTMat.hpp:53) */
-    int spec_dis_type;   /* "specDisType"; only 0 is built                            */
+    int spec_dis_type;   /* "specDisType": 0 log-amplitude MSE, 1 KLD, 2 amplitude MSE, 3 log
+                            spectral MSE, 4 spectral MSE, 5 amplitude ratio, 6 Itakura-Saito  */
     int max_length;      /* maxSeqLength in samples                                   */
     int max_waves;       /* waveforms per call, 1..32                                 */
 } cnt_dft_desc;

@@ -109,6 +109,9 @@ void orc_skipadd_backward(long count, float *errors, const float *errors_from_sk
 int orc_dft_frame_count(int signal_length, int frame_length, int frame_shift);
 void orc_dft_r2c(int n, const float *in, float *out);
 void orc_dft_c2r(int n, const float *in, float *out);
+float orc_dft_spectral_loss(int dis_type, int fft_length, int frame_length, int frame_shift, int window_type,
+                            int max_length, int length, float gamma, float log_floor, const float *source,
+                            const float *target, float *grad);
 float orc_dft_logamp_loss(int fft_length, int frame_length, int frame_shift, int window_type, int max_length,
                           int length, float gamma, float log_floor, const float *source, const float *target,
                           float *grad);

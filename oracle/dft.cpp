@@ -1,10 +1,14 @@
-// CPU oracle, DFT (STFT log-amplitude) loss -- TEST INFRASTRUCTURE ONLY (see oracle_common.h).
+// CPU oracle, DFT (STFT spectral) loss -- TEST INFRASTRUCTURE ONLY (see oracle_common.h).
 //
 // Restates /root/reference/CURRENNT_codes/currennt_lib/src:
 //   helpers/FFTMat.cu:282-312      FrameSignal: Hann window with the constant 3.141215, zero padding to the
 //                                  FFT length, evaluated in double and rounded once
 //   helpers/FFTMat.cu:473-496      log-amplitude distance per bin, d = safeLog(|S|^2+f) - safeLog(|T|^2+f)
 //   helpers/FFTMat.cu:760-782      gradient per bin, G = d * S / (|S|^2 + f)
+//   helpers/FFTMat.cu:498-628      the other amplitude / spectrum distances (specDisType 1..6), :784-900 their
+//                                  gradients; constants helpers/FFTMat.hpp (FFT_KLD_FLOOR_NUM, FFT_IS_FLOOR_NUM,
+//                                  FFT_SPEC_LOG_MSE_CONST); double literals in the reference promote the
+//                                  expression they stand in to double, restated as such
 //   helpers/FFTMat.cu:456-471      cleanDummyGradients
 //   helpers/FFTMat.cu:965-1006     collectGrad (windowed overlap-add, scale gamma / (bins * validFrames))
 //   helpers/FFTMat.cu:1137-1147    frame / bin counts;  :1152-1202 zero fill beyond the signal length
@@ -59,6 +63,92 @@ float window_product(float raw, int pos, int frame_length, int window_type) {
     return (float)(raw * 0.5 * (1 - std::cos(2.0 * kPiWindow * pos / (frame_length - 1))));
 }
 
+// helpers/FFTMat.hpp
+constexpr double kKldFloor = 0.00001, kIsFloor = 0.00001, kSpecLogMseConst = 1.0;
+
+// first pass of specAmpDistance (helpers/FFTMat.cu:1350-1475): x = distance, y = value kept for the gradient
+void bin_distance(int dis_type, float log_floor, float sx, float sy, float tx, float ty, float &x, float &y) {
+    switch (dis_type) {
+        case 1: {  // SpecAmpDistance_AMP_KLD
+            const float s = (float)std::sqrt(sx * sx + sy * sy + kKldFloor);
+            const float t = (float)std::sqrt(tx * tx + ty * ty + kKldFloor);
+            x = t * orc::safe_log(t / s) - t + s;
+            y = (float)(1.0 - t / s);
+            break;
+        }
+        case 2:  // SpecAmpDistance_AMP_MSE
+            y = (sx * sx + sy * sy) - (tx * tx + ty * ty);
+            x = y * y;
+            break;
+        case 3:  // SpecAmpDistance_SPEC_LOG_MSE
+            y = (float)((sx - tx) * (sx - tx) + (sy - ty) * (sy - ty) + kSpecLogMseConst);
+            x = orc::safe_log(y);
+            break;
+        case 4:  // SpecAmpDistance_SPEC_MSE
+            y = 0.0f;
+            x = (sx - tx) * (sx - tx) + (sy - ty) * (sy - ty);
+            break;
+        case 5:  // SpecAmpDistance_AMP_RATIO
+            y = (float)((sx * sx + sy * sy + kKldFloor) / (tx * tx + ty * ty + kKldFloor) - 1.0);
+            x = y * y;
+            break;
+        case 6: {  // SpecAmpDistance_AMP_IS
+            const float sa = (float)std::sqrt(sx * sx + sy * sy + kIsFloor);
+            const float ta = (float)std::sqrt(tx * tx + ty * ty + kIsFloor);
+            y = ta / sa;
+            x = (float)(y - orc::safe_log(y) - 1.0);
+            break;
+        }
+        default: {  // SpecAmpDistance_AMP_LOG_MSE
+            const float d = orc::safe_log(sx * sx + sy * sy + log_floor) - orc::safe_log(tx * tx + ty * ty + log_floor);
+            y = d;
+            x = d * d;
+        }
+    }
+}
+
+// second pass (helpers/FFTMat.cu:1637-1770): (x, y) <- gradient spectrum, y on entry is what pass one left
+void bin_gradient(int dis_type, float log_floor, float sx, float sy, float tx, float ty, float &x, float &y) {
+    const float keep = y;
+    switch (dis_type) {
+        case 1: {  // SpecAmpDistance_AMP_KLD_Grad
+            const float spec = (float)std::sqrt(sx * sx + sy * sy + kKldFloor);
+            x = keep * sx / spec;
+            y = keep * sy / spec;
+            break;
+        }
+        case 2:  // SpecAmpDistance_AMP_MSE_Grad
+            x = keep * sx;
+            y = keep * sy;
+            break;
+        case 3:  // SpecAmpDistance_SPEC_LOG_MSE_Grad
+            x = (sx - tx) / keep;
+            y = (sy - ty) / keep;
+            break;
+        case 4:  // SpecAmpDistance_SPEC_MSE_Grad
+            x = sx - tx;
+            y = sy - ty;
+            break;
+        case 5: {  // SpecAmpDistance_AMP_RATIO_Grad
+            const float spec = (float)(tx * tx + ty * ty + kKldFloor);
+            x = keep * sx / spec;
+            y = keep * sy / spec;
+            break;
+        }
+        case 6: {  // SpecAmpDistance_AMP_IS_Grad
+            const float spec = (float)(sx * sx + sy * sy + kIsFloor);
+            x = (float)(sx / spec * (1.0 - keep));
+            y = (float)(sy / spec * (1.0 - keep));
+            break;
+        }
+        default: {  // SpecAmpDistance_AMP_LOG_MSE_Grad
+            const float spec = sx * sx + sy * sy + log_floor;
+            x = keep * sx / spec;
+            y = keep * sy / spec;
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -92,9 +182,9 @@ void orc_dft_c2r(int n, const float *in, float *out) {
 
 // One resolution, one waveform.  source/target hold max_length samples (content beyond `length` is taken
 // as zero, as the reference's buffers are cleared there).  grad receives max_length values.
-float orc_dft_logamp_loss(int fft_length, int frame_length, int frame_shift, int window_type, int max_length,
-                          int length, float gamma, float log_floor, const float *source, const float *target,
-                          float *grad) {
+float orc_dft_spectral_loss(int dis_type, int fft_length, int frame_length, int frame_shift, int window_type,
+                            int max_length, int length, float gamma, float log_floor, const float *source,
+                            const float *target, float *grad) {
     const int N = fft_length, B = N / 2 + 1;
     const int Kmax = frame_count(max_length, frame_length, frame_shift);
     const int Kvalid = frame_count(length, frame_length, frame_shift);
@@ -119,22 +209,13 @@ float orc_dft_logamp_loss(int fft_length, int frame_length, int frame_shift, int
         orc_dft_r2c(N, &fs[(size_t)k * N], &S[(size_t)k * B * 2]);
         orc_dft_r2c(N, &ft[(size_t)k * N], &T[(size_t)k * B * 2]);
     }
-    for (size_t i = 0; i < (size_t)Kmax * B; ++i) {
-        const float sx = S[2 * i], sy = S[2 * i + 1], tx = T[2 * i], ty = T[2 * i + 1];
-        const float d = orc::safe_log(sx * sx + sy * sy + log_floor) - orc::safe_log(tx * tx + ty * ty + log_floor);
-        Dm[2 * i + 1] = d;
-        Dm[2 * i] = d * d;
-    }
+    for (size_t i = 0; i < (size_t)Kmax * B; ++i)
+        bin_distance(dis_type, log_floor, S[2 * i], S[2 * i + 1], T[2 * i], T[2 * i + 1], Dm[2 * i], Dm[2 * i + 1]);
     const float factor = (float)(B * Kvalid);
     float err = 0.0f;
     for (size_t i = 0; i < (size_t)B * Kvalid; ++i) err += Dm[2 * i] / factor;
-    for (size_t i = 0; i < (size_t)Kmax * B; ++i) {
-        const float sx = S[2 * i], sy = S[2 * i + 1];
-        const float spec = sx * sx + sy * sy + log_floor;
-        const float d = Dm[2 * i + 1];
-        Dm[2 * i] = d * sx / spec;
-        Dm[2 * i + 1] = d * sy / spec;
-    }
+    for (size_t i = 0; i < (size_t)Kmax * B; ++i)
+        bin_gradient(dis_type, log_floor, S[2 * i], S[2 * i + 1], T[2 * i], T[2 * i + 1], Dm[2 * i], Dm[2 * i + 1]);
     for (int k = 0; k < Kmax; ++k) orc_dft_c2r(N, &Dm[(size_t)k * B * 2], &fg[(size_t)k * N]);
     for (int k = 0; k < Kmax; ++k)
         for (int j = 0; j < N; ++j)
@@ -154,6 +235,13 @@ float orc_dft_logamp_loss(int fft_length, int frame_length, int frame_shift, int
         grad[t] = acc * scale;
     }
     return err;
+}
+
+float orc_dft_logamp_loss(int fft_length, int frame_length, int frame_shift, int window_type, int max_length,
+                          int length, float gamma, float log_floor, const float *source, const float *target,
+                          float *grad) {
+    return orc_dft_spectral_loss(0, fft_length, frame_length, frame_shift, window_type, max_length, length, gamma,
+                                 log_floor, source, target, grad);
 }
 
 }  // extern "C"

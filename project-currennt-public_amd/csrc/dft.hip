@@ -1,6 +1,7 @@
-// Multi-resolution STFT log-amplitude loss and its gradient for gfx950, with an in-house radix-2 FFT.
+// Multi-resolution STFT spectral loss (seven amplitude / spectrum distances) and its gradient for gfx950, with
+// an in-house radix-2 FFT.
 //
-// Reference behaviour: helpers/FFTMat.cu (FrameSignal :282-312, distance :473-496, gradient :760-782,
+// Reference behaviour: helpers/FFTMat.cu (FrameSignal :282-312, distances :473-628, gradients :760-900,
 // cleanDummyGradients :456-471, collectGrad :965-1006, drivers :1246-1274, :1350-1475, :1637-1770,
 // :1833-1886) and layers/DFTErrorPostoutputLayer.cu (:1186-1244, :1699-1714, :1782-1885).  The reference
 // runs about a dozen launches and three cuFFT calls per resolution and waveform, with every intermediate
@@ -46,7 +47,64 @@ __host__ __device__ inline int frame_count(int length, int Nw, int Hs) {
     return length < Nw ? 1 : 1 + (length - Nw) / Hs;
 }
 
-template <int LOGN>
+// The reference's floors and constants (helpers/FFTMat.hpp: FFT_KLD_FLOOR_NUM, FFT_IS_FLOOR_NUM,
+// FFT_SPEC_LOG_MSE_CONST)
+constexpr float kKldFloor = 0.00001f;
+constexpr float kIsFloor = 0.00001f;
+constexpr float kSpecLogMseConst = 1.0f;
+
+// Distance of one bin and the gradient spectrum of that bin, for source spectrum (sx, sy) and target spectrum
+// (tx, ty).  Distance functors: helpers/FFTMat.cu:473-628; gradient functors: :760-900.  DIS is the reference's
+// specDisType: 0 log-amplitude MSE, 1 KLD of amplitudes, 2 MSE of squared amplitudes, 3 log of the complex
+// spectral distance, 4 complex spectral MSE, 5 amplitude ratio, 6 Itakura-Saito.
+template <int DIS>
+__device__ inline void bin_distance(float sx, float sy, float tx, float ty, float log_floor, float &e, float &gx,
+                                    float &gy) {
+    const float s2 = sx * sx + sy * sy, t2 = tx * tx + ty * ty;
+    if (DIS == 1) {
+        const float s = sqrtf(s2 + kKldFloor), t = sqrtf(t2 + kKldFloor);
+        e = t * safe_log(t / s) - t + s;
+        const float aux = 1.0f - t / s;
+        gx = aux * sx / s;
+        gy = aux * sy / s;
+    } else if (DIS == 2) {
+        const float aux = s2 - t2;
+        e = aux * aux;
+        gx = aux * sx;
+        gy = aux * sy;
+    } else if (DIS == 3) {
+        const float dx = sx - tx, dy = sy - ty;
+        const float aux = dx * dx + dy * dy + kSpecLogMseConst;
+        e = safe_log(aux);
+        gx = dx / aux;
+        gy = dy / aux;
+    } else if (DIS == 4) {
+        const float dx = sx - tx, dy = sy - ty;
+        e = dx * dx + dy * dy;
+        gx = dx;
+        gy = dy;
+    } else if (DIS == 5) {
+        const float tf = t2 + kKldFloor;
+        const float aux = (s2 + kKldFloor) / tf - 1.0f;
+        e = aux * aux;
+        gx = aux * sx / tf;
+        gy = aux * sy / tf;
+    } else if (DIS == 6) {
+        const float sf = s2 + kIsFloor;
+        const float aux = sqrtf(t2 + kIsFloor) / sqrtf(sf);
+        e = aux - safe_log(aux) - 1.0f;
+        gx = sx / sf * (1.0f - aux);
+        gy = sy / sf * (1.0f - aux);
+    } else {
+        const float spec = s2 + log_floor;
+        const float d = safe_log(spec) - safe_log(t2 + log_floor);
+        e = d * d;
+        gx = d * sx / spec;
+        gy = d * sy / spec;
+    }
+}
+
+template <int LOGN, int DIS>
 __global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
     constexpr int N = 1 << LOGN;
     constexpr int HALF = N / 2;
@@ -104,10 +162,9 @@ __global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
         // S = (Z[b] + conj(Z[N-b])) / 2,  T = (Z[b] - conj(Z[N-b])) / (2i)
         const float sx = 0.5f * (zb.x + zn.x), sy = 0.5f * (zb.y - zn.y);
         const float tx = 0.5f * (zb.y + zn.y), ty = -0.5f * (zb.x - zn.x);
-        const float spec = sx * sx + sy * sy + p.log_floor;
-        const float d = safe_log(spec) - safe_log(tx * tx + ty * ty + p.log_floor);
-        if (active) err += d * d;
-        const float gx = d * sx / spec, gy = d * sy / spec;
+        float e, gx, gy;
+        bin_distance<DIS>(sx, sy, tx, ty, p.log_floor, e, gx, gy);
+        if (active) err += e;
         if (b == 0 || b == HALF) {
             z[fl][pb] = make_float2(gx, 0.0f);
         } else {
@@ -163,16 +220,29 @@ __global__ void dft_backward_kernel(int max_length, int n_waves, DftParams p, fl
 }
 
 typedef void (*dft_kernel_t)(const DftParams);
-dft_kernel_t pick_dft_kernel(int logn) {
+template <int DIS>
+dft_kernel_t pick_dft_length(int logn) {
     switch (logn) {
-        case 5: return dft_loss_kernel<5>;
-        case 6: return dft_loss_kernel<6>;
-        case 7: return dft_loss_kernel<7>;
-        case 8: return dft_loss_kernel<8>;
-        case 9: return dft_loss_kernel<9>;
-        case 10: return dft_loss_kernel<10>;
-        case 11: return dft_loss_kernel<11>;
-        case 12: return dft_loss_kernel<12>;
+        case 5: return dft_loss_kernel<5, DIS>;
+        case 6: return dft_loss_kernel<6, DIS>;
+        case 7: return dft_loss_kernel<7, DIS>;
+        case 8: return dft_loss_kernel<8, DIS>;
+        case 9: return dft_loss_kernel<9, DIS>;
+        case 10: return dft_loss_kernel<10, DIS>;
+        case 11: return dft_loss_kernel<11, DIS>;
+        case 12: return dft_loss_kernel<12, DIS>;
+        default: return nullptr;
+    }
+}
+dft_kernel_t pick_dft_kernel(int logn, int dis_type) {
+    switch (dis_type) {
+        case 0: return pick_dft_length<0>(logn);
+        case 1: return pick_dft_length<1>(logn);
+        case 2: return pick_dft_length<2>(logn);
+        case 3: return pick_dft_length<3>(logn);
+        case 4: return pick_dft_length<4>(logn);
+        case 5: return pick_dft_length<5>(logn);
+        case 6: return pick_dft_length<6>(logn);
         default: return nullptr;
     }
 }
@@ -210,9 +280,10 @@ int cnt_dft_create(const cnt_dft_desc *desc, cnt_dft **out) {
                 kMaxRes);
     CNT_REQUIRE(desc->max_length > 0 && desc->max_waves >= 1 && desc->max_waves <= kMaxWavesPerLaunch,
                 "dft_create: max_length must be positive and max_waves in 1..%d", kMaxWavesPerLaunch);
-    // the reference implements the Hann window (default) and the square window; other distances than the
-    // log-amplitude MSE (specDisType 0) are not built
-    CNT_REQUIRE(desc->spec_dis_type == 0, "dft_create: only specDisType 0 (log-amplitude MSE) is built");
+    // the reference implements the Hann window (default) and the square window, and the amplitude / spectrum
+    // distances 0..6; its phase distances are a separate driver and are not built
+    CNT_REQUIRE(desc->spec_dis_type >= 0 && desc->spec_dis_type <= 6, "dft_create: specDisType %d outside 0..6",
+                desc->spec_dis_type);
     cnt_dft *h = new (std::nothrow) cnt_dft();
     CNT_REQUIRE(h != nullptr, "dft_create: out of host memory");
     std::memset(h, 0, sizeof(*h));
@@ -222,7 +293,7 @@ int cnt_dft_create(const cnt_dft_desc *desc, cnt_dft **out) {
         const int N = desc->fft_length[r], Nw = desc->frame_length[r], Hs = desc->frame_shift[r];
         int logn = 0;
         while ((1 << logn) < N) ++logn;
-        if ((1 << logn) != N || !pick_dft_kernel(logn) || Nw < 2 || Nw > N || Hs < 1) {
+        if ((1 << logn) != N || !pick_dft_kernel(logn, 0) || Nw < 2 || Nw > N || Hs < 1) {
             set_error("dft_create: resolution %d has fftLength %d, frameLength %d, frameShift %d; supported: fftLength a "
                       "power of two in 32..4096, 2 <= frameLength <= fftLength, frameShift >= 1", r, N, Nw, Hs);
             cnt_dft_destroy(h);
@@ -293,7 +364,7 @@ int cnt_dft_forward(cnt_dft *h, void *stream_, int n_waves, const int *lengths, 
         const int kmax = frame_count(max_len, p.Nw, p.Hs);
         dim3 grid((kmax + fpb - 1) / fpb, n_waves);
         ProfileScope prof(stream, "dft_loss");
-        hipLaunchKernelGGL(pick_dft_kernel(h->logn[r]), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL(pick_dft_kernel(h->logn[r], h->desc.spec_dis_type), grid, dim3(256), 0, stream, p);
         CNT_HIP(hipGetLastError());
     }
     return CNT_OK;

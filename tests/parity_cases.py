@@ -522,7 +522,7 @@ def run_skipadd_case(n, seed):
     return 0.0
 
 
-def run_dft_case(resolutions, max_len, lengths, seed, gamma=1.0):
+def run_dft_case(resolutions, max_len, lengths, seed, gamma=1.0, dis_type=0):
     """Multi-resolution DFT loss: per-resolution losses and the summed gradient against the oracle."""
     import torch
 
@@ -536,10 +536,11 @@ def run_dft_case(resolutions, max_len, lengths, seed, gamma=1.0):
     for w in range(W):
         for r, (N, Nw, Hs) in enumerate(resolutions):
             g = np.zeros(max_len, dtype=np.float32)
-            err_o[w, r] = O.dft_logamp_loss(N, Nw, Hs, 0, max_len, lengths[w], gamma, 1e-5, src[w].copy(), tgt[w].copy(), g)
+            err_o[w, r] = O.dft_spectral_loss(dis_type, N, Nw, Hs, 0, max_len, lengths[w], gamma, 1e-5, src[w].copy(),
+                                              tgt[w].copy(), g)
             g[lengths[w]:] = 0  # the layer only passes on the first `length` samples
             grad_o[w] += g
-    layer = capi.Dft(resolutions, max_len, W, gamma=gamma)
+    layer = capi.Dft(resolutions, max_len, W, gamma=gamma, spec_dis_type=dis_type)
     err_d = torch.full((W * len(resolutions),), 7.0, dtype=torch.float32, device="cuda")
     prev_d = torch.full((W * max_len,), 7.0, dtype=torch.float32, device="cuda")
     layer.forward(lengths, dev(src.reshape(-1)), dev(tgt.reshape(-1)), err_d)

@@ -1,4 +1,4 @@
-"""GPU parity (through the C ABI) of the multi-resolution DFT log-amplitude loss with the in-house FFT against
+"""GPU parity (through the C ABI) of the multi-resolution DFT spectral loss (distance types 0..6) with the in-house FFT against
 the oracle's double-precision DFT: 1e-4 L2-normalised for losses and gradients; exact zeros beyond each
 waveform's length."""
 import pytest
@@ -21,6 +21,16 @@ def test_dft_loss(res, max_len, lengths):
     assert PC.run_dft_case(res, max_len, lengths, seed=len(res) + max_len, gamma=0.8) < TOL
 
 
+@pytest.mark.parametrize("dis_type", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("res,max_len,lengths", [
+    ([(64, 40, 10)], 333, [333, 120]),
+    ([(512, 512, 80), (128, 128, 40), (2048, 2048, 640)], 8000, [8000, 4500]),
+])
+def test_dft_other_distance_types(dis_type, res, max_len, lengths):
+    print("dft case", dis_type, res, max_len, lengths, flush=True)
+    assert PC.run_dft_case(res, max_len, lengths, seed=7 * dis_type + max_len, gamma=0.8, dis_type=dis_type) < TOL
+
+
 def test_dft_equal_signals_and_rejections():
     import torch
 
@@ -37,4 +47,4 @@ def test_dft_equal_signals_and_rejections():
     with pytest.raises(RuntimeError):
         capi.Dft([(100, 100, 25)], 1000, 1)          # not a power of two
     with pytest.raises(RuntimeError):
-        capi.Dft([(128, 128, 40)], 1000, 1, spec_dis_type=2)
+        capi.Dft([(128, 128, 40)], 1000, 1, spec_dis_type=7)   # the phase distances are not built

@@ -2,7 +2,9 @@
 numpy, and the (deliberately non-analytic) gradient against float64 autograd of an equivalent surrogate:
 the reference's gradient equals d/dx of  1/(4*B*K) * sum_k sum_b c_b d^2  with c_b = 1 for the DC and Nyquist
 bins and 2 for the others (its inverse transform counts interior bins twice and its per-bin term lacks the
-factor 4)."""
+factor 4).  The other distance types are pinned the same way; the factor between the reference's per-bin
+gradient and the true derivative of its per-bin distance is 1/4 for types 0, 2, 5, 1/2 for types 3, 4 and 1 for
+types 1, 6 (derived by hand from the distance definitions, not read off the oracle)."""
 import numpy as np
 import torch
 
@@ -42,7 +44,28 @@ def test_r2c_c2r_follow_cufft_conventions():
     assert relerr(O.dft_c2r(G.astype(np.complex64), n), brute) < 1e-6
 
 
-def surrogate(src, tgt, N, Nw, Hs, length, gamma, floor):
+def bin_distance64(dis_type, S, T, floor):
+    """Per-bin distance of every type in float64 torch, and the factor kappa with
+    reference gradient = kappa * true derivative."""
+    s2, t2 = S.abs() ** 2, T.abs() ** 2
+    if dis_type == 1:
+        s, t = torch.sqrt(s2 + 1e-5), torch.sqrt(t2 + 1e-5)
+        return t * torch.log(t / s) - t + s, 1.0
+    if dis_type == 2:
+        return (s2 - t2) ** 2, 0.25
+    if dis_type == 3:
+        return torch.log((S - T).abs() ** 2 + 1.0), 0.5
+    if dis_type == 4:
+        return (S - T).abs() ** 2, 0.5
+    if dis_type == 5:
+        return ((s2 + 1e-5) / (t2 + 1e-5) - 1.0) ** 2, 0.25
+    if dis_type == 6:
+        r = torch.sqrt(t2 + 1e-5) / torch.sqrt(s2 + 1e-5)
+        return r - torch.log(r) - 1.0, 1.0
+    return (torch.log(s2 + floor) - torch.log(t2 + floor)) ** 2, 0.25
+
+
+def surrogate(src, tgt, N, Nw, Hs, length, gamma, floor, dis_type=0):
     """float64 torch statement of the loss and of the surrogate whose autograd equals the reference gradient."""
     K = 1 if length < Nw else 1 + (length - Nw) // Hs
     B = N // 2 + 1
@@ -57,11 +80,11 @@ def surrogate(src, tgt, N, Nw, Hs, length, gamma, floor):
         return torch.fft.rfft(torch.nn.functional.pad(f, (0, N - Nw)), n=N)
 
     S, T = frames(x), frames(t)
-    d = torch.log(S.abs() ** 2 + floor) - torch.log(T.abs() ** 2 + floor)
-    loss = (d ** 2).sum() / (B * K)
+    e, kappa = bin_distance64(dis_type, S, T, floor)
+    loss = e.sum() / (B * K)
     c = torch.full((B,), 2.0, dtype=torch.float64)
     c[0] = c[-1] = 1.0
-    sur = gamma * (c * d ** 2).sum() / (4.0 * B * K)
+    sur = gamma * kappa * (c * e).sum() / (B * K)
     sur.backward()
     return float(loss.detach()), x.grad.numpy()
 
@@ -98,3 +121,42 @@ def test_equal_signals_give_zero():
     g = np.ones(300, dtype=np.float32)
     assert O.dft_logamp_loss(64, 64, 16, 0, 300, 300, 1.0, 1e-5, x, x.copy(), g) == 0.0
     assert not g.any()
+
+
+def run_type(dis_type, N, Nw, Hs, max_len, length, gamma=1.0, seed=0, tol=5e-5):
+    rng = np.random.default_rng(seed)
+    src = (0.3 * rng.standard_normal(max_len)).astype(np.float32)
+    tgt = (0.3 * rng.standard_normal(max_len)).astype(np.float32)
+    grad = np.zeros(max_len, dtype=np.float32)
+    err = O.dft_spectral_loss(dis_type, N, Nw, Hs, 0, max_len, length, gamma, 1e-5, src, tgt, grad)
+    ref_err, ref_grad = surrogate(src, tgt, N, Nw, Hs, length, gamma, 1e-5, dis_type)
+    assert abs(err - ref_err) <= tol * abs(ref_err), (dis_type, err, ref_err)
+    assert relerr(grad[:length], ref_grad) < tol, (dis_type, relerr(grad[:length], ref_grad))
+    assert not grad[length:].any()
+
+
+def test_every_distance_type_matches_its_surrogate():
+    for dis_type in range(7):
+        run_type(dis_type, 16, 16, 4, 64, 64, seed=10 + dis_type)
+        run_type(dis_type, 128, 100, 40, 1000, 900, gamma=0.7, seed=20 + dis_type)
+        run_type(dis_type, 512, 512, 80, 2000, 2000, seed=30 + dis_type)
+
+
+def test_type_zero_is_the_log_amplitude_loss():
+    rng = np.random.default_rng(40)
+    src, tgt = rng.standard_normal(500).astype(np.float32), rng.standard_normal(500).astype(np.float32)
+    g0, g1 = np.zeros(500, dtype=np.float32), np.zeros(500, dtype=np.float32)
+    e0 = O.dft_logamp_loss(64, 64, 16, 0, 500, 400, 0.5, 1e-5, src, tgt, g0)
+    e1 = O.dft_spectral_loss(0, 64, 64, 16, 0, 500, 400, 0.5, 1e-5, src, tgt, g1)
+    assert e0 == e1 and np.array_equal(g0, g1)
+
+
+def test_equal_signals_give_zero_for_every_type():
+    rng = np.random.default_rng(41)
+    x = rng.standard_normal(300).astype(np.float32)
+    for dis_type in (1, 2, 4, 5, 6):  # type 3 is log(0 + 1) = 0 as well, checked apart for its gradient
+        g = np.ones(300, dtype=np.float32)
+        assert abs(O.dft_spectral_loss(dis_type, 64, 64, 16, 0, 300, 300, 1.0, 1e-5, x, x.copy(), g)) < 1e-7
+        assert np.abs(g).max() < 1e-6
+    g = np.ones(300, dtype=np.float32)
+    assert O.dft_spectral_loss(3, 64, 64, 16, 0, 300, 300, 1.0, 1e-5, x, x.copy(), g) == 0.0 and not g.any()
