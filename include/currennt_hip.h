@@ -271,13 +271,20 @@ typedef struct {
                             spectral MSE, 4 spectral MSE, 5 amplitude ratio, 6 Itakura-Saito  */
     int max_length;      /* maxSeqLength in samples                                   */
     int max_waves;       /* waveforms per call, 1..32                                 */
+    float zeta;          /* "zeta": weight of the phase distance; 0 = none (the reference's default,
+                            layers/DFTErrorPostoutputLayer.cu:324, :613)              */
+    int phase_dis_type;  /* "phaseDisType"; 0 = cosine distance (helpers/FFTMat.cu:630-656, :862-878),
+                            the only one built                                        */
 } cnt_dft_desc;
 int cnt_dft_create(const cnt_dft_desc *desc, cnt_dft **out);
 int cnt_dft_destroy(cnt_dft *h);
 /* DFTPostoutputLayer::computeForwardPass in training mode (layers/DFTErrorPostoutputLayer.cu:1782-1839,
  * :1186-1244): computes the loss of every waveform and resolution into errors_dev[w*n_res + r] (device
  * memory) AND the gradient w.r.t. the source samples, which is kept inside the handle, as the reference
- * keeps it in m_fftDiffData.  lengths is a host array.  Samples at or beyond a waveform's length count as 0. */
+ * keeps it in m_fftDiffData.  lengths is a host array.  Samples at or beyond a waveform's length count as 0.
+ * With zeta > 0 (layers/DFTErrorPostoutputLayer.cu:1246-1295, :1672) errors_dev holds 2*n_waves*n_res floats:
+ * the phase distances follow at errors_dev[n_waves*n_res + w*n_res + r], and the kept gradient is
+ * gamma * amplitude part + zeta * phase part. */
 int cnt_dft_forward(cnt_dft *h, void *stream, int n_waves, const int *lengths, const float *source,
                     const float *target, float *errors_dev);
 /* DFTPostoutputLayer::computeBackwardPass (layers/DFTErrorPostoutputLayer.cu:1849-1885, :1699-1714):

@@ -112,6 +112,8 @@ void orc_dft_c2r(int n, const float *in, float *out);
 float orc_dft_spectral_loss(int dis_type, int fft_length, int frame_length, int frame_shift, int window_type,
                             int max_length, int length, float gamma, float log_floor, const float *source,
                             const float *target, float *grad);
+float orc_dft_phase_loss(int fft_length, int frame_length, int frame_shift, int window_type, int max_length,
+                         int length, float zeta, const float *source, const float *target, float *grad);
 float orc_dft_logamp_loss(int fft_length, int frame_length, int frame_shift, int window_type, int max_length,
                           int length, float gamma, float log_floor, const float *source, const float *target,
                           float *grad);

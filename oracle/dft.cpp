@@ -9,6 +9,9 @@
 //                                  gradients; constants helpers/FFTMat.hpp (FFT_KLD_FLOOR_NUM, FFT_IS_FLOOR_NUM,
 //                                  FFT_SPEC_LOG_MSE_CONST); double literals in the reference promote the
 //                                  expression they stand in to double, restated as such
+//   helpers/FFTMat.cu:630-656      phaseDistance (cosine distance), :862-878 PhaseGrad, drivers :1500-1636,
+//                                  :1775-1830; layers/DFTErrorPostoutputLayer.cu:1246-1295 (own framing, FFT,
+//                                  inverse FFT and collectGrad(zeta) for the phase term)
 //   helpers/FFTMat.cu:456-471      cleanDummyGradients
 //   helpers/FFTMat.cu:965-1006     collectGrad (windowed overlap-add, scale gamma / (bins * validFrames))
 //   helpers/FFTMat.cu:1137-1147    frame / bin counts;  :1152-1202 zero fill beyond the signal length
@@ -64,7 +67,8 @@ float window_product(float raw, int pos, int frame_length, int window_type) {
 }
 
 // helpers/FFTMat.hpp
-constexpr double kKldFloor = 0.00001, kIsFloor = 0.00001, kSpecLogMseConst = 1.0;
+constexpr double kKldFloor = 0.00001, kIsFloor = 0.00001, kSpecLogMseConst = 1.0, kAmpMin = 0.0000001;
+constexpr int kPhaseCos = 100;  // internal selector of the cosine phase distance
 
 // first pass of specAmpDistance (helpers/FFTMat.cu:1350-1475): x = distance, y = value kept for the gradient
 void bin_distance(int dis_type, float log_floor, float sx, float sy, float tx, float ty, float &x, float &y) {
@@ -92,6 +96,16 @@ void bin_distance(int dis_type, float log_floor, float sx, float sy, float tx, f
             y = (float)((sx * sx + sy * sy + kKldFloor) / (tx * tx + ty * ty + kKldFloor) - 1.0);
             x = y * y;
             break;
+        case kPhaseCos: {  // phaseDistance
+            y = (float)(std::sqrt(sx * sx + sy * sy) * std::sqrt(tx * tx + ty * ty));
+            if (y < kAmpMin) {
+                x = 0.0f;
+                y = (float)kAmpMin;
+            } else {
+                x = (float)(1.0 - (sx * tx + sy * ty) / y);
+            }
+            break;
+        }
         case 6: {  // SpecAmpDistance_AMP_IS
             const float sa = (float)std::sqrt(sx * sx + sy * sy + kIsFloor);
             const float ta = (float)std::sqrt(tx * tx + ty * ty + kIsFloor);
@@ -133,6 +147,13 @@ void bin_gradient(int dis_type, float log_floor, float sx, float sy, float tx, f
             const float spec = (float)(tx * tx + ty * ty + kKldFloor);
             x = keep * sx / spec;
             y = keep * sy / spec;
+            break;
+        }
+        case kPhaseCos: {  // PhaseGrad
+            const float spec = (float)(sx * sx + sy * sy + kKldFloor);
+            const float fac = (sy * tx - sx * ty) / keep;
+            x = (float)(fac * (-1.0) * sy / spec);
+            y = fac * sx / spec;
             break;
         }
         case 6: {  // SpecAmpDistance_AMP_IS_Grad
@@ -235,6 +256,13 @@ float orc_dft_spectral_loss(int dis_type, int fft_length, int frame_length, int 
         grad[t] = acc * scale;
     }
     return err;
+}
+
+// the phase term of one resolution: distance and gradient scaled by zeta
+float orc_dft_phase_loss(int fft_length, int frame_length, int frame_shift, int window_type, int max_length,
+                         int length, float zeta, const float *source, const float *target, float *grad) {
+    return orc_dft_spectral_loss(kPhaseCos, fft_length, frame_length, frame_shift, window_type, max_length, length,
+                                 zeta, 0.0f, source, target, grad);
 }
 
 float orc_dft_logamp_loss(int fft_length, int frame_length, int frame_shift, int window_type, int max_length,

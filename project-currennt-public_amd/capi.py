@@ -26,7 +26,8 @@ class CnnDesc(C.Structure):
 class DftDesc(C.Structure):
     _fields_ = [("n_res", C.c_int), ("fft_length", C.c_int * 3), ("frame_length", C.c_int * 3),
                 ("frame_shift", C.c_int * 3), ("window_type", C.c_int * 3), ("gamma", C.c_float),
-                ("log_floor", C.c_float), ("spec_dis_type", C.c_int), ("max_length", C.c_int), ("max_waves", C.c_int)]
+                ("log_floor", C.c_float), ("spec_dis_type", C.c_int), ("max_length", C.c_int), ("max_waves", C.c_int),
+                ("zeta", C.c_float), ("phase_dis_type", C.c_int)]
 
 
 class DatasetDesc(C.Structure):
@@ -405,13 +406,15 @@ def skipadd_backward(errors, errors_from_skip, targets, is_skip, stream=None):
 class Dft:
     """Thin owner of a cnt_dft handle.  resolutions: list of (fftLength, frameLength, frameShift)."""
 
-    def __init__(self, resolutions, max_length, max_waves, gamma=1.0, log_floor=1e-5, window_type=0, spec_dis_type=0):
+    def __init__(self, resolutions, max_length, max_waves, gamma=1.0, log_floor=1e-5, window_type=0, spec_dis_type=0,
+                 zeta=0.0, phase_dis_type=0):
         d = DftDesc()
         d.n_res = len(resolutions)
         for r, (n, nw, hs) in enumerate(resolutions[:3]):
             d.fft_length[r], d.frame_length[r], d.frame_shift[r], d.window_type[r] = n, nw, hs, window_type
         d.gamma, d.log_floor, d.spec_dis_type = gamma, log_floor, spec_dis_type
         d.max_length, d.max_waves = max_length, max_waves
+        d.zeta, d.phase_dis_type = zeta, phase_dis_type
         self.n_res = d.n_res
         self.handle = VP()
         check(lib().cnt_dft_create(C.byref(d), C.byref(self.handle)))

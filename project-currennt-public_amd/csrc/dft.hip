@@ -36,11 +36,12 @@ struct DftParams {
     int n_waves, n_res, res;
     int lengths[kMaxWavesPerLaunch];
     float gamma, log_floor;
+    float zeta;          // weight of the cosine phase distance; 0 = not evaluated
     const float2 *twiddle;  // N/2 entries exp(-2*pi*i*k/N)
     const float *window;    // Nw entries
     const float *source, *target;
     float *grad;    // n_waves x max_length, accumulated over resolutions
-    float *errors;  // n_waves x n_res
+    float *errors;  // n_waves x n_res amplitude distances, followed by n_waves x n_res phase distances if zeta > 0
 };
 
 __host__ __device__ inline int frame_count(int length, int Nw, int Hs) {
@@ -104,6 +105,24 @@ __device__ inline void bin_distance(float sx, float sy, float tx, float ty, floa
     }
 }
 
+// Cosine phase distance 1 - cos(arg S - arg T) of one bin and its gradient spectrum (helpers/FFTMat.cu:630-656
+// phaseDistance, :862-878 PhaseGrad; FFT_AMP_MIN_NUM floors the amplitude product, FFT_KLD_FLOOR_NUM the
+// gradient's denominator).
+constexpr float kAmpMin = 0.0000001f;
+__device__ inline void bin_phase(float sx, float sy, float tx, float ty, float &e, float &gx, float &gy) {
+    float amp = sqrtf(sx * sx + sy * sy) * sqrtf(tx * tx + ty * ty);
+    if (amp < kAmpMin) {
+        e = 0.0f;
+        amp = kAmpMin;
+    } else {
+        e = 1.0f - (sx * tx + sy * ty) / amp;
+    }
+    const float spec = sx * sx + sy * sy + kKldFloor;
+    const float fac = (sy * tx - sx * ty) / amp;
+    gx = -fac * sy / spec;
+    gy = fac * sx / spec;
+}
+
 template <int LOGN, int DIS>
 __global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
     constexpr int N = 1 << LOGN;
@@ -112,7 +131,7 @@ __global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
     constexpr int FPB = 256 / TPF;                // frames per block
     __shared__ float2 z[FPB][N];
     __shared__ float2 tw[HALF];
-    __shared__ float err_part[4];
+    __shared__ float err_part[2][4];
 
     const int tid = threadIdx.x;
     const int fl = tid / TPF, ft = tid % TPF;  // frame slot in the block, thread within the frame
@@ -153,7 +172,10 @@ __global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
     }
 
     // per-bin stage on the pairs (b, N-b); bin b lives at position bitrev(b)
-    float err = 0.0f;
+    // With the phase term both gradient spectra are weighted here and share the inverse transform (the reference
+    // runs a second framing / FFT / inverse FFT / overlap-add for it, layers/DFTErrorPostoutputLayer.cu:1246-1295).
+    const bool phase = p.zeta > 0.0f;
+    float err = 0.0f, err_ph = 0.0f;
     for (int b = ft; b <= HALF; b += TPF) {
         const int nb = (N - b) & (N - 1);
         const int pb = (int)(__brev((unsigned)b) >> (32 - LOGN));
@@ -165,6 +187,13 @@ __global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
         float e, gx, gy;
         bin_distance<DIS>(sx, sy, tx, ty, p.log_floor, e, gx, gy);
         if (active) err += e;
+        if (phase) {
+            float pe, px, py;
+            bin_phase(sx, sy, tx, ty, pe, px, py);
+            if (active) err_ph += pe;
+            gx = p.gamma * gx + p.zeta * px;
+            gy = p.gamma * gy + p.zeta * py;
+        }
         if (b == 0 || b == HALF) {
             z[fl][pb] = make_float2(gx, 0.0f);
         } else {
@@ -193,19 +222,25 @@ __global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
     // windowed overlap-add; frames at or beyond Kvalid contribute nothing
     const float inv = 1.0f / (float)((HALF + 1) * Kvalid);
     if (active) {
-        const float scale = p.gamma * inv;
+        const float scale = phase ? inv : p.gamma * inv;
         float *g = p.grad + (size_t)wave_id * p.max_length;
         for (int j = ft; j < p.Nw; j += TPF) {
             const int pos = k * p.Hs + j;
             if (pos < length) atomicAdd(&g[pos], scale * z[fl][j].x * p.window[j]);
         }
     }
-    for (int o = 32; o > 0; o >>= 1) err += __shfl_xor(err, o);
-    if ((tid & 63) == 0) err_part[tid >> 6] = err;
+    for (int o = 32; o > 0; o >>= 1) {
+        err += __shfl_xor(err, o);
+        err_ph += __shfl_xor(err_ph, o);
+    }
+    if ((tid & 63) == 0) {
+        err_part[0][tid >> 6] = err;
+        err_part[1][tid >> 6] = err_ph;
+    }
     __syncthreads();
-    if (tid == 0) {
-        const float e = (err_part[0] + err_part[1] + err_part[2] + err_part[3]) * inv;
-        if (e != 0.0f) atomicAdd(&p.errors[wave_id * p.n_res + p.res], e);
+    if (tid < 2 && (tid == 0 || phase)) {
+        const float e = (err_part[tid][0] + err_part[tid][1] + err_part[tid][2] + err_part[tid][3]) * inv;
+        if (e != 0.0f) atomicAdd(&p.errors[tid * p.n_waves * p.n_res + wave_id * p.n_res + p.res], e);
     }
 }
 
@@ -284,6 +319,9 @@ int cnt_dft_create(const cnt_dft_desc *desc, cnt_dft **out) {
     // distances 0..6; its phase distances are a separate driver and are not built
     CNT_REQUIRE(desc->spec_dis_type >= 0 && desc->spec_dis_type <= 6, "dft_create: specDisType %d outside 0..6",
                 desc->spec_dis_type);
+    CNT_REQUIRE(desc->zeta >= 0.0f, "dft_create: negative zeta");
+    CNT_REQUIRE(desc->zeta == 0.0f || desc->phase_dis_type == 0,
+                "dft_create: phaseDisType %d; only 0 (cosine distance) is built", desc->phase_dis_type);
     cnt_dft *h = new (std::nothrow) cnt_dft();
     CNT_REQUIRE(h != nullptr, "dft_create: out of host memory");
     std::memset(h, 0, sizeof(*h));
@@ -333,6 +371,7 @@ static void fill_params(const cnt_dft *h, cnt::DftParams &p) {
     for (int w = 0; w < h->n_waves; ++w) p.lengths[w] = h->lengths[w];
     p.gamma = h->desc.gamma;
     p.log_floor = h->desc.log_floor;
+    p.zeta = h->desc.zeta;
     p.grad = h->grad;
 }
 
@@ -349,7 +388,7 @@ int cnt_dft_forward(cnt_dft *h, void *stream_, int n_waves, const int *lengths, 
     h->n_waves = n_waves;
     for (int w = 0; w < n_waves; ++w) h->lengths[w] = lengths[w];
     CNT_TRY(fill_zero(stream, h->grad, (size_t)n_waves * h->desc.max_length));
-    CNT_TRY(fill_zero(stream, errors_dev, (size_t)n_waves * h->desc.n_res));
+    CNT_TRY(fill_zero(stream, errors_dev, (size_t)n_waves * h->desc.n_res * (h->desc.zeta > 0.0f ? 2 : 1)));
     int max_len = 0;
     for (int w = 0; w < n_waves; ++w) max_len = lengths[w] > max_len ? lengths[w] : max_len;
     for (int r = 0; r < h->desc.n_res; ++r) {

@@ -71,6 +71,7 @@ def lib():
         L.orc_sigmoid_error.restype = C.c_float
         L.orc_dft_logamp_loss.restype = C.c_float
         L.orc_dft_spectral_loss.restype = C.c_float
+        L.orc_dft_phase_loss.restype = C.c_float
         L.orc_opt_next_beta_accum.restype = C.c_float
         L.orc_opt_next_beta_accum.argtypes = [C.c_float, C.c_int]
         _lib = L
@@ -237,6 +238,11 @@ def dft_logamp_loss(N, Nw, Hs, window_type, max_len, length, gamma, floor, src, 
 def dft_spectral_loss(dis_type, N, Nw, Hs, window_type, max_len, length, gamma, floor, src, tgt, grad):
     return float(lib().orc_dft_spectral_loss(int(dis_type), N, Nw, Hs, window_type, max_len, length, C.c_float(gamma),
                                              C.c_float(floor), fptr(src), fptr(tgt), fptr(grad)))
+
+
+def dft_phase_loss(N, Nw, Hs, window_type, max_len, length, zeta, src, tgt, grad):
+    return float(lib().orc_dft_phase_loss(N, Nw, Hs, window_type, max_len, length, C.c_float(zeta), fptr(src),
+                                          fptr(tgt), fptr(grad)))
 
 
 def opt_accumulate(layer_updates, cur_updates, add):

@@ -522,7 +522,7 @@ def run_skipadd_case(n, seed):
     return 0.0
 
 
-def run_dft_case(resolutions, max_len, lengths, seed, gamma=1.0, dis_type=0):
+def run_dft_case(resolutions, max_len, lengths, seed, gamma=1.0, dis_type=0, zeta=0.0):
     """Multi-resolution DFT loss: per-resolution losses and the summed gradient against the oracle."""
     import torch
 
@@ -531,23 +531,28 @@ def run_dft_case(resolutions, max_len, lengths, seed, gamma=1.0, dis_type=0):
     W = len(lengths)
     src = (0.3 * rng.standard_normal((W, max_len))).astype(np.float32)
     tgt = (0.3 * rng.standard_normal((W, max_len))).astype(np.float32)
-    err_o = np.zeros((W, len(resolutions)))
+    err_o = np.zeros((2 if zeta > 0 else 1, W, len(resolutions)))
     grad_o = np.zeros((W, max_len), dtype=np.float64)
     for w in range(W):
         for r, (N, Nw, Hs) in enumerate(resolutions):
             g = np.zeros(max_len, dtype=np.float32)
-            err_o[w, r] = O.dft_spectral_loss(dis_type, N, Nw, Hs, 0, max_len, lengths[w], gamma, 1e-5, src[w].copy(),
+            err_o[0, w, r] = O.dft_spectral_loss(dis_type, N, Nw, Hs, 0, max_len, lengths[w], gamma, 1e-5, src[w].copy(),
                                               tgt[w].copy(), g)
             g[lengths[w]:] = 0  # the layer only passes on the first `length` samples
             grad_o[w] += g
-    layer = capi.Dft(resolutions, max_len, W, gamma=gamma, spec_dis_type=dis_type)
-    err_d = torch.full((W * len(resolutions),), 7.0, dtype=torch.float32, device="cuda")
+            if zeta > 0:
+                err_o[1, w, r] = O.dft_phase_loss(N, Nw, Hs, 0, max_len, lengths[w], zeta, src[w].copy(), tgt[w].copy(), g)
+                g[lengths[w]:] = 0
+                grad_o[w] += g
+    layer = capi.Dft(resolutions, max_len, W, gamma=gamma, spec_dis_type=dis_type, zeta=zeta)
+    err_d = torch.full((err_o.size,), 7.0, dtype=torch.float32, device="cuda")
     prev_d = torch.full((W * max_len,), 7.0, dtype=torch.float32, device="cuda")
     layer.forward(lengths, dev(src.reshape(-1)), dev(tgt.reshape(-1)), err_d)
     layer.backward(prev_d)
     torch.cuda.synchronize()
     got_g = prev_d.cpu().numpy().reshape(W, max_len)
-    worst = relerr(err_d.cpu().numpy(), err_o)
+    got_e = err_d.cpu().numpy().reshape(err_o.shape)
+    worst = max(relerr(got_e[i], err_o[i]) for i in range(err_o.shape[0]))
     for w in range(W):
         worst = max(worst, relerr(got_g[w], grad_o[w]))
         assert not got_g[w, lengths[w]:].any()

@@ -31,6 +31,16 @@ def test_dft_other_distance_types(dis_type, res, max_len, lengths):
     assert PC.run_dft_case(res, max_len, lengths, seed=7 * dis_type + max_len, gamma=0.8, dis_type=dis_type) < TOL
 
 
+@pytest.mark.parametrize("dis_type,gamma,zeta", [(0, 0.8, 0.5), (4, 1.0, 2.0), (0, 0.0, 1.0)])
+@pytest.mark.parametrize("res,max_len,lengths", [
+    ([(64, 40, 10)], 333, [333, 120]),
+    ([(512, 512, 80), (128, 128, 40), (2048, 2048, 640)], 8000, [8000, 4500]),
+])
+def test_dft_with_phase_distance(dis_type, gamma, zeta, res, max_len, lengths):
+    print("dft phase case", dis_type, gamma, zeta, res, max_len, lengths, flush=True)
+    assert PC.run_dft_case(res, max_len, lengths, seed=3 + max_len, gamma=gamma, dis_type=dis_type, zeta=zeta) < TOL
+
+
 def test_dft_equal_signals_and_rejections():
     import torch
 
@@ -47,4 +57,6 @@ def test_dft_equal_signals_and_rejections():
     with pytest.raises(RuntimeError):
         capi.Dft([(100, 100, 25)], 1000, 1)          # not a power of two
     with pytest.raises(RuntimeError):
-        capi.Dft([(128, 128, 40)], 1000, 1, spec_dis_type=7)   # the phase distances are not built
+        capi.Dft([(128, 128, 40)], 1000, 1, spec_dis_type=7)   # no such amplitude distance
+    with pytest.raises(RuntimeError):
+        capi.Dft([(128, 128, 40)], 1000, 1, zeta=1.0, phase_dis_type=1)   # instantaneous phase is not built

@@ -62,6 +62,11 @@ def bin_distance64(dis_type, S, T, floor):
     if dis_type == 6:
         r = torch.sqrt(t2 + 1e-5) / torch.sqrt(s2 + 1e-5)
         return r - torch.log(r) - 1.0, 1.0
+    if dis_type == "phase":
+        # 1 - cos(arg S - arg T); the reference divides its gradient by |S|^2 + 1e-5 where the derivative has
+        # |S|^2, which the detached weight restores
+        e = 1.0 - (S.real * T.real + S.imag * T.imag) / (S.abs() * T.abs())
+        return e, (s2 / (s2 + 1e-5)).detach()
     return (torch.log(s2 + floor) - torch.log(t2 + floor)) ** 2, 0.25
 
 
@@ -84,7 +89,7 @@ def surrogate(src, tgt, N, Nw, Hs, length, gamma, floor, dis_type=0):
     loss = e.sum() / (B * K)
     c = torch.full((B,), 2.0, dtype=torch.float64)
     c[0] = c[-1] = 1.0
-    sur = gamma * kappa * (c * e).sum() / (B * K)
+    sur = gamma * (kappa * c * e).sum() / (B * K)
     sur.backward()
     return float(loss.detach()), x.grad.numpy()
 
@@ -160,3 +165,21 @@ def test_equal_signals_give_zero_for_every_type():
         assert np.abs(g).max() < 1e-6
     g = np.ones(300, dtype=np.float32)
     assert O.dft_spectral_loss(3, 64, 64, 16, 0, 300, 300, 1.0, 1e-5, x, x.copy(), g) == 0.0 and not g.any()
+
+
+def test_cosine_phase_distance_matches_its_surrogate():
+    for N, Nw, Hs, max_len, length, zeta, seed in ((16, 16, 4, 64, 64, 1.0, 50), (128, 100, 40, 1000, 900, 0.6, 51),
+                                                  (512, 512, 80, 2000, 2000, 2.0, 52)):
+        rng = np.random.default_rng(seed)
+        src = (0.3 * rng.standard_normal(max_len)).astype(np.float32)
+        tgt = (0.3 * rng.standard_normal(max_len)).astype(np.float32)
+        grad = np.zeros(max_len, dtype=np.float32)
+        err = O.dft_phase_loss(N, Nw, Hs, 0, max_len, length, zeta, src, tgt, grad)
+        ref_err, ref_grad = surrogate(src, tgt, N, Nw, Hs, length, zeta, 0.0, "phase")
+        assert abs(err - ref_err) <= 5e-5 * abs(ref_err)
+        assert relerr(grad[:length], ref_grad) < 5e-5
+    # opposite signals: every bin has distance 1 - cos(pi) = 2, and the gradient vanishes
+    x = np.random.default_rng(53).standard_normal(300).astype(np.float32)
+    g = np.ones(300, dtype=np.float32)
+    assert abs(O.dft_phase_loss(64, 64, 16, 0, 300, 300, 1.0, x, -x, g) - 2.0) < 1e-5
+    assert np.abs(g).max() < 1e-5
