@@ -291,6 +291,71 @@ int cnt_dft_forward(cnt_dft *h, void *stream, int n_waves, const int *lengths, c
  * prev_errors (n_waves x max_length) = sum over resolutions of the stored gradients, 0 beyond each length. */
 int cnt_dft_backward(cnt_dft *h, void *stream, float *prev_errors);
 
+/* ---- network sequencer ------------------------------------------------------------------------------
+ * NeuralNetwork<TDevice> for the layer types of this library (NeuralNetwork.cpp): "input", "feedforward_identity /
+ * _tanh / _logistic / _relu", "lstm", "blstm", "skipini", "skipadd" (with "preSkipLayer"), "cnn" (1-D), "wavnetc",
+ * "feedback" (one step back, fed by one softmax unit) and the post-output layers "sse" and "mdn".  json_text is the
+ * text of a network file: "layers" in order, optionally "weights" with the "input" / "bias" / "internal" arrays of
+ * every trainable layer (layers/TrainableLayer.cu:135-220).  Without "weights" the weights are zero until the caller
+ * fills them (cnt_network_weights, cnt_network_randomize).  All weights of the network, and all weight updates, are
+ * one device array each, layers in file order, each layer's vector in the layout of its own entry points above. */
+typedef struct cnt_network cnt_network;
+typedef struct {
+    const float *mdn_config; /* content of the --mdn_config file (see cnt_mdn_create); NULL without an mdn layer */
+    int mdn_config_len;
+    int tie_variance;        /* --tieVariance; only 0 is supported                                               */
+    int no_overlap;          /* != 0: weight gradients on the caller's stream instead of a second stream         */
+} cnt_network_options;
+typedef struct {
+    char name[64];
+    char type[32];
+    int size;
+    long weight_offset;              /* of this layer inside the network's weight array            */
+    long n_input, n_bias, n_internal; /* lengths of the three sections of its weight vector         */
+    float *outputs;                  /* device, size x (maxSeqLength*S); a post-output layer keeps the targets here */
+    float *output_errors;            /* device, same shape; NULL for the input and post-output layers */
+} cnt_layer_info;
+/* NeuralNetwork::NeuralNetwork (NeuralNetwork.cpp:374-609, :805-812).  options may be NULL. */
+int cnt_network_create(const char *json_text, int parallel_sequences, int max_seq_length,
+                       const cnt_network_options *options, cnt_network **out);
+int cnt_network_destroy(cnt_network *net);
+int cnt_network_info(cnt_network *net, int *n_layers, int *input_size, int *output_size, long *n_weights);
+int cnt_network_layer_info(cnt_network *net, int index, cnt_layer_info *info);
+float *cnt_network_weights(cnt_network *net);        /* device, n_weights floats */
+float *cnt_network_weight_updates(cnt_network *net); /* device, n_weights floats */
+/* Uniform weights in (-range, range) from a seeded Mersenne twister (the reference draws from its own generator,
+ * layers/TrainableLayer.cu:221-300; the streams differ). */
+int cnt_network_randomize(cnt_network *net, unsigned seed, float range);
+/* Conditioning features of the wavnetc layers, contextDim x (maxSeqLength*S) in device memory, one column per
+ * slot (what the reference's first wavnetc layer builds in m_contextBuf from the layer flagged
+ * "wavenetConditionInputLayer", layers/wavNetCore.cu:455-492; cnt_wavnetc_load_context does that step).  The
+ * pointer is kept, not the data. */
+int cnt_network_set_context(cnt_network *net, const float *ctx);
+/* NeuralNetwork::loadSequences (NeuralNetwork.cpp:1367-1417): records the fraction's geometry and pattern types
+ * (device memory, char[T*S], kept by pointer), copies inputs (input size x T*S) and targets (post-output size x T*S)
+ * when given, and passes the call on to the layers that keep per-fraction state. */
+int cnt_network_load_sequences(cnt_network *net, void *stream, int T, int Tmin, const char *patTypes,
+                               const float *inputs, const float *targets);
+/* NeuralNetwork::computeForwardPass in training mode (NeuralNetwork.cpp:1419-1471, :1734-1760). */
+int cnt_network_forward(cnt_network *net, void *stream);
+/* NeuralNetwork::calculateError (NeuralNetwork.cpp:2897-2990): the post-output layer's error into *loss_dev. */
+int cnt_network_calculate_error(cnt_network *net, void *stream, float *loss_dev);
+/* NeuralNetwork::computeBackwardPass (NeuralNetwork.cpp:2744-2800, :2864-2895): layers in reverse order; on
+ * return the caller's stream has been made to wait for the second stream, so weight updates are complete in
+ * stream order. */
+int cnt_network_backward(cnt_network *net, void *stream);
+/* cnt_lstm_check for every LSTM layer. */
+int cnt_network_check(cnt_network *net, void *stream);
+/* One optimizer step over all weights in a single launch (see cnt_opt_step; the network keeps the optimizer's
+ * current updates, deltas, statistics and Adam's accumulated betas).  Layer-specific learning rates
+ * ("learningRate" of a layer) are not built. */
+int cnt_network_update(cnt_network *net, void *stream, int option, float learning_rate, float momentum,
+                       float frac_length);
+/* NeuralNetwork::exportLayers + exportWeights (NeuralNetwork.cpp:2993-3040): the layer objects as they stood in the
+ * network file plus the current weights.  *needed receives the size including the terminating 0; nothing is
+ * written if cap is smaller (call once with buf = NULL to learn the size). */
+int cnt_network_export_json(cnt_network *net, char *buf, size_t cap, size_t *needed);
+
 /* ---- weight update of the training loop (SURVEY "next": optimizer step on device) -----------------
  * optimizer option numbers are the reference's (MacroDefine.hpp:33-37): 0 plain SGD, 1 AdaGrad,
  * 2 gradient averaged over the fraction, 3 stochastic AdaGrad (statistics only), 4 SGD with decaying

@@ -35,6 +35,17 @@ class DatasetDesc(C.Structure):
                 ("fraction", C.c_float)]
 
 
+class NetworkOptions(C.Structure):
+    _fields_ = [("mdn_config", C.POINTER(C.c_float)), ("mdn_config_len", C.c_int), ("tie_variance", C.c_int),
+                ("no_overlap", C.c_int)]
+
+
+class LayerInfo(C.Structure):
+    _fields_ = [("name", C.c_char * 64), ("type", C.c_char * 32), ("size", C.c_int), ("weight_offset", C.c_long),
+                ("n_input", C.c_long), ("n_bias", C.c_long), ("n_internal", C.c_long), ("outputs", C.c_void_p),
+                ("output_errors", C.c_void_p)]
+
+
 class LstmDesc(C.Structure):
     _fields_ = [("P", C.c_int), ("L", C.c_int), ("bidir", C.c_int), ("S", C.c_int), ("maxT", C.c_int),
                 ("bias", C.c_float)]
@@ -105,6 +116,21 @@ _SIGNATURES = {
     "cnt_wavnetc_sum_context_grad": (I, [VP, I, I, I, I, I, VP, VP, VP, VP]),
     "cnt_gatedact_forward": (I, [VP, I, I, VP, VP, VP]),
     "cnt_gatedact_backward": (I, [VP, I, I, VP, VP, VP, VP]),
+    "cnt_network_create": (I, [C.c_char_p, I, I, C.POINTER(NetworkOptions), C.POINTER(VP)]),
+    "cnt_network_destroy": (I, [VP]),
+    "cnt_network_info": (I, [VP, C.POINTER(I), C.POINTER(I), C.POINTER(I), C.POINTER(C.c_long)]),
+    "cnt_network_layer_info": (I, [VP, I, C.POINTER(LayerInfo)]),
+    "cnt_network_weights": (VP, [VP]),
+    "cnt_network_weight_updates": (VP, [VP]),
+    "cnt_network_randomize": (I, [VP, C.c_uint, F]),
+    "cnt_network_set_context": (I, [VP, VP]),
+    "cnt_network_load_sequences": (I, [VP, VP, I, I, VP, VP, VP]),
+    "cnt_network_forward": (I, [VP, VP]),
+    "cnt_network_calculate_error": (I, [VP, VP, VP]),
+    "cnt_network_backward": (I, [VP, VP]),
+    "cnt_network_check": (I, [VP, VP]),
+    "cnt_network_update": (I, [VP, VP, I, F, F, F]),
+    "cnt_network_export_json": (I, [VP, C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]),
     "cnt_skipadd_forward": (I, [VP, C.c_long, I, C.POINTER(VP), VP, VP, VP]),
     "cnt_skipadd_backward": (I, [VP, C.c_long, VP, VP, I, C.POINTER(VP), C.POINTER(I)]),
 }
@@ -401,6 +427,114 @@ def skipadd_backward(errors, errors_from_skip, targets, is_skip, stream=None):
     flags = (I * len(is_skip))(*[int(v) for v in is_skip])
     check(lib().cnt_skipadd_backward(stream_ptr(stream), errors.numel(), ptr(errors), ptr(errors_from_skip),
                                      len(targets), _ptr_array(targets), flags))
+
+
+class Network:
+    """Thin owner of a cnt_network handle (the C++ sequencer).  Device memory belongs to the handle; `weights`,
+    `updates`, and a layer's `outputs` / `errors` are torch views of it (no copies)."""
+
+    def __init__(self, json_text, parallel_sequences, max_seq_length, mdn_config=None, overlap=True):
+        import torch
+
+        self.S, self.maxT = parallel_sequences, max_seq_length
+        opt = NetworkOptions()
+        self._cfg = None
+        if mdn_config is not None:
+            self._cfg = (F * len(mdn_config))(*[float(v) for v in mdn_config])
+            opt.mdn_config, opt.mdn_config_len = self._cfg, len(mdn_config)
+        opt.no_overlap = 0 if overlap else 1
+        self.handle = VP()
+        check(lib().cnt_network_create(json_text.encode(), parallel_sequences, max_seq_length, C.byref(opt),
+                                       C.byref(self.handle)))
+        n_layers, n_in, n_out, n_w = I(), I(), I(), C.c_long()
+        check(lib().cnt_network_info(self.handle, C.byref(n_layers), C.byref(n_in), C.byref(n_out), C.byref(n_w)))
+        self.n_layers, self.input_size, self.output_size, self.n_weights = n_layers.value, n_in.value, n_out.value, n_w.value
+        self.weights = _device_view(lib().cnt_network_weights(self.handle), self.n_weights, self)
+        self.updates = _device_view(lib().cnt_network_weight_updates(self.handle), self.n_weights, self)
+        self.layers = []
+        slots = parallel_sequences * max_seq_length
+        for i in range(self.n_layers):
+            info = LayerInfo()
+            check(lib().cnt_network_layer_info(self.handle, i, C.byref(info)))
+            n = info.n_input + info.n_bias + info.n_internal
+            self.layers.append({
+                "name": info.name.decode(), "type": info.type.decode(), "size": info.size,
+                "weight_offset": info.weight_offset, "weight_count": n,
+                "sections": (info.n_input, info.n_bias, info.n_internal),
+                "outputs": _device_view(info.outputs, info.size * slots, self),
+                "errors": _device_view(info.output_errors, info.size * slots, self),
+                "weights": self.weights[info.weight_offset:info.weight_offset + n] if n else None,
+                "updates": self.updates[info.weight_offset:info.weight_offset + n] if n else None,
+            })
+        self.loss = torch.zeros(1, dtype=torch.float32, device="cuda")
+
+    def layer(self, name):
+        for L in self.layers:
+            if L["name"] == name:
+                return L
+        raise KeyError(name)
+
+    def close(self):
+        if self.handle:
+            lib().cnt_network_destroy(self.handle)
+            self.handle = VP()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def randomize(self, seed, weight_range):
+        check(lib().cnt_network_randomize(self.handle, seed, weight_range))
+
+    def set_context(self, ctx):
+        self._ctx = ctx  # the library keeps the pointer only
+        check(lib().cnt_network_set_context(self.handle, ptr(ctx)))
+
+    def load_sequences(self, pat, T, Tmin, inputs=None, targets=None, stream=None):
+        self._pat = pat
+        check(lib().cnt_network_load_sequences(self.handle, stream_ptr(stream), T, Tmin, ptr(pat), ptr(inputs),
+                                               ptr(targets)))
+
+    def forward(self, stream=None):
+        check(lib().cnt_network_forward(self.handle, stream_ptr(stream)))
+
+    def calculate_error(self, stream=None):
+        check(lib().cnt_network_calculate_error(self.handle, stream_ptr(stream), ptr(self.loss)))
+        return self.loss
+
+    def backward(self, stream=None):
+        check(lib().cnt_network_backward(self.handle, stream_ptr(stream)))
+
+    def check(self, stream=None):
+        check(lib().cnt_network_check(self.handle, stream_ptr(stream)))
+
+    def update(self, option, learning_rate, momentum, frac_length, stream=None):
+        check(lib().cnt_network_update(self.handle, stream_ptr(stream), option, learning_rate, momentum, frac_length))
+
+    def export_json(self):
+        need = C.c_size_t()
+        check(lib().cnt_network_export_json(self.handle, None, 0, C.byref(need)))
+        buf = C.create_string_buffer(need.value)
+        check(lib().cnt_network_export_json(self.handle, buf, need.value, C.byref(need)))
+        return buf.value.decode()
+
+
+def _device_view(address, count, owner):
+    """float32 torch tensor over `count` floats of device memory that `owner` keeps alive (None for a null pointer)."""
+    import torch
+
+    if not address or count == 0:
+        return None
+
+    class _Span:
+        pass
+
+    span = _Span()
+    span.__cuda_array_interface__ = {"shape": (count,), "typestr": "<f4", "data": (int(address), False), "version": 3}
+    span.owner = owner
+    return torch.as_tensor(span, device="cuda")
 
 
 class Dft:

@@ -1,0 +1,923 @@
+// Network sequencer: builds the layer list of a network file and runs forward pass, error, backward pass and
+// weight update of one fraction through the layer entry points of this library.
+//
+// Reference behaviour: NeuralNetwork.cpp (:374-609 constructor with the skip-layer and wavnetc wiring, :805-812
+// feedback link, :1367-1417 loadSequences, :1419-1471 layer-by-layer forward pass, :2744-2800 backward pass in
+// reverse order, :2897-2990 calculateError, :2993-3040 exportLayers / exportWeights), layers/TrainableLayer.cu
+// (:93-220 weight sections of a network file, :441-492 export), layers/SkipAddLayer.cu (:77-170 preSkipLayer, :186-240, :305-346),
+// layers/FeedBackLayer.cu (:60-130, :607-650, :841-865), layers/MDNUnit.cu (:753-783 one-hot of the target).
+//
+// Differences by design: all weights (and all weight updates) of a network are ONE device allocation, layers in
+// file order, so the optimizer step is a single launch; error buffers of the skip layers are one allocation
+// cleared by one launch per forward pass; a skip layer with a single source (every skipini, and a skipadd with one
+// preSkipLayer) aliases that source's outputs instead of copying them; fan-in and fan-out of a skip layer are one
+// launch each, whatever the number of linked layers (pointer tables live in device memory); the weight-gradient
+// halves of dense and LSTM layers run on a second stream of the same priority.
+#include "common.hpp"
+
+#include <cerrno>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <random>
+#include <string>
+#include <utility>
+#include <vector>
+
+namespace cnt {
+namespace json {
+
+// A small JSON reader: objects, arrays of objects, arrays of numbers (kept as floats), strings, numbers, literals.
+struct Value {
+    enum Type { NUL, BOOL, NUM, STR, ARR, NUMS, OBJ } type = NUL;
+    double num = 0.0;
+    bool flag = false;
+    std::string str;
+    std::vector<Value> arr;
+    std::vector<float> nums;
+    std::vector<std::pair<std::string, Value>> obj;
+    size_t begin = 0, end = 0;  // extent in the source text
+
+    const Value *get(const char *key) const {
+        if (type != OBJ) return nullptr;
+        for (const auto &kv : obj)
+            if (kv.first == key) return &kv.second;
+        return nullptr;
+    }
+    bool has(const char *key) const { return get(key) != nullptr; }
+};
+
+struct Parser {
+    const char *s;
+    size_t n, i = 0;
+    std::string error;
+
+    bool fail(const char *what) {
+        if (error.empty()) {
+            char buf[160];
+            snprintf(buf, sizeof(buf), "%s at offset %zu", what, i);
+            error = buf;
+        }
+        return false;
+    }
+    void ws() {
+        while (i < n && (s[i] == ' ' || s[i] == '\t' || s[i] == '\n' || s[i] == '\r')) ++i;
+    }
+    bool string(std::string &out) {
+        if (i >= n || s[i] != '"') return fail("expected a string");
+        ++i;
+        out.clear();
+        while (i < n && s[i] != '"') {
+            char c = s[i++];
+            if (c == '\\') {
+                if (i >= n) return fail("unfinished escape");
+                const char e = s[i++];
+                switch (e) {
+                    case 'n': c = '\n'; break;
+                    case 't': c = '\t'; break;
+                    case 'r': c = '\r'; break;
+                    case 'b': c = '\b'; break;
+                    case 'f': c = '\f'; break;
+                    case 'u': {  // names and options of a network file are ASCII; keep the low byte
+                        if (i + 4 > n) return fail("unfinished \\u escape");
+                        c = (char)strtol(std::string(s + i, 4).c_str(), nullptr, 16);
+                        i += 4;
+                        break;
+                    }
+                    default: c = e;
+                }
+            }
+            out.push_back(c);
+        }
+        if (i >= n) return fail("unterminated string");
+        ++i;
+        return true;
+    }
+    bool number(double &out) {
+        char *endp = nullptr;
+        errno = 0;
+        out = strtod(s + i, &endp);
+        if (endp == s + i) return fail("expected a number");
+        i = (size_t)(endp - s);
+        return true;
+    }
+    bool value(Value &v, int depth) {
+        if (depth > 16) return fail("nesting too deep");
+        ws();
+        if (i >= n) return fail("unexpected end of text");
+        v.begin = i;
+        const char c = s[i];
+        if (c == '{') {
+            v.type = Value::OBJ;
+            ++i;
+            ws();
+            if (i < n && s[i] == '}') {
+                ++i;
+            } else {
+                for (;;) {
+                    ws();
+                    std::string key;
+                    if (!string(key)) return false;
+                    ws();
+                    if (i >= n || s[i] != ':') return fail("expected ':'");
+                    ++i;
+                    v.obj.emplace_back(std::move(key), Value());
+                    if (!value(v.obj.back().second, depth + 1)) return false;
+                    ws();
+                    if (i < n && s[i] == ',') { ++i; continue; }
+                    if (i < n && s[i] == '}') { ++i; break; }
+                    return fail("expected ',' or '}'");
+                }
+            }
+        } else if (c == '[') {
+            ++i;
+            ws();
+            v.type = Value::ARR;
+            if (i < n && s[i] == ']') {
+                ++i;
+            } else {
+                const bool numeric = (s[i] == '-' || s[i] == '+' || (s[i] >= '0' && s[i] <= '9'));
+                if (numeric) v.type = Value::NUMS;
+                for (;;) {
+                    ws();
+                    if (numeric) {
+                        double d;
+                        if (!number(d)) return false;
+                        v.nums.push_back((float)d);
+                    } else {
+                        v.arr.emplace_back();
+                        if (!value(v.arr.back(), depth + 1)) return false;
+                    }
+                    ws();
+                    if (i < n && s[i] == ',') { ++i; continue; }
+                    if (i < n && s[i] == ']') { ++i; break; }
+                    return fail("expected ',' or ']'");
+                }
+            }
+        } else if (c == '"') {
+            v.type = Value::STR;
+            if (!string(v.str)) return false;
+        } else if (!strncmp(s + i, "true", 4)) {
+            v.type = Value::BOOL; v.flag = true; i += 4;
+        } else if (!strncmp(s + i, "false", 5)) {
+            v.type = Value::BOOL; v.flag = false; i += 5;
+        } else if (!strncmp(s + i, "null", 4)) {
+            v.type = Value::NUL; i += 4;
+        } else {
+            v.type = Value::NUM;
+            if (!number(v.num)) return false;
+        }
+        v.end = i;
+        return true;
+    }
+};
+
+}  // namespace json
+
+namespace {
+
+enum Kind { K_INPUT, K_DENSE, K_LSTM, K_SKIPINI, K_SKIPADD, K_CNN, K_WAVNETC, K_FEEDBACK, K_SSE, K_MDN };
+
+inline bool is_skip_kind(int k) { return k == K_SKIPINI || k == K_SKIPADD; }
+
+struct NetLayer {
+    std::string name, type, text;  // text: the layer's object as it stands in the network file
+    int kind = K_INPUT;
+    int size = 0, prev = -1;
+    float bias = 0.0f;
+    int act = 0, bidir = 0;
+    std::vector<int> pre;  // skip layers: linked source layers
+    long w_off = 0, n_in = 0, n_bias = 0, n_int = 0;
+    float *out = nullptr, *err = nullptr, *eskip = nullptr;
+    cnt_lstm *lstm = nullptr;
+    cnt_cnn *cnn = nullptr;
+    cnt_mdn *mdn = nullptr;
+    float *core = nullptr, *cth = nullptr;  // wavnetc
+    int ctx_dim = 0;
+    int fb_start = 0, fb_end = 0;            // feedback: dimensions taken from the preceding layer
+    const float **in_ptrs = nullptr;         // skip layers: device tables
+    float **tgt_ptrs = nullptr;
+    int *tgt_is_skip = nullptr;
+    long weight_count() const { return n_in + n_bias + n_int; }
+};
+
+inline int blocks_for(size_t count) {
+    size_t b = (count + 255) / 256;
+    if (b > 4096) b = 4096;
+    return (int)(b < 1 ? 1 : b);
+}
+
+__global__ void skip_sum_kernel(size_t count, int n, const float *const *__restrict__ in, float *__restrict__ out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        float acc = 0.0f;
+        for (int k = 0; k < n; ++k) acc += in[k][i];
+        out[i] = acc;
+    }
+}
+
+// errors += errors_from_skip, then to every linked source in reverse order: added to a skip layer's side buffer,
+// written over any other layer's error buffer (layers/SkipAddLayer.cu:305-346)
+__global__ void skip_fan_kernel(size_t count, int n, float *const *__restrict__ target, const int *__restrict__ is_skip,
+                                float *__restrict__ errors, const float *__restrict__ errors_from_skip) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const float e = errors_from_skip[i] + errors[i];
+        errors[i] = e;
+        for (int k = n - 1; k >= 0; --k) {
+            float *t = target[k];
+            if (t == nullptr) continue;  // a source without an error buffer (the input layer)
+            t[i] = is_skip[k] ? e + t[i] : e;
+        }
+    }
+}
+
+// FeedBackLayer::computeForwardPass in training (layers/FeedBackLayer.cu:60-130, :607-650) with look-back of one
+// step, fed by a softmax unit's ground-truth one-hot vector (layers/MDNUnit.cu:753-783): dimensions
+// [0, d1) = preceding layer's [start, start+d1); the rest = one-hot of the previous step's target class, all zero
+// for the first step and where the previous slot is padding.
+__global__ void feedback_kernel(size_t count, int dim_out, int d1, int prev_total, int prev_start, int S, int target_dim,
+                                int target_start, const char *__restrict__ pat, const float *__restrict__ prev_out,
+                                const float *__restrict__ targets, float *__restrict__ out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const long slot = (long)(i / dim_out);
+        const int d = (int)(i % dim_out);
+        float v = 0.0f;
+        if (d < d1) {
+            v = prev_out[slot * prev_total + prev_start + d];
+        } else if (slot >= S && pat[slot - S] != 0) {
+            const int cls = (int)targets[(slot - S) * target_dim + target_start];
+            v = (cls == d - d1) ? 1.0f : 0.0f;
+        }
+        out[i] = v;
+    }
+}
+
+// FeedBackLayer::computeBackwardPass (layers/FeedBackLayer.cu:338-360, :841-865)
+__global__ void feedback_backward_kernel(size_t count, int prev_total, int prev_start, int prev_end, int dim_out,
+                                         const float *__restrict__ errors, float *__restrict__ prev_errors) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const long slot = (long)(i / prev_total);
+        const int d = (int)(i % prev_total);
+        prev_errors[i] = (d >= prev_start && d < prev_end) ? errors[slot * dim_out + d - prev_start] : 0.0f;
+    }
+}
+
+// "64*1_64*2": <count>*<value> runs joined by '_' (the reference's CNN option strings); one value per filter
+bool parse_runs(const std::string &opt, int D, std::vector<int> &out) {
+    out.clear();
+    size_t i = 0;
+    while (i < opt.size()) {
+        char *endp = nullptr;
+        const long a = strtol(opt.c_str() + i, &endp, 10);
+        if (endp == opt.c_str() + i) return false;
+        i = (size_t)(endp - opt.c_str());
+        if (i < opt.size() && opt[i] == '*') {
+            ++i;
+            const long b = strtol(opt.c_str() + i, &endp, 10);
+            if (endp == opt.c_str() + i || a < 0) return false;
+            i = (size_t)(endp - opt.c_str());
+            for (long k = 0; k < a; ++k) out.push_back((int)b);
+        } else {
+            out.push_back((int)a);
+        }
+        if (i < opt.size()) {
+            if (opt[i] != '_') return false;
+            ++i;
+        }
+    }
+    return (int)out.size() == D;
+}
+
+int get_int(const json::Value &o, const char *key, int def) {
+    const json::Value *v = o.get(key);
+    return (v && v->type == json::Value::NUM) ? (int)v->num : def;
+}
+std::string get_str(const json::Value &o, const char *key) {
+    const json::Value *v = o.get(key);
+    return (v && v->type == json::Value::STR) ? v->str : std::string();
+}
+
+}  // namespace
+}  // namespace cnt
+
+struct cnt_network {
+    std::vector<cnt::NetLayer> layers;
+    int S = 0, maxT = 0, T = 0, Tmin = 0;
+    const char *pat = nullptr;
+    long n_weights = 0;
+    float *weights = nullptr, *updates = nullptr;
+    float *skip_errors = nullptr;  // err and eskip of every skip layer, one allocation
+    size_t skip_error_count = 0;
+    const float *ctx = nullptr;    // conditioning features of the wavnetc layers, C x (maxT*S), set by the caller
+    std::vector<void *> allocations;
+    hipStream_t side = nullptr;
+    hipEvent_t ev_main = nullptr, ev_side = nullptr;
+    int overlap = 1;
+    // optimizer state (allocated by the first update)
+    float *cur_updates = nullptr, *deltas = nullptr, *stats = nullptr;
+    int stats_option = -1;
+    float beta1_accum = 1.0f, beta2_accum = 1.0f;
+    int mdn_target_start = 0, mdn_classes = 0;
+};
+
+namespace cnt {
+namespace {
+
+int device_alloc(cnt_network *n, void **p, size_t bytes, bool zero) {
+    CNT_HIP(hipMalloc(p, bytes ? bytes : 4));
+    n->allocations.push_back(*p);
+    if (zero) CNT_HIP(hipMemset(*p, 0, bytes ? bytes : 4));
+    return CNT_OK;
+}
+
+// TrainableLayer's three sections of a layer's weight vector (layers/TrainableLayer.cu:160-220)
+void weight_sections(NetLayer &L, int P) {
+    const long D = L.size;
+    L.n_in = L.n_bias = L.n_int = 0;
+    if (L.kind == K_DENSE) {
+        L.n_in = (long)P * D;
+        L.n_bias = D;
+    } else if (L.kind == K_LSTM) {
+        const long H = L.bidir ? D / 2 : D;
+        L.n_in = 4L * P * D;
+        L.n_bias = 4L * D;
+        L.n_int = 4L * D * H + 3L * D;
+    } else if (L.kind == K_CNN) {
+        L.n_int = cnt_cnn_weight_count(L.cnn);
+    } else if (L.kind == K_WAVNETC) {
+        L.n_int = 2L * L.ctx_dim * D;
+    }
+}
+
+int build_layer(cnt_network *net, const json::Value &obj, const char *text, const cnt_network_options *opt) {
+    const int index = (int)net->layers.size();
+    NetLayer L;
+    L.text.assign(text + obj.begin, obj.end - obj.begin);
+    L.name = get_str(obj, "name");
+    L.type = get_str(obj, "type");
+    L.size = get_int(obj, "size", 0);
+    const json::Value *bias = obj.get("bias");
+    L.bias = (bias && bias->type == json::Value::NUM) ? (float)bias->num : 0.0f;
+    L.prev = index - 1;
+    CNT_REQUIRE(L.size > 0, "network: layer %d ('%s') has no positive size", index, L.name.c_str());
+    CNT_REQUIRE(get_int(obj, "resolution", 1) == 1, "network: layer '%s' has a time resolution other than 1, which is "
+                "not built", L.name.c_str());
+    const int P = index > 0 ? net->layers[(size_t)index - 1].size : 0;
+    const size_t slots = (size_t)net->S * net->maxT;
+    const std::string &t = L.type;
+    static const char *ff[] = {"feedforward_identity", "feedforward_tanh", "feedforward_logistic", "feedforward_relu"};
+    bool trainable = true;
+    if (index == 0) {
+        CNT_REQUIRE(t == "input", "network: the first layer must be of type 'input'");
+        L.kind = K_INPUT;
+        trainable = false;
+    } else if (t == ff[0] || t == ff[1] || t == ff[2] || t == ff[3]) {
+        L.kind = K_DENSE;
+        for (int a = 0; a < 4; ++a)
+            if (t == ff[a]) L.act = a;
+    } else if (t == "lstm" || t == "blstm") {
+        L.kind = K_LSTM;
+        L.bidir = t == "blstm";
+        cnt_lstm_desc d = {P, L.size, L.bidir, net->S, net->maxT, L.bias};
+        CNT_TRY(cnt_lstm_create(&d, &L.lstm));
+    } else if (t == "skipini" || t == "skipadd") {
+        // NeuralNetwork.cpp:470-530 offers every earlier skip layer plus the layer right before; SkipAddLayer.cu:
+        // 96-138 keeps those named by preSkipLayer, or by default the last two of the offer (a skipini, and the
+        // first skip layer of a network, is offered the layer right before only)
+        L.kind = t == "skipini" ? K_SKIPINI : K_SKIPADD;
+        std::vector<int> offer;
+        if (L.kind == K_SKIPADD)
+            for (int j = 0; j < index; ++j)
+                if (is_skip_kind(net->layers[(size_t)j].kind)) offer.push_back(j);
+        offer.push_back(index - 1);
+        const std::string names = L.kind == K_SKIPADD ? get_str(obj, "preSkipLayer") : std::string();
+        if (!names.empty()) {
+            size_t b = 0;
+            while (b <= names.size()) {
+                size_t e = names.find(',', b);
+                if (e == std::string::npos) e = names.size();
+                const std::string one = names.substr(b, e - b);
+                for (int j : offer)
+                    if (net->layers[(size_t)j].name == one) {
+                        L.pre.push_back(j);
+                        break;
+                    }
+                b = e + 1;
+            }
+        } else if (offer.size() < 2) {
+            L.pre = offer;
+        } else {
+            L.pre.assign(offer.end() - 2, offer.end());
+        }
+        CNT_REQUIRE(!L.pre.empty(), "network: skip layer '%s' is linked to no layer", L.name.c_str());
+        for (int j : L.pre)
+            CNT_REQUIRE(net->layers[(size_t)j].size == L.size, "network: skip layer '%s' (size %d) is linked to '%s' of "
+                        "size %d", L.name.c_str(), L.size, net->layers[(size_t)j].name.c_str(), net->layers[(size_t)j].size);
+    } else if (t == "cnn") {
+        L.kind = K_CNN;
+        CNT_REQUIRE(!obj.has("window_height") && get_int(obj, "repeat_padding", 0) == 0,
+                    "network: cnn layer '%s' uses the 2-D path or repeat_padding, which are not built", L.name.c_str());
+        std::vector<int> hw, dil;
+        CNT_REQUIRE(parse_runs(get_str(obj, "window_width"), L.size, hw), "network: cnn layer '%s': window_width does "
+                    "not give one value per filter", L.name.c_str());
+        CNT_REQUIRE(parse_runs(get_str(obj, "window_tap_interval"), L.size, dil), "network: cnn layer '%s': "
+                    "window_tap_interval does not give one value per filter", L.name.c_str());
+        cnt_cnn_desc d = {P, L.size, net->S, net->maxT, get_int(obj, "causal", 0), get_int(obj, "tanhoutput", 1), L.bias};
+        CNT_TRY(cnt_cnn_create(&d, hw.data(), dil.data(), &L.cnn));
+    } else if (t == "wavnetc") {
+        L.kind = K_WAVNETC;
+        L.ctx_dim = get_int(obj, "contextDim", 0);
+        CNT_REQUIRE(P == 2 * L.size, "network: wavnetc layer '%s' of size %d needs a preceding layer of size %d",
+                    L.name.c_str(), L.size, 2 * L.size);
+        CNT_TRY(device_alloc(net, (void **)&L.core, 2 * (size_t)L.size * slots * sizeof(float), true));
+        CNT_TRY(device_alloc(net, (void **)&L.cth, 2 * (size_t)L.size * slots * sizeof(float), true));
+    } else if (t == "feedback") {
+        L.kind = K_FEEDBACK;
+        L.fb_start = get_int(obj, "previousDimStart", 0);
+        L.fb_end = get_int(obj, "previousDimEnd", P);
+        CNT_REQUIRE(L.fb_start >= 0 && L.fb_end >= L.fb_start && L.fb_end <= P, "network: feedback layer '%s': "
+                    "previousDimStart/End outside the preceding layer", L.name.c_str());
+        CNT_REQUIRE(!obj.has("lookBack") && !obj.has("aggregate") && !obj.has("lookbackStep"),
+                    "network: feedback layer '%s': look-back other than one step and aggregation are not built",
+                    L.name.c_str());
+        trainable = false;
+    } else if (t == "sse") {
+        L.kind = K_SSE;
+        CNT_REQUIRE(L.size == P, "network: sse layer of size %d after a layer of size %d", L.size, P);
+        trainable = false;
+    } else if (t == "mdn") {
+        L.kind = K_MDN;
+        CNT_REQUIRE(opt && opt->mdn_config && opt->mdn_config_len >= 6, "network: an mdn layer needs the mdn config "
+                    "(options.mdn_config)");
+        cnt_mdn_desc d = {P, L.size, net->S, net->maxT, opt->tie_variance, 0};
+        CNT_TRY(cnt_mdn_create(&d, opt->mdn_config, opt->mdn_config_len, &L.mdn));
+        if ((int)opt->mdn_config[0] == 1 && (int)opt->mdn_config[5] == -1) {
+            net->mdn_target_start = (int)opt->mdn_config[3];
+            net->mdn_classes = (int)opt->mdn_config[2] - (int)opt->mdn_config[1];
+        }
+        trainable = false;
+    } else {
+        set_error("network: layer '%s' has type '%s', which this path does not cover", L.name.c_str(), t.c_str());
+        return CNT_ERR_ARG;
+    }
+    // every trainable layer of a network file carries "bias" (layers/TrainableLayer.cu:118-120)
+    if (trainable) CNT_REQUIRE(bias != nullptr, "network: missing value 'bias' in layer '%s'", L.name.c_str());
+    weight_sections(L, P);
+    const size_t count = (size_t)L.size * slots;
+    const bool alias = is_skip_kind(L.kind) && L.pre.size() == 1;
+    if (alias) L.out = net->layers[(size_t)L.pre[0]].out;
+    else CNT_TRY(device_alloc(net, (void **)&L.out, count * sizeof(float), true));
+    if (L.kind != K_INPUT && L.kind != K_SSE && L.kind != K_MDN && !is_skip_kind(L.kind))
+        CNT_TRY(device_alloc(net, (void **)&L.err, count * sizeof(float), true));
+    net->layers.push_back(std::move(L));
+    return CNT_OK;
+}
+
+int finish_build(cnt_network *net, const json::Value *weights) {
+    const size_t slots = (size_t)net->S * net->maxT;
+    // flat weights
+    long total = 0;
+    for (auto &L : net->layers) {
+        L.w_off = total;
+        total += L.weight_count();
+    }
+    net->n_weights = total;
+    CNT_TRY(device_alloc(net, (void **)&net->weights, (size_t)total * sizeof(float), true));
+    CNT_TRY(device_alloc(net, (void **)&net->updates, (size_t)total * sizeof(float), true));
+    if (weights && weights->type == json::Value::OBJ) {
+        std::vector<float> host((size_t)total, 0.0f);
+        for (auto &L : net->layers) {
+            if (L.weight_count() == 0) continue;
+            const json::Value *sec = weights->get(L.name.c_str());
+            CNT_REQUIRE(sec && sec->type == json::Value::OBJ, "network: missing weights section for layer '%s'",
+                        L.name.c_str());
+            const char *keys[3] = {"input", "bias", "internal"};
+            const long want[3] = {L.n_in, L.n_bias, L.n_int};
+            long at = L.w_off;
+            for (int k = 0; k < 3; ++k) {
+                const json::Value *a = sec->get(keys[k]);
+                CNT_REQUIRE(a && (a->type == json::Value::NUMS || a->type == json::Value::ARR),
+                            "network: missing array 'weights/%s/%s'", L.name.c_str(), keys[k]);
+                CNT_REQUIRE((long)a->nums.size() == want[k], "network: layer '%s' has %zu %s weights, expected %ld",
+                            L.name.c_str(), a->nums.size(), keys[k], want[k]);
+                std::memcpy(host.data() + at, a->nums.data(), (size_t)want[k] * sizeof(float));
+                at += want[k];
+            }
+        }
+        CNT_HIP(hipMemcpy(net->weights, host.data(), (size_t)total * sizeof(float), hipMemcpyHostToDevice));
+    }
+    // error buffers of the skip layers: one allocation, [err | eskip] per layer
+    size_t skip_total = 0;
+    for (auto &L : net->layers)
+        if (is_skip_kind(L.kind)) skip_total += 2 * (size_t)L.size * slots;
+    net->skip_error_count = skip_total;
+    if (skip_total) {
+        CNT_TRY(device_alloc(net, (void **)&net->skip_errors, skip_total * sizeof(float), true));
+        size_t at = 0;
+        for (auto &L : net->layers)
+            if (is_skip_kind(L.kind)) {
+                L.err = net->skip_errors + at;
+                L.eskip = L.err + (size_t)L.size * slots;
+                at += 2 * (size_t)L.size * slots;
+            }
+    }
+    // pointer tables of the skip layers
+    for (auto &L : net->layers) {
+        if (!is_skip_kind(L.kind)) continue;
+        const size_t n = L.pre.size();
+        std::vector<const float *> in(n);
+        std::vector<float *> tgt(n);
+        std::vector<int> flag(n);
+        for (size_t k = 0; k < n; ++k) {
+            const NetLayer &src = net->layers[(size_t)L.pre[k]];
+            in[k] = src.out;
+            flag[k] = is_skip_kind(src.kind) ? 1 : 0;
+            tgt[k] = flag[k] ? src.eskip : src.err;
+        }
+        CNT_TRY(device_alloc(net, (void **)&L.in_ptrs, n * sizeof(float *), false));
+        CNT_TRY(device_alloc(net, (void **)&L.tgt_ptrs, n * sizeof(float *), false));
+        CNT_TRY(device_alloc(net, (void **)&L.tgt_is_skip, n * sizeof(int), false));
+        CNT_HIP(hipMemcpy(L.in_ptrs, in.data(), n * sizeof(float *), hipMemcpyHostToDevice));
+        CNT_HIP(hipMemcpy(L.tgt_ptrs, tgt.data(), n * sizeof(float *), hipMemcpyHostToDevice));
+        CNT_HIP(hipMemcpy(L.tgt_is_skip, flag.data(), n * sizeof(int), hipMemcpyHostToDevice));
+    }
+    // checks that need the whole list
+    const NetLayer &post = net->layers.back();
+    CNT_REQUIRE(post.kind == K_SSE || post.kind == K_MDN, "network: the last layer must be a post-output layer (sse or "
+                "mdn), found '%s'", post.type.c_str());
+    for (size_t i = 0; i + 1 < net->layers.size(); ++i)
+        CNT_REQUIRE(net->layers[i].kind != K_SSE && net->layers[i].kind != K_MDN, "network: post-output layer '%s' is "
+                    "not the last layer", net->layers[i].name.c_str());
+    for (auto &L : net->layers)
+        if (L.kind == K_FEEDBACK) {
+            // NeuralNetwork.cpp:805-812 links every feedback layer to the post-output layer
+            CNT_REQUIRE(post.kind == K_MDN && net->mdn_classes > 0, "network: a feedback layer needs an mdn post-output "
+                        "layer with one softmax unit");
+            CNT_REQUIRE(L.size == (L.fb_end - L.fb_start) + net->mdn_classes, "network: feedback layer '%s' has size "
+                        "%d, expected %d + %d classes", L.name.c_str(), L.size, L.fb_end - L.fb_start, net->mdn_classes);
+        }
+    CNT_HIP(hipStreamCreateWithFlags(&net->side, hipStreamNonBlocking));
+    CNT_HIP(hipEventCreateWithFlags(&net->ev_main, hipEventDisableTiming));
+    CNT_HIP(hipEventCreateWithFlags(&net->ev_side, hipEventDisableTiming));
+    return CNT_OK;
+}
+
+}  // namespace
+}  // namespace cnt
+
+extern "C" {
+
+int cnt_network_destroy(cnt_network *net) {
+    if (!net) return CNT_OK;
+    for (auto &L : net->layers) {
+        if (L.lstm) cnt_lstm_destroy(L.lstm);
+        if (L.cnn) cnt_cnn_destroy(L.cnn);
+        if (L.mdn) cnt_mdn_destroy(L.mdn);
+    }
+    for (void *p : net->allocations) (void)hipFree(p);
+    if (net->side) (void)hipStreamDestroy(net->side);
+    if (net->ev_main) (void)hipEventDestroy(net->ev_main);
+    if (net->ev_side) (void)hipEventDestroy(net->ev_side);
+    delete net;
+    return CNT_OK;
+}
+
+int cnt_network_create(const char *json_text, int parallel_sequences, int max_seq_length,
+                       const cnt_network_options *options, cnt_network **out) {
+    using namespace cnt;
+    CNT_REQUIRE(json_text && out, "network_create: null argument");
+    CNT_REQUIRE(parallel_sequences >= 1 && max_seq_length >= 1, "network_create: non-positive geometry");
+    json::Parser parser{json_text, std::strlen(json_text)};
+    json::Value doc;
+    if (!parser.value(doc, 0)) {
+        set_error("network_create: JSON error: %s", parser.error.c_str());
+        return CNT_ERR_ARG;
+    }
+    CNT_REQUIRE(doc.type == json::Value::OBJ, "network_create: the network file is not a JSON object");
+    const json::Value *layers = doc.get("layers");
+    CNT_REQUIRE(layers && layers->type == json::Value::ARR, "network_create: missing section 'layers'");
+    CNT_REQUIRE(layers->arr.size() >= 3, "network_create: a network needs an input layer, a hidden or output layer and "
+                "a post-output layer");
+    cnt_network *net = new (std::nothrow) cnt_network();
+    CNT_REQUIRE(net != nullptr, "network_create: out of host memory");
+    net->S = parallel_sequences;
+    net->maxT = max_seq_length;
+    if (options) net->overlap = options->no_overlap ? 0 : 1;
+    int status = CNT_OK;
+    for (const auto &obj : layers->arr) {
+        if (obj.type != json::Value::OBJ) {
+            set_error("network_create: an entry of 'layers' is not an object");
+            status = CNT_ERR_ARG;
+        } else {
+            status = build_layer(net, obj, json_text, options);
+        }
+        if (status != CNT_OK) break;
+    }
+    if (status == CNT_OK) status = finish_build(net, doc.get("weights"));
+    if (status != CNT_OK) {
+        cnt_network_destroy(net);
+        return status;
+    }
+    *out = net;
+    return CNT_OK;
+}
+
+int cnt_network_info(cnt_network *net, int *n_layers, int *input_size, int *output_size, long *n_weights) {
+    using namespace cnt;
+    CNT_REQUIRE(net, "network_info: null handle");
+    if (n_layers) *n_layers = (int)net->layers.size();
+    if (input_size) *input_size = net->layers.front().size;
+    if (output_size) *output_size = net->layers.back().size;
+    if (n_weights) *n_weights = net->n_weights;
+    return CNT_OK;
+}
+
+int cnt_network_layer_info(cnt_network *net, int index, cnt_layer_info *info) {
+    using namespace cnt;
+    CNT_REQUIRE(net && info, "network_layer_info: null argument");
+    CNT_REQUIRE(index >= 0 && index < (int)net->layers.size(), "network_layer_info: no layer %d", index);
+    const NetLayer &L = net->layers[(size_t)index];
+    std::memset(info, 0, sizeof(*info));
+    std::strncpy(info->name, L.name.c_str(), sizeof(info->name) - 1);
+    std::strncpy(info->type, L.type.c_str(), sizeof(info->type) - 1);
+    info->size = L.size;
+    info->weight_offset = L.w_off;
+    info->n_input = L.n_in;
+    info->n_bias = L.n_bias;
+    info->n_internal = L.n_int;
+    info->outputs = L.out;
+    info->output_errors = L.err;
+    return CNT_OK;
+}
+
+float *cnt_network_weights(cnt_network *net) { return net ? net->weights : nullptr; }
+float *cnt_network_weight_updates(cnt_network *net) { return net ? net->updates : nullptr; }
+
+int cnt_network_randomize(cnt_network *net, unsigned seed, float range) {
+    using namespace cnt;
+    CNT_REQUIRE(net, "network_randomize: null handle");
+    std::mt19937 gen(seed);
+    std::uniform_real_distribution<float> dist(-range, range);
+    std::vector<float> host((size_t)net->n_weights);
+    for (auto &v : host) v = dist(gen);
+    CNT_HIP(hipMemcpy(net->weights, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice));
+    return CNT_OK;
+}
+
+int cnt_network_set_context(cnt_network *net, const float *ctx) {
+    using namespace cnt;
+    CNT_REQUIRE(net, "network_set_context: null handle");
+    net->ctx = ctx;
+    return CNT_OK;
+}
+
+int cnt_network_load_sequences(cnt_network *net, void *stream_, int T, int Tmin, const char *patTypes,
+                               const float *inputs, const float *targets) {
+    using namespace cnt;
+    CNT_REQUIRE(net && patTypes, "network_load_sequences: null argument");
+    CNT_REQUIRE(T >= 1 && T <= net->maxT && Tmin >= 1 && Tmin <= T, "network_load_sequences: lengths %d / %d outside "
+                "1..%d", T, Tmin, net->maxT);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    net->T = T;
+    net->Tmin = Tmin;
+    net->pat = patTypes;
+    const size_t slots = (size_t)T * net->S;
+    NetLayer &in = net->layers.front(), &post = net->layers.back();
+    if (inputs)
+        CNT_HIP(hipMemcpyAsync(in.out, inputs, slots * in.size * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    // a post-output layer keeps the targets in its own outputs() (layers/PostOutputLayer.cu:108-124)
+    if (targets)
+        CNT_HIP(hipMemcpyAsync(post.out, targets, slots * post.size * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    for (auto &L : net->layers) {
+        if (L.lstm) CNT_TRY(cnt_lstm_load_sequences(L.lstm, stream, patTypes, T, Tmin));
+        if (L.mdn) CNT_TRY(cnt_mdn_load_sequences(L.mdn, stream, patTypes, T));
+    }
+    return CNT_OK;
+}
+
+int cnt_network_forward(cnt_network *net, void *stream_) {
+    using namespace cnt;
+    CNT_REQUIRE(net && net->T > 0, "network_forward: no fraction loaded");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int N = net->T * net->S;
+    // what the skip layers' forward passes clear (layers/SkipAddLayer.cu:195-205)
+    if (net->skip_error_count) CNT_TRY(fill_zero(stream, net->skip_errors, net->skip_error_count));
+    for (size_t i = 1; i < net->layers.size(); ++i) {
+        NetLayer &L = net->layers[i];
+        const NetLayer &prev = net->layers[i - 1];
+        const float *W = net->weights + L.w_off;
+        const size_t count = (size_t)L.size * N;
+        switch (L.kind) {
+            case K_DENSE:
+                CNT_TRY(cnt_dense_forward(stream, prev.size, L.size, N, L.act, L.bias, W, prev.out, L.out));
+                break;
+            case K_LSTM:
+                CNT_TRY(cnt_lstm_forward(L.lstm, stream, W, prev.out, L.out));
+                break;
+            case K_SKIPINI:
+            case K_SKIPADD:
+                if (L.pre.size() > 1) {
+                    ProfileScope prof(stream, "skip_sum");
+                    hipLaunchKernelGGL(skip_sum_kernel, dim3(blocks_for(count)), dim3(256), 0, stream, count,
+                                       (int)L.pre.size(), L.in_ptrs, L.out);
+                    CNT_HIP(hipGetLastError());
+                }
+                break;
+            case K_CNN:
+                CNT_TRY(cnt_cnn_forward(L.cnn, stream, net->pat, net->T, W, prev.out, L.out));
+                break;
+            case K_WAVNETC:
+                CNT_REQUIRE(L.ctx_dim == 0 || net->ctx, "network_forward: wavnetc layer '%s' has no conditioning features "
+                            "(cnt_network_set_context)", L.name.c_str());
+                CNT_TRY(cnt_wavnetc_forward(stream, L.size, L.ctx_dim, N, net->pat, W, net->ctx, prev.out, L.core, L.cth,
+                                            L.out));
+                break;
+            case K_FEEDBACK: {
+                const NetLayer &post = net->layers.back();
+                ProfileScope prof(stream, "feedback");
+                hipLaunchKernelGGL(feedback_kernel, dim3(blocks_for(count)), dim3(256), 0, stream, count, L.size,
+                                   L.fb_end - L.fb_start, prev.size, L.fb_start, net->S, post.size, net->mdn_target_start,
+                                   net->pat, prev.out, post.out, L.out);
+                CNT_HIP(hipGetLastError());
+                break;
+            }
+            case K_MDN:
+                CNT_TRY(cnt_mdn_forward(L.mdn, stream, prev.out));
+                break;
+            default:
+                break;
+        }
+    }
+    return CNT_OK;
+}
+
+int cnt_network_calculate_error(cnt_network *net, void *stream_, float *loss_dev) {
+    using namespace cnt;
+    CNT_REQUIRE(net && loss_dev && net->T > 0, "network_calculate_error: null argument or no fraction loaded");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int N = net->T * net->S;
+    NetLayer &post = net->layers.back();
+    const NetLayer &last = net->layers[net->layers.size() - 2];
+    if (post.kind == K_SSE) return cnt_sse_error(stream, post.size, N, net->pat, last.out, post.out, loss_dev);
+    return cnt_mdn_calculate_error(post.mdn, stream, post.out, loss_dev);
+}
+
+int cnt_network_backward(cnt_network *net, void *stream_) {
+    using namespace cnt;
+    CNT_REQUIRE(net && net->T > 0, "network_backward: no fraction loaded");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t wstream = net->overlap ? net->side : stream;
+    const int N = net->T * net->S;
+    bool side_used = false;
+    for (size_t i = net->layers.size() - 1; i >= 1; --i) {
+        NetLayer &L = net->layers[i];
+        NetLayer &prev = net->layers[i - 1];
+        const float *W = net->weights + L.w_off;
+        float *dW = net->updates + L.w_off;
+        // the input layer has no error buffer; a feedback layer that takes nothing from its preceding layer passes
+        // nothing on, and neither does anything that feeds such a feedback layer's one-hot part
+        float *prev_err = prev.err;
+        if (prev.kind == K_FEEDBACK && prev.fb_end == prev.fb_start) prev_err = nullptr;
+        const size_t count = (size_t)L.size * N;
+        switch (L.kind) {
+            case K_SSE:
+                CNT_TRY(cnt_sse_backward(stream, L.size, N, net->pat, prev.out, L.out, prev.err));
+                break;
+            case K_MDN:
+                CNT_TRY(cnt_mdn_backward(L.mdn, stream, L.out, prev.err));
+                break;
+            case K_DENSE:
+            case K_LSTM:
+                if (L.kind == K_DENSE)
+                    CNT_TRY(cnt_dense_backward_errors(stream, prev.size, L.size, N, L.act, W, L.out, L.err, prev_err));
+                else
+                    CNT_TRY(cnt_lstm_backward_errors(L.lstm, stream, W, L.err, prev_err));
+                // the weight half has no consumer before the optimizer: second stream, after the error half
+                if (net->overlap) {
+                    CNT_HIP(hipEventRecord(net->ev_main, stream));
+                    CNT_HIP(hipStreamWaitEvent(net->side, net->ev_main, 0));
+                    side_used = true;
+                }
+                if (L.kind == K_DENSE)
+                    CNT_TRY(cnt_dense_backward_weights(wstream, prev.size, L.size, N, L.bias, prev.out, L.err, dW));
+                else
+                    CNT_TRY(cnt_lstm_backward_weights(L.lstm, wstream, prev.out, dW));
+                break;
+            case K_SKIPINI:
+            case K_SKIPADD: {
+                ProfileScope prof(stream, "skip_fan");
+                hipLaunchKernelGGL(skip_fan_kernel, dim3(blocks_for(count)), dim3(256), 0, stream, count,
+                                   (int)L.pre.size(), L.tgt_ptrs, L.tgt_is_skip, L.err, L.eskip);
+                CNT_HIP(hipGetLastError());
+                break;
+            }
+            case K_CNN:
+                CNT_TRY(cnt_cnn_backward(L.cnn, stream, net->pat, net->T, W, prev.out, L.out, L.err, prev_err, dW));
+                break;
+            case K_WAVNETC:
+                CNT_TRY(cnt_wavnetc_backward(stream, L.size, L.ctx_dim, N, net->pat, W, net->ctx, L.core, L.cth, L.err,
+                                             prev.err, dW, nullptr));
+                break;
+            case K_FEEDBACK:
+                if (L.fb_end > L.fb_start && prev.err) {
+                    const size_t pc = (size_t)prev.size * N;
+                    hipLaunchKernelGGL(feedback_backward_kernel, dim3(blocks_for(pc)), dim3(256), 0, stream, pc,
+                                       prev.size, L.fb_start, L.fb_end, L.size, L.err, prev.err);
+                    CNT_HIP(hipGetLastError());
+                }
+                break;
+            default:
+                break;
+        }
+    }
+    if (side_used) {
+        CNT_HIP(hipEventRecord(net->ev_side, net->side));
+        CNT_HIP(hipStreamWaitEvent(stream, net->ev_side, 0));
+    }
+    return CNT_OK;
+}
+
+int cnt_network_check(cnt_network *net, void *stream) {
+    using namespace cnt;
+    CNT_REQUIRE(net, "network_check: null handle");
+    for (auto &L : net->layers)
+        if (L.lstm) CNT_TRY(cnt_lstm_check(L.lstm, stream));
+    return CNT_OK;
+}
+
+int cnt_network_update(cnt_network *net, void *stream_, int option, float learning_rate, float momentum,
+                       float frac_length) {
+    using namespace cnt;
+    CNT_REQUIRE(net, "network_update: null handle");
+    const size_t n = (size_t)net->n_weights;
+    if (!net->cur_updates) {
+        CNT_TRY(device_alloc(net, (void **)&net->cur_updates, n * sizeof(float), true));
+        CNT_TRY(device_alloc(net, (void **)&net->deltas, n * sizeof(float), true));
+    }
+    const bool adagrad = option == 1 || option == 3, adam = option == 5;
+    if ((adagrad || adam) && net->stats_option != option) {
+        CNT_REQUIRE(net->stats_option < 0, "network_update: the optimizer option changed from %d to %d", net->stats_option,
+                    option);
+        // optimizers/Optimizer.cu:427-447: AdaGrad statistics start at 1e-6, Adam's (m, v) pairs at 0
+        std::vector<float> init(adam ? 2 * n : n, adam ? 0.0f : 1e-6f);
+        CNT_TRY(device_alloc(net, (void **)&net->stats, init.size() * sizeof(float), false));
+        CNT_HIP(hipMemcpy(net->stats, init.data(), init.size() * sizeof(float), hipMemcpyHostToDevice));
+        net->stats_option = option;
+    }
+    if (adam) {
+        net->beta1_accum = cnt_opt_next_beta_accum(net->beta1_accum, 1);
+        net->beta2_accum = cnt_opt_next_beta_accum(net->beta2_accum, 2);
+    }
+    return cnt_opt_step(stream_, option, (long)n, net->weights, net->updates, net->cur_updates, net->stats, net->deltas,
+                        nullptr, frac_length, net->beta1_accum, net->beta2_accum, learning_rate, momentum);
+}
+
+int cnt_network_export_json(cnt_network *net, char *buf, size_t cap, size_t *needed) {
+    using namespace cnt;
+    CNT_REQUIRE(net && needed, "network_export_json: null argument");
+    std::vector<float> host((size_t)net->n_weights);
+    CNT_HIP(hipDeviceSynchronize());
+    if (!host.empty())
+        CNT_HIP(hipMemcpy(host.data(), net->weights, host.size() * sizeof(float), hipMemcpyDeviceToHost));
+    std::string s = "{\"layers\":[";
+    for (size_t i = 0; i < net->layers.size(); ++i) {
+        if (i) s += ",";
+        s += net->layers[i].text;
+    }
+    s += "],\"weights\":{";
+    bool first = true;
+    char num[32];
+    for (const auto &L : net->layers) {
+        if (L.weight_count() == 0) continue;
+        if (!first) s += ",";
+        first = false;
+        s += "\"" + L.name + "\":{";
+        const char *keys[3] = {"input", "bias", "internal"};
+        const long len[3] = {L.n_in, L.n_bias, L.n_int};
+        long at = L.w_off;
+        for (int k = 0; k < 3; ++k) {
+            s += std::string(k ? "," : "") + "\"" + keys[k] + "\":[";
+            for (long j = 0; j < len[k]; ++j) {
+                snprintf(num, sizeof(num), j ? ",%.9g" : "%.9g", (double)host[(size_t)(at + j)]);
+                s += num;
+            }
+            s += "]";
+            at += len[k];
+        }
+        s += "}";
+    }
+    s += "}}";
+    *needed = s.size() + 1;
+    if (buf && cap >= s.size() + 1) std::memcpy(buf, s.c_str(), s.size() + 1);
+    return CNT_OK;
+}
+
+}  // extern "C"

@@ -33,3 +33,20 @@ def test_version_and_argument_errors_without_gpu():
     assert b"null" in L.cnt_last_error()
     assert L.cnt_lstm_weight_count(382, 256, 0) == 655104
     assert L.cnt_lstm_weight_count(512, 512, 1) == 1576448
+
+
+def test_network_file_syntax_errors_without_gpu():
+    """The network file is parsed before any device call: malformed JSON and a missing 'layers' section are
+    reported with the parser's message."""
+    import ctypes as C
+
+    import pytest
+
+    capi = load_package().capi
+    capi.lib()
+    for text, what in (('{"layers": [', "JSON error"), ('{"layers": [{"size": 3,}]}', "JSON error"),
+                       ('{"weights": {}}', "missing section 'layers'"), ('[1, 2]', "not a JSON object"),
+                       ('{"layers": [{"size": 1, "name": "input", "type": "input"}]}', "needs an input layer")):
+        h = C.c_void_p()
+        with pytest.raises(RuntimeError, match=what):
+            capi.check(capi.lib().cnt_network_create(text.encode(), 2, 10, None, C.byref(h)))

@@ -1,0 +1,225 @@
+"""GPU tests of the C++ network sequencer (cnt_network_*): a network file in the reference's JSON structure is
+turned into the layer list, and forward pass, error, backward pass and optimizer step of a fraction are compared
+with the CPU oracle doing the same steps.  Tolerance 1e-4 on L2-normalised differences (fp32, different summation
+orders), the tolerance of the layer kernels themselves."""
+import json
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+import oracle_models as OM
+import parity_cases as PC
+import wavenet_data as WD
+from torch_models import make_pat_types
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def _sections(doc_weights, name, w, n_in, n_bias):
+    doc_weights[name] = {"input": w[:n_in].tolist(), "bias": w[n_in:n_in + n_bias].tolist(),
+                         "internal": w[n_in + n_bias:].tolist()}
+
+
+@pytest.mark.parametrize("option,momentum,overlap", [(0, 0.9, True), (5, 0.0, True), (0, 0.0, False)])
+def test_stacked_network_trains_like_the_oracle(option, momentum, overlap):
+    import torch
+
+    print("network case", option, momentum, overlap, flush=True)
+    pkg = PC.pkg()
+    capi, networks = pkg.capi, pkg.networks
+    P, Q, S = 20, 6, 4
+    specs = [{"name": "ff1", "type": "feedforward_tanh", "size": 32, "bias": 1.0},
+             {"name": "bl1", "type": "blstm", "size": 128, "bias": 1.0},
+             {"name": "l2", "type": "lstm", "size": 64, "bias": 1.0},
+             {"name": "out", "type": "feedforward_identity", "size": Q, "bias": 1.0},
+             {"name": "postoutput", "type": "sse", "size": Q}]
+    weights = OM.init_weights(P, specs, 4, 0.1)
+    doc = {"layers": [{"size": P, "name": "input", "type": "input"}] + specs, "weights": {}}
+    wi, prev = iter(weights), P
+    for sp in specs:
+        n_in, n_bias, _ = networks.weight_sections(sp, prev)
+        if n_in:
+            _sections(doc["weights"], sp["name"], next(wi), n_in, n_bias)
+        prev = sp["size"]
+    maxT = 30
+    net = capi.Network(json.dumps(doc, indent=1), S, maxT, overlap=overlap)
+    assert net.input_size == P and net.output_size == Q and net.n_weights == sum(w.size for w in weights)
+    assert [L["type"] for L in net.layers] == ["input"] + [s["type"] for s in specs]
+    for L, w in zip([L for L in net.layers if L["weight_count"]], weights):
+        assert np.array_equal(L["weights"].cpu().numpy(), w)
+
+    rng = np.random.default_rng(6)
+    ow = [w.copy() for w in weights]
+    deltas = [np.zeros_like(w) for w in ow]
+    stats = [np.zeros(2 * w.size, np.float32) for w in ow]
+    b1 = b2 = 1.0
+    for step, lengths in enumerate(([30, 22, 13, 9], [17, 26, 28, 11], [19, 24, 8, 15])):
+        T, Tmin = max(lengths), min(lengths)
+        pat = make_pat_types(lengths, T)
+        x = rng.standard_normal((T, S, P)).astype(np.float32)
+        tgt = (0.3 * rng.standard_normal((T, S, Q))).astype(np.float32)
+        valid = (pat != 0).reshape(T, S)
+        x[~valid] = 0
+        tgt[~valid] = 0
+        net.load_sequences(PC.dev(pat), T, Tmin, PC.dev(x.reshape(-1)), PC.dev(tgt.reshape(-1)))
+        net.forward()
+        loss = float(net.calculate_error().item())
+        net.backward()
+        ref = OM.OracleNetwork(P, specs, S, T, Tmin, pat, ow)
+        ref.forward(x.reshape(-1), tgt.reshape(-1))
+        assert abs(loss - ref.error()) <= TOL * max(1.0, abs(ref.error()))
+        ref.backward()
+        grads = [L["updates"] for L in ref.layers if "updates" in L]
+        torch.cuda.synchronize()
+        for L, g in zip([L for L in net.layers if L["weight_count"]], grads):
+            assert PC.relerr(L["updates"].cpu().numpy(), g) < TOL, (step, L["name"])
+        frac = float(sum(lengths))
+        net.update(option, 1e-3, momentum, frac)
+        if option == 5:
+            b1 = O.opt_next_beta_accum(b1, 1)
+            b2 = O.opt_next_beta_accum(b2, 2)
+        for w, g, d, st in zip(ow, grads, deltas, stats):
+            cur = np.empty_like(g)
+            O.opt_accumulate(g, cur, False)
+            O.opt_adjust_gradient(option, cur, st, None, frac, b1, b2)
+            O.opt_update_weights(w, cur, d, None, 1e-3, momentum)
+    net.check()
+    got = [L["weights"].cpu().numpy() for L in net.layers if L["weight_count"]]
+    for g, w, w0 in zip(got, ow, weights):
+        assert PC.relerr(g, w) < TOL
+        assert PC.relerr(g, w0) > 1e-5  # the weights did move
+    # export and re-import: same layers, bit-identical weights
+    text = net.export_json()
+    back = json.loads(text)
+    assert [l["name"] for l in back["layers"]] == ["input"] + [s["name"] for s in specs]
+    assert back["layers"][2] == specs[1]
+    again = capi.Network(text, S, maxT)
+    assert np.array_equal(again.weights.cpu().numpy(), net.weights.cpu().numpy())
+    again.close()
+    net.close()
+
+
+def wavenet_json(nb, Q, R, K, C, cnn_tanh, dilation_cycle):
+    """Network file with the topology of the reference's example obsolete/scripts/EXAMPLE/MODEL_WAVENET/network.jsn
+    (without its frame-rate conditioning sub-network: the conditioning features are handed to the library)."""
+    def ff(name, size, kind="feedforward_identity"):
+        return {"size": size, "name": name, "bias": 1.0, "type": kind}
+
+    layers = [{"size": 1, "name": "input", "type": "input"},
+              {"size": Q, "name": "feedbackBottom", "bias": 1.0, "type": "feedback", "previousDimEnd": 0,
+               "previousDimStart": 0},
+              ff("emb", R), {"size": R, "name": "causalSkip", "bias": 1.0, "type": "skipini"}]
+    res = "causalSkip"
+    for l in range(nb):
+        dil = 2 ** (l % dilation_cycle)
+        layers += [
+            {"size": 2 * R, "name": "cnn%d" % l, "bias": 1.0, "type": "cnn", "window_width": "%d*1" % (2 * R),
+             "window_tap_interval": "%d*%d" % (2 * R, dil), "causal": 1, "tanhoutput": cnn_tanh},
+            {"size": R, "name": "wav%d" % l, "bias": 1.0, "type": "wavnetc", "contextDim": C},
+            ff("out%d" % l, R),
+            {"size": R, "name": "sadd%d" % l, "bias": 1.0, "type": "skipadd", "preSkipLayer": "%s,out%d" % (res, l)},
+            {"size": R, "name": "temp%d" % l, "bias": 1.0, "type": "skipini"},
+            ff("sot%d" % l, K),
+            {"size": K, "name": "skip%d" % l, "bias": 1.0, "type": "skipini"},
+            {"size": R, "name": "temp2_%d" % l, "bias": 1.0, "type": "skipadd", "preSkipLayer": "temp%d" % l}]
+        res = "temp2_%d" % l
+    layers += [{"size": K, "name": "postAdd", "bias": 1.0, "type": "skipadd",
+                "preSkipLayer": ",".join("skip%d" % l for l in range(nb))},
+               ff("postL1", K, "feedforward_tanh"), ff("output", Q), {"size": 1, "name": "postoutput", "type": "mdn"}]
+    return {"layers": layers}
+
+
+@pytest.mark.parametrize("nb,cnn_tanh", [(4, 1), (11, 0)])
+def test_wavenet_network_file_against_oracle_graph(nb, cnn_tanh):
+    import torch
+
+    print("wavenet network file", nb, cnn_tanh, flush=True)
+    pkg = PC.pkg()
+    capi, networks = pkg.capi, pkg.networks
+    Q, R, K, C = 64, 32, 64, 20
+    lengths = [120, 90]
+    S, T = len(lengths), max(lengths)
+    pat, onehot, ctx, target, N = WD.make(lengths, Q, C, upsample=20, seed=2)
+    ref = networks.WaveNet(OM.OracleBackend(), nb, S, T, Q=Q, R=R, K=K, C=C, cnn_tanh=cnn_tanh, dilation_cycle=3)
+    shapes = {k: len(ref.buf[k]["W"]) for k in ref.weight_names()}
+    W = WD.init_weights(shapes, seed=3)
+    for k, w in W.items():
+        ref.buf[k]["W"][:] = w
+    ref.set_inputs(pat, onehot, ctx, target)
+    ref.forward()
+    ref.calculate_error()
+    ref.backward()
+
+    doc = wavenet_json(nb, Q, R, K, C, cnn_tanh, 3)
+    net = capi.Network(json.dumps(doc), S, T + 7, mdn_config=[1, 0, Q, 0, 1, -1])   # buffers longer than the fraction
+    names = [L["name"] for L in net.layers if L["weight_count"]]
+    assert sorted(names) == sorted(W)
+    for L in net.layers:
+        if L["weight_count"]:
+            assert L["weight_count"] == W[L["name"]].size
+            L["weights"].copy_(torch.from_numpy(W[L["name"]]))
+    ctx_d = torch.zeros(C * S * (T + 7), dtype=torch.float32, device="cuda")
+    ctx_d[: ctx.size].copy_(torch.from_numpy(ctx))
+    net.set_context(ctx_d)
+    dummy_in = torch.zeros(S * T, dtype=torch.float32, device="cuda")
+    for _ in range(2):  # a second pass over the same fraction gives the same result (buffers cleared properly)
+        net.load_sequences(PC.dev(pat), T, min(lengths), dummy_in, PC.dev(target))
+        net.forward()
+        loss = float(net.calculate_error().item())
+        net.backward()
+        torch.cuda.synchronize()
+        ref_loss = float(ref.loss[0])
+        assert abs(loss - ref_loss) <= TOL * abs(ref_loss)
+        # teacher-forced one-hot input: equal on every valid slot (a padding slot right after a sequence's end holds
+        # the one-hot of the last sample, as in the reference, where the oracle's input has zeros)
+        fb = net.layer("feedbackBottom")["outputs"][: N * Q].cpu().numpy().reshape(N, Q)
+        valid = pat != 0
+        assert np.array_equal(fb[valid], onehot.reshape(N, Q)[valid])
+        worst = 0.0
+        for L in net.layers:
+            if L["weight_count"]:
+                e = PC.relerr(L["updates"].cpu().numpy(), ref.buf[L["name"]]["dW"])
+                worst = max(worst, e)
+                if e > TOL:
+                    print("   ", L["name"], e, flush=True)
+        assert worst < TOL
+    net.update(0, 1e-4, 0.0, float(sum(lengths)))
+    torch.cuda.synchronize()
+    moved = net.layer("cnn0")["weights"].cpu().numpy()
+    assert PC.relerr(moved, W["cnn0"] - 1e-4 * ref.buf["cnn0"]["dW"]) < TOL
+    net.close()
+
+
+def test_network_file_rejections():
+    capi = PC.pkg().capi
+
+    def make(layers, weights=None):
+        doc = {"layers": layers}
+        if weights is not None:
+            doc["weights"] = weights
+        return json.dumps(doc)
+
+    inp = {"size": 3, "name": "input", "type": "input"}
+    post = {"size": 4, "name": "post", "type": "sse"}
+    with pytest.raises(RuntimeError, match="does not cover"):
+        capi.Network(make([inp, {"size": 4, "name": "c", "type": "maxpooling", "bias": 1.0}, post]), 2, 10)
+    with pytest.raises(RuntimeError, match="expected 12"):
+        capi.Network(make([inp, {"size": 4, "name": "o", "type": "feedforward_identity", "bias": 1.0}, post],
+                          {"o": {"input": [0.0] * 11, "bias": [0.0] * 4, "internal": []}}), 2, 10)
+    with pytest.raises(RuntimeError, match="Missing value 'bias'|missing value 'bias'"):
+        capi.Network(make([inp, {"size": 4, "name": "o", "type": "feedforward_identity"}, post]), 2, 10)
+    with pytest.raises(RuntimeError, match="post-output"):
+        capi.Network(make([inp, {"size": 4, "name": "o", "type": "feedforward_identity", "bias": 1.0},
+                           {"size": 4, "name": "o2", "type": "feedforward_identity", "bias": 1.0}]), 2, 10)
+    with pytest.raises(RuntimeError, match="linked to"):
+        capi.Network(make([inp, {"size": 4, "name": "o", "type": "feedforward_identity", "bias": 1.0},
+                           {"size": 5, "name": "s", "type": "skipini", "bias": 1.0}, post]), 2, 10)
+    with pytest.raises(RuntimeError, match="resolution"):
+        capi.Network(make([inp, {"size": 4, "name": "o", "type": "feedforward_identity", "bias": 1.0, "resolution": 80},
+                           post]), 2, 10)
+    net = capi.Network(make([inp, {"size": 4, "name": "o", "type": "feedforward_identity", "bias": 1.0}, post]), 2, 10)
+    with pytest.raises(RuntimeError, match="no fraction"):
+        net.forward()
+    net.close()
