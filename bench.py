@@ -138,28 +138,24 @@ def main():
     lengths, T, x, tgt, pat = make_fraction(seed, S, Tmax, 300, input_size, 187)
     frames = sum(lengths)
 
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    net = networks.StackedNetwork(input_size, specs, S, T)
+    # the network file a user of the reference would write for this model, handed to the library's sequencer
+    layers = [{"size": input_size, "name": "input", "type": "input"}]
+    for i, sp in enumerate(specs):
+        layers.append(dict(sp, name="%s_%d" % (sp["type"], i + 1)))
+    net = capi.Network(json.dumps({"layers": layers}), S, T)
     # weights: seeded U(-0.08, 0.08), generated on the host with the same generator the parity tests use
     rng = np.random.default_rng(seed + 1)
-    weights, prev = [], input_size
-    for sp in specs:
-        n = networks.layer_weight_count(sp, prev)
-        if n:
-            weights.append(rng.uniform(-0.08, 0.08, n).astype(np.float32))
-        prev = sp["size"]
-    net.set_weights(weights)
+    for L in net.layers:
+        if L["weight_count"]:
+            L["weights"].copy_(torch.from_numpy(rng.uniform(-0.08, 0.08, L["weight_count"]).astype(np.float32)))
     pat_d = torch.from_numpy(pat).cuda()
     net.load_sequences(pat_d, T, min(lengths), torch.from_numpy(x).cuda(), torch.from_numpy(tgt).cuda())
     net.forward()
     net.check()
 
-    side = torch.cuda.Stream()  # default priority; carries the weight-gradient halves
-
     def step():
         net.load_sequences(pat_d, T, min(lengths))  # per-fraction clearing of the stored output-gate deltas
-        net.backward_overlapped(side)
-        torch.cuda.current_stream().wait_stream(side)
+        net.backward()  # weight-gradient halves on the library's second stream, joined before it returns
 
     for _ in range(args.warmup):
         step()
@@ -179,8 +175,7 @@ def main():
     for _ in range(args.steps):
         net.load_sequences(pat_d, T, min(lengths))
         net.forward()
-        net.backward_overlapped(side)
-        torch.cuda.current_stream().wait_stream(side)
+        net.backward()
     torch.cuda.synchronize()
     fb_ms = 1e3 * (time.perf_counter() - t0) / args.steps
 

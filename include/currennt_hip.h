@@ -209,6 +209,14 @@ int cnt_cnn_backward(cnt_cnn *h, void *stream, const char *patTypes, int curT, c
                      const float *x, const float *outputs, float *output_errors, float *prev_errors,
                      float *weight_updates);
 
+/* The two halves of cnt_cnn_backward for callers that put the weight gradients on another stream (the reference
+ * has no such split): _errors = tanh derivative in place and prev_errors; _weights reads x and the finished
+ * output_errors.  Calling both in this order on one stream is cnt_cnn_backward. */
+int cnt_cnn_backward_errors(cnt_cnn *h, void *stream, const char *patTypes, int curT, const float *weights,
+                            const float *outputs, float *output_errors, float *prev_errors);
+int cnt_cnn_backward_weights(cnt_cnn *h, void *stream, const char *patTypes, int curT, const float *x,
+                             const float *output_errors, float *weight_updates);
+
 /* ---- gated activation, conditioned ("wavnetc") and plain ("gatedact") ------------------------------
  * WavNetCore<TDevice> (layers/wavNetCore.cu) and GatedActLayer<TDevice> (layers/GatedActLayer.cu).
  * D = layer size, the preceding layer has 2D units; C = contextDim; N = T*S slots.
@@ -231,6 +239,13 @@ int cnt_wavnetc_forward(void *stream, int D, int C, int N, const char *patTypes,
 int cnt_wavnetc_backward(void *stream, int D, int C, int N, const char *patTypes, const float *weights,
                          const float *ctx, const float *core_buf, float *ctx_tanh, const float *output_errors,
                          float *prev_errors, float *weight_updates, float *ctx_grad);
+/* The two halves of cnt_wavnetc_backward (same split as above): _errors = prev_errors, the gradient left in
+ * ctx_tanh and the optional context gradient; _weights = weight_updates from ctx and that gradient. */
+int cnt_wavnetc_backward_errors(void *stream, int D, int C, int N, const char *patTypes, const float *weights,
+                                const float *core_buf, float *ctx_tanh, const float *output_errors, float *prev_errors,
+                                float *ctx_grad);
+int cnt_wavnetc_backward_weights(void *stream, int D, int C, int N, const float *ctx, const float *ctx_tanh,
+                                 float *weight_updates);
 /* SumGradientsForExternalInput (layers/wavNetCore.cu:237-270, driver :895-913): frame_grad (C x
  * n_frame_slots) = sum of ctx_grad over the `resolution` samples of each frame. */
 int cnt_wavnetc_sum_context_grad(void *stream, int C, int S, int resolution, int n_frame_slots, int N,

@@ -796,10 +796,18 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 break;
             case K_DENSE:
             case K_LSTM:
+            case K_CNN:
+            case K_WAVNETC:
                 if (L.kind == K_DENSE)
                     CNT_TRY(cnt_dense_backward_errors(stream, prev.size, L.size, N, L.act, W, L.out, L.err, prev_err));
-                else
+                else if (L.kind == K_LSTM)
                     CNT_TRY(cnt_lstm_backward_errors(L.lstm, stream, W, L.err, prev_err));
+                else if (L.kind == K_CNN)
+                    CNT_TRY(cnt_cnn_backward_errors(L.cnn, stream, net->pat, net->T, W, L.out, L.err, prev_err));
+                else
+                    CNT_TRY(cnt_wavnetc_backward_errors(stream, L.size, L.ctx_dim, N, net->pat, W, L.core, L.cth, L.err,
+                                                        prev.err, nullptr));
+                if (L.kind == K_WAVNETC && L.ctx_dim == 0) break;
                 // the weight half has no consumer before the optimizer: second stream, after the error half
                 if (net->overlap) {
                     CNT_HIP(hipEventRecord(net->ev_main, stream));
@@ -808,8 +816,12 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 }
                 if (L.kind == K_DENSE)
                     CNT_TRY(cnt_dense_backward_weights(wstream, prev.size, L.size, N, L.bias, prev.out, L.err, dW));
-                else
+                else if (L.kind == K_LSTM)
                     CNT_TRY(cnt_lstm_backward_weights(L.lstm, wstream, prev.out, dW));
+                else if (L.kind == K_CNN)
+                    CNT_TRY(cnt_cnn_backward_weights(L.cnn, wstream, net->pat, net->T, prev.out, L.err, dW));
+                else
+                    CNT_TRY(cnt_wavnetc_backward_weights(wstream, L.size, L.ctx_dim, N, net->ctx, L.cth, dW));
                 break;
             case K_SKIPINI:
             case K_SKIPADD: {
@@ -819,13 +831,6 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 CNT_HIP(hipGetLastError());
                 break;
             }
-            case K_CNN:
-                CNT_TRY(cnt_cnn_backward(L.cnn, stream, net->pat, net->T, W, prev.out, L.out, L.err, prev_err, dW));
-                break;
-            case K_WAVNETC:
-                CNT_TRY(cnt_wavnetc_backward(stream, L.size, L.ctx_dim, N, net->pat, W, net->ctx, L.core, L.cth, L.err,
-                                             prev.err, dW, nullptr));
-                break;
             case K_FEEDBACK:
                 if (L.fb_end > L.fb_start && prev.err) {
                     const size_t pc = (size_t)prev.size * N;

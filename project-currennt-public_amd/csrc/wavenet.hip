@@ -251,12 +251,11 @@ int cnt_cnn_forward(cnt_cnn *h, void *stream_, const char *patTypes, int curT, c
     return CNT_OK;
 }
 
-int cnt_cnn_backward(cnt_cnn *h, void *stream_, const char *patTypes, int curT, const float *weights, const float *x,
-                     const float *outputs, float *output_errors, float *prev_errors, float *weight_updates) {
+int cnt_cnn_backward_errors(cnt_cnn *h, void *stream_, const char *patTypes, int curT, const float *weights,
+                            const float *outputs, float *output_errors, float *prev_errors) {
     using namespace cnt;
-    CNT_REQUIRE(h && patTypes && weights && x && outputs && output_errors && weight_updates,
-                "cnn_backward: null argument");
-    CNT_REQUIRE(curT >= 1 && curT <= h->desc.maxT, "cnn_backward: curT %d outside 1..%d", curT, h->desc.maxT);
+    CNT_REQUIRE(h && patTypes && weights && outputs && output_errors, "cnn_backward_errors: null argument");
+    CNT_REQUIRE(curT >= 1 && curT <= h->desc.maxT, "cnn_backward_errors: curT %d outside 1..%d", curT, h->desc.maxT);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const cnt_cnn_desc &d = h->desc;
     const int P = d.P, D = d.D, S = d.S, N = curT * S;
@@ -297,6 +296,17 @@ int cnt_cnn_backward(cnt_cnn *h, void *stream_, const char *patTypes, int curT, 
             first = false;
         }
     }
+    return CNT_OK;
+}
+
+int cnt_cnn_backward_weights(cnt_cnn *h, void *stream_, const char *patTypes, int curT, const float *x,
+                             const float *output_errors, float *weight_updates) {
+    using namespace cnt;
+    CNT_REQUIRE(h && patTypes && x && output_errors && weight_updates, "cnn_backward_weights: null argument");
+    CNT_REQUIRE(curT >= 1 && curT <= h->desc.maxT, "cnn_backward_weights: curT %d outside 1..%d", curT, h->desc.maxT);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const cnt_cnn_desc &d = h->desc;
+    const int P = d.P, D = d.D, S = d.S, N = curT * S;
 
     CNT_TRY(fill_zero(stream, weight_updates, (size_t)P * h->Lw + D));
     for (const cnt_cnn_group &g : h->groups) {
@@ -322,6 +332,14 @@ int cnt_cnn_backward(cnt_cnn *h, void *stream_, const char *patTypes, int curT, 
     }
     // bias gradient over every slot, padding included, as the reference's ones-vector product does
     return column_sum(stream, output_errors, D, N, d.bias, weight_updates + (size_t)P * h->Lw);
+}
+
+int cnt_cnn_backward(cnt_cnn *h, void *stream, const char *patTypes, int curT, const float *weights, const float *x,
+                     const float *outputs, float *output_errors, float *prev_errors, float *weight_updates) {
+    using namespace cnt;
+    CNT_REQUIRE(x && weight_updates, "cnn_backward: null argument");
+    CNT_TRY(cnt_cnn_backward_errors(h, stream, patTypes, curT, weights, outputs, output_errors, prev_errors));
+    return cnt_cnn_backward_weights(h, stream, patTypes, curT, x, output_errors, weight_updates);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -395,14 +413,14 @@ int cnt_wavnetc_forward(void *stream_, int D, int C, int N, const char *patTypes
     return cnt_gatedact_forward(stream_, D, N, patTypes, core_buf, outputs);
 }
 
-int cnt_wavnetc_backward(void *stream_, int D, int C, int N, const char *patTypes, const float *weights, const float *ctx,
-                         const float *core_buf, float *ctx_tanh, const float *output_errors, float *prev_errors,
-                         float *weight_updates, float *ctx_grad) {
+int cnt_wavnetc_backward_errors(void *stream_, int D, int C, int N, const char *patTypes, const float *weights,
+                                const float *core_buf, float *ctx_tanh, const float *output_errors, float *prev_errors,
+                                float *ctx_grad) {
     using namespace cnt;
     CNT_REQUIRE(patTypes && core_buf && output_errors && prev_errors, "wavnetc_backward: null argument");
     CNT_REQUIRE(D > 0 && N > 0 && C >= 0, "wavnetc_backward: bad size");
-    CNT_REQUIRE(C == 0 || (weights && ctx && ctx_tanh && weight_updates),
-                "wavnetc_backward: conditioning needs weights, context, tanh buffer and weight updates");
+    CNT_REQUIRE(C == 0 || ctx_tanh, "wavnetc_backward: conditioning needs the tanh buffer");
+    CNT_REQUIRE(!ctx_grad || weights, "wavnetc_backward: the context gradient needs the weights");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const size_t count = (size_t)D * N;
     {
@@ -411,21 +429,7 @@ int cnt_wavnetc_backward(void *stream_, int D, int C, int N, const char *patType
                            core_buf, output_errors, prev_errors, C > 0 ? ctx_tanh : static_cast<float *>(nullptr));
         CNT_HIP(hipGetLastError());
     }
-    if (C == 0) return CNT_OK;
-    CNT_TRY(fill_zero(stream, weight_updates, (size_t)C * 2 * D));
-    {
-        GemmArgs ga = {};
-        ga.m = C; ga.n = 2 * D; ga.k = N;
-        ga.a_kcontig = 0; ga.lda = C;
-        ga.b_kcontig = 0; ga.ldb = 2 * D;
-        ga.ldc = C;
-        ga.nseg = 1; ga.nprob = 1; ga.epilogue = EPI_ATOMIC;
-        ga.splitk = 0;  // chosen by the launcher
-        ga.prob[0].A[0] = ctx; ga.prob[0].B[0] = ctx_tanh; ga.prob[0].C = weight_updates;
-        ga.label = "gemm:wavnetc_dW";
-        CNT_TRY(gemm_launch(stream, ga));
-    }
-    if (ctx_grad) {
+    if (C > 0 && ctx_grad) {
         GemmArgs ga = {};
         ga.m = C; ga.n = N; ga.k = 2 * D;
         ga.a_kcontig = 0; ga.lda = C;
@@ -437,6 +441,37 @@ int cnt_wavnetc_backward(void *stream_, int D, int C, int N, const char *patType
         CNT_TRY(gemm_launch(stream, ga));
     }
     return CNT_OK;
+}
+
+int cnt_wavnetc_backward_weights(void *stream_, int D, int C, int N, const float *ctx, const float *ctx_tanh,
+                                 float *weight_updates) {
+    using namespace cnt;
+    CNT_REQUIRE(D > 0 && N > 0 && C >= 0, "wavnetc_backward_weights: bad size");
+    if (C == 0) return CNT_OK;
+    CNT_REQUIRE(ctx && ctx_tanh && weight_updates, "wavnetc_backward_weights: null argument");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    CNT_TRY(fill_zero(stream, weight_updates, (size_t)C * 2 * D));
+    GemmArgs ga = {};
+    ga.m = C; ga.n = 2 * D; ga.k = N;
+    ga.a_kcontig = 0; ga.lda = C;
+    ga.b_kcontig = 0; ga.ldb = 2 * D;
+    ga.ldc = C;
+    ga.nseg = 1; ga.nprob = 1; ga.epilogue = EPI_ATOMIC;
+    ga.splitk = 0;  // chosen by the launcher
+    ga.prob[0].A[0] = ctx; ga.prob[0].B[0] = ctx_tanh; ga.prob[0].C = weight_updates;
+    ga.label = "gemm:wavnetc_dW";
+    return gemm_launch(stream, ga);
+}
+
+int cnt_wavnetc_backward(void *stream, int D, int C, int N, const char *patTypes, const float *weights, const float *ctx,
+                         const float *core_buf, float *ctx_tanh, const float *output_errors, float *prev_errors,
+                         float *weight_updates, float *ctx_grad) {
+    using namespace cnt;
+    CNT_REQUIRE(C == 0 || (weights && ctx && ctx_tanh && weight_updates),
+                "wavnetc_backward: conditioning needs weights, context, tanh buffer and weight updates");
+    CNT_TRY(cnt_wavnetc_backward_errors(stream, D, C, N, patTypes, weights, core_buf, ctx_tanh, output_errors, prev_errors,
+                                        ctx_grad));
+    return cnt_wavnetc_backward_weights(stream, D, C, N, ctx, ctx_tanh, weight_updates);
 }
 
 int cnt_wavnetc_sum_context_grad(void *stream_, int C, int S, int resolution, int n_frame_slots, int N,

@@ -1,8 +1,9 @@
 """BASELINE config 4 as a benchmark workload: backward pass of the 30-block WaveNet-style stack,
-2 waveforms x 16000 samples.  A backward pass consumes state that only the forward pass rebuilds (the skip
-layers' cleared error buffers, the tanh(context) buffer that the gated layer overwrites with its gradient), so
-every timed backward is preceded by an untimed restore of exactly that state; the backward itself is timed with
-events on the launch stream."""
+2 waveforms x 16000 samples, driven through the library's network sequencer from a network file.  A backward pass
+consumes state that only the forward pass rebuilds (the skip layers' cleared error buffers, the tanh(context)
+buffer that the gated layer overwrites with its gradient), so every timed backward is preceded by an untimed
+forward pass; the backward itself is timed with events on the launch stream."""
+import json
 import os
 import time
 
@@ -30,24 +31,19 @@ def run(args, pkg):
     lengths = [16000, 16000]
     S, T = 2, 16000
     pat, onehot, ctx, target, N = WD.make(lengths, Q, C, upsample=80, seed=4)
-    net = networks.WaveNet(networks.HipBackend(), nb, S, T, Q=Q, R=R, K=K, C=C, cnn_tanh=1)
-    shapes = {k: len(net.buf[k]["W"]) for k in net.weight_names()}
+    net = capi.Network(json.dumps(WD.network_json(nb, Q, R, K, C, 1, 10)), S, T, mdn_config=[1, 0, Q, 0, 1, -1])
+    shapes = {L["name"]: L["weight_count"] for L in net.layers if L["weight_count"]}
     for k, w in WD.init_weights(shapes, seed=5).items():
-        net.buf[k]["W"].copy_(torch.from_numpy(w))
-    net.set_inputs(BW._dev(pat), BW._dev(onehot), BW._dev(ctx), BW._dev(target))
-    net.forward()
-    net.calculate_error()
-    saved = {k: v["cth"].clone() for k, v in net.buf.items() if "cth" in v}
-
-    def restore():
-        net.reset_skip_errors()
-        for k, v in saved.items():
-            net.buf[k]["cth"].copy_(v)
+        net.layer(k)["weights"].copy_(torch.from_numpy(w))
+    ctx_d, pat_d = BW._dev(ctx), BW._dev(pat)
+    net.set_context(ctx_d)
+    net.load_sequences(pat_d, T, T, torch.zeros(N, dtype=torch.float32, device="cuda"), BW._dev(target))
+    del onehot  # the feedback layer builds the teacher-forced one-hot input from the targets
 
     def timed_backward(n):
         total = 0.0
         for _ in range(n):
-            restore()
+            net.forward()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             net.backward()
@@ -58,8 +54,9 @@ def run(args, pkg):
 
     timed_backward(args.warmup)
     sec = timed_backward(args.steps)
+    net.forward()
+    torch.cuda.synchronize()
     capi.profile_enable(True)
-    restore()
     net.backward()
     torch.cuda.synchronize()
     prof = capi.profile_read()

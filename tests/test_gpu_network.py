@@ -101,36 +101,6 @@ def test_stacked_network_trains_like_the_oracle(option, momentum, overlap):
     net.close()
 
 
-def wavenet_json(nb, Q, R, K, C, cnn_tanh, dilation_cycle):
-    """Network file with the topology of the reference's example obsolete/scripts/EXAMPLE/MODEL_WAVENET/network.jsn
-    (without its frame-rate conditioning sub-network: the conditioning features are handed to the library)."""
-    def ff(name, size, kind="feedforward_identity"):
-        return {"size": size, "name": name, "bias": 1.0, "type": kind}
-
-    layers = [{"size": 1, "name": "input", "type": "input"},
-              {"size": Q, "name": "feedbackBottom", "bias": 1.0, "type": "feedback", "previousDimEnd": 0,
-               "previousDimStart": 0},
-              ff("emb", R), {"size": R, "name": "causalSkip", "bias": 1.0, "type": "skipini"}]
-    res = "causalSkip"
-    for l in range(nb):
-        dil = 2 ** (l % dilation_cycle)
-        layers += [
-            {"size": 2 * R, "name": "cnn%d" % l, "bias": 1.0, "type": "cnn", "window_width": "%d*1" % (2 * R),
-             "window_tap_interval": "%d*%d" % (2 * R, dil), "causal": 1, "tanhoutput": cnn_tanh},
-            {"size": R, "name": "wav%d" % l, "bias": 1.0, "type": "wavnetc", "contextDim": C},
-            ff("out%d" % l, R),
-            {"size": R, "name": "sadd%d" % l, "bias": 1.0, "type": "skipadd", "preSkipLayer": "%s,out%d" % (res, l)},
-            {"size": R, "name": "temp%d" % l, "bias": 1.0, "type": "skipini"},
-            ff("sot%d" % l, K),
-            {"size": K, "name": "skip%d" % l, "bias": 1.0, "type": "skipini"},
-            {"size": R, "name": "temp2_%d" % l, "bias": 1.0, "type": "skipadd", "preSkipLayer": "temp%d" % l}]
-        res = "temp2_%d" % l
-    layers += [{"size": K, "name": "postAdd", "bias": 1.0, "type": "skipadd",
-                "preSkipLayer": ",".join("skip%d" % l for l in range(nb))},
-               ff("postL1", K, "feedforward_tanh"), ff("output", Q), {"size": 1, "name": "postoutput", "type": "mdn"}]
-    return {"layers": layers}
-
-
 @pytest.mark.parametrize("nb,cnn_tanh", [(4, 1), (11, 0)])
 def test_wavenet_network_file_against_oracle_graph(nb, cnn_tanh):
     import torch
@@ -152,7 +122,7 @@ def test_wavenet_network_file_against_oracle_graph(nb, cnn_tanh):
     ref.calculate_error()
     ref.backward()
 
-    doc = wavenet_json(nb, Q, R, K, C, cnn_tanh, 3)
+    doc = WD.network_json(nb, Q, R, K, C, cnn_tanh, 3)
     net = capi.Network(json.dumps(doc), S, T + 7, mdn_config=[1, 0, Q, 0, 1, -1])   # buffers longer than the fraction
     names = [L["name"] for L in net.layers if L["weight_count"]]
     assert sorted(names) == sorted(W)

@@ -36,3 +36,33 @@ def make(lengths, Q, C, upsample, seed):
 def init_weights(net_weight_shapes, seed, scale=0.1):
     rng = np.random.default_rng(seed)
     return {k: rng.uniform(-scale, scale, n).astype(np.float32) for k, n in net_weight_shapes.items()}
+
+
+def network_json(nb, Q, R, K, C, cnn_tanh, dilation_cycle):
+    """Network file with the topology of the reference's example obsolete/scripts/EXAMPLE/MODEL_WAVENET/network.jsn
+    (without its frame-rate conditioning sub-network: the conditioning features are handed to the library)."""
+    def ff(name, size, kind="feedforward_identity"):
+        return {"size": size, "name": name, "bias": 1.0, "type": kind}
+
+    layers = [{"size": 1, "name": "input", "type": "input"},
+              {"size": Q, "name": "feedbackBottom", "bias": 1.0, "type": "feedback", "previousDimEnd": 0,
+               "previousDimStart": 0},
+              ff("emb", R), {"size": R, "name": "causalSkip", "bias": 1.0, "type": "skipini"}]
+    res = "causalSkip"
+    for l in range(nb):
+        dil = 2 ** (l % dilation_cycle)
+        layers += [
+            {"size": 2 * R, "name": "cnn%d" % l, "bias": 1.0, "type": "cnn", "window_width": "%d*1" % (2 * R),
+             "window_tap_interval": "%d*%d" % (2 * R, dil), "causal": 1, "tanhoutput": cnn_tanh},
+            {"size": R, "name": "wav%d" % l, "bias": 1.0, "type": "wavnetc", "contextDim": C},
+            ff("out%d" % l, R),
+            {"size": R, "name": "sadd%d" % l, "bias": 1.0, "type": "skipadd", "preSkipLayer": "%s,out%d" % (res, l)},
+            {"size": R, "name": "temp%d" % l, "bias": 1.0, "type": "skipini"},
+            ff("sot%d" % l, K),
+            {"size": K, "name": "skip%d" % l, "bias": 1.0, "type": "skipini"},
+            {"size": R, "name": "temp2_%d" % l, "bias": 1.0, "type": "skipadd", "preSkipLayer": "temp%d" % l}]
+        res = "temp2_%d" % l
+    layers += [{"size": K, "name": "postAdd", "bias": 1.0, "type": "skipadd",
+                "preSkipLayer": ",".join("skip%d" % l for l in range(nb))},
+               ff("postL1", K, "feedforward_tanh"), ff("output", Q), {"size": 1, "name": "postoutput", "type": "mdn"}]
+    return {"layers": layers}
