@@ -196,6 +196,9 @@ struct NetLayer {
     float *core = nullptr, *cth = nullptr;  // wavnetc
     int ctx_dim = 0;
     int fb_start = 0, fb_end = 0;            // feedback: dimensions taken from the preceding layer
+    const float *total = nullptr;            // skip layers: where the summed error stands after the layer's step
+    bool needs_sum = false;                  // skip layers: errors += side buffer is not a no-op
+    int live_targets = 0;                    // skip layers: sources that receive the sum through a launch
     const float **in_ptrs = nullptr;         // skip layers: device tables
     float **tgt_ptrs = nullptr;
     int *tgt_is_skip = nullptr;
@@ -220,16 +223,19 @@ __global__ void skip_sum_kernel(size_t count, int n, const float *const *__restr
 
 // errors += errors_from_skip, then to every linked source in reverse order: added to a skip layer's side buffer,
 // written over any other layer's error buffer (layers/SkipAddLayer.cu:305-346)
+// errors_from_skip == NULL: nothing to add, `errors` is only read
 __global__ void skip_fan_kernel(size_t count, int n, float *const *__restrict__ target, const int *__restrict__ is_skip,
-                                float *__restrict__ errors, const float *__restrict__ errors_from_skip) {
+                                float *errors, const float *__restrict__ errors_from_skip) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (; i < count; i += stride) {
-        const float e = errors_from_skip[i] + errors[i];
-        errors[i] = e;
-        for (int k = n - 1; k >= 0; --k) {
+        float e = errors[i];
+        if (errors_from_skip) {
+            e = errors_from_skip[i] + e;
+            errors[i] = e;
+        }
+        for (int k = 0; k < n; ++k) {
             float *t = target[k];
-            if (t == nullptr) continue;  // a source without an error buffer (the input layer)
             t[i] = is_skip[k] ? e + t[i] : e;
         }
     }
@@ -514,40 +520,107 @@ int finish_build(cnt_network *net, const json::Value *weights) {
         }
         CNT_HIP(hipMemcpy(net->weights, host.data(), (size_t)total * sizeof(float), hipMemcpyHostToDevice));
     }
-    // error buffers of the skip layers: one allocation, [err | eskip] per layer
+    // ---- routing of the skip layers' errors -------------------------------------------------------------------
+    // The reference gives every skip layer an error buffer and a side buffer, adds the two in the layer's backward
+    // step and hands the sum to every linked source (layers/SkipAddLayer.cu:305-346).  Which of these buffers ever
+    // differ is known once the layer list stands:
+    //   * a skip layer that no ordinary layer follows (nothing writes its error buffer) and that exactly one later
+    //     skip layer links to only forwards that layer's sum: it shares the sum by pointer and owns no buffers;
+    //   * a skip layer that no later skip layer links to has an all-zero side buffer: no addition, no side buffer;
+    //   * a source that is a feedforward_identity layer (its backward step only reads its errors) and that receives
+    //     its errors from this link alone shares the sum by pointer instead of receiving a copy.
+    // What remains is one launch per skip layer that still has something to add or to hand on.
+    const int n_layers = (int)net->layers.size();
+    std::vector<int> links(n_layers, 0), linker(n_layers, -1), link_slot(n_layers, -1);
+    for (int y = 0; y < n_layers; ++y)
+        if (is_skip_kind(net->layers[(size_t)y].kind))
+            for (size_t k = 0; k < net->layers[(size_t)y].pre.size(); ++k) {
+                const int x = net->layers[(size_t)y].pre[k];
+                ++links[x];
+                linker[x] = y;
+                link_slot[x] = (int)k;
+            }
+    auto followed_by_writer = [&](int i) {
+        if (i + 1 >= n_layers) return false;
+        const NetLayer &nx = net->layers[(size_t)i + 1];
+        if (is_skip_kind(nx.kind)) return false;
+        return !(nx.kind == K_FEEDBACK && nx.fb_end == nx.fb_start);
+    };
+    std::vector<char> shares(n_layers, 0);  // skip layer that shares its linker's sum
     size_t skip_total = 0;
-    for (auto &L : net->layers)
-        if (is_skip_kind(L.kind)) skip_total += 2 * (size_t)L.size * slots;
+    for (int i = 0; i < n_layers; ++i) {
+        NetLayer &L = net->layers[(size_t)i];
+        if (!is_skip_kind(L.kind)) continue;
+        shares[i] = (!followed_by_writer(i) && links[i] == 1) ? 1 : 0;
+        L.needs_sum = !shares[i] && links[i] > 0;
+        if (!shares[i]) skip_total += (size_t)L.size * slots * (links[i] > 0 ? 2 : 1);
+    }
     net->skip_error_count = skip_total;
     if (skip_total) {
         CNT_TRY(device_alloc(net, (void **)&net->skip_errors, skip_total * sizeof(float), true));
         size_t at = 0;
-        for (auto &L : net->layers)
-            if (is_skip_kind(L.kind)) {
-                L.err = net->skip_errors + at;
-                L.eskip = L.err + (size_t)L.size * slots;
-                at += 2 * (size_t)L.size * slots;
+        for (int i = 0; i < n_layers; ++i) {
+            NetLayer &L = net->layers[(size_t)i];
+            if (!is_skip_kind(L.kind) || shares[i]) continue;
+            L.err = net->skip_errors + at;
+            at += (size_t)L.size * slots;
+            if (links[i] > 0) {
+                L.eskip = net->skip_errors + at;
+                at += (size_t)L.size * slots;
             }
+        }
     }
-    // pointer tables of the skip layers
-    for (auto &L : net->layers) {
+    // sums, from the last layer to the first (a linker comes after the layers it links to)
+    for (int i = n_layers - 1; i >= 0; --i) {
+        NetLayer &L = net->layers[(size_t)i];
+        if (!is_skip_kind(L.kind)) continue;
+        L.total = shares[i] ? net->layers[(size_t)linker[i]].total : L.err;
+        if (shares[i]) L.err = const_cast<float *>(L.total);  // what cnt_network_layer_info reports as this layer's errors
+    }
+    // pointer tables.  A source that shares the sum needs no write; what a sharing skip layer hands on is handed on
+    // by the layer that owns the sum, in that layer's launch (sums into side buffers commute, and a source whose
+    // error buffer an ordinary layer writes later is overwritten then either way).
+    std::vector<int> owner(n_layers, -1);
+    for (int i = n_layers - 1; i >= 0; --i)
+        if (is_skip_kind(net->layers[(size_t)i].kind)) owner[i] = shares[i] ? owner[linker[i]] : i;
+    std::vector<std::vector<float *>> tgt(n_layers);
+    std::vector<std::vector<int>> flag(n_layers);
+    for (int i = n_layers - 1; i >= 0; --i) {
+        NetLayer &L = net->layers[(size_t)i];
+        if (!is_skip_kind(L.kind)) continue;
+        for (size_t k = L.pre.size(); k-- > 0;) {  // last source first, as the reference walks them
+            const int x = L.pre[k];
+            NetLayer &src = net->layers[(size_t)x];
+            float *t = nullptr;
+            const int skip = is_skip_kind(src.kind) ? 1 : 0;
+            if (skip) {
+                t = shares[x] ? nullptr : src.eskip;
+            } else if (src.kind == K_DENSE && src.act == ACT_IDENTITY && links[x] == 1 && !followed_by_writer(x)) {
+                src.err = const_cast<float *>(L.total);  // the buffer allocated for it stays unused
+            } else {
+                t = src.err;
+            }
+            if (t) {
+                tgt[(size_t)owner[i]].push_back(t);
+                flag[(size_t)owner[i]].push_back(skip);
+            }
+        }
+    }
+    for (int i = 0; i < n_layers; ++i) {
+        NetLayer &L = net->layers[(size_t)i];
         if (!is_skip_kind(L.kind)) continue;
         const size_t n = L.pre.size();
         std::vector<const float *> in(n);
-        std::vector<float *> tgt(n);
-        std::vector<int> flag(n);
-        for (size_t k = 0; k < n; ++k) {
-            const NetLayer &src = net->layers[(size_t)L.pre[k]];
-            in[k] = src.out;
-            flag[k] = is_skip_kind(src.kind) ? 1 : 0;
-            tgt[k] = flag[k] ? src.eskip : src.err;
-        }
+        for (size_t k = 0; k < n; ++k) in[k] = net->layers[(size_t)L.pre[k]].out;
         CNT_TRY(device_alloc(net, (void **)&L.in_ptrs, n * sizeof(float *), false));
-        CNT_TRY(device_alloc(net, (void **)&L.tgt_ptrs, n * sizeof(float *), false));
-        CNT_TRY(device_alloc(net, (void **)&L.tgt_is_skip, n * sizeof(int), false));
         CNT_HIP(hipMemcpy(L.in_ptrs, in.data(), n * sizeof(float *), hipMemcpyHostToDevice));
-        CNT_HIP(hipMemcpy(L.tgt_ptrs, tgt.data(), n * sizeof(float *), hipMemcpyHostToDevice));
-        CNT_HIP(hipMemcpy(L.tgt_is_skip, flag.data(), n * sizeof(int), hipMemcpyHostToDevice));
+        std::vector<float *> &t = tgt[(size_t)i];
+        L.live_targets = (int)t.size();
+        if (t.empty()) continue;
+        CNT_TRY(device_alloc(net, (void **)&L.tgt_ptrs, t.size() * sizeof(float *), false));
+        CNT_TRY(device_alloc(net, (void **)&L.tgt_is_skip, t.size() * sizeof(int), false));
+        CNT_HIP(hipMemcpy(L.tgt_ptrs, t.data(), t.size() * sizeof(float *), hipMemcpyHostToDevice));
+        CNT_HIP(hipMemcpy(L.tgt_is_skip, flag[(size_t)i].data(), t.size() * sizeof(int), hipMemcpyHostToDevice));
     }
     // checks that need the whole list
     const NetLayer &post = net->layers.back();
@@ -825,9 +898,11 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 break;
             case K_SKIPINI:
             case K_SKIPADD: {
+                if (!L.needs_sum && L.live_targets == 0) break;
                 ProfileScope prof(stream, "skip_fan");
                 hipLaunchKernelGGL(skip_fan_kernel, dim3(blocks_for(count)), dim3(256), 0, stream, count,
-                                   (int)L.pre.size(), L.tgt_ptrs, L.tgt_is_skip, L.err, L.eskip);
+                                   L.live_targets, L.tgt_ptrs, L.tgt_is_skip, const_cast<float *>(L.total),
+                                   L.needs_sum ? L.eskip : static_cast<const float *>(nullptr));
                 CNT_HIP(hipGetLastError());
                 break;
             }
