@@ -309,7 +309,9 @@ int cnt_dft_backward(cnt_dft *h, void *stream, float *prev_errors);
 /* ---- network sequencer ------------------------------------------------------------------------------
  * NeuralNetwork<TDevice> for the layer types of this library (NeuralNetwork.cpp): "input", "feedforward_identity /
  * _tanh / _logistic / _relu", "lstm", "blstm", "skipini", "skipadd" (with "preSkipLayer"), "cnn" (1-D), "wavnetc",
- * "feedback" (one step back, fed by one softmax unit) and the post-output layers "sse" and "mdn".  json_text is the
+ * "feedback" (one step back, fed by one softmax unit), "skipcat" (with "preSkipLayerDim"), "externalloader" and the
+ * post-output layers "sse" and "mdn"; layers may run at a lower time "resolution" (layers/Layer.cu:254-305), and a
+ * layer flagged "wavenetConditionInputLayer" feeds the wavnetc layers (NeuralNetwork.cpp:544-561).  json_text is the
  * text of a network file: "layers" in order, optionally "weights" with the "input" / "bias" / "internal" arrays of
  * every trainable layer (layers/TrainableLayer.cu:135-220).  Without "weights" the weights are zero until the caller
  * fills them (cnt_network_weights, cnt_network_randomize).  All weights of the network, and all weight updates, are
@@ -329,6 +331,8 @@ typedef struct {
     long n_input, n_bias, n_internal; /* lengths of the three sections of its weight vector         */
     float *outputs;                  /* device, size x (maxSeqLength*S); a post-output layer keeps the targets here */
     float *output_errors;            /* device, same shape; NULL for the input and post-output layers */
+    int resolution;                  /* "resolution": the layer has one slot per so many time steps; its buffers hold
+                                        size x (ceil(maxSeqLength / resolution) * S) floats                      */
 } cnt_layer_info;
 /* NeuralNetwork::NeuralNetwork (NeuralNetwork.cpp:374-609, :805-812).  options may be NULL. */
 int cnt_network_create(const char *json_text, int parallel_sequences, int max_seq_length,
@@ -346,6 +350,13 @@ int cnt_network_randomize(cnt_network *net, unsigned seed, float range);
  * "wavenetConditionInputLayer", layers/wavNetCore.cu:455-492; cnt_wavnetc_load_context does that step).  The
  * pointer is kept, not the data. */
 int cnt_network_set_context(cnt_network *net, const float *ctx);
+/* External data of an "externalloader" layer (layers/ExternalLoader.cu:58-110, :205-250; the reference reads the
+ * fraction's files there): data is [frame][sequence][dimension] in device memory with max_frames frames per
+ * sequence; slot (t', s) of the layer takes the frame whose index the network's input layer (size 1) holds at time
+ * step t' * resolution.  mean_std = [size means | size standard deviations] ("externalDataMV") or NULL.  The
+ * pointers are kept, not the data. */
+int cnt_network_set_external_input(cnt_network *net, int layer_index, const float *data, int max_frames,
+                                   const float *mean_std);
 /* NeuralNetwork::loadSequences (NeuralNetwork.cpp:1367-1417): records the fraction's geometry and pattern types
  * (device memory, char[T*S], kept by pointer), copies inputs (input size x T*S) and targets (post-output size x T*S)
  * when given, and passes the call on to the layers that keep per-fraction state. */

@@ -43,7 +43,7 @@ class NetworkOptions(C.Structure):
 class LayerInfo(C.Structure):
     _fields_ = [("name", C.c_char * 64), ("type", C.c_char * 32), ("size", C.c_int), ("weight_offset", C.c_long),
                 ("n_input", C.c_long), ("n_bias", C.c_long), ("n_internal", C.c_long), ("outputs", C.c_void_p),
-                ("output_errors", C.c_void_p)]
+                ("output_errors", C.c_void_p), ("resolution", C.c_int)]
 
 
 class LstmDesc(C.Structure):
@@ -128,6 +128,7 @@ _SIGNATURES = {
     "cnt_network_weight_updates": (VP, [VP]),
     "cnt_network_randomize": (I, [VP, C.c_uint, F]),
     "cnt_network_set_context": (I, [VP, VP]),
+    "cnt_network_set_external_input": (I, [VP, I, VP, I, VP]),
     "cnt_network_load_sequences": (I, [VP, VP, I, I, VP, VP, VP]),
     "cnt_network_forward": (I, [VP, VP]),
     "cnt_network_calculate_error": (I, [VP, VP, VP]),
@@ -456,15 +457,15 @@ class Network:
         self.weights = _device_view(lib().cnt_network_weights(self.handle), self.n_weights, self)
         self.updates = _device_view(lib().cnt_network_weight_updates(self.handle), self.n_weights, self)
         self.layers = []
-        slots = parallel_sequences * max_seq_length
         for i in range(self.n_layers):
             info = LayerInfo()
             check(lib().cnt_network_layer_info(self.handle, i, C.byref(info)))
             n = info.n_input + info.n_bias + info.n_internal
+            slots = parallel_sequences * (-(-max_seq_length // info.resolution))
             self.layers.append({
                 "name": info.name.decode(), "type": info.type.decode(), "size": info.size,
                 "weight_offset": info.weight_offset, "weight_count": n,
-                "sections": (info.n_input, info.n_bias, info.n_internal),
+                "sections": (info.n_input, info.n_bias, info.n_internal), "resolution": info.resolution,
                 "outputs": _device_view(info.outputs, info.size * slots, self),
                 "errors": _device_view(info.output_errors, info.size * slots, self),
                 "weights": self.weights[info.weight_offset:info.weight_offset + n] if n else None,
@@ -495,6 +496,12 @@ class Network:
     def set_context(self, ctx):
         self._ctx = ctx  # the library keeps the pointer only
         check(lib().cnt_network_set_context(self.handle, ptr(ctx)))
+
+    def set_external_input(self, layer_name, data, max_frames, mean_std=None):
+        index = [L["name"] for L in self.layers].index(layer_name)
+        self._ext = getattr(self, "_ext", {})
+        self._ext[layer_name] = (data, mean_std)  # the library keeps the pointers only
+        check(lib().cnt_network_set_external_input(self.handle, index, ptr(data), max_frames, ptr(mean_std)))
 
     def load_sequences(self, pat, T, Tmin, inputs=None, targets=None, stream=None):
         self._pat = pat

@@ -177,9 +177,11 @@ struct Parser {
 
 namespace {
 
-enum Kind { K_INPUT, K_DENSE, K_LSTM, K_SKIPINI, K_SKIPADD, K_CNN, K_WAVNETC, K_FEEDBACK, K_SSE, K_MDN };
+enum Kind { K_INPUT, K_DENSE, K_LSTM, K_SKIPINI, K_SKIPADD, K_SKIPCAT, K_CNN, K_WAVNETC, K_FEEDBACK, K_EXTERNAL, K_SSE,
+            K_MDN };
 
-inline bool is_skip_kind(int k) { return k == K_SKIPINI || k == K_SKIPADD; }
+inline bool is_sum_skip(int k) { return k == K_SKIPINI || k == K_SKIPADD; }
+inline bool is_skip_kind(int k) { return is_sum_skip(k) || k == K_SKIPCAT; }
 
 struct NetLayer {
     std::string name, type, text;  // text: the layer's object as it stands in the network file
@@ -196,6 +198,15 @@ struct NetLayer {
     float *core = nullptr, *cth = nullptr;  // wavnetc
     int ctx_dim = 0;
     int fb_start = 0, fb_end = 0;            // feedback: dimensions taken from the preceding layer
+    // time base: a layer with "resolution" r has one slot per r time steps (layers/Layer.cu:254-305)
+    int res = 1, maxTr = 0;
+    int T = 0, Tmin = 0, N = 0;              // of the current fraction, at this layer's resolution
+    const char *pat = nullptr;               // pattern types at this layer's resolution
+    std::string flag;                        // "layerFlag"
+    std::vector<int> cat_lo, cat_hi;         // skipcat: dimension range taken from each source
+    const float *ext_data = nullptr;         // externalloader: [frame][sequence][dimension], set by the caller
+    const float *ext_mean_std = nullptr;
+    int ext_frames = 0, index_load_method = 0;
     const float *total = nullptr;            // skip layers: where the summed error stands after the layer's step
     bool needs_sum = false;                  // skip layers: errors += side buffer is not a no-op
     int live_targets = 0;                    // skip layers: sources that receive the sum through a launch
@@ -276,6 +287,93 @@ __global__ void feedback_backward_kernel(size_t count, int prev_total, int prev_
     }
 }
 
+// Pattern types at a lower time resolution, as data_sets/DataSet.cpp:993-1012 leaves them: slot t' covers the time
+// steps [t'*res, (t'+1)*res); none if the sequence has ended before it, first for t' = 0, otherwise the type of the
+// last time step of the sequence inside the block (normal, or last if the sequence ends there).
+__global__ void lowres_pat_kernel(int S, int T, int Tr, int res, const char *__restrict__ pat, char *__restrict__ out) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= Tr * S) return;
+    const int tr = i / S, s = i % S;
+    const int t0 = tr * res;
+    char v = 0;
+    if (pat[(size_t)t0 * S + s] != 0) {
+        if (tr == 0) {
+            v = 1;
+        } else {
+            const int tl = min(t0 + res - 1, T - 1);
+            const char p = pat[(size_t)tl * S + s];
+            v = p == 0 ? 3 : p;
+        }
+    }
+    out[i] = v;
+}
+
+// ExternalLoader::loadSequences (layers/ExternalLoader.cu:58-110, :205-250): slot (t', s) takes frame
+// frame_index[(t'*res)*S + s] (divided by res for indexLoadMethod 1) of sequence s from the external data,
+// optionally (x - mean) / std with std < 1e-5 taken as 1; 0 on padding slots and beyond the data.
+__global__ void external_load_kernel(size_t count, int dim, int S, int res, int method, int max_frames,
+                                     const float *__restrict__ data, const float *__restrict__ frame_index,
+                                     const float *__restrict__ mean_std, const char *__restrict__ pat,
+                                     float *__restrict__ out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const int d = (int)(i % dim);
+        const long slot = (long)(i / dim);
+        const long tr = slot / S;
+        const int s = (int)(slot % S);
+        float v = 0.0f;
+        if (pat[slot] != 0) {
+            int frame = (int)frame_index[(size_t)tr * res * S + s];
+            if (method == 1) frame /= res;
+            if (frame < max_frames) {
+                v = data[((size_t)frame * S + s) * dim + d];
+                if (mean_std) {
+                    const float sd = mean_std[dim + d];
+                    v = (v - mean_std[d]) / (sd < 1e-5f ? 1.0f : sd);
+                }
+            }
+        }
+        out[i] = v;
+    }
+}
+
+// SkipCatLayer (layers/SkipCatLayer.cu:52-91): dimensions [lo, lo+n) of the source into [at, at+n) of this layer
+// (forward), and the errors back (backward: added to a skip layer's side buffer on non-padding slots, written to
+// any other layer's error buffer, which the caller has zero-filled, on non-padding slots).
+__global__ void skipcat_forward_kernel(size_t count, int n, int src_dim, int lo, int dst_dim, int at,
+                                       const float *__restrict__ src, float *__restrict__ dst) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const size_t slot = i / n;
+        const int j = (int)(i % n);
+        dst[slot * dst_dim + at + j] = src[slot * src_dim + lo + j];
+    }
+}
+__global__ void skipcat_backward_kernel(size_t count, int n, int src_dim, int lo, int dst_dim, int at, int accumulate,
+                                        const char *__restrict__ pat, const float *__restrict__ errors,
+                                        float *__restrict__ target) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const size_t slot = i / n;
+        const int j = (int)(i % n);
+        float *t = target + slot * src_dim + lo + j;
+        if (pat[slot] == 0) {
+            if (!accumulate) *t = 0.0f;
+            continue;
+        }
+        const float e = errors[slot * dst_dim + at + j];
+        *t = accumulate ? *t + e : e;
+    }
+}
+__global__ void add_inplace_kernel(size_t count, float *__restrict__ a, const float *__restrict__ b) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) a[i] += b[i];
+}
+
 // "64*1_64*2": <count>*<value> runs joined by '_' (the reference's CNN option strings); one value per filter
 bool parse_runs(const std::string &opt, int D, std::vector<int> &out) {
     out.clear();
@@ -322,7 +420,12 @@ struct cnt_network {
     float *weights = nullptr, *updates = nullptr;
     float *skip_errors = nullptr;  // err and eskip of every skip layer, one allocation
     size_t skip_error_count = 0;
-    const float *ctx = nullptr;    // conditioning features of the wavnetc layers, C x (maxT*S), set by the caller
+    const float *ctx = nullptr;    // conditioning features of the wavnetc layers, C x (maxT*S)
+    // conditioning sub-network: the layer flagged "wavenetConditionInputLayer" feeds the wavnetc layers
+    int flagged = -1, first_wavnetc = -1;
+    float *ctx_own = nullptr, *ctx_grad = nullptr;
+    struct LowRes { int res; char *pat; };
+    std::vector<LowRes> low_res;
     std::vector<void *> allocations;
     hipStream_t side = nullptr;
     hipEvent_t ev_main = nullptr, ev_side = nullptr;
@@ -374,10 +477,13 @@ int build_layer(cnt_network *net, const json::Value &obj, const char *text, cons
     L.bias = (bias && bias->type == json::Value::NUM) ? (float)bias->num : 0.0f;
     L.prev = index - 1;
     CNT_REQUIRE(L.size > 0, "network: layer %d ('%s') has no positive size", index, L.name.c_str());
-    CNT_REQUIRE(get_int(obj, "resolution", 1) == 1, "network: layer '%s' has a time resolution other than 1, which is "
-                "not built", L.name.c_str());
+    L.res = get_int(obj, "resolution", 1);
+    CNT_REQUIRE(L.res >= 1, "network: layer '%s' has resolution %d", L.name.c_str(), L.res);
+    L.maxTr = (net->maxT + L.res - 1) / L.res;
+    L.flag = get_str(obj, "layerFlag");
     const int P = index > 0 ? net->layers[(size_t)index - 1].size : 0;
-    const size_t slots = (size_t)net->S * net->maxT;
+    const int prev_res = index > 0 ? net->layers[(size_t)index - 1].res : 1;
+    const size_t slots = (size_t)net->S * L.maxTr;
     const std::string &t = L.type;
     static const char *ff[] = {"feedforward_identity", "feedforward_tanh", "feedforward_logistic", "feedforward_relu"};
     bool trainable = true;
@@ -392,7 +498,7 @@ int build_layer(cnt_network *net, const json::Value &obj, const char *text, cons
     } else if (t == "lstm" || t == "blstm") {
         L.kind = K_LSTM;
         L.bidir = t == "blstm";
-        cnt_lstm_desc d = {P, L.size, L.bidir, net->S, net->maxT, L.bias};
+        cnt_lstm_desc d = {P, L.size, L.bidir, net->S, L.maxTr, L.bias};
         CNT_TRY(cnt_lstm_create(&d, &L.lstm));
     } else if (t == "skipini" || t == "skipadd") {
         // NeuralNetwork.cpp:470-530 offers every earlier skip layer plus the layer right before; SkipAddLayer.cu:
@@ -424,9 +530,73 @@ int build_layer(cnt_network *net, const json::Value &obj, const char *text, cons
             L.pre.assign(offer.end() - 2, offer.end());
         }
         CNT_REQUIRE(!L.pre.empty(), "network: skip layer '%s' is linked to no layer", L.name.c_str());
-        for (int j : L.pre)
+        for (int j : L.pre) {
             CNT_REQUIRE(net->layers[(size_t)j].size == L.size, "network: skip layer '%s' (size %d) is linked to '%s' of "
                         "size %d", L.name.c_str(), L.size, net->layers[(size_t)j].name.c_str(), net->layers[(size_t)j].size);
+            CNT_REQUIRE(net->layers[(size_t)j].res == L.res, "network: skip layer '%s' is linked to '%s' of another "
+                        "resolution", L.name.c_str(), net->layers[(size_t)j].name.c_str());
+        }
+    } else if (t == "skipcat") {
+        // SkipCatLayer::SkipCatLayer (layers/SkipCatLayer.cu:100-200): the layers named by preSkipLayer, of each the
+        // dimension range [a, b) given by preSkipLayerDim "a_b_a_b..." (default: all of it)
+        L.kind = K_SKIPCAT;
+        std::vector<int> offer;
+        for (int j = 0; j < index; ++j)
+            if (is_skip_kind(net->layers[(size_t)j].kind)) offer.push_back(j);
+        offer.push_back(index - 1);
+        const std::string names = get_str(obj, "preSkipLayer");
+        CNT_REQUIRE(!names.empty(), "network: no preSkipLayer configuration in skipcat layer '%s'", L.name.c_str());
+        size_t b = 0;
+        while (b <= names.size()) {
+            size_t e = names.find(',', b);
+            if (e == std::string::npos) e = names.size();
+            const std::string one = names.substr(b, e - b);
+            for (int j : offer)
+                if (net->layers[(size_t)j].name == one) {
+                    L.pre.push_back(j);
+                    break;
+                }
+            b = e + 1;
+        }
+        CNT_REQUIRE(!L.pre.empty(), "network: skipcat layer '%s' is linked to no layer", L.name.c_str());
+        std::vector<int> dims;
+        const std::string ds = get_str(obj, "preSkipLayerDim");
+        if (!ds.empty()) {
+            size_t i = 0;
+            while (i < ds.size()) {
+                char *endp = nullptr;
+                const long v = strtol(ds.c_str() + i, &endp, 10);
+                CNT_REQUIRE(endp != ds.c_str() + i, "network: skipcat layer '%s': bad preSkipLayerDim", L.name.c_str());
+                dims.push_back((int)v);
+                i = (size_t)(endp - ds.c_str());
+                if (i < ds.size() && ds[i] == '_') ++i;
+            }
+        } else {
+            for (int j : L.pre) {
+                dims.push_back(0);
+                dims.push_back(net->layers[(size_t)j].size);
+            }
+        }
+        CNT_REQUIRE(dims.size() == 2 * L.pre.size(), "network: skipcat layer '%s': preSkipLayerDim needs two numbers per "
+                    "layer of preSkipLayer", L.name.c_str());
+        int total = 0;
+        for (size_t k = 0; k < L.pre.size(); ++k) {
+            const NetLayer &src = net->layers[(size_t)L.pre[k]];
+            const int lo = dims[2 * k], hi = dims[2 * k + 1];
+            CNT_REQUIRE(lo >= 0 && hi >= lo && hi <= src.size, "network: skipcat layer '%s': range %d..%d outside layer "
+                        "'%s'", L.name.c_str(), lo, hi, src.name.c_str());
+            CNT_REQUIRE(src.res == L.res, "network: skipcat layer '%s' needs layers of its own resolution", L.name.c_str());
+            L.cat_lo.push_back(lo);
+            L.cat_hi.push_back(hi);
+            total += hi - lo;
+        }
+        CNT_REQUIRE(total == L.size, "network: skipcat layer '%s' has size %d, its sources give %d", L.name.c_str(), L.size,
+                    total);
+    } else if (t == "externalloader") {
+        L.kind = K_EXTERNAL;
+        L.index_load_method = get_int(obj, "indexLoadMethod", 0);
+        CNT_REQUIRE(net->layers.front().size == 1, "network: externalloader layer '%s' reads the frame index from an input "
+                    "layer of size 1", L.name.c_str());
     } else if (t == "cnn") {
         L.kind = K_CNN;
         CNT_REQUIRE(!obj.has("window_height") && get_int(obj, "repeat_padding", 0) == 0,
@@ -436,13 +606,17 @@ int build_layer(cnt_network *net, const json::Value &obj, const char *text, cons
                     "not give one value per filter", L.name.c_str());
         CNT_REQUIRE(parse_runs(get_str(obj, "window_tap_interval"), L.size, dil), "network: cnn layer '%s': "
                     "window_tap_interval does not give one value per filter", L.name.c_str());
-        cnt_cnn_desc d = {P, L.size, net->S, net->maxT, get_int(obj, "causal", 0), get_int(obj, "tanhoutput", 1), L.bias};
+        cnt_cnn_desc d = {P, L.size, net->S, L.maxTr, get_int(obj, "causal", 0), get_int(obj, "tanhoutput", 1), L.bias};
         CNT_TRY(cnt_cnn_create(&d, hw.data(), dil.data(), &L.cnn));
     } else if (t == "wavnetc") {
         L.kind = K_WAVNETC;
         L.ctx_dim = get_int(obj, "contextDim", 0);
         CNT_REQUIRE(P == 2 * L.size, "network: wavnetc layer '%s' of size %d needs a preceding layer of size %d",
                     L.name.c_str(), L.size, 2 * L.size);
+        CNT_REQUIRE(L.res == 1, "network: wavnetc layer '%s' must have resolution 1", L.name.c_str());
+        CNT_REQUIRE(get_str(obj, "contextMV").empty(), "network: wavnetc layer '%s': contextMV is not built",
+                    L.name.c_str());
+        if (net->first_wavnetc < 0) net->first_wavnetc = index;
         CNT_TRY(device_alloc(net, (void **)&L.core, 2 * (size_t)L.size * slots * sizeof(float), true));
         CNT_TRY(device_alloc(net, (void **)&L.cth, 2 * (size_t)L.size * slots * sizeof(float), true));
     } else if (t == "feedback") {
@@ -474,14 +648,19 @@ int build_layer(cnt_network *net, const json::Value &obj, const char *text, cons
         set_error("network: layer '%s' has type '%s', which this path does not cover", L.name.c_str(), t.c_str());
         return CNT_ERR_ARG;
     }
+    // a layer runs on the time base of the layer before it; an externalloader starts one, a feedback layer that takes
+    // nothing from the layer before it is independent of that layer's
+    if (index > 0 && L.kind != K_EXTERNAL && !(L.kind == K_FEEDBACK && L.fb_end == L.fb_start))
+        CNT_REQUIRE(prev_res == L.res, "network: layer '%s' has resolution %d, the layer before it %d", L.name.c_str(),
+                    L.res, prev_res);
     // every trainable layer of a network file carries "bias" (layers/TrainableLayer.cu:118-120)
     if (trainable) CNT_REQUIRE(bias != nullptr, "network: missing value 'bias' in layer '%s'", L.name.c_str());
     weight_sections(L, P);
     const size_t count = (size_t)L.size * slots;
-    const bool alias = is_skip_kind(L.kind) && L.pre.size() == 1;
+    const bool alias = is_sum_skip(L.kind) && L.pre.size() == 1;
     if (alias) L.out = net->layers[(size_t)L.pre[0]].out;
     else CNT_TRY(device_alloc(net, (void **)&L.out, count * sizeof(float), true));
-    if (L.kind != K_INPUT && L.kind != K_SSE && L.kind != K_MDN && !is_skip_kind(L.kind))
+    if (L.kind != K_INPUT && L.kind != K_EXTERNAL && L.kind != K_SSE && L.kind != K_MDN && !is_skip_kind(L.kind))
         CNT_TRY(device_alloc(net, (void **)&L.err, count * sizeof(float), true));
     net->layers.push_back(std::move(L));
     return CNT_OK;
@@ -536,14 +715,23 @@ int finish_build(cnt_network *net, const json::Value *weights) {
         if (is_skip_kind(net->layers[(size_t)y].kind))
             for (size_t k = 0; k < net->layers[(size_t)y].pre.size(); ++k) {
                 const int x = net->layers[(size_t)y].pre[k];
-                ++links[x];
+                // a skipcat hands on parts of its sum: whatever it links to keeps buffers of its own
+                links[x] += net->layers[(size_t)y].kind == K_SKIPCAT ? 2 : 1;
                 linker[x] = y;
                 link_slot[x] = (int)k;
+            }
+    // the layer that feeds the wavnetc layers receives its errors from them
+    if (net->first_wavnetc >= 0 && net->layers[(size_t)net->first_wavnetc].ctx_dim > 0)
+        for (int j = 0; j < net->first_wavnetc; ++j)
+            if (net->layers[(size_t)j].flag == "wavenetConditionInputLayer") {
+                net->flagged = j;
+                break;
             }
     auto followed_by_writer = [&](int i) {
         if (i + 1 >= n_layers) return false;
         const NetLayer &nx = net->layers[(size_t)i + 1];
-        if (is_skip_kind(nx.kind)) return false;
+        if (i == net->flagged) return true;
+        if (is_skip_kind(nx.kind) || nx.kind == K_EXTERNAL) return false;
         return !(nx.kind == K_FEEDBACK && nx.fb_end == nx.fb_start);
     };
     std::vector<char> shares(n_layers, 0);  // skip layer that shares its linker's sum
@@ -551,9 +739,11 @@ int finish_build(cnt_network *net, const json::Value *weights) {
     for (int i = 0; i < n_layers; ++i) {
         NetLayer &L = net->layers[(size_t)i];
         if (!is_skip_kind(L.kind)) continue;
-        shares[i] = (!followed_by_writer(i) && links[i] == 1) ? 1 : 0;
+        const size_t lslots = (size_t)net->S * L.maxTr;
+        if (L.kind == K_SKIPCAT) links[i] = std::max(links[i], 2);  // always keeps both buffers
+        shares[i] = (is_sum_skip(L.kind) && !followed_by_writer(i) && links[i] == 1) ? 1 : 0;
         L.needs_sum = !shares[i] && links[i] > 0;
-        if (!shares[i]) skip_total += (size_t)L.size * slots * (links[i] > 0 ? 2 : 1);
+        if (!shares[i]) skip_total += (size_t)L.size * lslots * (links[i] > 0 ? 2 : 1);
     }
     net->skip_error_count = skip_total;
     if (skip_total) {
@@ -562,11 +752,12 @@ int finish_build(cnt_network *net, const json::Value *weights) {
         for (int i = 0; i < n_layers; ++i) {
             NetLayer &L = net->layers[(size_t)i];
             if (!is_skip_kind(L.kind) || shares[i]) continue;
+            const size_t lslots = (size_t)net->S * L.maxTr;
             L.err = net->skip_errors + at;
-            at += (size_t)L.size * slots;
+            at += (size_t)L.size * lslots;
             if (links[i] > 0) {
                 L.eskip = net->skip_errors + at;
-                at += (size_t)L.size * slots;
+                at += (size_t)L.size * lslots;
             }
         }
     }
@@ -587,7 +778,7 @@ int finish_build(cnt_network *net, const json::Value *weights) {
     std::vector<std::vector<int>> flag(n_layers);
     for (int i = n_layers - 1; i >= 0; --i) {
         NetLayer &L = net->layers[(size_t)i];
-        if (!is_skip_kind(L.kind)) continue;
+        if (!is_sum_skip(L.kind)) continue;
         for (size_t k = L.pre.size(); k-- > 0;) {  // last source first, as the reference walks them
             const int x = L.pre[k];
             NetLayer &src = net->layers[(size_t)x];
@@ -608,7 +799,7 @@ int finish_build(cnt_network *net, const json::Value *weights) {
     }
     for (int i = 0; i < n_layers; ++i) {
         NetLayer &L = net->layers[(size_t)i];
-        if (!is_skip_kind(L.kind)) continue;
+        if (!is_sum_skip(L.kind)) continue;
         const size_t n = L.pre.size();
         std::vector<const float *> in(n);
         for (size_t k = 0; k < n; ++k) in[k] = net->layers[(size_t)L.pre[k]].out;
@@ -622,6 +813,36 @@ int finish_build(cnt_network *net, const json::Value *weights) {
         CNT_HIP(hipMemcpy(L.tgt_ptrs, t.data(), t.size() * sizeof(float *), hipMemcpyHostToDevice));
         CNT_HIP(hipMemcpy(L.tgt_is_skip, flag[(size_t)i].data(), t.size() * sizeof(int), hipMemcpyHostToDevice));
     }
+    // pattern types of the lower time resolutions, one buffer per resolution
+    for (auto &L : net->layers) {
+        if (L.res == 1) continue;
+        bool have = false;
+        for (auto &lr : net->low_res) have = have || lr.res == L.res;
+        if (have) continue;
+        cnt_network::LowRes lr = {L.res, nullptr};
+        CNT_TRY(device_alloc(net, (void **)&lr.pat, (size_t)net->S * L.maxTr, true));
+        net->low_res.push_back(lr);
+    }
+    // conditioning sub-network (NeuralNetwork.cpp:544-561, layers/wavNetCore.cu:455-492, :895-913): the wavnetc
+    // layers read the flagged layer's outputs through the frame index in the input layer and send their summed
+    // gradient back to it
+    if (net->flagged >= 0) {
+        const NetLayer &f = net->layers[(size_t)net->flagged];
+        const int C = net->layers[(size_t)net->first_wavnetc].ctx_dim;
+        CNT_REQUIRE(f.kind != K_WAVNETC && f.size == C, "network: layer '%s' feeds the wavnetc layers but has size %d, "
+                    "contextDim is %d", f.name.c_str(), f.size, C);
+        CNT_REQUIRE(net->layers.front().size == 1, "network: the conditioning sub-network reads the frame index from an "
+                    "input layer of size 1");
+        CNT_REQUIRE(f.err != nullptr, "network: layer '%s' feeds the wavnetc layers but has no error buffer",
+                    f.name.c_str());
+        CNT_TRY(device_alloc(net, (void **)&net->ctx_own, (size_t)C * slots * sizeof(float), true));
+        CNT_TRY(device_alloc(net, (void **)&net->ctx_grad, (size_t)C * slots * sizeof(float), true));
+        net->ctx = net->ctx_own;
+    }
+    for (auto &L : net->layers)
+        if (L.kind == K_WAVNETC)
+            CNT_REQUIRE(L.ctx_dim == net->layers[(size_t)net->first_wavnetc].ctx_dim, "network: wavnetc layer '%s' has "
+                        "another contextDim than the first one", L.name.c_str());
     // checks that need the whole list
     const NetLayer &post = net->layers.back();
     CNT_REQUIRE(post.kind == K_SSE || post.kind == K_MDN, "network: the last layer must be a post-output layer (sse or "
@@ -728,6 +949,7 @@ int cnt_network_layer_info(cnt_network *net, int index, cnt_layer_info *info) {
     info->n_internal = L.n_int;
     info->outputs = L.out;
     info->output_errors = L.err;
+    info->resolution = L.res;
     return CNT_OK;
 }
 
@@ -748,7 +970,24 @@ int cnt_network_randomize(cnt_network *net, unsigned seed, float range) {
 int cnt_network_set_context(cnt_network *net, const float *ctx) {
     using namespace cnt;
     CNT_REQUIRE(net, "network_set_context: null handle");
+    CNT_REQUIRE(net->flagged < 0, "network_set_context: this network computes the conditioning features itself (layer "
+                "'%s')", net->layers[(size_t)net->flagged].name.c_str());
     net->ctx = ctx;
+    return CNT_OK;
+}
+
+int cnt_network_set_external_input(cnt_network *net, int layer_index, const float *data, int max_frames,
+                                   const float *mean_std) {
+    using namespace cnt;
+    CNT_REQUIRE(net && data, "network_set_external_input: null argument");
+    CNT_REQUIRE(layer_index >= 0 && layer_index < (int)net->layers.size() &&
+                net->layers[(size_t)layer_index].kind == K_EXTERNAL,
+                "network_set_external_input: layer %d is not an externalloader layer", layer_index);
+    CNT_REQUIRE(max_frames >= 1, "network_set_external_input: no frames");
+    NetLayer &L = net->layers[(size_t)layer_index];
+    L.ext_data = data;
+    L.ext_frames = max_frames;
+    L.ext_mean_std = mean_std;
     return CNT_OK;
 }
 
@@ -769,9 +1008,23 @@ int cnt_network_load_sequences(cnt_network *net, void *stream_, int T, int Tmin,
     // a post-output layer keeps the targets in its own outputs() (layers/PostOutputLayer.cu:108-124)
     if (targets)
         CNT_HIP(hipMemcpyAsync(post.out, targets, slots * post.size * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    // Layer::loadSequences (layers/Layer.cu:254-305): lengths and pattern types at each layer's resolution
+    for (auto &lr : net->low_res) {
+        const int Tr = (T + lr.res - 1) / lr.res;
+        const int n = Tr * net->S;
+        hipLaunchKernelGGL(lowres_pat_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, net->S, T, Tr, lr.res,
+                           patTypes, lr.pat);
+        CNT_HIP(hipGetLastError());
+    }
     for (auto &L : net->layers) {
-        if (L.lstm) CNT_TRY(cnt_lstm_load_sequences(L.lstm, stream, patTypes, T, Tmin));
-        if (L.mdn) CNT_TRY(cnt_mdn_load_sequences(L.mdn, stream, patTypes, T));
+        L.T = (T + L.res - 1) / L.res;
+        L.Tmin = (Tmin + L.res - 1) / L.res;
+        L.N = L.T * net->S;
+        L.pat = patTypes;
+        for (auto &lr : net->low_res)
+            if (lr.res == L.res) L.pat = lr.pat;
+        if (L.lstm) CNT_TRY(cnt_lstm_load_sequences(L.lstm, stream, L.pat, L.T, L.Tmin));
+        if (L.mdn) CNT_TRY(cnt_mdn_load_sequences(L.mdn, stream, L.pat, L.T));
     }
     return CNT_OK;
 }
@@ -780,13 +1033,13 @@ int cnt_network_forward(cnt_network *net, void *stream_) {
     using namespace cnt;
     CNT_REQUIRE(net && net->T > 0, "network_forward: no fraction loaded");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    const int N = net->T * net->S;
     // what the skip layers' forward passes clear (layers/SkipAddLayer.cu:195-205)
     if (net->skip_error_count) CNT_TRY(fill_zero(stream, net->skip_errors, net->skip_error_count));
     for (size_t i = 1; i < net->layers.size(); ++i) {
         NetLayer &L = net->layers[i];
         const NetLayer &prev = net->layers[i - 1];
         const float *W = net->weights + L.w_off;
+        const int N = L.N;
         const size_t count = (size_t)L.size * N;
         switch (L.kind) {
             case K_DENSE:
@@ -804,13 +1057,43 @@ int cnt_network_forward(cnt_network *net, void *stream_) {
                     CNT_HIP(hipGetLastError());
                 }
                 break;
+            case K_SKIPCAT: {
+                int at = 0;
+                for (size_t k = 0; k < L.pre.size(); ++k) {
+                    const NetLayer &src = net->layers[(size_t)L.pre[k]];
+                    const int n = L.cat_hi[k] - L.cat_lo[k];
+                    if (n == 0) continue;
+                    const size_t c = (size_t)n * N;
+                    hipLaunchKernelGGL(skipcat_forward_kernel, dim3(blocks_for(c)), dim3(256), 0, stream, c, n, src.size,
+                                       L.cat_lo[k], L.size, at, src.out, L.out);
+                    CNT_HIP(hipGetLastError());
+                    at += n;
+                }
+                break;
+            }
+            case K_EXTERNAL:
+                CNT_REQUIRE(L.ext_data, "network_forward: externalloader layer '%s' has no data "
+                            "(cnt_network_set_external_input)", L.name.c_str());
+                hipLaunchKernelGGL(external_load_kernel, dim3(blocks_for(count)), dim3(256), 0, stream, count, L.size,
+                                   net->S, L.res, L.index_load_method, L.ext_frames, L.ext_data, net->layers.front().out,
+                                   L.ext_mean_std, L.pat, L.out);
+                CNT_HIP(hipGetLastError());
+                break;
             case K_CNN:
-                CNT_TRY(cnt_cnn_forward(L.cnn, stream, net->pat, net->T, W, prev.out, L.out));
+                CNT_TRY(cnt_cnn_forward(L.cnn, stream, L.pat, L.T, W, prev.out, L.out));
                 break;
             case K_WAVNETC:
                 CNT_REQUIRE(L.ctx_dim == 0 || net->ctx, "network_forward: wavnetc layer '%s' has no conditioning features "
                             "(cnt_network_set_context)", L.name.c_str());
-                CNT_TRY(cnt_wavnetc_forward(stream, L.size, L.ctx_dim, N, net->pat, W, net->ctx, prev.out, L.core, L.cth,
+                if ((int)i == net->first_wavnetc && net->flagged >= 0) {
+                    // WavNetCore::__loadContextBuff (layers/wavNetCore.cu:455-492) and the clearing of the gradient
+                    // buffer for the conditioning sub-network (:645-647)
+                    const NetLayer &f = net->layers[(size_t)net->flagged];
+                    CNT_TRY(fill_zero(stream, net->ctx_grad, (size_t)L.ctx_dim * N));
+                    CNT_TRY(cnt_wavnetc_load_context(stream, L.ctx_dim, net->S, N, f.T, f.res == 1 ? 1 : 0, f.out,
+                                                     net->layers.front().out, nullptr, L.pat, net->ctx_own));
+                }
+                CNT_TRY(cnt_wavnetc_forward(stream, L.size, L.ctx_dim, N, L.pat, W, net->ctx, prev.out, L.core, L.cth,
                                             L.out));
                 break;
             case K_FEEDBACK: {
@@ -818,7 +1101,7 @@ int cnt_network_forward(cnt_network *net, void *stream_) {
                 ProfileScope prof(stream, "feedback");
                 hipLaunchKernelGGL(feedback_kernel, dim3(blocks_for(count)), dim3(256), 0, stream, count, L.size,
                                    L.fb_end - L.fb_start, prev.size, L.fb_start, net->S, post.size, net->mdn_target_start,
-                                   net->pat, prev.out, post.out, L.out);
+                                   L.pat, prev.out, post.out, L.out);
                 CNT_HIP(hipGetLastError());
                 break;
             }
@@ -836,10 +1119,9 @@ int cnt_network_calculate_error(cnt_network *net, void *stream_, float *loss_dev
     using namespace cnt;
     CNT_REQUIRE(net && loss_dev && net->T > 0, "network_calculate_error: null argument or no fraction loaded");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    const int N = net->T * net->S;
     NetLayer &post = net->layers.back();
     const NetLayer &last = net->layers[net->layers.size() - 2];
-    if (post.kind == K_SSE) return cnt_sse_error(stream, post.size, N, net->pat, last.out, post.out, loss_dev);
+    if (post.kind == K_SSE) return cnt_sse_error(stream, post.size, post.N, post.pat, last.out, post.out, loss_dev);
     return cnt_mdn_calculate_error(post.mdn, stream, post.out, loss_dev);
 }
 
@@ -848,13 +1130,13 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     CNT_REQUIRE(net && net->T > 0, "network_backward: no fraction loaded");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     hipStream_t wstream = net->overlap ? net->side : stream;
-    const int N = net->T * net->S;
     bool side_used = false;
     for (size_t i = net->layers.size() - 1; i >= 1; --i) {
         NetLayer &L = net->layers[i];
         NetLayer &prev = net->layers[i - 1];
         const float *W = net->weights + L.w_off;
         float *dW = net->updates + L.w_off;
+        const int N = L.N;
         // the input layer has no error buffer; a feedback layer that takes nothing from its preceding layer passes
         // nothing on, and neither does anything that feeds such a feedback layer's one-hot part
         float *prev_err = prev.err;
@@ -862,7 +1144,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
         const size_t count = (size_t)L.size * N;
         switch (L.kind) {
             case K_SSE:
-                CNT_TRY(cnt_sse_backward(stream, L.size, N, net->pat, prev.out, L.out, prev.err));
+                CNT_TRY(cnt_sse_backward(stream, L.size, N, L.pat, prev.out, L.out, prev.err));
                 break;
             case K_MDN:
                 CNT_TRY(cnt_mdn_backward(L.mdn, stream, L.out, prev.err));
@@ -876,10 +1158,18 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 else if (L.kind == K_LSTM)
                     CNT_TRY(cnt_lstm_backward_errors(L.lstm, stream, W, L.err, prev_err));
                 else if (L.kind == K_CNN)
-                    CNT_TRY(cnt_cnn_backward_errors(L.cnn, stream, net->pat, net->T, W, L.out, L.err, prev_err));
-                else
-                    CNT_TRY(cnt_wavnetc_backward_errors(stream, L.size, L.ctx_dim, N, net->pat, W, L.core, L.cth, L.err,
-                                                        prev.err, nullptr));
+                    CNT_TRY(cnt_cnn_backward_errors(L.cnn, stream, L.pat, L.T, W, L.out, L.err, prev_err));
+                else {
+                    CNT_TRY(cnt_wavnetc_backward_errors(stream, L.size, L.ctx_dim, N, L.pat, W, L.core, L.cth, L.err,
+                                                        prev.err, net->flagged >= 0 ? net->ctx_grad : nullptr));
+                    if ((int)i == net->first_wavnetc && net->flagged >= 0) {
+                        // every wavnetc layer has added its share; hand the sum per frame to the layer that feeds them
+                        // (layers/wavNetCore.cu:895-913)
+                        NetLayer &f = net->layers[(size_t)net->flagged];
+                        CNT_TRY(cnt_wavnetc_sum_context_grad(stream, L.ctx_dim, net->S, f.res, f.N, N, f.pat, L.pat,
+                                                             net->ctx_grad, f.err));
+                    }
+                }
                 if (L.kind == K_WAVNETC && L.ctx_dim == 0) break;
                 // the weight half has no consumer before the optimizer: second stream, after the error half
                 if (net->overlap) {
@@ -892,7 +1182,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 else if (L.kind == K_LSTM)
                     CNT_TRY(cnt_lstm_backward_weights(L.lstm, wstream, prev.out, dW));
                 else if (L.kind == K_CNN)
-                    CNT_TRY(cnt_cnn_backward_weights(L.cnn, wstream, net->pat, net->T, prev.out, L.err, dW));
+                    CNT_TRY(cnt_cnn_backward_weights(L.cnn, wstream, L.pat, L.T, prev.out, L.err, dW));
                 else
                     CNT_TRY(cnt_wavnetc_backward_weights(wstream, L.size, L.ctx_dim, N, net->ctx, L.cth, dW));
                 break;
@@ -904,6 +1194,29 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                                    L.live_targets, L.tgt_ptrs, L.tgt_is_skip, const_cast<float *>(L.total),
                                    L.needs_sum ? L.eskip : static_cast<const float *>(nullptr));
                 CNT_HIP(hipGetLastError());
+                break;
+            }
+            case K_SKIPCAT: {
+                // SkipCatLayer::computeBackwardPass (layers/SkipCatLayer.cu:340-397)
+                hipLaunchKernelGGL(add_inplace_kernel, dim3(blocks_for(count)), dim3(256), 0, stream, count, L.err, L.eskip);
+                CNT_HIP(hipGetLastError());
+                int at = 0;
+                for (size_t k = 0; k < L.pre.size(); ++k) {
+                    NetLayer &src = net->layers[(size_t)L.pre[k]];
+                    const int n = L.cat_hi[k] - L.cat_lo[k];
+                    const int skip = is_skip_kind(src.kind) ? 1 : 0;
+                    float *target = skip ? src.eskip : src.err;
+                    if (target != nullptr) {
+                        if (!skip) CNT_TRY(fill_zero(stream, src.err, (size_t)src.size * net->S * src.maxTr));
+                        if (n > 0) {
+                            const size_t c = (size_t)n * N;
+                            hipLaunchKernelGGL(skipcat_backward_kernel, dim3(blocks_for(c)), dim3(256), 0, stream, c, n,
+                                               src.size, L.cat_lo[k], L.size, at, skip, L.pat, L.err, target);
+                            CNT_HIP(hipGetLastError());
+                        }
+                    }
+                    at += n;
+                }
                 break;
             }
             case K_FEEDBACK:

@@ -28,7 +28,12 @@ def test_matrix_product_rejects_double_transpose():
         capi.matrix_product(a, 2, 2, 2, a, 1, a, 1, 0)
 
 
-@pytest.mark.parametrize("P,D,N,act", [(382, 512, 600, 1), (512, 187, 600, 0), (33, 65, 130, 2), (64, 64, 256, 3)])
+@pytest.mark.parametrize("P,D,N,act", [
+    (382, 512, 600, 1), (512, 187, 600, 0), (33, 65, 130, 2), (64, 64, 256, 3),
+    # small layers, long contraction (the shapes of a WaveNet-style stack's 1x1 layers): split-K weight gradients
+    # with one, several and ragged tiles, sizes that are not multiples of the tile
+    (64, 128, 3000, 0), (128, 1024, 777, 1), (80, 20, 1501, 2), (12, 8, 200, 0), (128, 132, 999, 3),
+])
 def test_dense(P, D, N, act):
     print("dense case", P, D, N, act, flush=True)
     assert PC.run_dense_case(P, D, N, act, 1.0, seed=P + D) < TOL

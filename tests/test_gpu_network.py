@@ -193,3 +193,127 @@ def test_network_file_rejections():
     with pytest.raises(RuntimeError, match="no fraction"):
         net.forward()
     net.close()
+
+
+class _CondOracleBackend(OM.OracleBackend):
+    """Oracle back end whose gated layers also accumulate the gradient with respect to the conditioning features."""
+    ctx_grad = None
+
+    def wavnetc_backward(self, D, C, N, pat, W, ctx, core, cth, err, prev_err, dW):
+        O.wavnetc_backward(D, C, N, pat, W, ctx, core, cth, err, prev_err, dW, self.ctx_grad)
+
+
+def test_wavenet_with_frame_rate_conditioning_network():
+    """The reference example's layout in full: externalloader -> skipini -> blstm -> cnn -> skipcat at one slot per
+    R time steps, flagged as the wavnetc layers' input; the oracle side walks the same graph with the oracle's
+    primitives (conditioning part spelled out here, sample-rate part by the shared graph walk)."""
+    import torch
+
+    print("wavenet network file with conditioning sub-network", flush=True)
+    pkg = PC.pkg()
+    capi, networks = pkg.capi, pkg.networks
+    nb, Q, R, K = 3, 64, 32, 64
+    E, HB, DC, C, RES = 12, 128, 10, 11, 4
+    lengths = [120, 90]
+    S, T = len(lengths), max(lengths)
+    Tr = -(-T // RES)
+    lengths_r = [-(-n // RES) for n in lengths]
+    pat, onehot, _, target, N = WD.make(lengths, Q, C, upsample=RES, seed=2)
+    pat_r = make_pat_types(lengths_r, Tr)
+    Nr = S * Tr
+    rng = np.random.default_rng(11)
+    frame_index = np.zeros((T, S), dtype=np.float32)
+    for s, n in enumerate(lengths):
+        frame_index[:n, s] = np.arange(n) // RES
+    data = rng.standard_normal((Tr, S, E)).astype(np.float32)
+    mean_std = np.concatenate([0.1 * rng.standard_normal(E), rng.uniform(0.5, 2.0, E)]).astype(np.float32)
+    mean_std[E + 3] = 1e-7   # a vanishing deviation counts as 1
+
+    # ---- oracle: conditioning part -----------------------------------------------------------------------------
+    valid_r = (pat_r != 0)
+    sd = np.where(mean_std[E:] < 1e-5, 1.0, mean_std[E:])
+    ext = ((data - mean_std[:E]) / sd).astype(np.float32).reshape(Nr, E)
+    ext[~valid_r] = 0
+    ext = np.ascontiguousarray(ext.reshape(-1))
+    w_lstm = rng.uniform(-0.1, 0.1, OM.weight_count({"type": "blstm", "size": HB}, E)).astype(np.float32)
+    hw, it = np.ones(DC, dtype=np.int32), np.ones(DC, dtype=np.int32)
+    w_cnn = rng.uniform(-0.1, 0.1, HB * 3 * DC + DC).astype(np.float32)
+    desc = O.LstmDesc(E, HB, 1, S, Tr, min(lengths_r), 1.0)
+    fw, bw = O.LstmState(HB // 2, Nr), O.LstmState(HB // 2, Nr)
+    l2 = np.zeros(HB * Nr, dtype=np.float32)
+    O.lstm_forward(desc, w_lstm, pat_r, ext, fw, bw, l2)
+    l3 = np.zeros(DC * Nr, dtype=np.float32)
+    con = np.zeros(3 * DC * Nr, dtype=np.float32)
+    O.cnn_forward(HB, DC, S, Tr, 0, 0, 1.0, hw, it, pat_r, w_cnn, l2, con, l3)
+    cat = np.concatenate([l3.reshape(Nr, DC), ext.reshape(Nr, E)[:, 11:12]], axis=1).astype(np.float32)
+    ctx = np.zeros(C * N, dtype=np.float32)
+    O.wavnetc_load_context(C, S, N, Tr, False, np.ascontiguousarray(cat.reshape(-1)), frame_index.reshape(-1), None, pat, ctx)
+
+    # ---- oracle: sample-rate part --------------------------------------------------------------------------------
+    backend = _CondOracleBackend()
+    backend.ctx_grad = np.zeros(C * N, dtype=np.float32)
+    ref = networks.WaveNet(backend, nb, S, T, Q=Q, R=R, K=K, C=C, cnn_tanh=1, dilation_cycle=3)
+    W = WD.init_weights({k: len(ref.buf[k]["W"]) for k in ref.weight_names()}, seed=3)
+    for k, w in W.items():
+        ref.buf[k]["W"][:] = w
+    ref.set_inputs(pat, onehot, ctx, target)
+    ref.forward()
+    ref.calculate_error()
+    ref.backward()
+    cat_err = np.zeros(C * Nr, dtype=np.float32)
+    O.wavnetc_sum_context_grad(C, S, RES, Nr, N, pat_r, pat, backend.ctx_grad, cat_err)
+    cat_err = cat_err.reshape(Nr, C)
+    l3_err = np.zeros((Nr, DC), dtype=np.float32)
+    l3_err[valid_r] = cat_err[valid_r, :DC]
+    l3_err = np.ascontiguousarray(l3_err.reshape(-1))
+    l2_err = np.zeros(HB * Nr, dtype=np.float32)
+    dw_cnn = np.zeros_like(w_cnn)
+    O.cnn_backward(HB, DC, S, Tr, 0, 0, 1.0, hw, it, pat_r, w_cnn, l2, l3, l3_err, con, l2_err, dw_cnn)
+    skip_err = np.zeros(E * Nr, dtype=np.float32)
+    dw_lstm = np.zeros_like(w_lstm)
+    O.lstm_backward(desc, w_lstm, pat_r, ext, l2_err, fw, bw, skip_err, dw_lstm)
+    W["exL2"], W["exL3"] = w_lstm, w_cnn
+    dW_ref = {k: ref.buf[k]["dW"] for k in ref.weight_names()}
+    dW_ref["exL2"], dW_ref["exL3"] = dw_lstm, dw_cnn
+
+    # ---- the library, from the network file ---------------------------------------------------------------------
+    doc = WD.network_json(nb, Q, R, K, C, 1, 3)
+    cond = [{"size": E, "name": "exL1", "type": "externalloader", "bias": 1.0, "resolution": RES},
+            {"size": E, "name": "exSkip", "bias": 1.0, "type": "skipini", "resolution": RES},
+            {"size": HB, "name": "exL2", "bias": 1.0, "type": "blstm", "resolution": RES},
+            {"size": DC, "name": "exL3", "bias": 1.0, "type": "cnn", "window_width": "%d*1" % DC,
+             "window_tap_interval": "%d*1" % DC, "tanhoutput": 0, "resolution": RES},
+            {"size": C, "name": "exAdd", "bias": 1.0, "type": "skipcat", "resolution": RES,
+             "preSkipLayer": "exL3,exSkip", "preSkipLayerDim": "0_%d_11_12" % DC,
+             "layerFlag": "wavenetConditionInputLayer"}]
+    doc["layers"] = doc["layers"][:1] + cond + doc["layers"][1:]
+    net = capi.Network(json.dumps(doc), S, T + 6, mdn_config=[1, 0, Q, 0, 1, -1])
+    assert net.layer("exL2")["resolution"] == RES and net.layer("emb")["resolution"] == 1
+    for L in net.layers:
+        if L["weight_count"]:
+            assert L["weight_count"] == W[L["name"]].size, L["name"]
+            L["weights"].copy_(torch.from_numpy(W[L["name"]]))
+    net.set_external_input("exL1", PC.dev(data.reshape(-1)), Tr, PC.dev(mean_std))
+    with pytest.raises(RuntimeError, match="computes the conditioning features itself"):
+        net.set_context(PC.dev(ctx))
+    for _ in range(2):
+        net.load_sequences(PC.dev(pat), T, min(lengths), PC.dev(frame_index.reshape(-1)), PC.dev(target))
+        net.forward()
+        loss = float(net.calculate_error().item())
+        net.backward()
+        net.check()
+        torch.cuda.synchronize()
+        assert PC.relerr(net.layer("exL1")["outputs"][: ext.size].cpu().numpy(), ext) < 1e-6
+        assert PC.relerr(net.layer("exAdd")["outputs"][: cat.size].cpu().numpy(), cat.reshape(-1)) < TOL
+        ref_loss = float(ref.loss[0])
+        assert abs(loss - ref_loss) <= TOL * abs(ref_loss)
+        assert PC.relerr(net.layer("exAdd")["errors"][: cat_err.size].cpu().numpy(), cat_err.reshape(-1)) < TOL
+        worst = 0.0
+        for L in net.layers:
+            if L["weight_count"]:
+                e = PC.relerr(L["updates"].cpu().numpy(), dW_ref[L["name"]])
+                worst = max(worst, e)
+                if e > TOL:
+                    print("   ", L["name"], e, flush=True)
+        assert worst < TOL
+    net.close()
