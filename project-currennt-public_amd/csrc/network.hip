@@ -15,6 +15,7 @@
 // halves of dense and LSTM layers run on a second stream of the same priority.
 #include "common.hpp"
 
+#include <algorithm>
 #include <cerrno>
 #include <cmath>
 #include <cstdlib>
@@ -427,8 +428,11 @@ struct cnt_network {
     struct LowRes { int res; char *pat; };
     std::vector<LowRes> low_res;
     std::vector<void *> allocations;
-    hipStream_t side = nullptr;
-    hipEvent_t ev_main = nullptr, ev_side = nullptr;
+    // weight gradients go round-robin to these streams (default priority); CNT_NET_SIDE_STREAMS overrides the count
+    static constexpr int kMaxSide = 4;
+    hipStream_t side[kMaxSide] = {};
+    hipEvent_t ev_main = nullptr, ev_side[kMaxSide] = {};
+    int n_side = 2;
     int overlap = 1;
     // optimizer state (allocated by the first update)
     float *cur_updates = nullptr, *deltas = nullptr, *stats = nullptr;
@@ -858,9 +862,13 @@ int finish_build(cnt_network *net, const json::Value *weights) {
             CNT_REQUIRE(L.size == (L.fb_end - L.fb_start) + net->mdn_classes, "network: feedback layer '%s' has size "
                         "%d, expected %d + %d classes", L.name.c_str(), L.size, L.fb_end - L.fb_start, net->mdn_classes);
         }
-    CNT_HIP(hipStreamCreateWithFlags(&net->side, hipStreamNonBlocking));
+    if (const char *e = std::getenv("CNT_NET_SIDE_STREAMS"))
+        net->n_side = std::max(1, std::min((int)cnt_network::kMaxSide, std::atoi(e)));
     CNT_HIP(hipEventCreateWithFlags(&net->ev_main, hipEventDisableTiming));
-    CNT_HIP(hipEventCreateWithFlags(&net->ev_side, hipEventDisableTiming));
+    for (int k = 0; k < net->n_side; ++k) {
+        CNT_HIP(hipStreamCreateWithFlags(&net->side[k], hipStreamNonBlocking));
+        CNT_HIP(hipEventCreateWithFlags(&net->ev_side[k], hipEventDisableTiming));
+    }
     return CNT_OK;
 }
 
@@ -877,9 +885,11 @@ int cnt_network_destroy(cnt_network *net) {
         if (L.mdn) cnt_mdn_destroy(L.mdn);
     }
     for (void *p : net->allocations) (void)hipFree(p);
-    if (net->side) (void)hipStreamDestroy(net->side);
+    for (int k = 0; k < cnt_network::kMaxSide; ++k) {
+        if (net->side[k]) (void)hipStreamDestroy(net->side[k]);
+        if (net->ev_side[k]) (void)hipEventDestroy(net->ev_side[k]);
+    }
     if (net->ev_main) (void)hipEventDestroy(net->ev_main);
-    if (net->ev_side) (void)hipEventDestroy(net->ev_side);
     delete net;
     return CNT_OK;
 }
@@ -1129,8 +1139,9 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     using namespace cnt;
     CNT_REQUIRE(net && net->T > 0, "network_backward: no fraction loaded");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    hipStream_t wstream = net->overlap ? net->side : stream;
-    bool side_used = false;
+    hipStream_t wstream = stream;
+    int next_side = 0;
+    bool side_used[cnt_network::kMaxSide] = {};
     for (size_t i = net->layers.size() - 1; i >= 1; --i) {
         NetLayer &L = net->layers[i];
         NetLayer &prev = net->layers[i - 1];
@@ -1173,9 +1184,11 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 if (L.kind == K_WAVNETC && L.ctx_dim == 0) break;
                 // the weight half has no consumer before the optimizer: second stream, after the error half
                 if (net->overlap) {
+                    wstream = net->side[next_side];
                     CNT_HIP(hipEventRecord(net->ev_main, stream));
-                    CNT_HIP(hipStreamWaitEvent(net->side, net->ev_main, 0));
-                    side_used = true;
+                    CNT_HIP(hipStreamWaitEvent(wstream, net->ev_main, 0));
+                    side_used[next_side] = true;
+                    next_side = (next_side + 1) % net->n_side;
                 }
                 if (L.kind == K_DENSE)
                     CNT_TRY(cnt_dense_backward_weights(wstream, prev.size, L.size, N, L.bias, prev.out, L.err, dW));
@@ -1231,9 +1244,10 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 break;
         }
     }
-    if (side_used) {
-        CNT_HIP(hipEventRecord(net->ev_side, net->side));
-        CNT_HIP(hipStreamWaitEvent(stream, net->ev_side, 0));
+    for (int k = 0; k < net->n_side; ++k) {
+        if (!side_used[k]) continue;
+        CNT_HIP(hipEventRecord(net->ev_side[k], net->side[k]));
+        CNT_HIP(hipStreamWaitEvent(stream, net->ev_side[k], 0));
     }
     return CNT_OK;
 }
