@@ -211,9 +211,10 @@ int cnt_cnn_backward(cnt_cnn *h, void *stream, const char *patTypes, int curT, c
 
 /* The two halves of cnt_cnn_backward for callers that put the weight gradients on another stream (the reference
  * has no such split): _errors = tanh derivative in place and prev_errors; _weights reads x and the finished
- * output_errors.  Calling both in this order on one stream is cnt_cnn_backward. */
+ * output_errors.  Calling both in this order on one stream (delta_applied = 0) is cnt_cnn_backward.
+ * delta_applied != 0: output_errors already holds tanh'(y) * error (see cnt_wavnetc_backward_errors). */
 int cnt_cnn_backward_errors(cnt_cnn *h, void *stream, const char *patTypes, int curT, const float *weights,
-                            const float *outputs, float *output_errors, float *prev_errors);
+                            const float *outputs, float *output_errors, float *prev_errors, int delta_applied);
 int cnt_cnn_backward_weights(cnt_cnn *h, void *stream, const char *patTypes, int curT, const float *x,
                              const float *output_errors, float *weight_updates);
 
@@ -240,10 +241,13 @@ int cnt_wavnetc_backward(void *stream, int D, int C, int N, const char *patTypes
                          const float *ctx, const float *core_buf, float *ctx_tanh, const float *output_errors,
                          float *prev_errors, float *weight_updates, float *ctx_grad);
 /* The two halves of cnt_wavnetc_backward (same split as above): _errors = prev_errors, the gradient left in
- * ctx_tanh and the optional context gradient; _weights = weight_updates from ctx and that gradient. */
+ * ctx_tanh and the optional context gradient; _weights = weight_updates from ctx and that gradient.
+ * prev_tanh_outputs (may be NULL): the outputs of the preceding layer when that is a cnn layer with tanh output;
+ * prev_errors then receives that layer's delta tanh'(y) * error right away, which saves the pass over the buffer
+ * that cnt_cnn_backward_errors would make (call it with delta_applied = 1). */
 int cnt_wavnetc_backward_errors(void *stream, int D, int C, int N, const char *patTypes, const float *weights,
                                 const float *core_buf, float *ctx_tanh, const float *output_errors, float *prev_errors,
-                                float *ctx_grad);
+                                float *ctx_grad, const float *prev_tanh_outputs);
 int cnt_wavnetc_backward_weights(void *stream, int D, int C, int N, const float *ctx, const float *ctx_tanh,
                                  float *weight_updates);
 /* SumGradientsForExternalInput (layers/wavNetCore.cu:237-270, driver :895-913): frame_grad (C x

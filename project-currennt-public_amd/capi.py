@@ -110,9 +110,9 @@ _SIGNATURES = {
     "cnt_cnn_weight_count": (C.c_long, [VP]),
     "cnt_cnn_forward": (I, [VP, VP, VP, I, VP, VP, VP]),
     "cnt_cnn_backward": (I, [VP, VP, VP, I, VP, VP, VP, VP, VP, VP]),
-    "cnt_cnn_backward_errors": (I, [VP, VP, VP, I, VP, VP, VP, VP]),
+    "cnt_cnn_backward_errors": (I, [VP, VP, VP, I, VP, VP, VP, VP, I]),
     "cnt_cnn_backward_weights": (I, [VP, VP, VP, I, VP, VP, VP]),
-    "cnt_wavnetc_backward_errors": (I, [VP, I, I, I, VP, VP, VP, VP, VP, VP, VP]),
+    "cnt_wavnetc_backward_errors": (I, [VP, I, I, I, VP, VP, VP, VP, VP, VP, VP, VP]),
     "cnt_wavnetc_backward_weights": (I, [VP, I, I, I, VP, VP, VP]),
     "cnt_wavnetc_load_context": (I, [VP, I, I, I, I, I, VP, VP, VP, VP, VP]),
     "cnt_wavnetc_forward": (I, [VP, I, I, I, VP, VP, VP, VP, VP, VP, VP]),

@@ -208,6 +208,8 @@ struct NetLayer {
     const float *ext_data = nullptr;         // externalloader: [frame][sequence][dimension], set by the caller
     const float *ext_mean_std = nullptr;
     int ext_frames = 0, index_load_method = 0;
+    int cnn_tanh = 0;                        // cnn: "tanhoutput"
+    bool delta_fused = false;                // cnn followed by a wavnetc layer: that layer writes this layer's delta
     const float *total = nullptr;            // skip layers: where the summed error stands after the layer's step
     bool needs_sum = false;                  // skip layers: errors += side buffer is not a no-op
     int live_targets = 0;                    // skip layers: sources that receive the sum through a launch
@@ -610,7 +612,8 @@ int build_layer(cnt_network *net, const json::Value &obj, const char *text, cons
                     "not give one value per filter", L.name.c_str());
         CNT_REQUIRE(parse_runs(get_str(obj, "window_tap_interval"), L.size, dil), "network: cnn layer '%s': "
                     "window_tap_interval does not give one value per filter", L.name.c_str());
-        cnt_cnn_desc d = {P, L.size, net->S, L.maxTr, get_int(obj, "causal", 0), get_int(obj, "tanhoutput", 1), L.bias};
+        L.cnn_tanh = get_int(obj, "tanhoutput", 1);
+        cnt_cnn_desc d = {P, L.size, net->S, L.maxTr, get_int(obj, "causal", 0), L.cnn_tanh, L.bias};
         CNT_TRY(cnt_cnn_create(&d, hw.data(), dil.data(), &L.cnn));
     } else if (t == "wavnetc") {
         L.kind = K_WAVNETC;
@@ -621,6 +624,8 @@ int build_layer(cnt_network *net, const json::Value &obj, const char *text, cons
         CNT_REQUIRE(get_str(obj, "contextMV").empty(), "network: wavnetc layer '%s': contextMV is not built",
                     L.name.c_str());
         if (net->first_wavnetc < 0) net->first_wavnetc = index;
+        NetLayer &before = net->layers[(size_t)index - 1];
+        if (before.kind == K_CNN && before.cnn_tanh) before.delta_fused = true;
         CNT_TRY(device_alloc(net, (void **)&L.core, 2 * (size_t)L.size * slots * sizeof(float), true));
         CNT_TRY(device_alloc(net, (void **)&L.cth, 2 * (size_t)L.size * slots * sizeof(float), true));
     } else if (t == "feedback") {
@@ -1169,10 +1174,12 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 else if (L.kind == K_LSTM)
                     CNT_TRY(cnt_lstm_backward_errors(L.lstm, stream, W, L.err, prev_err));
                 else if (L.kind == K_CNN)
-                    CNT_TRY(cnt_cnn_backward_errors(L.cnn, stream, L.pat, L.T, W, L.out, L.err, prev_err));
+                    CNT_TRY(cnt_cnn_backward_errors(L.cnn, stream, L.pat, L.T, W, L.out, L.err, prev_err,
+                                                    L.delta_fused ? 1 : 0));
                 else {
                     CNT_TRY(cnt_wavnetc_backward_errors(stream, L.size, L.ctx_dim, N, L.pat, W, L.core, L.cth, L.err,
-                                                        prev.err, net->flagged >= 0 ? net->ctx_grad : nullptr));
+                                                        prev.err, net->flagged >= 0 ? net->ctx_grad : nullptr,
+                                                        prev.delta_fused ? prev.out : nullptr));
                     if ((int)i == net->first_wavnetc && net->flagged >= 0) {
                         // every wavnetc layer has added its share; hand the sum per frame to the layer that feeds them
                         // (layers/wavNetCore.cu:895-913)

@@ -83,9 +83,11 @@ __global__ void core_copy_kernel(int D2, size_t count, const char *__restrict__ 
 
 // One thread per (slot, d): both halves of the gate gradient from the same three loads, and -- when the
 // core is conditioned -- the gradient through tanh(X_c) written over ctx_tanh in the same pass.
+// prev_out (optional): outputs of a preceding layer with tanh output; its delta tanh'(y) * error is then written
+// instead of the error.
 __global__ void gated_backward_kernel(int D, size_t count, const char *__restrict__ pat, const float *__restrict__ pre,
                                       const float *__restrict__ err, float *__restrict__ prev_err,
-                                      float *__restrict__ ctx_tanh) {
+                                      float *__restrict__ ctx_tanh, const float *__restrict__ prev_out) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (; i < count; i += stride) {
@@ -99,8 +101,13 @@ __global__ void gated_backward_kernel(int D, size_t count, const char *__restric
             g1 = (1.0f - th * th) * sg * e;
             g2 = th * (sg * (1.0f - sg)) * e;
         }
-        prev_err[i1] = g1;
-        prev_err[i2] = g2;
+        if (prev_out) {
+            prev_err[i1] = tanh_deriv(prev_out[i1]) * g1;
+            prev_err[i2] = tanh_deriv(prev_out[i2]) * g2;
+        } else {
+            prev_err[i1] = g1;
+            prev_err[i2] = g2;
+        }
         if (ctx_tanh) {
             ctx_tanh[i1] = tanh_deriv(ctx_tanh[i1]) * g1;
             ctx_tanh[i2] = tanh_deriv(ctx_tanh[i2]) * g2;
@@ -252,7 +259,7 @@ int cnt_cnn_forward(cnt_cnn *h, void *stream_, const char *patTypes, int curT, c
 }
 
 int cnt_cnn_backward_errors(cnt_cnn *h, void *stream_, const char *patTypes, int curT, const float *weights,
-                            const float *outputs, float *output_errors, float *prev_errors) {
+                            const float *outputs, float *output_errors, float *prev_errors, int delta_applied) {
     using namespace cnt;
     CNT_REQUIRE(h && patTypes && weights && outputs && output_errors, "cnn_backward_errors: null argument");
     CNT_REQUIRE(curT >= 1 && curT <= h->desc.maxT, "cnn_backward_errors: curT %d outside 1..%d", curT, h->desc.maxT);
@@ -261,7 +268,7 @@ int cnt_cnn_backward_errors(cnt_cnn *h, void *stream_, const char *patTypes, int
     const int P = d.P, D = d.D, S = d.S, N = curT * S;
     const size_t count = (size_t)D * N;
 
-    if (d.output_tanh) {
+    if (d.output_tanh && !delta_applied) {
         ProfileScope prof(stream, "cnn_tanh_delta");
         hipLaunchKernelGGL(tanh_delta_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, output_errors, outputs,
                            count);
@@ -338,7 +345,7 @@ int cnt_cnn_backward(cnt_cnn *h, void *stream, const char *patTypes, int curT, c
                      const float *outputs, float *output_errors, float *prev_errors, float *weight_updates) {
     using namespace cnt;
     CNT_REQUIRE(x && weight_updates, "cnn_backward: null argument");
-    CNT_TRY(cnt_cnn_backward_errors(h, stream, patTypes, curT, weights, outputs, output_errors, prev_errors));
+    CNT_TRY(cnt_cnn_backward_errors(h, stream, patTypes, curT, weights, outputs, output_errors, prev_errors, 0));
     return cnt_cnn_backward_weights(h, stream, patTypes, curT, x, output_errors, weight_updates);
 }
 
@@ -379,7 +386,7 @@ int cnt_gatedact_backward(void *stream_, int D, int N, const char *patTypes, con
     ProfileScope prof(static_cast<hipStream_t>(stream_), "gated_backward");
     hipLaunchKernelGGL(gated_backward_kernel, dim3(stream_blocks(count)), dim3(256), 0,
                        static_cast<hipStream_t>(stream_), D, count, patTypes, pre, output_errors, prev_errors,
-                       static_cast<float *>(nullptr));
+                       static_cast<float *>(nullptr), static_cast<const float *>(nullptr));
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
@@ -415,7 +422,7 @@ int cnt_wavnetc_forward(void *stream_, int D, int C, int N, const char *patTypes
 
 int cnt_wavnetc_backward_errors(void *stream_, int D, int C, int N, const char *patTypes, const float *weights,
                                 const float *core_buf, float *ctx_tanh, const float *output_errors, float *prev_errors,
-                                float *ctx_grad) {
+                                float *ctx_grad, const float *prev_tanh_outputs) {
     using namespace cnt;
     CNT_REQUIRE(patTypes && core_buf && output_errors && prev_errors, "wavnetc_backward: null argument");
     CNT_REQUIRE(D > 0 && N > 0 && C >= 0, "wavnetc_backward: bad size");
@@ -426,7 +433,8 @@ int cnt_wavnetc_backward_errors(void *stream_, int D, int C, int N, const char *
     {
         ProfileScope prof(stream, "gated_backward");
         hipLaunchKernelGGL(gated_backward_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, D, count, patTypes,
-                           core_buf, output_errors, prev_errors, C > 0 ? ctx_tanh : static_cast<float *>(nullptr));
+                           core_buf, output_errors, prev_errors, C > 0 ? ctx_tanh : static_cast<float *>(nullptr),
+                           prev_tanh_outputs);
         CNT_HIP(hipGetLastError());
     }
     if (C > 0 && ctx_grad) {
@@ -470,7 +478,7 @@ int cnt_wavnetc_backward(void *stream, int D, int C, int N, const char *patTypes
     CNT_REQUIRE(C == 0 || (weights && ctx && ctx_tanh && weight_updates),
                 "wavnetc_backward: conditioning needs weights, context, tanh buffer and weight updates");
     CNT_TRY(cnt_wavnetc_backward_errors(stream, D, C, N, patTypes, weights, core_buf, ctx_tanh, output_errors, prev_errors,
-                                        ctx_grad));
+                                        ctx_grad, nullptr));
     return cnt_wavnetc_backward_weights(stream, D, C, N, ctx, ctx_tanh, weight_updates);
 }
 
