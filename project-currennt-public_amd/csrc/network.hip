@@ -472,9 +472,26 @@ void weight_sections(NetLayer &L, int P) {
     }
 }
 
+int build_layer_into(cnt_network *net, NetLayer &L, const json::Value &obj, const char *text,
+                     const cnt_network_options *opt);
+
+// a layer that fails half way must not leave its handles behind
 int build_layer(cnt_network *net, const json::Value &obj, const char *text, const cnt_network_options *opt) {
-    const int index = (int)net->layers.size();
     NetLayer L;
+    const int status = build_layer_into(net, L, obj, text, opt);
+    if (status != CNT_OK) {
+        if (L.lstm) cnt_lstm_destroy(L.lstm);
+        if (L.cnn) cnt_cnn_destroy(L.cnn);
+        if (L.mdn) cnt_mdn_destroy(L.mdn);
+        return status;
+    }
+    net->layers.push_back(std::move(L));
+    return CNT_OK;
+}
+
+int build_layer_into(cnt_network *net, NetLayer &L, const json::Value &obj, const char *text,
+                     const cnt_network_options *opt) {
+    const int index = (int)net->layers.size();
     L.text.assign(text + obj.begin, obj.end - obj.begin);
     L.name = get_str(obj, "name");
     L.type = get_str(obj, "type");
@@ -671,7 +688,6 @@ int build_layer(cnt_network *net, const json::Value &obj, const char *text, cons
     else CNT_TRY(device_alloc(net, (void **)&L.out, count * sizeof(float), true));
     if (L.kind != K_INPUT && L.kind != K_EXTERNAL && L.kind != K_SSE && L.kind != K_MDN && !is_skip_kind(L.kind))
         CNT_TRY(device_alloc(net, (void **)&L.err, count * sizeof(float), true));
-    net->layers.push_back(std::move(L));
     return CNT_OK;
 }
 

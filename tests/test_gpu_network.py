@@ -317,3 +317,95 @@ def test_wavenet_with_frame_rate_conditioning_network():
                     print("   ", L["name"], e, flush=True)
         assert worst < TOL
     net.close()
+
+
+def test_full_size_acoustic_backward_is_affine_in_the_targets():
+    """BASELINE configs[1] at its real size (T = 600, S = 10, 382-512-512-blstm512-blstm512-187), where the oracle
+    would take minutes: with the forward state fixed, the SSE error is y - target and every later step of the
+    backward pass is linear in it as long as no LSTM delta reaches the clipping bound, so
+    dW(t1) + dW(t2) = dW(t1 + t2) + dW(0) for every weight tensor.  A wrong accumulation, a stale buffer (the stored
+    output-gate deltas are read-modify-write) or a race between the streams breaks it."""
+    import torch
+
+    print("full-size acoustic linearity", flush=True)
+    pkg = PC.pkg()
+    capi, networks = pkg.capi, pkg.networks
+    S, Tmax = 10, 600
+    input_size, specs = networks.acoustic_model_spec()
+    rng = np.random.default_rng(77)
+    lengths = [int(v) for v in rng.integers(300, Tmax + 1, size=S)]
+    T = max(lengths)
+    pat = make_pat_types(lengths, T)
+    valid = (pat != 0).reshape(T, S)
+    x = rng.standard_normal((T, S, input_size)).astype(np.float32)
+    x[~valid] = 0
+    layers = [{"size": input_size, "name": "input", "type": "input"}]
+    layers += [dict(sp, name="l%d" % i) for i, sp in enumerate(specs)]
+    net = capi.Network(json.dumps({"layers": layers}), S, Tmax)
+    net.randomize(5, 0.08)
+    pat_d, x_d = PC.dev(pat), PC.dev(x.reshape(-1))
+
+    def grads(target):
+        tgt = target.copy()
+        tgt[~valid] = 0
+        net.load_sequences(pat_d, T, min(lengths), x_d, PC.dev(tgt.reshape(-1)))
+        net.forward()
+        net.backward()
+        net.check()
+        torch.cuda.synchronize()
+        return net.updates.clone()
+
+    t1 = (0.05 * rng.standard_normal((T, S, 187))).astype(np.float32)
+    t2 = (0.05 * rng.standard_normal((T, S, 187))).astype(np.float32)
+    g1, g2, g12, g0 = grads(t1), grads(t2), grads(t1 + t2), grads(np.zeros_like(t1))
+    assert float(g1.abs().max()) > 0
+    for L in net.layers:
+        if not L["weight_count"]:
+            continue
+        a, b = L["weight_offset"], L["weight_offset"] + L["weight_count"]
+        lhs = (g1[a:b] + g2[a:b]).cpu().numpy()
+        rhs = (g12[a:b] + g0[a:b]).cpu().numpy()
+        assert PC.relerr(lhs, rhs) < TOL, L["name"]
+    net.close()
+
+
+def test_full_size_wavenet_sequencer_matches_layer_by_layer_walk():
+    """BASELINE configs[3] at its real size (30 blocks, 2 x 16000 samples, 1024 classes): the sequencer (shared sums,
+    aliased buffers, fan-in / fan-out tables, side streams, fused delta) against the plain layer-by-layer walk over
+    the same kernels, which the shortened-stack tests tie to the oracle.  Loss equal to 1e-6, every weight gradient
+    to the tolerance of the split-K atomics' summation order."""
+    import torch
+
+    print("full-size wavenet sequencer vs walk", flush=True)
+    pkg = PC.pkg()
+    capi, networks = pkg.capi, pkg.networks
+    nb, Q, R, K, C = 30, 1024, 64, 128, 80
+    lengths = [16000, 15000]
+    S, T = 2, 16000
+    pat, onehot, ctx, target, N = WD.make(lengths, Q, C, upsample=80, seed=4)
+    walk = networks.WaveNet(networks.HipBackend(), nb, S, T, Q=Q, R=R, K=K, C=C, cnn_tanh=1)
+    W = WD.init_weights({k: len(walk.buf[k]["W"]) for k in walk.weight_names()}, seed=5)
+    for k, w in W.items():
+        walk.buf[k]["W"].copy_(torch.from_numpy(w))
+    pat_d, ctx_d, tgt_d = PC.dev(pat), PC.dev(ctx), PC.dev(target)
+    walk.set_inputs(pat_d, PC.dev(onehot), ctx_d, tgt_d)
+    walk.forward()
+    walk.calculate_error()
+    walk.backward()
+    net = capi.Network(json.dumps(WD.network_json(nb, Q, R, K, C, 1, 10)), S, T, mdn_config=[1, 0, Q, 0, 1, -1])
+    for L in net.layers:
+        if L["weight_count"]:
+            L["weights"].copy_(torch.from_numpy(W[L["name"]]))
+    net.set_context(ctx_d)
+    net.load_sequences(pat_d, T, min(lengths), torch.zeros(N, dtype=torch.float32, device="cuda"), tgt_d)
+    net.forward()
+    loss = float(net.calculate_error().item())
+    net.backward()
+    torch.cuda.synchronize()
+    ref_loss = float(walk.loss.item())
+    assert abs(loss - ref_loss) <= 1e-6 * abs(ref_loss)
+    for L in net.layers:
+        if L["weight_count"]:
+            assert PC.relerr(L["updates"].cpu().numpy(), walk.buf[L["name"]]["dW"].cpu().numpy()) < TOL, L["name"]
+    walk.close()
+    net.close()
