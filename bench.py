@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the backward hot path on one MI355X.
 
-Workload: BASELINE config 2, the acoustic model 382 -> 2 x feedforward_tanh 512 -> 2 x blstm 512
+Workload: benchmark config 2, the acoustic model 382 -> 2 x feedforward_tanh 512 -> 2 x blstm 512
 (256 cells per direction) -> feedforward_identity 187 -> sse, T = 600 frames, 10 parallel sequences
 with lengths U{300..600}, fp32, synthetic seeded data, weights U(-0.08, 0.08).
 
@@ -100,7 +100,7 @@ def main():
     ap.add_argument("--cpu-sample-T", type=int, default=160)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--workload", default="acoustic", choices=["acoustic", "lstm_c1", "mdn_c3", "dft_c5", "wavenet_c4", "opt_step", "nc_fraction"],
-                    help="acoustic = BASELINE configs[1] (the headline metric); the others are the remaining configs")
+                    help="acoustic = benchmark configs[1] (the headline metric); the others are the remaining configs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters)")

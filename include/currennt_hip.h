@@ -386,7 +386,7 @@ int cnt_network_update(cnt_network *net, void *stream, int option, float learnin
  * written if cap is smaller (call once with buf = NULL to learn the size). */
 int cnt_network_export_json(cnt_network *net, char *buf, size_t cap, size_t *needed);
 
-/* ---- weight update of the training loop (SURVEY "next": optimizer step on device) -----------------
+/* ---- weight update of the training loop (optimizer step on device) ------------------------------------
  * optimizer option numbers are the reference's (MacroDefine.hpp:33-37): 0 plain SGD, 1 AdaGrad,
  * 2 gradient averaged over the fraction, 3 stochastic AdaGrad (statistics only), 4 SGD with decaying
  * learning rate (the decay is host logic; treated as 0 here), 5 Adam.  `stats` holds one float per weight
@@ -415,7 +415,7 @@ int cnt_opt_step(void *stream, int option, long n, float *weights, const float *
                  float beta2_accum, float learning_rate, float momentum);
 float cnt_opt_next_beta_accum(float accum, int which);
 
-/* ---- the .nc data path (SURVEY "next": NetCDF reader and fraction builder; host memory only) --------
+/* ---- the .nc data path (NetCDF reader and fraction builder; host memory only) ------------------------
  * data_sets::DataSet's constructor for ONE .nc file (data_sets/DataSet.cpp:1376-1907): reads the
  * dimensions and seqLengths / seqTags, keeps the first max(1, int(numSeqs * fraction)) sequences, cuts a
  * sequence longer than 1.5 * truncate_seq into segments of truncate_seq (0 = off), and in training mode

@@ -270,7 +270,7 @@ class Trainer:
 
 
 def acoustic_model_spec():
-    """BASELINE config 2: 382 -> 2 x feedforward_tanh 512 -> 2 x blstm 512 -> feedforward_identity 187 -> sse."""
+    """benchmark config 2: 382 -> 2 x feedforward_tanh 512 -> 2 x blstm 512 -> feedforward_identity 187 -> sse."""
     return 382, [
         {"type": "feedforward_tanh", "size": 512, "bias": 1.0},
         {"type": "feedforward_tanh", "size": 512, "bias": 1.0},
@@ -282,7 +282,7 @@ def acoustic_model_spec():
 
 
 # ---------------------------------------------------------------------------------------------------------
-# WaveNet-style stack (BASELINE config 4), topology of the reference's example network
+# WaveNet-style stack (benchmark config 4), topology of the reference's example network
 # obsolete/scripts/EXAMPLE/MODEL_WAVENET/network.jsn: embedding of the fed-back one-hot sample, then per block
 #   cnn (causal, dilated, 2R filters) -> wavnetc (gate, conditioned) -> out (R->R) -> skipadd(residual, out)
 #   -> temp (skipini) -> skipouttrans (R->K) -> skip (skipini) ; temp2 = skipadd(temp) feeds the next block,

@@ -1,4 +1,4 @@
-"""BASELINE config 4 as a benchmark workload: backward pass of the 30-block WaveNet-style stack,
+"""benchmark config 4 as a benchmark workload: backward pass of the 30-block WaveNet-style stack,
 2 waveforms x 16000 samples, driven through the library's network sequencer from a network file.  A backward pass
 consumes state that only the forward pass rebuilds (the skip layers' cleared error buffers, the tanh(context)
 buffer that the gated layer overwrites with its gradient), so every timed backward is preceded by an untimed

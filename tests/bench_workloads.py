@@ -1,4 +1,4 @@
-"""Secondary benchmark workloads (BASELINE configs 1, 3, 4, 5), reached through `bench.py --workload ...`.
+"""Secondary benchmark workloads (benchmark configs 1, 3, 4, 5), reached through `bench.py --workload ...`.
 Each returns the same JSON fields as the headline workload: value in the config's unit, a roofline entry for
 the dominant kernel (duration from the library's HIP-event hooks) and a cpu_baseline (the oracle, one core)."""
 import os

@@ -72,7 +72,7 @@ def test_lstm_clip_and_repeat_backward():
 
 
 def test_lstm_config1_unidirectional():
-    """BASELINE config 1: P=382, H=256, T=200, S=4 with one sequence of 150 frames."""
+    """benchmark config 1: P=382, H=256, T=200, S=4 with one sequence of 150 frames."""
     print("lstm config 1", flush=True)
     assert PC.run_lstm_case(382, 256, False, [200, 200, 200, 150], seed=1) < TOL
 

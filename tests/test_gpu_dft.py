@@ -12,7 +12,7 @@ TOL = 1e-4
 @pytest.mark.parametrize("res,max_len,lengths", [
     ([(32, 32, 8)], 200, [200]),
     ([(64, 40, 10)], 333, [333, 120]),                       # zero padding inside the frames, ragged lengths
-    ([(512, 512, 80), (128, 128, 40), (2048, 2048, 640)], 16000, [16000, 9000]),  # BASELINE config 5 resolutions
+    ([(512, 512, 80), (128, 128, 40), (2048, 2048, 640)], 16000, [16000, 9000]),  # benchmark config 5 resolutions
     ([(1024, 800, 200), (4096, 4096, 1024)], 6000, [6000, 5000, 4097]),
     ([(128, 128, 40)], 300, [60]),                           # waveform shorter than one frame
 ])

@@ -1,4 +1,4 @@
-"""GPU parity of the whole acoustic model of BASELINE config 2 (382 -> 512t -> 512t -> blstm512 -> blstm512
+"""GPU parity of the whole acoustic model of benchmark config 2 (382 -> 512t -> 512t -> blstm512 -> blstm512
 -> 187 -> sse) against the CPU oracle on a shortened fraction, every gradient tensor at 1e-4 (L2-normalised)."""
 import numpy as np
 import pytest

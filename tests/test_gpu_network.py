@@ -320,7 +320,7 @@ def test_wavenet_with_frame_rate_conditioning_network():
 
 
 def test_full_size_acoustic_backward_is_affine_in_the_targets():
-    """BASELINE configs[1] at its real size (T = 600, S = 10, 382-512-512-blstm512-blstm512-187), where the oracle
+    """benchmark configs[1] at its real size (T = 600, S = 10, 382-512-512-blstm512-blstm512-187), where the oracle
     would take minutes: with the forward state fixed, the SSE error is y - target and every later step of the
     backward pass is linear in it as long as no LSTM delta reaches the clipping bound, so
     dW(t1) + dW(t2) = dW(t1 + t2) + dW(0) for every weight tensor.  A wrong accumulation, a stale buffer (the stored
@@ -370,7 +370,7 @@ def test_full_size_acoustic_backward_is_affine_in_the_targets():
 
 
 def test_full_size_wavenet_sequencer_matches_layer_by_layer_walk():
-    """BASELINE configs[3] at its real size (30 blocks, 2 x 16000 samples, 1024 classes): the sequencer (shared sums,
+    """benchmark configs[3] at its real size (30 blocks, 2 x 16000 samples, 1024 classes): the sequencer (shared sums,
     aliased buffers, fan-in / fan-out tables, side streams, fused delta) against the plain layer-by-layer walk over
     the same kernels, which the shortened-stack tests tie to the oracle.  Loss equal to 1e-6, every weight gradient
     to the tolerance of the split-K atomics' summation order."""

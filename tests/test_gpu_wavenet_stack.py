@@ -1,4 +1,4 @@
-"""GPU parity of a whole WaveNet-style stack (reference example topology, BASELINE config 4 layer sizes, few
+"""GPU parity of a whole WaveNet-style stack (reference example topology, benchmark config 4 layer sizes, few
 blocks, short waveforms) against the same graph on the CPU oracle: loss and every weight-update vector."""
 import numpy as np
 import pytest

@@ -1,4 +1,4 @@
-"""Seeded synthetic inputs of the WaveNet workload (BASELINE config 4): mu-law quantised U(-1,1) waveforms, the
+"""Seeded synthetic inputs of the WaveNet workload (benchmark config 4): mu-law quantised U(-1,1) waveforms, the
 teacher-forced one-hot of the previous sample, frame-rate conditioning up-sampled by a frame index."""
 import numpy as np
 
