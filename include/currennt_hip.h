@@ -92,7 +92,10 @@ typedef struct {
     float bias;  /* the layer's constant bias input ("bias" in the JSON)    */
 } cnt_lstm_desc;
 
-/* LstmLayer::LstmLayer (layers/LstmLayer.cu:1078-1268): allocates the per-direction state. */
+/* LstmLayer::LstmLayer (layers/LstmLayer.cu:1078-1268): allocates the per-direction state.  Layers with 64, 128,
+ * 256 or 512 cells per direction and at most 32 parallel sequences run their recursions as persistent kernels;
+ * any other geometry runs them step by step (one batched recurrent product and one cell kernel per time step, the
+ * reference's own schedule), with the same results. */
 int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out);
 int cnt_lstm_destroy(cnt_lstm *h);
 /* LstmLayer::loadSequences (layers/LstmLayer.cu:1488-1533): records the fraction's geometry and

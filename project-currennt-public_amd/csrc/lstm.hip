@@ -819,6 +819,104 @@ __global__ void lstm_small_grads(const SmallGradParams p) {
     atomicAdd(p.g_peep + 2 * L + u, q_og);
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Step-by-step recursion for geometries the persistent kernels do not cover (cells per direction other than 64,
+// 128, 256, 512, or more than 32 parallel sequences): per time step one batched recurrent product through the
+// matrix-product kernel and one cell kernel, i.e. the reference's own schedule (LstmLayer.cu:1743-1949,
+// :2066-2255).  One thread per (direction, sequence, cell).
+// ---------------------------------------------------------------------------------------------------
+__global__ void lstm_forward_step(const ChainParams p, int step) {
+    const int H = p.H, S = p.S, n = S * H;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= p.ndir * n) return;
+    const int dir = idx / n, r = idx % n, s = r / H, j = r % H;
+    const DirPtrs &D = p.d[dir];
+    const int t = dir ? (p.T - 1 - step) : step;
+    const int prev = dir ? t + 1 : t - 1;
+    const bool first = step == 0;
+    const size_t i = (size_t)t * n + (size_t)s * H + j;
+    float *out = p.out ? p.out + ((size_t)t * S + s) * p.L + dir * H + j : nullptr;
+    // padding is only looked for at or after the shortest sequence's end (LstmLayer.cu:1800-1803)
+    if (t >= p.Tmin && p.pat[t * S + s] == 0) {
+        if (dir) D.c[i] = 0.0f;  // only the time-reversed direction clears the cell state
+        D.h[i] = 0.0f;
+        if (out) *out = 0.0f;
+        return;
+    }
+    const size_t ip = (size_t)prev * n + (size_t)s * H + j;
+    float a_ni = D.ni[i] + p.bias * D.b[0][j];
+    float a_ig = D.ig[i] + p.bias * D.b[1][j];
+    float a_fg = D.fg[i] + p.bias * D.b[2][j];
+    float a_og = D.og[i] + p.bias * D.b[3][j];
+    float cp = 0.0f;
+    if (!first) {
+        cp = D.c[ip];
+        a_ig += cp * D.peep[0][j];
+        a_fg += cp * D.peep[1][j];
+    }
+    const float ni = tanh_act(a_ni), ig = logistic(a_ig), fg = logistic(a_fg);
+    D.ni[i] = ni; D.ig[i] = ig; D.fg[i] = fg;
+    float c = ni * ig;
+    if (!first) c += cp * fg;
+    D.c[i] = c;
+    a_og += c * D.peep[2][j];
+    const float og = logistic(a_og);
+    D.og[i] = og;
+    const float hv = tanh_act(c) * og;
+    D.h[i] = hv;
+    if (out) *out = hv;
+}
+
+// herr of both directions from the interleaved output errors (LstmLayer.cu:210-235)
+__global__ void lstm_split_errors(const ChainParams p, size_t count) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride) {
+        const size_t slot = i / p.L;
+        const int v = (int)(i % p.L);
+        const float e = p.outerr[i];
+        if (v < p.H) p.d[0].herr[slot * p.H + v] = e;
+        else p.d[1].herr[slot * p.H + v - p.H] = e;
+    }
+}
+
+__global__ void lstm_backward_step(const ChainParams p, int step) {
+    const int H = p.H, S = p.S, n = S * H;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= p.ndir * n) return;
+    const int dir = idx / n, r = idx % n, s = r / H, j = r % H;
+    const DirPtrs &D = p.d[dir];
+    const int t = dir ? step : (p.T - 1 - step);
+    const int later = dir ? t - 1 : t + 1;    // the slot handled one step before this one
+    const int earlier = dir ? t + 1 : t - 1;  // the slot the forward pass came from
+    const bool first = step == 0, last = step == p.T - 1;
+    const size_t i = (size_t)t * n + (size_t)s * H + j;
+    if (t >= p.Tmin && p.pat[t * S + s] == 0) {
+        D.dni[i] = 0.0f; D.dig[i] = 0.0f; D.dfg[i] = 0.0f; D.dog[i] = 0.0f;
+        D.cerr[i] = 0.0f;
+        return;
+    }
+    const float e = D.herr[i];
+    const float ni = D.ni[i], ig = D.ig[i], og = D.og[i], c = D.c[i];
+    const float tc = tanh_act(c);
+    // the stored output-gate delta is read back before it is overwritten (LstmLayer.cu:300-310)
+    const float d_og = (logistic_deriv(og) * tc * e) + D.dog[i];
+    float ce = og * tanh_deriv(tc) * e + D.peep[2][j] * d_og;
+    if (!first) {
+        const size_t il = (size_t)later * n + (size_t)s * H + j;
+        ce += (D.fg[il] * D.cerr[il] + D.peep[0][j] * D.dig[il] + D.peep[1][j] * D.dfg[il]);
+    }
+    const float d_ni = ig * tanh_deriv(ni) * ce;
+    float d_fg = 0.0f;
+    if (!last) d_fg = logistic_deriv(D.fg[i]) * D.c[(size_t)earlier * n + (size_t)s * H + j] * ce;
+    const float d_ig = logistic_deriv(ig) * ni * ce;
+    D.dni[i] = clip1(d_ni);
+    D.dig[i] = clip1(d_ig);
+    D.dfg[i] = clip1(d_fg);
+    D.dog[i] = clip1(d_og);
+    D.cerr[i] = ce;
+}
+
 }  // namespace
 }  // namespace cnt
 
@@ -844,6 +942,7 @@ struct cnt_lstm {
     int poll_delay, poll_gap, poll_delay_fwd;
     int last_was_forward;  // which recursion the diagnostic buffer describes
     int bmail_dirty;       // the backward mailbox may hold words that are not empty
+    int stepwise;          // no persistent recursion kernel for this geometry: one product + one cell kernel per step
 };
 
 namespace cnt {
@@ -922,6 +1021,81 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     return CNT_OK;
 }
 
+// The recursions of both directions step by step (see lstm_forward_step): per step the recurrent products of all
+// gates and directions are one launch of the matrix-product kernel, accumulating into the slices of that step.
+int stepwise_forward(cnt_lstm *h, hipStream_t stream, ChainParams &p) {
+    const int H = h->H, S = h->desc.S, L = h->desc.L, n = S * H;
+    const int threads = h->ndir * n;
+    ProfileScope prof(stream, "lstm_forward_steps");
+    for (int step = 0; step < h->T; ++step) {
+        if (step > 0) {
+            GemmArgs ga = {};
+            ga.m = H; ga.n = S; ga.k = H;
+            ga.a_kcontig = 1; ga.lda = H;  // W_int block [from + to*H]: element (to, from) at [to*H + from]
+            ga.b_kcontig = 1; ga.ldb = H;
+            ga.ldc = H;
+            ga.nseg = 1; ga.splitk = 1; ga.epilogue = EPI_ADD;
+            ga.nprob = 4 * h->ndir;
+            for (int dir = 0; dir < h->ndir; ++dir) {
+                const int t = dir ? (h->T - 1 - step) : step, prev = dir ? t + 1 : t - 1;
+                for (int g = 0; g < 4; ++g) {
+                    GemmProblem &pb = ga.prob[dir * 4 + g];
+                    pb.A[0] = p.d[dir].w_int + (size_t)g * L * H;
+                    pb.B[0] = p.d[dir].h + (size_t)prev * n;
+                    pb.C = h->state[dir][g] + (size_t)t * n;
+                }
+            }
+            CNT_TRY(gemm_launch(stream, ga));
+        }
+        hipLaunchKernelGGL(lstm_forward_step, dim3((threads + 255) / 256), dim3(256), 0, stream, p, step);
+        CNT_HIP(hipGetLastError());
+    }
+    return CNT_OK;
+}
+
+int stepwise_backward(cnt_lstm *h, hipStream_t stream, ChainParams &p) {
+    const int H = h->H, S = h->desc.S, L = h->desc.L, n = S * H;
+    const int threads = h->ndir * n;
+    const size_t count = (size_t)L * h->T * S;
+    ProfileScope prof(stream, "lstm_backward_steps");
+    if (h->ndir == 2) {
+        size_t blocks = (count + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(lstm_split_errors, dim3((unsigned)blocks), dim3(256), 0, stream, p, count);
+        CNT_HIP(hipGetLastError());
+    } else {
+        CNT_HIP(hipMemcpyAsync(p.d[0].herr, p.outerr, count * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    }
+    for (int step = 0; step < h->T; ++step) {
+        if (step > 0) {
+            // herr[t] += sum over gates of W_int[g] * delta_g[later]
+            GemmArgs ga = {};
+            ga.m = H; ga.n = S; ga.k = H;
+            ga.a_kcontig = 0; ga.lda = H;
+            ga.b_kcontig = 1; ga.ldb = H;
+            ga.ldc = H;
+            ga.nseg = 4; ga.splitk = 1; ga.epilogue = EPI_ADD;
+            ga.nprob = h->ndir;
+            for (int dir = 0; dir < h->ndir; ++dir) {
+                const int t = dir ? step : (h->T - 1 - step), later = dir ? t - 1 : t + 1;
+                GemmProblem &pb = ga.prob[dir];
+                for (int g = 0; g < 4; ++g) {
+                    pb.A[g] = p.d[dir].w_int + (size_t)g * L * H;
+                    pb.B[g] = h->state[dir][7 + g] + (size_t)later * n;
+                }
+                pb.C = p.d[dir].herr + (size_t)t * n;
+            }
+            CNT_TRY(gemm_launch(stream, ga));
+        }
+        hipLaunchKernelGGL(lstm_backward_step, dim3((threads + 255) / 256), dim3(256), 0, stream, p, step);
+        CNT_HIP(hipGetLastError());
+    }
+    // a unidirectional layer leaves the summed errors in the caller's buffer (LstmLayer.cu:2086-2087, :2378-2381)
+    if (p.herr_out)
+        CNT_HIP(hipMemcpyAsync(p.herr_out, p.d[0].herr, count * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    return CNT_OK;
+}
+
 }  // namespace
 }  // namespace cnt
 
@@ -940,14 +1114,15 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     const int NT = (desc->S + 15) / 16;
     int JB = default_jb(H);
     if (const char *e = std::getenv("CNT_LSTM_JB")) JB = std::atoi(e);
-    CNT_REQUIRE(pick_kernel(true, H, JB, NT) != nullptr,
-                "lstm_create: cells per direction H=%d with S=%d parallel sequences has no recursion kernel "
-                "(H in {64,128,256,512}, S <= 32)", H, desc->S);
+    // H in {64, 128, 256, 512} with S <= 32 run as persistent recursion kernels; everything else step by step
+    const bool stepwise = pick_kernel(true, H, JB, NT) == nullptr || std::getenv("CNT_LSTM_STEPWISE") != nullptr;
+    if (stepwise) JB = 1;
 
     cnt_lstm *h = new (std::nothrow) cnt_lstm();
     CNT_REQUIRE(h != nullptr, "lstm_create: out of host memory");
     std::memset(h, 0, sizeof(*h));
     h->desc = *desc; h->ndir = ndir; h->H = H; h->JB = JB; h->NT = NT;
+    h->stepwise = stepwise ? 1 : 0;
     h->bmail_dirty = 1;
     h->spin_limit = 1u << 22;
     if (const char *e = std::getenv("CNT_LSTM_SPIN_LIMIT")) h->spin_limit = (unsigned)std::strtoul(e, nullptr, 10);
@@ -966,8 +1141,8 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     const size_t nstate = (size_t)H * desc->maxT * desc->S;
     const int G = H / JB;
     // mailboxes, kMailSlots slots each: forward H*S words, backward G*G*JB*S words
-    h->fmail_words = (size_t)kMailSlots * H * desc->S;
-    h->bmail_words = (size_t)kMailSlots * G * H * desc->S;
+    h->fmail_words = stepwise ? 1 : (size_t)kMailSlots * H * desc->S;
+    h->bmail_words = stepwise ? 1 : (size_t)kMailSlots * G * H * desc->S;
     for (int dir = 0; dir < ndir && err == hipSuccess; ++dir) {
         for (int w = 0; w < 12 && err == hipSuccess; ++w) {
             err = hipMalloc(reinterpret_cast<void **>(&h->state[dir][w]), nstate * sizeof(float));
@@ -1099,6 +1274,7 @@ int cnt_lstm_forward(cnt_lstm *h, void *stream_, const float *weights, const flo
     fill_chain_params(h, weights, p);
     // the reference lets a unidirectional layer write its outputs directly (buffer swap, :1747-1749)
     p.out = outputs;
+    if (h->stepwise) return stepwise_forward(h, stream, p);
     return launch_chain(h, stream, true, p);
 }
 
@@ -1114,7 +1290,8 @@ int cnt_lstm_backward_errors(cnt_lstm *h, void *stream_, const float *weights, f
     fill_chain_params(h, weights, p);
     p.outerr = output_errors;
     p.herr_out = (h->ndir == 1) ? output_errors : nullptr;
-    CNT_TRY(launch_chain(h, stream, false, p));
+    if (h->stepwise) CNT_TRY(stepwise_backward(h, stream, p));
+    else CNT_TRY(launch_chain(h, stream, false, p));
 
     // 2. error to the preceding layer
     if (prev_errors) return cnt_lstm_backward_prev_errors(h, stream_, weights, prev_errors);

@@ -57,6 +57,12 @@ def test_sse():
     (32, 1024, True, [7, 5, 7]),
     (20, 256, False, [5] * 24),            # more than 16 parallel sequences with 256 cells
     (16, 128, True, [1, 1]),               # a single time step, two sequences
+    # geometries without a persistent recursion kernel: step-by-step recursion
+    (12, 64, True, [30, 23]),              # 32 cells per direction (the reference example's conditioning BLSTM)
+    (7, 20, False, [9, 4, 9]),             # 20 cells, sizes that are no multiple of anything
+    (25, 200, True, [11, 11, 6, 2]),       # 100 cells per direction
+    (10, 64, False, [6] * 40),             # more than 32 parallel sequences
+    (9, 6, True, [1, 1, 1]),               # a single time step
 ])
 def test_lstm(P, L, bidir, lengths):
     print("lstm case", P, L, bidir, lengths, flush=True)
@@ -123,9 +129,18 @@ def test_lstm_gives_up_cleanly_and_recovers():
     layer.close()
 
 
-def test_lstm_unsupported_geometry_is_an_error():
+def test_lstm_step_by_step_recursion_equals_the_persistent_kernels(monkeypatch):
+    """The two implementations of the recursion on a geometry both cover (clip active, ragged lengths): the handle
+    created with CNT_LSTM_STEPWISE set runs step by step."""
+    print("lstm stepwise vs persistent", flush=True)
+    monkeypatch.setenv("CNT_LSTM_STEPWISE", "1")
+    assert PC.run_lstm_case(24, 128, True, [10, 6, 10], seed=5, wscale=0.5, escale=20.0, repeat_backward=True) < TOL
+    assert PC.run_lstm_case(30, 256, False, [12, 12, 7], seed=6) < TOL
+
+
+def test_lstm_invalid_geometry_is_an_error():
     capi = PC.pkg().capi
     with pytest.raises(RuntimeError):
-        capi.Lstm(10, 100, False, 4, 10)
+        capi.Lstm(10, 129, True, 4, 10)      # odd size of a bidirectional layer
     with pytest.raises(RuntimeError):
-        capi.Lstm(10, 129, True, 4, 10)
+        capi.Lstm(10, 0, False, 4, 10)
