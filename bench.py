@@ -29,9 +29,9 @@ sys.path.insert(0, ROOT)
 import numpy as np  # noqa: E402
 
 # HBM bytes one launch of lstm_backward_chain moves on this workload (T=588, S=10, H=256, two directions), from
-# two rocprofv3 --pmc runs scaled by a copy of known size: 1071 MiB read + 1605 MiB written
+# two rocprofv3 --pmc runs scaled by a copy of known size: 1070 MiB read + 1605 MiB written
 # (profiles/acoustic_backward_hbm_traffic.md).  Algorithmic bytes of the same launch: 120 MB.
-CHAIN_TRAFFIC_BYTES = int((1070.8 + 1605.3) * 2 ** 20)
+CHAIN_TRAFFIC_BYTES = int((1070.0 + 1605.3) * 2 ** 20)
 
 METRIC = "BLSTM backward frames/sec at 1 MI355X; % HBM/MFMA roofline vs host CPU"
 PEAK_FP32_MFMA_TFLOPS = 157.3
