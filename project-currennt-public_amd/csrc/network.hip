@@ -178,8 +178,10 @@ struct Parser {
 
 namespace {
 
-enum Kind { K_INPUT, K_DENSE, K_LSTM, K_SKIPINI, K_SKIPADD, K_SKIPCAT, K_CNN, K_WAVNETC, K_FEEDBACK, K_EXTERNAL, K_SSE,
-            K_MDN };
+enum Kind { K_INPUT, K_DENSE, K_LSTM, K_SKIPINI, K_SKIPADD, K_SKIPCAT, K_CNN, K_WAVNETC, K_GATED, K_FEEDBACK, K_EXTERNAL,
+            K_SSE, K_MDN, K_DFT };
+
+inline bool is_post_kind(int k) { return k == K_SSE || k == K_MDN || k == K_DFT; }
 
 inline bool is_sum_skip(int k) { return k == K_SKIPINI || k == K_SKIPADD; }
 inline bool is_skip_kind(int k) { return is_sum_skip(k) || k == K_SKIPCAT; }
@@ -196,6 +198,9 @@ struct NetLayer {
     cnt_lstm *lstm = nullptr;
     cnt_cnn *cnn = nullptr;
     cnt_mdn *mdn = nullptr;
+    cnt_dft *dft = nullptr;
+    float *dft_errors = nullptr;             // dft: per-resolution distances written by the forward pass
+    int dft_error_count = 0;
     float *core = nullptr, *cth = nullptr;  // wavnetc
     int ctx_dim = 0;
     int fb_start = 0, fb_end = 0;            // feedback: dimensions taken from the preceding layer
@@ -371,6 +376,13 @@ __global__ void skipcat_backward_kernel(size_t count, int n, int src_dim, int lo
         *t = accumulate ? *t + e : e;
     }
 }
+__global__ void sum_few_kernel(int n, const float *__restrict__ v, float *__restrict__ out) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        float acc = 0.0f;
+        for (int i = 0; i < n; ++i) acc += v[i];
+        *out = acc;
+    }
+}
 __global__ void add_inplace_kernel(size_t count, float *__restrict__ a, const float *__restrict__ b) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -483,6 +495,7 @@ int build_layer(cnt_network *net, const json::Value &obj, const char *text, cons
         if (L.lstm) cnt_lstm_destroy(L.lstm);
         if (L.cnn) cnt_cnn_destroy(L.cnn);
         if (L.mdn) cnt_mdn_destroy(L.mdn);
+        if (L.dft) cnt_dft_destroy(L.dft);
         return status;
     }
     net->layers.push_back(std::move(L));
@@ -645,6 +658,57 @@ int build_layer_into(cnt_network *net, NetLayer &L, const json::Value &obj, cons
         if (before.kind == K_CNN && before.cnn_tanh) before.delta_fused = true;
         CNT_TRY(device_alloc(net, (void **)&L.core, 2 * (size_t)L.size * slots * sizeof(float), true));
         CNT_TRY(device_alloc(net, (void **)&L.cth, 2 * (size_t)L.size * slots * sizeof(float), true));
+    } else if (t == "gatedact") {
+        // GatedActLayer::GatedActLayer (layers/GatedActLayer.cu:131-143)
+        L.kind = K_GATED;
+        CNT_REQUIRE(P == 2 * L.size, "network: gatedact layer '%s' of size %d needs a preceding layer of size %d",
+                    L.name.c_str(), L.size, 2 * L.size);
+    } else if (t == "dft") {
+        // DFTPostoutputLayer::DFTPostoutputLayer (layers/DFTErrorPostoutputLayer.cu:599-849)
+        L.kind = K_DFT;
+        trainable = false;
+        CNT_REQUIRE(L.size == 1 && P == 1, "network: the dft layer evaluates one waveform (size 1), found size %d after "
+                    "a layer of size %d", L.size, P);
+        CNT_REQUIRE(net->S == 1, "network: the dft layer needs parallel_sequences = 1 (one waveform per fraction)");
+        const char *off[] = {"beta", "eta", "kappa", "tau", "iota"};
+        for (const char *key : off) {
+            const json::Value *v = obj.get(key);
+            CNT_REQUIRE(!v || v->type != json::Value::NUM || v->num <= 0.0, "network: dft layer '%s': the '%s' term is not "
+                        "built", L.name.c_str(), key);
+        }
+        const char *flags[] = {"preEmphasisNaturalWav", "hnmMode", "multiDimSignalMode", "lpcOrder", "lpcOrder2", "lpcOrder3"};
+        for (const char *key : flags)
+            CNT_REQUIRE(get_int(obj, key, 0) == 0, "network: dft layer '%s': '%s' is not built", L.name.c_str(), key);
+        CNT_REQUIRE(get_str(obj, "specWeightVec").empty() && get_str(obj, "specWeightVec2").empty() &&
+                    get_str(obj, "specWeightVec3").empty(), "network: dft layer '%s': spectral weight vectors are not "
+                    "built", L.name.c_str());
+        auto real = [&](const char *key, double def) {
+            const json::Value *v = obj.get(key);
+            return (v && v->type == json::Value::NUM) ? v->num : def;
+        };
+        cnt_dft_desc d = {};
+        const char *suffix[3] = {"", "2", "3"};
+        const int def_len[3] = {320, 80, 80}, def_shift[3] = {80, 40, 40};
+        for (int r = 0; r < 3; ++r) {
+            const std::string sx = suffix[r];
+            const int fft = get_int(obj, ("fftLength" + sx).c_str(), r == 0 ? 512 : 0);
+            if (fft <= 0) continue;
+            d.fft_length[d.n_res] = fft;
+            d.frame_length[d.n_res] = get_int(obj, ("frameLength" + sx).c_str(), def_len[r]);
+            d.frame_shift[d.n_res] = get_int(obj, ("frameShift" + sx).c_str(), def_shift[r]);
+            d.window_type[d.n_res] = get_int(obj, ("windowType" + sx).c_str(), 0);
+            ++d.n_res;
+        }
+        d.gamma = (float)real("gamma", 0.0);
+        d.zeta = (float)real("zeta", 0.0);
+        d.log_floor = (float)real("logSpecAmpFloor", 0.00001);
+        d.spec_dis_type = get_int(obj, "specDisType", 0);
+        d.phase_dis_type = get_int(obj, "phaseDisType", 0);
+        d.max_length = net->maxT;
+        d.max_waves = 1;
+        CNT_TRY(cnt_dft_create(&d, &L.dft));
+        L.dft_error_count = d.n_res * (d.zeta > 0.0f ? 2 : 1);
+        CNT_TRY(device_alloc(net, (void **)&L.dft_errors, 8 * sizeof(float), true));
     } else if (t == "feedback") {
         L.kind = K_FEEDBACK;
         L.fb_start = get_int(obj, "previousDimStart", 0);
@@ -686,7 +750,7 @@ int build_layer_into(cnt_network *net, NetLayer &L, const json::Value &obj, cons
     const bool alias = is_sum_skip(L.kind) && L.pre.size() == 1;
     if (alias) L.out = net->layers[(size_t)L.pre[0]].out;
     else CNT_TRY(device_alloc(net, (void **)&L.out, count * sizeof(float), true));
-    if (L.kind != K_INPUT && L.kind != K_EXTERNAL && L.kind != K_SSE && L.kind != K_MDN && !is_skip_kind(L.kind))
+    if (L.kind != K_INPUT && L.kind != K_EXTERNAL && !is_post_kind(L.kind) && !is_skip_kind(L.kind))
         CNT_TRY(device_alloc(net, (void **)&L.err, count * sizeof(float), true));
     return CNT_OK;
 }
@@ -870,11 +934,11 @@ int finish_build(cnt_network *net, const json::Value *weights) {
                         "another contextDim than the first one", L.name.c_str());
     // checks that need the whole list
     const NetLayer &post = net->layers.back();
-    CNT_REQUIRE(post.kind == K_SSE || post.kind == K_MDN, "network: the last layer must be a post-output layer (sse or "
-                "mdn), found '%s'", post.type.c_str());
+    CNT_REQUIRE(is_post_kind(post.kind), "network: the last layer must be a post-output layer (sse, mdn or dft), found "
+                "'%s'", post.type.c_str());
     for (size_t i = 0; i + 1 < net->layers.size(); ++i)
-        CNT_REQUIRE(net->layers[i].kind != K_SSE && net->layers[i].kind != K_MDN, "network: post-output layer '%s' is "
-                    "not the last layer", net->layers[i].name.c_str());
+        CNT_REQUIRE(!is_post_kind(net->layers[i].kind), "network: post-output layer '%s' is not the last layer",
+                    net->layers[i].name.c_str());
     for (auto &L : net->layers)
         if (L.kind == K_FEEDBACK) {
             // NeuralNetwork.cpp:805-812 links every feedback layer to the post-output layer
@@ -904,6 +968,7 @@ int cnt_network_destroy(cnt_network *net) {
         if (L.lstm) cnt_lstm_destroy(L.lstm);
         if (L.cnn) cnt_cnn_destroy(L.cnn);
         if (L.mdn) cnt_mdn_destroy(L.mdn);
+        if (L.dft) cnt_dft_destroy(L.dft);
     }
     for (void *p : net->allocations) (void)hipFree(p);
     for (int k = 0; k < cnt_network::kMaxSide; ++k) {
@@ -1139,6 +1204,15 @@ int cnt_network_forward(cnt_network *net, void *stream_) {
             case K_MDN:
                 CNT_TRY(cnt_mdn_forward(L.mdn, stream, prev.out));
                 break;
+            case K_GATED:
+                CNT_TRY(cnt_gatedact_forward(stream, L.size, N, L.pat, prev.out, L.out));
+                break;
+            case K_DFT: {
+                // distances and gradient are both computed here (layers/DFTErrorPostoutputLayer.cu:1782-1839)
+                const int len = L.T;
+                CNT_TRY(cnt_dft_forward(L.dft, stream, 1, &len, prev.out, L.out, L.dft_errors));
+                break;
+            }
             default:
                 break;
         }
@@ -1153,6 +1227,13 @@ int cnt_network_calculate_error(cnt_network *net, void *stream_, float *loss_dev
     NetLayer &post = net->layers.back();
     const NetLayer &last = net->layers[net->layers.size() - 2];
     if (post.kind == K_SSE) return cnt_sse_error(stream, post.size, post.N, post.pat, last.out, post.out, loss_dev);
+    if (post.kind == K_DFT) {
+        // DFTPostoutputLayer::calculateError (layers/DFTErrorPostoutputLayer.cu:2105-2150): the plain sum of the
+        // distances of every resolution
+        hipLaunchKernelGGL(sum_few_kernel, dim3(1), dim3(64), 0, stream, post.dft_error_count, post.dft_errors, loss_dev);
+        CNT_HIP(hipGetLastError());
+        return CNT_OK;
+    }
     return cnt_mdn_calculate_error(post.mdn, stream, post.out, loss_dev);
 }
 
@@ -1180,6 +1261,14 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 break;
             case K_MDN:
                 CNT_TRY(cnt_mdn_backward(L.mdn, stream, L.out, prev.err));
+                break;
+            case K_DFT:
+                // writes the whole preceding error buffer: gradients up to the waveform's length, zeros beyond
+                // (the reference clears the buffer first, :1855-1856)
+                CNT_TRY(cnt_dft_backward(L.dft, stream, prev.err));
+                break;
+            case K_GATED:
+                CNT_TRY(cnt_gatedact_backward(stream, L.size, N, L.pat, prev.out, L.err, prev.err));
                 break;
             case K_DENSE:
             case K_LSTM:

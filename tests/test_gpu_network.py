@@ -409,3 +409,107 @@ def test_full_size_wavenet_sequencer_matches_layer_by_layer_walk():
             assert PC.relerr(L["updates"].cpu().numpy(), walk.buf[L["name"]]["dW"].cpu().numpy()) < TOL, L["name"]
     walk.close()
     net.close()
+
+
+def test_gatedact_layer_and_dft_post_output_in_a_network_file():
+    """Two more layer types of the reference's registry through the sequencer: `gatedact` inside a small stack with
+    an sse output, and a `dft` post-output layer (two resolutions, spectral distance type 1, phase term) after a
+    stack that produces a waveform -- each against the oracle's primitives."""
+    import torch
+
+    print("gatedact and dft layers in network files", flush=True)
+    capi = PC.pkg().capi
+    rng = np.random.default_rng(21)
+
+    # ---- gatedact ------------------------------------------------------------------------------------------------
+    P, D, Q, lengths = 6, 8, 5, [20, 13, 17]
+    S, T = len(lengths), max(lengths)
+    N = S * T
+    pat = make_pat_types(lengths, T)
+    valid = pat != 0
+    x = rng.standard_normal((N, P)).astype(np.float32); x[~valid] = 0
+    tgt = rng.standard_normal((N, Q)).astype(np.float32); tgt[~valid] = 0
+    w1 = rng.uniform(-0.5, 0.5, P * 2 * D + 2 * D).astype(np.float32)
+    w2 = rng.uniform(-0.5, 0.5, D * Q + Q).astype(np.float32)
+    h1, g, y = np.zeros(2 * D * N, np.float32), np.zeros(D * N, np.float32), np.zeros(Q * N, np.float32)
+    O.dense_forward(P, 2 * D, N, 0, 1.0, w1, x.reshape(-1), h1)
+    O.gated_forward(D, N, pat, h1, g)
+    O.dense_forward(D, Q, N, 1, 1.0, w2, g, y)
+    ref_loss = O.sse_error(Q, N, pat, y, tgt.reshape(-1))
+    ey, eg, eh1 = np.zeros(Q * N, np.float32), np.zeros(D * N, np.float32), np.zeros(2 * D * N, np.float32)
+    dw1, dw2 = np.zeros_like(w1), np.zeros_like(w2)
+    O.sse_backward(Q, N, pat, y, tgt.reshape(-1), ey)
+    O.dense_backward(D, Q, N, 1, 1.0, w2, g, y, ey, eg, dw2)
+    O.gated_backward(D, N, pat, h1, eg, eh1)
+    O.dense_backward(P, 2 * D, N, 0, 1.0, w1, x.reshape(-1), h1, eh1, None, dw1)
+    doc = {"layers": [{"size": P, "name": "input", "type": "input"},
+                      {"size": 2 * D, "name": "pre", "type": "feedforward_identity", "bias": 1.0},
+                      {"size": D, "name": "gate", "type": "gatedact", "bias": 1.0},
+                      {"size": Q, "name": "out", "type": "feedforward_tanh", "bias": 1.0},
+                      {"size": Q, "name": "post", "type": "sse"}]}
+    net = capi.Network(json.dumps(doc), S, T)
+    net.layer("pre")["weights"].copy_(torch.from_numpy(w1))
+    net.layer("out")["weights"].copy_(torch.from_numpy(w2))
+    net.load_sequences(PC.dev(pat), T, min(lengths), PC.dev(x.reshape(-1)), PC.dev(tgt.reshape(-1)))
+    net.forward()
+    loss = float(net.calculate_error().item())
+    net.backward()
+    torch.cuda.synchronize()
+    assert abs(loss - ref_loss) <= TOL * abs(ref_loss)
+    assert PC.relerr(net.layer("gate")["outputs"][: g.size].cpu().numpy(), g) < TOL
+    assert PC.relerr(net.layer("pre")["updates"].cpu().numpy(), dw1) < TOL
+    assert PC.relerr(net.layer("out")["updates"].cpu().numpy(), dw2) < TOL
+    net.close()
+
+    # ---- dft -------------------------------------------------------------------------------------------------------
+    P, Hd, T, maxT = 4, 16, 900, 1000
+    pat = make_pat_types([T], T)
+    x = rng.standard_normal((T, P)).astype(np.float32)
+    tgt = (0.3 * rng.standard_normal(T)).astype(np.float32)
+    w1 = rng.uniform(-0.5, 0.5, P * Hd + Hd).astype(np.float32)
+    w2 = rng.uniform(-0.5, 0.5, Hd + 1).astype(np.float32)
+    h1, y = np.zeros(Hd * T, np.float32), np.zeros(T, np.float32)
+    O.dense_forward(P, Hd, T, 1, 1.0, w1, x.reshape(-1), h1)
+    O.dense_forward(Hd, 1, T, 0, 1.0, w2, h1, y)
+    res = [(128, 100, 25), (64, 64, 16)]
+    gamma, zeta, dis = 0.7, 0.4, 1
+    src = np.zeros(maxT, np.float32); src[:T] = y
+    tg = np.zeros(maxT, np.float32); tg[:T] = tgt
+    ey, ref_loss = np.zeros(maxT, np.float64), 0.0
+    for (Nf, Nw, Hs) in res:
+        gbuf = np.zeros(maxT, np.float32)
+        ref_loss += O.dft_spectral_loss(dis, Nf, Nw, Hs, 0, maxT, T, gamma, 1e-5, src.copy(), tg.copy(), gbuf)
+        gbuf[T:] = 0
+        ey += gbuf
+        ref_loss += O.dft_phase_loss(Nf, Nw, Hs, 0, maxT, T, zeta, src.copy(), tg.copy(), gbuf)
+        gbuf[T:] = 0
+        ey += gbuf
+    ey = ey[:T].astype(np.float32)
+    eh1, dw1, dw2 = np.zeros(Hd * T, np.float32), np.zeros_like(w1), np.zeros_like(w2)
+    O.dense_backward(Hd, 1, T, 0, 1.0, w2, h1, y, ey, eh1, dw2)
+    O.dense_backward(P, Hd, T, 1, 1.0, w1, x.reshape(-1), h1, eh1, None, dw1)
+    doc = {"layers": [{"size": P, "name": "input", "type": "input"},
+                      {"size": Hd, "name": "h", "type": "feedforward_tanh", "bias": 1.0},
+                      {"size": 1, "name": "wave", "type": "feedforward_identity", "bias": 1.0},
+                      {"size": 1, "name": "post", "type": "dft", "gamma": gamma, "zeta": zeta, "specDisType": dis,
+                       "fftLength": 128, "frameLength": 100, "frameShift": 25,
+                       "fftLength2": 64, "frameLength2": 64, "frameShift2": 16}]}
+    net = capi.Network(json.dumps(doc), 1, maxT)
+    net.layer("h")["weights"].copy_(torch.from_numpy(w1))
+    net.layer("wave")["weights"].copy_(torch.from_numpy(w2))
+    for _ in range(2):
+        net.load_sequences(PC.dev(pat), T, T, PC.dev(x.reshape(-1)), PC.dev(tgt))
+        net.forward()
+        loss = float(net.calculate_error().item())
+        net.backward()
+        torch.cuda.synchronize()
+        assert abs(loss - ref_loss) <= TOL * abs(ref_loss)
+        assert PC.relerr(net.layer("wave")["errors"][:T].cpu().numpy(), ey) < TOL
+        assert PC.relerr(net.layer("h")["updates"].cpu().numpy(), dw1) < TOL
+        assert PC.relerr(net.layer("wave")["updates"].cpu().numpy(), dw2) < TOL
+    net.close()
+    with pytest.raises(RuntimeError, match="parallel_sequences = 1"):
+        capi.Network(json.dumps(doc), 2, maxT)
+    doc["layers"][-1]["beta"] = 1.0
+    with pytest.raises(RuntimeError, match="'beta' term"):
+        capi.Network(json.dumps(doc), 1, maxT)
