@@ -513,3 +513,55 @@ def test_gatedact_layer_and_dft_post_output_in_a_network_file():
     doc["layers"][-1]["beta"] = 1.0
     with pytest.raises(RuntimeError, match="'beta' term"):
         capi.Network(json.dumps(doc), 1, maxT)
+
+
+def test_mixture_density_network_file():
+    """benchmark config 3's layout in small: ... -> feedforward_identity -> mdn with one untied-variance mixture unit
+    (mdn config [1, 0, Lp, 0, D, M]); loss, the error handed to the output layer and the weight gradients against
+    the oracle."""
+    import torch
+
+    print("mixture density network file", flush=True)
+    capi = PC.pkg().capi
+    rng = np.random.default_rng(31)
+    P, Hd, M, D = 5, 8, 4, 3
+    Lp = M + 2 * M * D
+    lengths = [14, 9, 14, 11]
+    S, T = len(lengths), max(lengths)
+    N = S * T
+    pat = make_pat_types(lengths, T)
+    valid = pat != 0
+    x = rng.standard_normal((N, P)).astype(np.float32); x[~valid] = 0
+    tgt = rng.standard_normal((N, D)).astype(np.float32); tgt[~valid] = 0
+    w1 = rng.uniform(-0.5, 0.5, P * Hd + Hd).astype(np.float32)
+    w2 = rng.uniform(-0.5, 0.5, Hd * Lp + Lp).astype(np.float32)
+    h1, y = np.zeros(Hd * N, np.float32), np.zeros(Lp * N, np.float32)
+    O.dense_forward(P, Hd, N, 1, 1.0, w1, x.reshape(-1), h1)
+    O.dense_forward(Hd, Lp, N, 0, 1.0, w2, h1, y)
+    para, tmp = np.zeros(N * M * (1 + 2 * D), np.float32), np.zeros(N * M + N, np.float32)
+    O.mdn_mixture_forward(N, Lp, 0, M, D, 0.0, pat, y, para)
+    ref_loss = O.mdn_mixture_error(N, D, 0, M, D, pat, tgt.reshape(-1), para, tmp)
+    ey = np.zeros(Lp * N, np.float32)
+    O.mdn_mixture_backward(N, Lp, D, 0, 0, M, D, 0.0, pat, tgt.reshape(-1), para, tmp, ey)
+    eh1, dw1, dw2 = np.zeros(Hd * N, np.float32), np.zeros_like(w1), np.zeros_like(w2)
+    O.dense_backward(Hd, Lp, N, 0, 1.0, w2, h1, y, ey.copy(), eh1, dw2)
+    O.dense_backward(P, Hd, N, 1, 1.0, w1, x.reshape(-1), h1, eh1, None, dw1)
+    doc = {"layers": [{"size": P, "name": "input", "type": "input"},
+                      {"size": Hd, "name": "h", "type": "feedforward_tanh", "bias": 1.0},
+                      {"size": Lp, "name": "out", "type": "feedforward_identity", "bias": 1.0},
+                      {"size": D, "name": "post", "type": "mdn"}]}
+    net = capi.Network(json.dumps(doc), S, T + 3, mdn_config=[1, 0, Lp, 0, D, M])
+    net.layer("h")["weights"].copy_(torch.from_numpy(w1))
+    net.layer("out")["weights"].copy_(torch.from_numpy(w2))
+    net.load_sequences(PC.dev(pat), T, min(lengths), PC.dev(x.reshape(-1)), PC.dev(tgt.reshape(-1)))
+    net.forward()
+    loss = float(net.calculate_error().item())
+    net.backward()
+    torch.cuda.synchronize()
+    assert abs(loss - ref_loss) <= TOL * abs(ref_loss)
+    assert PC.relerr(net.layer("out")["errors"][: ey.size].cpu().numpy(), ey) < TOL
+    assert PC.relerr(net.layer("h")["updates"].cpu().numpy(), dw1) < TOL
+    assert PC.relerr(net.layer("out")["updates"].cpu().numpy(), dw2) < TOL
+    net.close()
+    with pytest.raises(RuntimeError, match="mdn config"):
+        capi.Network(json.dumps(doc), S, T)
