@@ -382,8 +382,8 @@ int cnt_network_backward(cnt_network *net, void *stream);
 /* cnt_lstm_check for every LSTM layer. */
 int cnt_network_check(cnt_network *net, void *stream);
 /* One optimizer step over all weights in a single launch (see cnt_opt_step; the network keeps the optimizer's
- * current updates, deltas, statistics and Adam's accumulated betas).  Layer-specific learning rates
- * ("learningRate" of a layer) are not built. */
+ * current updates, deltas, statistics and Adam's accumulated betas).  If a layer of the network file carries its
+ * own "learningRate" (layers/TrainableLayer.cu:110-111), the step is one launch per trainable layer instead. */
 int cnt_network_update(cnt_network *net, void *stream, int option, float learning_rate, float momentum,
                        float frac_length);
 /* NeuralNetwork::exportLayers + exportWeights (NeuralNetwork.cpp:2993-3040): the layer objects as they stood in the

@@ -191,6 +191,7 @@ struct NetLayer {
     int kind = K_INPUT;
     int size = 0, prev = -1;
     float bias = 0.0f;
+    float learning_rate = -1.0f;  // "learningRate" of a trainable layer; below -0.5: the optimizer's
     int act = 0, bidir = 0;
     std::vector<int> pre;  // skip layers: linked source layers
     long w_off = 0, n_in = 0, n_bias = 0, n_int = 0;
@@ -512,6 +513,8 @@ int build_layer_into(cnt_network *net, NetLayer &L, const json::Value &obj, cons
     const json::Value *bias = obj.get("bias");
     L.bias = (bias && bias->type == json::Value::NUM) ? (float)bias->num : 0.0f;
     L.prev = index - 1;
+    if (const json::Value *lr = obj.get("learningRate"))
+        if (lr->type == json::Value::NUM) L.learning_rate = (float)lr->num;
     CNT_REQUIRE(L.size > 0, "network: layer %d ('%s') has no positive size", index, L.name.c_str());
     L.res = get_int(obj, "resolution", 1);
     CNT_REQUIRE(L.res >= 1, "network: layer '%s' has resolution %d", L.name.c_str(), L.res);
@@ -1395,8 +1398,23 @@ int cnt_network_update(cnt_network *net, void *stream_, int option, float learni
         net->beta1_accum = cnt_opt_next_beta_accum(net->beta1_accum, 1);
         net->beta2_accum = cnt_opt_next_beta_accum(net->beta2_accum, 2);
     }
-    return cnt_opt_step(stream_, option, (long)n, net->weights, net->updates, net->cur_updates, net->stats, net->deltas,
-                        nullptr, frac_length, net->beta1_accum, net->beta2_accum, learning_rate, momentum);
+    bool own_rates = false;
+    for (const auto &L : net->layers) own_rates = own_rates || (L.weight_count() > 0 && L.learning_rate > -0.5f);
+    if (!own_rates)
+        return cnt_opt_step(stream_, option, (long)n, net->weights, net->updates, net->cur_updates, net->stats, net->deltas,
+                            nullptr, frac_length, net->beta1_accum, net->beta2_accum, learning_rate, momentum);
+    // a layer's own "learningRate" replaces the optimizer's (optimizers/SteepestDescentOptimizer.cu:402-403, :425-426): one
+    // launch per trainable layer
+    for (const auto &L : net->layers) {
+        const long c = L.weight_count();
+        if (c == 0) continue;
+        const long o = L.w_off;
+        float *st = net->stats ? net->stats + (adam ? 2 * o : o) : nullptr;
+        CNT_TRY(cnt_opt_step(stream_, option, c, net->weights + o, net->updates + o, net->cur_updates + o, st,
+                             net->deltas + o, nullptr, frac_length, net->beta1_accum, net->beta2_accum,
+                             L.learning_rate > -0.5f ? L.learning_rate : learning_rate, momentum));
+    }
+    return CNT_OK;
 }
 
 int cnt_network_export_json(cnt_network *net, char *buf, size_t cap, size_t *needed) {

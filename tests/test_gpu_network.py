@@ -195,6 +195,36 @@ def test_network_file_rejections():
     net.close()
 
 
+def test_layer_specific_learning_rate():
+    """A layer's own "learningRate" replaces the optimizer's for that layer (0 freezes it)."""
+    import torch
+
+    capi = PC.pkg().capi
+    doc = {"layers": [{"size": 3, "name": "input", "type": "input"},
+                      {"size": 5, "name": "frozen", "type": "feedforward_tanh", "bias": 1.0, "learningRate": 0.0},
+                      {"size": 4, "name": "fast", "type": "feedforward_identity", "bias": 1.0, "learningRate": 0.5},
+                      {"size": 4, "name": "plain", "type": "feedforward_identity", "bias": 1.0},
+                      {"size": 4, "name": "post", "type": "sse"}]}
+    S, T = 2, 6
+    net = capi.Network(json.dumps(doc), S, T)
+    net.randomize(3, 0.3)
+    w0 = net.weights.clone()
+    rng = np.random.default_rng(2)
+    pat = make_pat_types([T, T], T)
+    net.load_sequences(PC.dev(pat), T, T, PC.dev(rng.standard_normal(3 * S * T).astype(np.float32)),
+                       PC.dev(rng.standard_normal(4 * S * T).astype(np.float32)))
+    net.forward()
+    net.backward()
+    net.update(0, 0.01, 0.0, float(S * T))
+    torch.cuda.synchronize()
+    g = net.updates
+    for name, lr in (("frozen", 0.0), ("fast", 0.5), ("plain", 0.01)):
+        L = net.layer(name)
+        a, b = L["weight_offset"], L["weight_offset"] + L["weight_count"]
+        assert torch.allclose(net.weights[a:b], w0[a:b] - lr * g[a:b], rtol=1e-6, atol=1e-7), name
+    net.close()
+
+
 class _CondOracleBackend(OM.OracleBackend):
     """Oracle back end whose gated layers also accumulate the gradient with respect to the conditioning features."""
     ctx_grad = None
