@@ -318,7 +318,7 @@ int cnt_dft_backward(cnt_dft *h, void *stream, float *prev_errors);
  * _tanh / _logistic / _relu", "lstm", "blstm", "skipini", "skipadd" (with "preSkipLayer"), "cnn" (1-D), "wavnetc",
  * "gatedact", "feedback" (one step back, fed by one softmax unit), "skipcat" (with "preSkipLayerDim"),
  * "externalloader" and the post-output layers "sse", "mdn" and "dft" (keys fftLength / frameLength / frameShift /
- * windowType with suffix "", "2", "3", gamma, zeta, specDisType, phaseDisType, logSpecAmpFloor; one waveform per
+ * windowType with suffix "", "2", "3", beta, gamma, zeta, specDisType, phaseDisType, logSpecAmpFloor; one waveform per
  * fraction, i.e. parallel_sequences = 1); layers may run at a lower time "resolution" (layers/Layer.cu:254-305), and a
  * layer flagged "wavenetConditionInputLayer" feeds the wavnetc layers (NeuralNetwork.cpp:544-561).  json_text is the
  * text of a network file: "layers" in order, optionally "weights" with the "input" / "bias" / "internal" arrays of

@@ -202,6 +202,7 @@ struct NetLayer {
     cnt_dft *dft = nullptr;
     float *dft_errors = nullptr;             // dft: per-resolution distances written by the forward pass
     int dft_error_count = 0;
+    float dft_beta = 0.0f;                   // dft: weight of the waveform MSE gradient
     float *core = nullptr, *cth = nullptr;  // wavnetc
     int ctx_dim = 0;
     int fb_start = 0, fb_end = 0;            // feedback: dimensions taken from the preceding layer
@@ -383,6 +384,16 @@ __global__ void sum_few_kernel(int n, const float *__restrict__ v, float *__rest
         for (int i = 0; i < n; ++i) acc += v[i];
         *out = acc;
     }
+}
+// gradient of the dft layer's waveform MSE term, added to the spectral gradients (ComputeMseWaveformGrad,
+// layers/DFTErrorPostoutputLayer.cu:87-120, :1157-1183)
+__global__ void waveform_mse_grad_kernel(size_t count, int dim, float beta, const char *__restrict__ pat,
+                                         const float *__restrict__ y, const float *__restrict__ target,
+                                         float *__restrict__ err) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count; i += stride)
+        if (pat[i / dim] != 0) err[i] += (y[i] - target[i]) * beta;
 }
 __global__ void add_inplace_kernel(size_t count, float *__restrict__ a, const float *__restrict__ b) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -673,7 +684,7 @@ int build_layer_into(cnt_network *net, NetLayer &L, const json::Value &obj, cons
         CNT_REQUIRE(L.size == 1 && P == 1, "network: the dft layer evaluates one waveform (size 1), found size %d after "
                     "a layer of size %d", L.size, P);
         CNT_REQUIRE(net->S == 1, "network: the dft layer needs parallel_sequences = 1 (one waveform per fraction)");
-        const char *off[] = {"beta", "eta", "kappa", "tau", "iota"};
+        const char *off[] = {"eta", "kappa", "tau", "iota"};
         for (const char *key : off) {
             const json::Value *v = obj.get(key);
             CNT_REQUIRE(!v || v->type != json::Value::NUM || v->num <= 0.0, "network: dft layer '%s': the '%s' term is not "
@@ -702,6 +713,7 @@ int build_layer_into(cnt_network *net, NetLayer &L, const json::Value &obj, cons
             d.window_type[d.n_res] = get_int(obj, ("windowType" + sx).c_str(), 0);
             ++d.n_res;
         }
+        L.dft_beta = (float)real("beta", 0.0);
         d.gamma = (float)real("gamma", 0.0);
         d.zeta = (float)real("zeta", 0.0);
         d.log_floor = (float)real("logSpecAmpFloor", 0.00001);
@@ -1269,6 +1281,11 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 // writes the whole preceding error buffer: gradients up to the waveform's length, zeros beyond
                 // (the reference clears the buffer first, :1855-1856)
                 CNT_TRY(cnt_dft_backward(L.dft, stream, prev.err));
+                if (L.dft_beta > 0.0f) {
+                    hipLaunchKernelGGL(waveform_mse_grad_kernel, dim3(blocks_for(count)), dim3(256), 0, stream, count,
+                                       L.size, L.dft_beta, L.pat, prev.out, L.out, prev.err);
+                    CNT_HIP(hipGetLastError());
+                }
                 break;
             case K_GATED:
                 CNT_TRY(cnt_gatedact_backward(stream, L.size, N, L.pat, prev.out, L.err, prev.err));

@@ -502,7 +502,7 @@ def test_gatedact_layer_and_dft_post_output_in_a_network_file():
     O.dense_forward(P, Hd, T, 1, 1.0, w1, x.reshape(-1), h1)
     O.dense_forward(Hd, 1, T, 0, 1.0, w2, h1, y)
     res = [(128, 100, 25), (64, 64, 16)]
-    gamma, zeta, dis = 0.7, 0.4, 1
+    gamma, zeta, dis, beta = 0.7, 0.4, 1, 0.3
     src = np.zeros(maxT, np.float32); src[:T] = y
     tg = np.zeros(maxT, np.float32); tg[:T] = tgt
     ey, ref_loss = np.zeros(maxT, np.float64), 0.0
@@ -514,14 +514,14 @@ def test_gatedact_layer_and_dft_post_output_in_a_network_file():
         ref_loss += O.dft_phase_loss(Nf, Nw, Hs, 0, maxT, T, zeta, src.copy(), tg.copy(), gbuf)
         gbuf[T:] = 0
         ey += gbuf
-    ey = ey[:T].astype(np.float32)
+    ey = (ey[:T] + beta * (y.astype(np.float64) - tgt)).astype(np.float32)   # waveform MSE term: gradient only
     eh1, dw1, dw2 = np.zeros(Hd * T, np.float32), np.zeros_like(w1), np.zeros_like(w2)
     O.dense_backward(Hd, 1, T, 0, 1.0, w2, h1, y, ey, eh1, dw2)
     O.dense_backward(P, Hd, T, 1, 1.0, w1, x.reshape(-1), h1, eh1, None, dw1)
     doc = {"layers": [{"size": P, "name": "input", "type": "input"},
                       {"size": Hd, "name": "h", "type": "feedforward_tanh", "bias": 1.0},
                       {"size": 1, "name": "wave", "type": "feedforward_identity", "bias": 1.0},
-                      {"size": 1, "name": "post", "type": "dft", "gamma": gamma, "zeta": zeta, "specDisType": dis,
+                      {"size": 1, "name": "post", "type": "dft", "gamma": gamma, "zeta": zeta, "specDisType": dis, "beta": beta,
                        "fftLength": 128, "frameLength": 100, "frameShift": 25,
                        "fftLength2": 64, "frameLength2": 64, "frameShift2": 16}]}
     net = capi.Network(json.dumps(doc), 1, maxT)
@@ -540,8 +540,8 @@ def test_gatedact_layer_and_dft_post_output_in_a_network_file():
     net.close()
     with pytest.raises(RuntimeError, match="parallel_sequences = 1"):
         capi.Network(json.dumps(doc), 2, maxT)
-    doc["layers"][-1]["beta"] = 1.0
-    with pytest.raises(RuntimeError, match="'beta' term"):
+    doc["layers"][-1]["kappa"] = 1.0
+    with pytest.raises(RuntimeError, match="'kappa' term"):
         capi.Network(json.dumps(doc), 1, maxT)
 
 
