@@ -50,3 +50,22 @@ def test_network_file_syntax_errors_without_gpu():
         h = C.c_void_p()
         with pytest.raises(RuntimeError, match=what):
             capi.check(capi.lib().cnt_network_create(text.encode(), 2, 10, None, C.byref(h)))
+
+
+def test_truncated_network_files_are_rejected_without_gpu():
+    """Every prefix of a valid network file is an error (never a crash): the reader validates as it goes."""
+    import ctypes as C
+    import json
+
+    capi = load_package().capi
+    L = capi.lib()
+    doc = {"layers": [{"size": 3, "name": "input", "type": "input"},
+                      {"size": 4, "name": "h", "type": "feedforward_tanh", "bias": 1.0},
+                      {"size": 4, "name": "s", "type": "skipini", "bias": 1.0},
+                      {"size": 4, "name": "post", "type": "sse"}],
+           "weights": {"h": {"input": [0.5, -1e-3, 2.0e1], "bias": [1, 2], "internal": []}}}
+    text = json.dumps(doc)
+    for cut in range(len(text)):
+        h = C.c_void_p()
+        assert L.cnt_network_create(text[:cut].encode(), 2, 10, None, C.byref(h)) != 0
+        assert L.cnt_last_error()
