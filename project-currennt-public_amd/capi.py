@@ -162,7 +162,7 @@ def lib():
 
 def check(status):
     if status != CNT_OK:
-        raise RuntimeError("currennt_hip error %d: %s" % (status, lib().cnt_last_error().decode()))
+        raise RuntimeError("currennt_hip error %d: %s" % (status, lib().cnt_last_error().decode(errors="replace")))
 
 
 def ptr(t):

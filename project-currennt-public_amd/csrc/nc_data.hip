@@ -265,6 +265,13 @@ int cnt_dataset_open(const char *nc_path, const cnt_dataset_desc *desc, cnt_data
     else if (!d->file.dimension("targetPattSize", out_size)) return bail("Cannot get dimension 'targetPattSize'");
     if (!d->file.dimension("numSeqs", n_seq)) return bail("Cannot get dimension 'numSeqs'");
     d->file.dimension("numTimesteps", n_steps);
+    // sizes a damaged header could claim
+    constexpr long kMaxPattern = 1L << 20, kMaxTag = 1L << 16;
+    if (in_size < 1 || in_size > kMaxPattern) return bail("dataset_open: dimension 'inputPattSize' out of range");
+    if (out_size < 1 || out_size > kMaxPattern) return bail("dataset_open: target dimension out of range");
+    if (max_tag < 1 || max_tag > kMaxTag) return bail("dataset_open: dimension 'maxSeqTagLength' out of range");
+    if (n_seq < 1 || n_seq > (1L << 31) - 1) return bail("dataset_open: dimension 'numSeqs' out of range");
+    if (n_steps < 0) return bail("dataset_open: dimension 'numTimesteps' out of range");
     d->input_size = (int)in_size;
     d->output_size = (int)out_size;
 

@@ -142,3 +142,30 @@ def test_reader_errors(tmp_path):
     with pytest.raises(RuntimeError, match="unlimited"):
         ds.fraction(0)
     ds.close()
+
+
+def test_damaged_header_is_rejected(tmp_path):
+    """A dimension a damaged header claims (here inputPattSize = 2^32 - 1, read as a negative size) is refused, and
+    a file cut anywhere in its header or data is an error, never a crash."""
+    capi = load_package().capi
+    p = str(tmp_path / "ok.nc")
+    write_nc(p, [4, 6], 3, 2, 1)
+    good = open(p, "rb").read()
+    at = good.index(b"inputPattSize")
+    pad = (4 - len(b"inputPattSize") % 4) % 4
+    q = tmp_path / "dim.nc"
+    q.write_bytes(good[:at + 13 + pad] + b"\xff\xff\xff\xff" + good[at + 13 + pad + 4:])
+    with pytest.raises(RuntimeError, match="out of range|dimension"):
+        capi.Dataset(str(q), 2)
+    for cut in range(8, len(good), 37):
+        c = tmp_path / "cut.nc"
+        c.write_bytes(good[:cut])
+        try:
+            ds = capi.Dataset(str(c), 2)
+        except RuntimeError:
+            continue
+        try:
+            ds.fraction(0)
+        except RuntimeError:
+            pass
+        ds.close()
