@@ -7,7 +7,8 @@
 // runs about a dozen launches and three cuFFT calls per resolution and waveform, with every intermediate
 // (framed signals, spectra, per-bin differences, framed gradients) in device memory.
 //
-// Here one workgroup owns one frame end to end and nothing but the waveforms and the gradient touches HBM:
+// Here one workgroup owns one frame end to end, all resolutions of a call are one launch, and nothing but the
+// waveforms and the gradient touches HBM:
 //   frame + window source and target  ->  ONE complex FFT of z = source + i*target in LDS (both real
 //   spectra are recovered from Z[b] and Z[N-b])  ->  per-bin log-amplitude difference, loss partial and
 //   gradient spectrum, written back as its Hermitian extension  ->  inverse FFT in LDS  ->  windowed
@@ -31,14 +32,16 @@ constexpr int kMaxRes = 3;
 constexpr int kMaxWavesPerLaunch = 32;
 
 struct DftParams {
-    int N, Nw, Hs;       // fft length, frame length, frame shift
+    // per resolution: log2 of the fft length, frame length, frame shift, blocks along x that carry frames
+    int logn[kMaxRes], Nw[kMaxRes], Hs[kMaxRes], nblocks[kMaxRes];
+    const float2 *twiddle[kMaxRes];  // N entries, stage by stage: entry 2^s + k = exp(-2*pi*i*k / 2^(s+1)), k < 2^s
+    const float *window[kMaxRes];    // Nw entries
     int max_length;      // samples per waveform buffer
-    int n_waves, n_res, res;
+    int n_waves, n_res;
+
     int lengths[kMaxWavesPerLaunch];
     float gamma, log_floor;
     float zeta;          // weight of the cosine phase distance; 0 = not evaluated
-    const float2 *twiddle;  // N/2 entries exp(-2*pi*i*k/N)
-    const float *window;    // Nw entries
     const float *source, *target;
     float *grad;    // n_waves x max_length, accumulated over resolutions
     float *errors;  // n_waves x n_res amplitude distances, followed by n_waves x n_res phase distances if zeta > 0
@@ -123,112 +126,146 @@ __device__ inline void bin_phase(float sx, float sy, float tx, float ty, float &
     gy = fac * sx / spec;
 }
 
+constexpr int kMaxLogN = 12;
+
+// One block = passes of FPB frames of resolution `res` of one waveform.  lds: max(512, N) + N complex words.
 template <int LOGN, int DIS>
-__global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
+__device__ __forceinline__ void dft_frames(const DftParams &p, const int res, float2 *__restrict__ lds,
+                                           float (*err_part)[4]) {
     constexpr int N = 1 << LOGN;
+    float2 *__restrict__ zbuf = lds;                    // frame storage: FPB * N = max(512, N) complex words
+    float2 *__restrict__ tw = lds + (N > 512 ? N : 512);  // N twiddles
     constexpr int HALF = N / 2;
     constexpr int TPF = HALF < 256 ? HALF : 256;  // threads per frame
     constexpr int FPB = 256 / TPF;                // frames per block
-    __shared__ float2 z[FPB][N];
-    __shared__ float2 tw[HALF];
-    __shared__ float err_part[2][4];
+    static_assert(FPB * N <= (N > 512 ? N : 512), "frame storage: max(512, N) complex words");
+
+    constexpr int EPT = N / TPF;  // samples per thread and frame
 
     const int tid = threadIdx.x;
     const int fl = tid / TPF, ft = tid % TPF;  // frame slot in the block, thread within the frame
+    float2 *zf = zbuf + fl * N;                // this frame's storage
+    const int Nw = p.Nw[res], Hs = p.Hs[res];
+    const float *__restrict__ win = p.window[res];
     const int wave_id = blockIdx.y;
     const int length = p.lengths[wave_id];
-    const int Kvalid = frame_count(length, p.Nw, p.Hs);
-    const int k = blockIdx.x * FPB + fl;
-    const bool active = k < Kvalid;  // every thread stays for the barriers
+    const int Kvalid = frame_count(length, Nw, Hs);
+    const int kstep = p.nblocks[res] * FPB;  // frames between two passes of this block
     const float *src = p.source + (size_t)wave_id * p.max_length;
     const float *tgt = p.target + (size_t)wave_id * p.max_length;
-
-    for (int i = tid; i < HALF; i += 256) tw[i] = p.twiddle[i];
-    for (int j = ft; j < N; j += TPF) {
-        float2 v = make_float2(0.0f, 0.0f);
-        const int pos = k * p.Hs + j;
-        if (active && j < p.Nw && pos < length) {
-            const float w = p.window[j];
-            v = make_float2(src[pos] * w, tgt[pos] * w);
-        }
-        z[fl][j] = v;
-    }
-    __syncthreads();
-
-    // forward: decimation in frequency
-#pragma unroll 1
-    for (int s = LOGN - 1; s >= 0; --s) {
-        const int half = 1 << s;
-        for (int i = ft; i < HALF; i += TPF) {
-            const int pos = i & (half - 1);
-            const int a = ((i >> s) << (s + 1)) + pos, b = a + half;
-            const float2 u = z[fl][a], v = z[fl][b];
-            const float2 w = tw[pos << (LOGN - 1 - s)];
-            const float dx = u.x - v.x, dy = u.y - v.y;
-            z[fl][a] = make_float2(u.x + v.x, u.y + v.y);
-            z[fl][b] = make_float2(dx * w.x - dy * w.y, dx * w.y + dy * w.x);
-        }
-        __syncthreads();
-    }
-
-    // per-bin stage on the pairs (b, N-b); bin b lives at position bitrev(b)
-    // With the phase term both gradient spectra are weighted here and share the inverse transform (the reference
-    // runs a second framing / FFT / inverse FFT / overlap-add for it, layers/DFTErrorPostoutputLayer.cu:1246-1295).
+    float *g = p.grad + (size_t)wave_id * p.max_length;
     const bool phase = p.zeta > 0.0f;
-    float err = 0.0f, err_ph = 0.0f;
-    for (int b = ft; b <= HALF; b += TPF) {
-        const int nb = (N - b) & (N - 1);
-        const int pb = (int)(__brev((unsigned)b) >> (32 - LOGN));
-        const int pnb = (int)(__brev((unsigned)nb) >> (32 - LOGN));
-        const float2 zb = z[fl][pb], zn = z[fl][pnb];
-        // S = (Z[b] + conj(Z[N-b])) / 2,  T = (Z[b] - conj(Z[N-b])) / (2i)
-        const float sx = 0.5f * (zb.x + zn.x), sy = 0.5f * (zb.y - zn.y);
-        const float tx = 0.5f * (zb.y + zn.y), ty = -0.5f * (zb.x - zn.x);
-        float e, gx, gy;
-        bin_distance<DIS>(sx, sy, tx, ty, p.log_floor, e, gx, gy);
-        if (active) err += e;
-        if (phase) {
-            float pe, px, py;
-            bin_phase(sx, sy, tx, ty, pe, px, py);
-            if (active) err_ph += pe;
-            gx = p.gamma * gx + p.zeta * px;
-            gy = p.gamma * gy + p.zeta * py;
-        }
-        if (b == 0 || b == HALF) {
-            z[fl][pb] = make_float2(gx, 0.0f);
-        } else {
-            z[fl][pb] = make_float2(gx, gy);
-            z[fl][pnb] = make_float2(gx, -gy);
-        }
-    }
-    __syncthreads();
-
-    // inverse: decimation in time with conjugated twiddles, unnormalised
-#pragma unroll 1
-    for (int s = 0; s < LOGN; ++s) {
-        const int half = 1 << s;
-        for (int i = ft; i < HALF; i += TPF) {
-            const int pos = i & (half - 1);
-            const int a = ((i >> s) << (s + 1)) + pos, b = a + half;
-            const float2 u = z[fl][a], x = z[fl][b];
-            const float2 w = tw[pos << (LOGN - 1 - s)];
-            const float vx = x.x * w.x + x.y * w.y, vy = x.y * w.x - x.x * w.y;
-            z[fl][a] = make_float2(u.x + vx, u.y + vy);
-            z[fl][b] = make_float2(u.x - vx, u.y - vy);
-        }
-        __syncthreads();
-    }
-
-    // windowed overlap-add; frames at or beyond Kvalid contribute nothing
     const float inv = 1.0f / (float)((HALF + 1) * Kvalid);
-    if (active) {
-        const float scale = phase ? inv : p.gamma * inv;
-        float *g = p.grad + (size_t)wave_id * p.max_length;
-        for (int j = ft; j < p.Nw; j += TPF) {
-            const int pos = k * p.Hs + j;
-            if (pos < length) atomicAdd(&g[pos], scale * z[fl][j].x * p.window[j]);
+    const float scale = phase ? inv : p.gamma * inv;
+    float err = 0.0f, err_ph = 0.0f;
+
+    // windowed samples of frame k, source in x and target in y; zero outside the window, the waveform and Kvalid
+    auto fetch = [&](const int k, float2 (&v)[EPT]) {
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) {
+            const int j = ft + e * TPF, pos = k * Hs + j;
+            v[e] = make_float2(0.0f, 0.0f);
+            if (k < Kvalid && j < Nw && pos < length) {
+                const float w = win[j];
+                v[e] = make_float2(src[pos] * w, tgt[pos] * w);
+            }
         }
+    };
+
+    int k0 = blockIdx.x * FPB;  // first frame of the pass; the same for every thread, so the barriers are uniform
+    if (k0 >= Kvalid) return;
+    for (int i = tid; i < N; i += 256) tw[i] = p.twiddle[res][i];
+    float2 cur[EPT];
+    fetch(k0 + fl, cur);
+    for (; k0 < Kvalid; k0 += kstep) {
+        const int k = k0 + fl;
+        const bool active = k < Kvalid;
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) zf[ft + e * TPF] = cur[e];
+        __syncthreads();
+        // the next pass's samples travel while this pass computes
+        if (k0 + kstep < Kvalid) fetch(k + kstep, cur);
+
+        // forward: decimation in frequency
+#pragma unroll 1
+        for (int s = LOGN - 1; s >= 0; --s) {
+            const int half = 1 << s;
+            for (int i = ft; i < HALF; i += TPF) {
+                const int pos = i & (half - 1);
+                const int a = ((i >> s) << (s + 1)) + pos, b = a + half;
+                const float2 u = zf[a], v = zf[b];
+                const float2 w = tw[half + pos];
+                const float dx = u.x - v.x, dy = u.y - v.y;
+                zf[a] = make_float2(u.x + v.x, u.y + v.y);
+                zf[b] = make_float2(dx * w.x - dy * w.y, dx * w.y + dy * w.x);
+            }
+            __syncthreads();
+        }
+
+        // per-bin stage on the pairs (b, N-b); bin b lives at position bitrev(b)
+        // With the phase term both gradient spectra are weighted here and share the inverse transform (the
+        // reference runs a second framing / FFT / inverse FFT / overlap-add for it,
+        // layers/DFTErrorPostoutputLayer.cu:1246-1295).
+        // Stored position q holds bin bitrev(q).  Thread index t walks the even positions 2t (bins below N/2) and
+        // pairs each with the position of bin N - b, which for a wave's consecutive t are consecutive words too;
+        // walking the bins in natural order instead puts a wave's reads into two LDS banks.  Bins 0 (position 0)
+        // and N/2 (position 1) pair with themselves.
+        auto bin = [&](const int pb, const int pnb) {
+            const float2 zb = zf[pb], zn = zf[pnb];
+            // S = (Z[b] + conj(Z[N-b])) / 2,  T = (Z[b] - conj(Z[N-b])) / (2i)
+            const float sx = 0.5f * (zb.x + zn.x), sy = 0.5f * (zb.y - zn.y);
+            const float tx = 0.5f * (zb.y + zn.y), ty = -0.5f * (zb.x - zn.x);
+            float e, gx, gy;
+            bin_distance<DIS>(sx, sy, tx, ty, p.log_floor, e, gx, gy);
+            if (active) err += e;
+            if (phase) {
+                float pe, px, py;
+                bin_phase(sx, sy, tx, ty, pe, px, py);
+                if (active) err_ph += pe;
+                gx = p.gamma * gx + p.zeta * px;
+                gy = p.gamma * gy + p.zeta * py;
+            }
+            if (pb == pnb) {
+                zf[pb] = make_float2(gx, 0.0f);
+            } else {
+                zf[pb] = make_float2(gx, gy);
+                zf[pnb] = make_float2(gx, -gy);
+            }
+        };
+        for (int t = ft; t < HALF; t += TPF) {
+            const int b = (int)(__brev((unsigned)(2 * t)) >> (32 - LOGN));
+            const int pnb = (int)(__brev((unsigned)((N - b) & (N - 1))) >> (32 - LOGN));
+            bin(2 * t, pnb);
+        }
+        if (ft == 0) bin(1, 1);
+        __syncthreads();
+
+        // inverse: decimation in time with conjugated twiddles, unnormalised
+#pragma unroll 1
+        for (int s = 0; s < LOGN; ++s) {
+            const int half = 1 << s;
+            for (int i = ft; i < HALF; i += TPF) {
+                const int pos = i & (half - 1);
+                const int a = ((i >> s) << (s + 1)) + pos, b = a + half;
+                const float2 u = zf[a], x = zf[b];
+                const float2 w = tw[half + pos];
+                const float vx = x.x * w.x + x.y * w.y, vy = x.y * w.x - x.x * w.y;
+                zf[a] = make_float2(u.x + vx, u.y + vy);
+                zf[b] = make_float2(u.x - vx, u.y - vy);
+            }
+            __syncthreads();
+        }
+
+        // windowed overlap-add; frames at or beyond Kvalid contribute nothing
+        if (active) {
+            for (int j = ft; j < Nw; j += TPF) {
+                const int pos = k * Hs + j;
+                if (pos < length) atomicAdd(&g[pos], scale * zf[j].x * win[j]);
+            }
+        }
+        __syncthreads();  // the next pass overwrites the frame storage
     }
+
     for (int o = 32; o > 0; o >>= 1) {
         err += __shfl_xor(err, o);
         err_ph += __shfl_xor(err_ph, o);
@@ -240,7 +277,28 @@ __global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
     __syncthreads();
     if (tid < 2 && (tid == 0 || phase)) {
         const float e = (err_part[tid][0] + err_part[tid][1] + err_part[tid][2] + err_part[tid][3]) * inv;
-        if (e != 0.0f) atomicAdd(&p.errors[tid * p.n_waves * p.n_res + wave_id * p.n_res + p.res], e);
+        if (e != 0.0f) atomicAdd(&p.errors[tid * p.n_waves * p.n_res + wave_id * p.n_res + res], e);
+    }
+}
+
+// All resolutions of a call in one launch: blockIdx.z selects the resolution, blockIdx.x the group of frames
+// (blocks beyond a resolution's last frame leave at once), blockIdx.y the waveform.
+template <int DIS>
+__global__ __launch_bounds__(256) void dft_loss_kernel(const DftParams p) {
+    // sized by the launch for the call's longest transform; every instantiation places its tables at fixed offsets
+    extern __shared__ __attribute__((aligned(16))) float2 dft_lds[];
+    __shared__ float err_part[2][4];
+    const int res = blockIdx.z;
+    if ((int)blockIdx.x >= p.nblocks[res]) return;
+    switch (p.logn[res]) {
+        case 5: dft_frames<5, DIS>(p, res, dft_lds, err_part); break;
+        case 6: dft_frames<6, DIS>(p, res, dft_lds, err_part); break;
+        case 7: dft_frames<7, DIS>(p, res, dft_lds, err_part); break;
+        case 8: dft_frames<8, DIS>(p, res, dft_lds, err_part); break;
+        case 9: dft_frames<9, DIS>(p, res, dft_lds, err_part); break;
+        case 10: dft_frames<10, DIS>(p, res, dft_lds, err_part); break;
+        case 11: dft_frames<11, DIS>(p, res, dft_lds, err_part); break;
+        default: dft_frames<12, DIS>(p, res, dft_lds, err_part); break;
     }
 }
 
@@ -255,29 +313,15 @@ __global__ void dft_backward_kernel(int max_length, int n_waves, DftParams p, fl
 }
 
 typedef void (*dft_kernel_t)(const DftParams);
-template <int DIS>
-dft_kernel_t pick_dft_length(int logn) {
-    switch (logn) {
-        case 5: return dft_loss_kernel<5, DIS>;
-        case 6: return dft_loss_kernel<6, DIS>;
-        case 7: return dft_loss_kernel<7, DIS>;
-        case 8: return dft_loss_kernel<8, DIS>;
-        case 9: return dft_loss_kernel<9, DIS>;
-        case 10: return dft_loss_kernel<10, DIS>;
-        case 11: return dft_loss_kernel<11, DIS>;
-        case 12: return dft_loss_kernel<12, DIS>;
-        default: return nullptr;
-    }
-}
-dft_kernel_t pick_dft_kernel(int logn, int dis_type) {
+dft_kernel_t pick_dft_kernel(int dis_type) {
     switch (dis_type) {
-        case 0: return pick_dft_length<0>(logn);
-        case 1: return pick_dft_length<1>(logn);
-        case 2: return pick_dft_length<2>(logn);
-        case 3: return pick_dft_length<3>(logn);
-        case 4: return pick_dft_length<4>(logn);
-        case 5: return pick_dft_length<5>(logn);
-        case 6: return pick_dft_length<6>(logn);
+        case 0: return dft_loss_kernel<0>;
+        case 1: return dft_loss_kernel<1>;
+        case 2: return dft_loss_kernel<2>;
+        case 3: return dft_loss_kernel<3>;
+        case 4: return dft_loss_kernel<4>;
+        case 5: return dft_loss_kernel<5>;
+        case 6: return dft_loss_kernel<6>;
         default: return nullptr;
     }
 }
@@ -331,18 +375,20 @@ int cnt_dft_create(const cnt_dft_desc *desc, cnt_dft **out) {
         const int N = desc->fft_length[r], Nw = desc->frame_length[r], Hs = desc->frame_shift[r];
         int logn = 0;
         while ((1 << logn) < N) ++logn;
-        if ((1 << logn) != N || !pick_dft_kernel(logn, 0) || Nw < 2 || Nw > N || Hs < 1) {
+        if ((1 << logn) != N || logn < 5 || logn > kMaxLogN || Nw < 2 || Nw > N || Hs < 1) {
             set_error("dft_create: resolution %d has fftLength %d, frameLength %d, frameShift %d; supported: fftLength a "
                       "power of two in 32..4096, 2 <= frameLength <= fftLength, frameShift >= 1", r, N, Nw, Hs);
             cnt_dft_destroy(h);
             return CNT_ERR_ARG;
         }
         h->logn[r] = logn;
-        std::vector<float2> tw((size_t)N / 2);
-        for (int k2 = 0; k2 < N / 2; ++k2) {
-            const double a = -2.0 * 3.14159265358979323846 * k2 / N;
-            tw[(size_t)k2] = make_float2((float)std::cos(a), (float)std::sin(a));
-        }
+        // one run of twiddles per butterfly stage, so that a stage reads consecutive LDS words
+        std::vector<float2> tw((size_t)N, make_float2(1.0f, 0.0f));
+        for (int half = 1; half < N; half *= 2)
+            for (int k2 = 0; k2 < half; ++k2) {
+                const double a = -3.14159265358979323846 * k2 / half;
+                tw[(size_t)(half + k2)] = make_float2((float)std::cos(a), (float)std::sin(a));
+            }
         std::vector<float> win((size_t)Nw);
         for (int j = 0; j < Nw; ++j)
             win[(size_t)j] = desc->window_type[r] == 1 ? 1.0f
@@ -354,6 +400,11 @@ int cnt_dft_create(const cnt_dft_desc *desc, cnt_dft **out) {
     }
     if (err == hipSuccess)
         err = hipMalloc(reinterpret_cast<void **>(&h->grad), (size_t)desc->max_waves * desc->max_length * sizeof(float));
+    // a 4096-point transform takes 64 KB of LDS for its frame and twiddles, beyond what a launch may ask for unannounced
+    for (int r = 0; r < desc->n_res && err == hipSuccess; ++r)
+        if (desc->fft_length[r] > 2048)
+            err = hipFuncSetAttribute(reinterpret_cast<const void *>(pick_dft_kernel(desc->spec_dis_type)),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 4096 * (int)sizeof(float2));
     if (err != hipSuccess) {
         set_error("dft_create: %s", hipGetErrorString(err));
         cnt_dft_destroy(h);
@@ -373,6 +424,13 @@ static void fill_params(const cnt_dft *h, cnt::DftParams &p) {
     p.log_floor = h->desc.log_floor;
     p.zeta = h->desc.zeta;
     p.grad = h->grad;
+    for (int r = 0; r < h->desc.n_res; ++r) {
+        p.logn[r] = h->logn[r];
+        p.Nw[r] = h->desc.frame_length[r];
+        p.Hs[r] = h->desc.frame_shift[r];
+        p.twiddle[r] = h->twiddle[r];
+        p.window[r] = h->window[r];
+    }
 }
 
 int cnt_dft_forward(cnt_dft *h, void *stream_, int n_waves, const int *lengths, const float *source,
@@ -391,19 +449,42 @@ int cnt_dft_forward(cnt_dft *h, void *stream_, int n_waves, const int *lengths, 
     CNT_TRY(fill_zero(stream, errors_dev, (size_t)n_waves * h->desc.n_res * (h->desc.zeta > 0.0f ? 2 : 1)));
     int max_len = 0;
     for (int w = 0; w < n_waves; ++w) max_len = lengths[w] > max_len ? lengths[w] : max_len;
+    DftParams p;
+    fill_params(h, p);
+    p.source = source; p.target = target; p.errors = errors_dev;
+    // A block of a short transform makes several passes over its waveform's frames, so that the blocks of all
+    // resolutions carry about the work of one pass of the longest transform (butterflies per pass: N/2 * log2 N
+    // per frame, 256 / (N/2) frames per pass below N = 512).
+    static const int max_passes = [] {
+        const char *e = getenv("CNT_DFT_PASSES");
+        const int v = e ? atoi(e) : 8;
+        return v < 1 ? 1 : v;
+    }();
+    int gx = 1;
+    long work_max = 1;
+    size_t lds_bytes = 0;
     for (int r = 0; r < h->desc.n_res; ++r) {
-        DftParams p;
-        fill_params(h, p);
-        p.N = h->desc.fft_length[r]; p.Nw = h->desc.frame_length[r]; p.Hs = h->desc.frame_shift[r];
-        p.res = r;
-        p.twiddle = h->twiddle[r]; p.window = h->window[r];
-        p.source = source; p.target = target; p.errors = errors_dev;
-        const int half = p.N / 2;
+        const long n = h->desc.fft_length[r];
+        const long w = (n < 512 ? 512 : n) * p.logn[r];
+        work_max = w > work_max ? w : work_max;
+        const size_t b = (size_t)((n < 512 ? 512 : n) + n) * sizeof(float2);
+        lds_bytes = b > lds_bytes ? b : lds_bytes;
+    }
+    for (int r = 0; r < h->desc.n_res; ++r) {
+        const long n = h->desc.fft_length[r];
+        const int half = (int)(n / 2);
         const int fpb = half < 256 ? 256 / half : 1;
-        const int kmax = frame_count(max_len, p.Nw, p.Hs);
-        dim3 grid((kmax + fpb - 1) / fpb, n_waves);
+        const int kmax = frame_count(max_len, p.Nw[r], p.Hs[r]);
+        long passes = work_max / ((n < 512 ? 512 : n) * p.logn[r]);
+        passes = passes < 1 ? 1 : passes > max_passes ? max_passes : passes;
+        const int groups = (kmax + fpb - 1) / fpb;
+        p.nblocks[r] = (int)((groups + passes - 1) / passes);
+        gx = p.nblocks[r] > gx ? p.nblocks[r] : gx;
+    }
+    {
         ProfileScope prof(stream, "dft_loss");
-        hipLaunchKernelGGL(pick_dft_kernel(h->logn[r], h->desc.spec_dis_type), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL(pick_dft_kernel(h->desc.spec_dis_type), dim3(gx, n_waves, h->desc.n_res), dim3(256), lds_bytes, stream,
+                           p);
         CNT_HIP(hipGetLastError());
     }
     return CNT_OK;
