@@ -1,5 +1,5 @@
 // Multi-resolution STFT spectral loss (seven amplitude / spectrum distances) and its gradient for gfx950, with
-// an in-house radix-2 FFT.
+// an in-house radix-4 FFT.
 //
 // Reference behaviour: helpers/FFTMat.cu (FrameSignal :282-312, distances :473-628, gradients :760-900,
 // cleanDummyGradients :456-471, collectGrad :965-1006, drivers :1246-1274, :1350-1475, :1637-1770,
@@ -7,17 +7,21 @@
 // runs about a dozen launches and three cuFFT calls per resolution and waveform, with every intermediate
 // (framed signals, spectra, per-bin differences, framed gradients) in device memory.
 //
-// Here one workgroup owns one frame end to end, all resolutions of a call are one launch, and nothing but the
-// waveforms and the gradient touches HBM:
+// Here a frame stays in one workgroup's LDS end to end, all resolutions of a call are one launch, and nothing
+// but the waveforms and the gradient touches HBM:
 //   frame + window source and target  ->  ONE complex FFT of z = source + i*target in LDS (both real
-//   spectra are recovered from Z[b] and Z[N-b])  ->  per-bin log-amplitude difference, loss partial and
-//   gradient spectrum, written back as its Hermitian extension  ->  inverse FFT in LDS  ->  windowed
-//   overlap-add straight into the per-sample gradient with float atomics.
+//   spectra are recovered from Z[b] and Z[N-b])  ->  per-bin distance, loss partial and gradient spectrum,
+//   written back as its Hermitian extension  ->  inverse FFT in LDS  ->  windowed overlap-add straight into
+//   the per-sample gradient with float atomics.
+// A workgroup makes several such passes (short transforms more than long ones, so that the workgroups of all
+// resolutions carry similar work), loads its twiddles once, fetches the next pass's samples while it computes,
+// and adds its loss partial to the per-waveform sums once at its end.
 // The forward transform is decimation-in-frequency (natural order in, bit-reversed out), the per-bin stage
 // addresses bins through the bit-reversal, and the inverse is decimation-in-time (bit-reversed in, natural
-// out), so no reordering pass exists.  Twiddles and the window (with the reference's constant 3.141215) are
-// tabulated in double on the host.  Transform conventions are cuFFT's: unnormalised, N/2+1 bins, the
-// imaginary parts of the DC and Nyquist bins do not enter the inverse.
+// out), so no reordering pass exists; two butterfly stages share a barrier as one radix-4 butterfly.  Twiddles
+// (one run per stage, so that a stage reads consecutive LDS words) and the window (with the reference's
+// constant 3.141215) are tabulated in double on the host.  Transform conventions are cuFFT's: unnormalised,
+// N/2+1 bins, the imaginary parts of the DC and Nyquist bins do not enter the inverse.
 #include "common.hpp"
 
 #include <cmath>
@@ -128,17 +132,18 @@ __device__ inline void bin_phase(float sx, float sy, float tx, float ty, float &
 
 constexpr int kMaxLogN = 12;
 
-// One block = passes of FPB frames of resolution `res` of one waveform.  lds: max(512, N) + N complex words.
+// One block = passes of FPB frames of resolution `res` of one waveform.  lds: max(1024, N) + N complex words.
 template <int LOGN, int DIS>
 __device__ __forceinline__ void dft_frames(const DftParams &p, const int res, float2 *__restrict__ lds,
                                            float (*err_part)[4]) {
     constexpr int N = 1 << LOGN;
-    float2 *__restrict__ zbuf = lds;                    // frame storage: FPB * N = max(512, N) complex words
-    float2 *__restrict__ tw = lds + (N > 512 ? N : 512);  // N twiddles
+    float2 *__restrict__ zbuf = lds;                      // frame storage: FPB * N = max(1024, N) complex words
+    float2 *__restrict__ tw = lds + (N > 1024 ? N : 1024);  // N twiddles
     constexpr int HALF = N / 2;
-    constexpr int TPF = HALF < 256 ? HALF : 256;  // threads per frame
-    constexpr int FPB = 256 / TPF;                // frames per block
-    static_assert(FPB * N <= (N > 512 ? N : 512), "frame storage: max(512, N) complex words");
+    constexpr int QUARTER = N / 4;
+    constexpr int TPF = QUARTER < 256 ? QUARTER : 256;  // threads per frame: one per radix-4 butterfly up to N = 1024
+    constexpr int FPB = 256 / TPF;                      // frames per block
+    static_assert(FPB * N <= (N > 1024 ? N : 1024), "frame storage: max(1024, N) complex words");
 
     constexpr int EPT = N / TPF;  // samples per thread and frame
 
@@ -186,18 +191,33 @@ __device__ __forceinline__ void dft_frames(const DftParams &p, const int res, fl
         // the next pass's samples travel while this pass computes
         if (k0 + kstep < Kvalid) fetch(k + kstep, cur);
 
-        // forward: decimation in frequency
+        // forward: decimation in frequency, two stages (s, s - 1) per barrier as one radix-4 butterfly on the words
+        // base + {0, q, 2q, 3q}, q = 2^(s-1); the twiddle of the second pair of stage s is -i times the first's
 #pragma unroll 1
-        for (int s = LOGN - 1; s >= 0; --s) {
-            const int half = 1 << s;
+        for (int s = LOGN - 1; s >= 1; s -= 2) {
+            const int q = 1 << (s - 1);
+            for (int i = ft; i < QUARTER; i += TPF) {
+                const int j = i & (q - 1);
+                const int base = ((i >> (s - 1)) << (s + 1)) + j;
+                const float2 x0 = zf[base], x1 = zf[base + q], x2 = zf[base + 2 * q], x3 = zf[base + 3 * q];
+                const float2 w1 = tw[2 * q + j], w2 = tw[q + j];
+                const float2 y0 = make_float2(x0.x + x2.x, x0.y + x2.y), d02 = make_float2(x0.x - x2.x, x0.y - x2.y);
+                const float2 y1 = make_float2(x1.x + x3.x, x1.y + x3.y), d13 = make_float2(x1.y - x3.y, x3.x - x1.x);
+                const float2 y2 = make_float2(d02.x * w1.x - d02.y * w1.y, d02.x * w1.y + d02.y * w1.x);
+                const float2 y3 = make_float2(d13.x * w1.x - d13.y * w1.y, d13.x * w1.y + d13.y * w1.x);
+                const float2 e01 = make_float2(y0.x - y1.x, y0.y - y1.y), e23 = make_float2(y2.x - y3.x, y2.y - y3.y);
+                zf[base] = make_float2(y0.x + y1.x, y0.y + y1.y);
+                zf[base + q] = make_float2(e01.x * w2.x - e01.y * w2.y, e01.x * w2.y + e01.y * w2.x);
+                zf[base + 2 * q] = make_float2(y2.x + y3.x, y2.y + y3.y);
+                zf[base + 3 * q] = make_float2(e23.x * w2.x - e23.y * w2.y, e23.x * w2.y + e23.y * w2.x);
+            }
+            __syncthreads();
+        }
+        if (LOGN & 1) {  // the last stage on its own: neighbours, twiddle 1
             for (int i = ft; i < HALF; i += TPF) {
-                const int pos = i & (half - 1);
-                const int a = ((i >> s) << (s + 1)) + pos, b = a + half;
-                const float2 u = zf[a], v = zf[b];
-                const float2 w = tw[half + pos];
-                const float dx = u.x - v.x, dy = u.y - v.y;
-                zf[a] = make_float2(u.x + v.x, u.y + v.y);
-                zf[b] = make_float2(dx * w.x - dy * w.y, dx * w.y + dy * w.x);
+                const float2 u = zf[2 * i], v = zf[2 * i + 1];
+                zf[2 * i] = make_float2(u.x + v.x, u.y + v.y);
+                zf[2 * i + 1] = make_float2(u.x - v.x, u.y - v.y);
             }
             __syncthreads();
         }
@@ -240,18 +260,34 @@ __device__ __forceinline__ void dft_frames(const DftParams &p, const int res, fl
         if (ft == 0) bin(1, 1);
         __syncthreads();
 
-        // inverse: decimation in time with conjugated twiddles, unnormalised
-#pragma unroll 1
-        for (int s = 0; s < LOGN; ++s) {
-            const int half = 1 << s;
+        // inverse: decimation in time with conjugated twiddles, unnormalised; stages (s - 1, s) per barrier
+        if (LOGN & 1) {
             for (int i = ft; i < HALF; i += TPF) {
-                const int pos = i & (half - 1);
-                const int a = ((i >> s) << (s + 1)) + pos, b = a + half;
-                const float2 u = zf[a], x = zf[b];
-                const float2 w = tw[half + pos];
-                const float vx = x.x * w.x + x.y * w.y, vy = x.y * w.x - x.x * w.y;
-                zf[a] = make_float2(u.x + vx, u.y + vy);
-                zf[b] = make_float2(u.x - vx, u.y - vy);
+                const float2 u = zf[2 * i], v = zf[2 * i + 1];
+                zf[2 * i] = make_float2(u.x + v.x, u.y + v.y);
+                zf[2 * i + 1] = make_float2(u.x - v.x, u.y - v.y);
+            }
+            __syncthreads();
+        }
+#pragma unroll 1
+        for (int s = 1 + (LOGN & 1); s < LOGN; s += 2) {
+            const int q = 1 << (s - 1);
+            for (int i = ft; i < QUARTER; i += TPF) {
+                const int j = i & (q - 1);
+                const int base = ((i >> (s - 1)) << (s + 1)) + j;
+                const float2 x0 = zf[base], x1 = zf[base + q], x2 = zf[base + 2 * q], x3 = zf[base + 3 * q];
+                const float2 w1 = tw[2 * q + j], w2 = tw[q + j];
+                const float2 v1 = make_float2(x1.x * w2.x + x1.y * w2.y, x1.y * w2.x - x1.x * w2.y);
+                const float2 v3 = make_float2(x3.x * w2.x + x3.y * w2.y, x3.y * w2.x - x3.x * w2.y);
+                const float2 y0 = make_float2(x0.x + v1.x, x0.y + v1.y), y1 = make_float2(x0.x - v1.x, x0.y - v1.y);
+                const float2 y2 = make_float2(x2.x + v3.x, x2.y + v3.y), y3 = make_float2(x2.x - v3.x, x2.y - v3.y);
+                const float2 u2 = make_float2(y2.x * w1.x + y2.y * w1.y, y2.y * w1.x - y2.x * w1.y);
+                const float2 t3 = make_float2(y3.x * w1.x + y3.y * w1.y, y3.y * w1.x - y3.x * w1.y);
+                const float2 u3 = make_float2(-t3.y, t3.x);  // conj(-i * w1) = i * conj(w1)
+                zf[base] = make_float2(y0.x + u2.x, y0.y + u2.y);
+                zf[base + q] = make_float2(y1.x + u3.x, y1.y + u3.y);
+                zf[base + 2 * q] = make_float2(y0.x - u2.x, y0.y - u2.y);
+                zf[base + 3 * q] = make_float2(y1.x - u3.x, y1.y - u3.y);
             }
             __syncthreads();
         }
@@ -453,29 +489,25 @@ int cnt_dft_forward(cnt_dft *h, void *stream_, int n_waves, const int *lengths, 
     fill_params(h, p);
     p.source = source; p.target = target; p.errors = errors_dev;
     // A block of a short transform makes several passes over its waveform's frames, so that the blocks of all
-    // resolutions carry about the work of one pass of the longest transform (butterflies per pass: N/2 * log2 N
-    // per frame, 256 / (N/2) frames per pass below N = 512).
-    static const int max_passes = [] {
-        const char *e = getenv("CNT_DFT_PASSES");
-        const int v = e ? atoi(e) : 8;
-        return v < 1 ? 1 : v;
-    }();
+    // resolutions carry about the work of one pass of the longest transform (work per pass: N * log2 N per frame,
+    // 256 / (N/4) frames per pass below N = 1024).
+    const long max_passes = 8;
     int gx = 1;
     long work_max = 1;
     size_t lds_bytes = 0;
     for (int r = 0; r < h->desc.n_res; ++r) {
         const long n = h->desc.fft_length[r];
-        const long w = (n < 512 ? 512 : n) * p.logn[r];
+        const long w = (n < 1024 ? 1024 : n) * p.logn[r];
         work_max = w > work_max ? w : work_max;
-        const size_t b = (size_t)((n < 512 ? 512 : n) + n) * sizeof(float2);
+        const size_t b = (size_t)((n < 1024 ? 1024 : n) + n) * sizeof(float2);
         lds_bytes = b > lds_bytes ? b : lds_bytes;
     }
     for (int r = 0; r < h->desc.n_res; ++r) {
         const long n = h->desc.fft_length[r];
-        const int half = (int)(n / 2);
-        const int fpb = half < 256 ? 256 / half : 1;
+        const int quarter = (int)(n / 4);
+        const int fpb = quarter < 256 ? 256 / quarter : 1;
         const int kmax = frame_count(max_len, p.Nw[r], p.Hs[r]);
-        long passes = work_max / ((n < 512 ? 512 : n) * p.logn[r]);
+        long passes = work_max / ((n < 1024 ? 1024 : n) * p.logn[r]);
         passes = passes < 1 ? 1 : passes > max_passes ? max_passes : passes;
         const int groups = (kmax + fpb - 1) / fpb;
         p.nblocks[r] = (int)((groups + passes - 1) / passes);
