@@ -157,6 +157,8 @@ int gemm_simple(hipStream_t stream, float *C, int m, int n, int k, const float *
 
 // ----- small streaming kernels (elementwise.hip) ----------------------------------------------------
 int fill_zero(hipStream_t stream, float *p, size_t count);
+// two buffers in one launch
+int fill_zero_pair(hipStream_t stream, float *p, size_t count, float *q, size_t count_q);
 int fill_words(hipStream_t stream, unsigned *p, size_t count, unsigned word);
 // out[d] += scale * sum over the N columns of a D x N column-major matrix (out pre-zeroed by the caller)
 int column_sum(hipStream_t stream, const float *v, int D, int N, float scale, float *out);

@@ -481,8 +481,8 @@ int cnt_dft_forward(cnt_dft *h, void *stream_, int n_waves, const int *lengths, 
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     h->n_waves = n_waves;
     for (int w = 0; w < n_waves; ++w) h->lengths[w] = lengths[w];
-    CNT_TRY(fill_zero(stream, h->grad, (size_t)n_waves * h->desc.max_length));
-    CNT_TRY(fill_zero(stream, errors_dev, (size_t)n_waves * h->desc.n_res * (h->desc.zeta > 0.0f ? 2 : 1)));
+    CNT_TRY(fill_zero_pair(stream, h->grad, (size_t)n_waves * h->desc.max_length, errors_dev,
+                           (size_t)n_waves * h->desc.n_res * (h->desc.zeta > 0.0f ? 2 : 1)));
     int max_len = 0;
     for (int w = 0; w < n_waves; ++w) max_len = lengths[w] > max_len ? lengths[w] : max_len;
     DftParams p;

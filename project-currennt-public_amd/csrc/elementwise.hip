@@ -15,6 +15,15 @@ __global__ void fill_zero_kernel(float *__restrict__ p, size_t count) {
     for (; i < count; i += stride) p[i] = 0.0f;
 }
 
+__global__ void fill_zero_pair_kernel(float *__restrict__ p, size_t count, float *__restrict__ q, size_t count_q) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < count + count_q; i += stride) {
+        if (i < count) p[i] = 0.0f;
+        else q[i - count] = 0.0f;
+    }
+}
+
 __global__ void fill_words_kernel(unsigned *__restrict__ p, size_t count, unsigned word) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -91,6 +100,14 @@ inline int stream_blocks(size_t count) {
 int fill_zero(hipStream_t stream, float *p, size_t count) {
     if (count == 0) return CNT_OK;
     hipLaunchKernelGGL(fill_zero_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, p, count);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+int fill_zero_pair(hipStream_t stream, float *p, size_t count, float *q, size_t count_q) {
+    if (count + count_q == 0) return CNT_OK;
+    hipLaunchKernelGGL(fill_zero_pair_kernel, dim3(stream_blocks(count + count_q)), dim3(256), 0, stream, p, count, q,
+                       count_q);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
