@@ -1256,14 +1256,39 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     using namespace cnt;
     CNT_REQUIRE(net && net->T > 0, "network_backward: no fraction loaded");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    hipStream_t wstream = stream;
     int next_side = 0;
     bool side_used[cnt_network::kMaxSide] = {};
+
+    // The weight half of a layer's backward pass has no consumer before the optimizer, so it runs on a side stream
+    // after the layer's error half.  Handing work to another stream costs the host two event calls; a network of
+    // many small layers cannot afford them per layer (the host's enqueue rate then bounds its backward pass), so the
+    // weight halves of small layers are collected and handed over a few at a time, those of large layers at once.
+    std::vector<size_t> pending;
+    auto weight_half = [&](size_t i, hipStream_t ws) -> int {
+        NetLayer &L = net->layers[i];
+        NetLayer &prev = net->layers[i - 1];
+        float *dW = net->updates + L.w_off;
+        if (L.kind == K_DENSE)
+            return cnt_dense_backward_weights(ws, prev.size, L.size, L.N, L.bias, prev.out, L.err, dW);
+        if (L.kind == K_LSTM) return cnt_lstm_backward_weights(L.lstm, ws, prev.out, dW);
+        if (L.kind == K_CNN) return cnt_cnn_backward_weights(L.cnn, ws, L.pat, L.T, prev.out, L.err, dW);
+        return cnt_wavnetc_backward_weights(ws, L.size, L.ctx_dim, L.N, net->ctx, L.cth, dW);
+    };
+    auto hand_over = [&]() -> int {
+        if (pending.empty()) return CNT_OK;
+        hipStream_t ws = net->side[next_side];
+        CNT_HIP(hipEventRecord(net->ev_main, stream));
+        CNT_HIP(hipStreamWaitEvent(ws, net->ev_main, 0));
+        side_used[next_side] = true;
+        next_side = (next_side + 1) % net->n_side;
+        for (size_t i : pending) CNT_TRY(weight_half(i, ws));
+        pending.clear();
+        return CNT_OK;
+    };
     for (size_t i = net->layers.size() - 1; i >= 1; --i) {
         NetLayer &L = net->layers[i];
         NetLayer &prev = net->layers[i - 1];
         const float *W = net->weights + L.w_off;
-        float *dW = net->updates + L.w_off;
         const int N = L.N;
         // the input layer has no error buffer; a feedback layer that takes nothing from its preceding layer passes
         // nothing on, and neither does anything that feeds such a feedback layer's one-hot part
@@ -1314,22 +1339,18 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                     }
                 }
                 if (L.kind == K_WAVNETC && L.ctx_dim == 0) break;
-                // the weight half has no consumer before the optimizer: second stream, after the error half
-                if (net->overlap) {
-                    wstream = net->side[next_side];
-                    CNT_HIP(hipEventRecord(net->ev_main, stream));
-                    CNT_HIP(hipStreamWaitEvent(wstream, net->ev_main, 0));
-                    side_used[next_side] = true;
-                    next_side = (next_side + 1) % net->n_side;
+                if (!net->overlap) {
+                    CNT_TRY(weight_half(i, stream));
+                    break;
                 }
-                if (L.kind == K_DENSE)
-                    CNT_TRY(cnt_dense_backward_weights(wstream, prev.size, L.size, N, L.bias, prev.out, L.err, dW));
-                else if (L.kind == K_LSTM)
-                    CNT_TRY(cnt_lstm_backward_weights(L.lstm, wstream, prev.out, dW));
-                else if (L.kind == K_CNN)
-                    CNT_TRY(cnt_cnn_backward_weights(L.cnn, wstream, L.pat, L.T, prev.out, L.err, dW));
-                else
-                    CNT_TRY(cnt_wavnetc_backward_weights(wstream, L.size, L.ctx_dim, N, net->ctx, L.cth, dW));
+                pending.push_back(i);
+                {
+                    // small: below 4e8 multiply-adds (a WaveNet block's 64..128-wide layers over 32 000 samples are
+                    // 1.6-2.6e8, the acoustic model's dense layers over 5 880 frames 5.6e8 and more); four at a time
+                    // measured best on the 30-block WaveNet stack (5.36 -> 5.23 ms; two: no gain, eight: 5.31 ms)
+                    const double macs = (double)prev.size * L.size * N;
+                    if (L.kind == K_LSTM || macs >= 4e8 || pending.size() >= 4) CNT_TRY(hand_over());
+                }
                 break;
             case K_SKIPINI:
             case K_SKIPADD: {
@@ -1376,6 +1397,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 break;
         }
     }
+    CNT_TRY(hand_over());
     for (int k = 0; k < net->n_side; ++k) {
         if (!side_used[k]) continue;
         CNT_HIP(hipEventRecord(net->ev_side[k], net->side[k]));
