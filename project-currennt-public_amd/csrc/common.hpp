@@ -118,7 +118,9 @@ enum GemmEpilogue {
     EPI_ATOMIC = 2,         // atomicAdd(C, acc)   (split-K; C zeroed by the caller)
     EPI_BIAS_ACT = 3,       // C = act(acc + bias_scale * bias_vec[row])
     EPI_BIAS_ACT_SKIP = 4,  // as above, but columns whose pattern type is "none" are left untouched
-    EPI_CONTEXT = 5         // th = tanh(acc); aux_out = th; C = aux_in + th; both 0 on "none" columns
+    EPI_CONTEXT = 5,        // th = tanh(acc); aux_out = th; C = aux_in + th; both 0 on "none" columns
+    EPI_PARTIAL = 6         // split-K without atomics: every split stores its m x n partial product into the
+                            // launcher's scratch, and a second kernel sums the splits into C (set by gemm_plan)
 };
 
 struct GemmProblem {
@@ -147,8 +149,21 @@ struct GemmArgs {
     const char *pat;  // masked mode and the *_SKIP / CONTEXT epilogues
     GemmProblem prob[kGemmMaxProb];
     const char *label;  // name under which the launch is timed when profiling is on (may be NULL)
+    // Split-K products with a small output (EPI_ATOMIC, splitk = 0): `overwrite_ok` allows gemm_plan to choose
+    // EPI_PARTIAL, which overwrites C instead of adding to a cleared C.  With `rowsum_out` (one problem, one operand
+    // pair, unmasked) the same pass also sums the B operand over k: rowsum_out[j] = rowsum_scale * sum_k B(j, k),
+    // the bias gradient of a dense layer, for which the atomic path needs a separate column-sum launch.
+    int overwrite_ok;
+    float *rowsum_out;
+    float rowsum_scale;
+    float *partial;        // set by the launcher: scratch of splitk * partial_stride floats
+    size_t partial_stride;  // floats per split: nprob * m * n (+ n with rowsum_out)
 };
 
+// Resolves splitk = 0 (chosen by the launcher) and, where the arguments allow it and it pays, switches an
+// EPI_ATOMIC product to EPI_PARTIAL.  A caller that needs to know whether C must be cleared first calls this
+// before gemm_launch and looks at args.epilogue; gemm_launch calls it for everyone else.
+void gemm_plan(GemmArgs &args);
 int gemm_launch(hipStream_t stream, const GemmArgs &args);
 
 // Convenience: single problem, BLAS-like transposes on column-major matrices.

@@ -185,19 +185,24 @@ int cnt_dense_backward_weights(void *stream_, int P, int D, int N, float bias, c
     CNT_REQUIRE(x && err && weight_updates, "dense_backward_weights: null argument");
     CNT_REQUIRE(P > 0 && D > 0 && N > 0, "dense_backward_weights: non-positive size");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    GemmArgs ga = {};
+    ga.m = P; ga.n = D; ga.k = N;
+    ga.a_kcontig = 0; ga.lda = P;
+    ga.b_kcontig = 0; ga.ldb = D;
+    ga.ldc = P;
+    ga.nseg = 1; ga.nprob = 1; ga.epilogue = EPI_ATOMIC;
+    ga.splitk = 0;  // chosen by the launcher
+    ga.prob[0].A[0] = x; ga.prob[0].B[0] = err; ga.prob[0].C = weight_updates;
+    ga.label = "gemm:dense_dW";
+    // narrow layers: the launcher sums partial products instead of adding atomically, which overwrites the
+    // weight part and brings the bias part (row sums of the errors) along
+    ga.overwrite_ok = 1;
+    ga.rowsum_out = weight_updates + (size_t)P * D;
+    ga.rowsum_scale = bias;
+    gemm_plan(ga);
+    if (ga.epilogue == EPI_PARTIAL) return gemm_launch(stream, ga);
     CNT_TRY(fill_zero(stream, weight_updates, (size_t)P * D + D));
-    {
-        GemmArgs ga = {};
-        ga.m = P; ga.n = D; ga.k = N;
-        ga.a_kcontig = 0; ga.lda = P;
-        ga.b_kcontig = 0; ga.ldb = D;
-        ga.ldc = P;
-        ga.nseg = 1; ga.nprob = 1; ga.epilogue = EPI_ATOMIC;
-        ga.splitk = 0;  // chosen by the launcher
-        ga.prob[0].A[0] = x; ga.prob[0].B[0] = err; ga.prob[0].C = weight_updates;
-        ga.label = "gemm:dense_dW";
-        CNT_TRY(gemm_launch(stream, ga));
-    }
+    CNT_TRY(gemm_launch(stream, ga));
     return column_sum(stream, err, D, N, bias, weight_updates + (size_t)P * D);
 }
 

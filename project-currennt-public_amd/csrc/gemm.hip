@@ -18,6 +18,8 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
+#include <vector>
 
 namespace cnt {
 namespace {
@@ -53,7 +55,100 @@ int pick_tile(const GemmArgs &a) {
     return t128 < 2048 ? 64 : 128;
 }
 
+// ----- split-K through partial products ---------------------------------------------------------------------
+// Weight gradients of narrow layers over long inputs (a 64 x 128 output summed over 32 000 slots) need a few
+// hundred splits to fill the machine, and with the atomic epilogue every output element then receives a few
+// hundred atomic adds; atomics to one address serialise, and they, not the loads, set the run time of such a
+// launch.  Here every split stores its partial product with plain stores into a scratch buffer and a second,
+// small kernel sums the splits into C.  That also replaces the clearing launch in front of the atomic path and,
+// for dense layers, the separate column sum for the bias gradient (the splits carry the row sums of B along).
+constexpr size_t kSplitScratchFloats = (size_t)4 << 20;  // 16 MB per (device, stream)
+constexpr long kPartialMaxOutput = 64 << 10;             // floats of output (all problems) up to which it pays
+
+struct SplitScratch {
+    int device;
+    hipStream_t stream;
+    float *buf;
+};
+std::mutex g_split_mu;  // held while a product and its reduction are enqueued, so that they stay adjacent
+std::vector<SplitScratch> g_split_scratch;
+
+// One scratch buffer per stream: launches on a stream execute in order, so the next product on the same stream
+// cannot overwrite partial sums that a reduction has yet to read.  Never freed.
+float *split_scratch(hipStream_t stream) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    for (const SplitScratch &e : g_split_scratch)
+        if (e.device == dev && e.stream == stream) return e.buf;
+    float *buf = nullptr;
+    if (hipMalloc(reinterpret_cast<void **>(&buf), kSplitScratchFloats * sizeof(float)) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    g_split_scratch.push_back({dev, stream, buf});
+    return buf;
+}
+
+// 64 consecutive outputs per block, the splits dealt to four groups of 64 threads whose sums meet in LDS
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs args) {
+    __shared__ float part[4][64];
+    const int tx = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const size_t mn = (size_t)args.m * args.n;
+    const size_t products = mn * args.nprob;
+    const size_t total = products + (args.rowsum_out ? (size_t)args.n : 0);
+    const size_t e = (size_t)blockIdx.x * 64 + tx;
+    float a0 = 0.0f, a1 = 0.0f;
+    if (e < total) {
+        const float *__restrict__ p = args.partial + e;
+        int s = g;
+        for (; s + 4 < args.splitk; s += 8) {
+            a0 += p[(size_t)s * args.partial_stride];
+            a1 += p[(size_t)(s + 4) * args.partial_stride];
+        }
+        if (s < args.splitk) a0 += p[(size_t)s * args.partial_stride];
+    }
+    part[g][tx] = a0 + a1;
+    __syncthreads();
+    if (g == 0 && e < total) {
+        const float v = (part[0][tx] + part[1][tx]) + (part[2][tx] + part[3][tx]);
+        if (e < products) {
+            const size_t z = e / mn, r = e % mn;
+            args.prob[z].C[(r / args.m) * args.ldc + r % args.m] = v;
+        } else {
+            args.rowsum_out[e - products] = args.rowsum_scale * v;
+        }
+    }
+}
+
 }  // namespace
+
+void gemm_plan(GemmArgs &args) {
+    if (args.splitk != 0) return;
+    // Long-K products with a small output (weight gradients): cut K so that the launch has about
+    // `target` workgroups of 64 x 64 tiles, but leave every workgroup at least eight k-iterations -- each
+    // one ends with an atomic add (or a store) of its whole tile, and those, not the products, dominate short
+    // ranges.
+    static const int target = [] { const char *e = std::getenv("CNT_GEMM_SPLIT_TARGET"); return e ? std::atoi(e) : 512; }();
+    const long tiles = (long)((args.m + 63) / 64) * ((args.n + 63) / 64) * args.nprob;
+    const long kt = ((long)args.k + BK - 1) / BK * args.nseg;
+    long s = (target + tiles - 1) / tiles;
+    s = std::min(s, std::max(1L, kt / 8));
+    s = std::max(1L, s);
+    // no empty split: every split of the partial-product path has to write its share
+    while (s > 1 && (s - 1) * ((kt + s - 1) / s) >= kt) --s;
+    args.splitk = (int)s;
+    static const bool partial_on = [] { const char *e = std::getenv("CNT_GEMM_PARTIAL"); return !e || std::atoi(e) != 0; }();
+    const long out = (long)args.m * args.n * args.nprob;
+    const size_t stride = (size_t)out + (args.rowsum_out ? (size_t)args.n : 0);
+    const bool rowsum_ok = !args.rowsum_out || (args.nprob == 1 && args.nseg == 1 && !args.masked);
+    if (partial_on && args.epilogue == EPI_ATOMIC && args.overwrite_ok && rowsum_ok && s >= 8 &&
+        out <= kPartialMaxOutput && stride * (size_t)s <= kSplitScratchFloats) {
+        args.epilogue = EPI_PARTIAL;
+        args.partial_stride = stride;
+    } else {
+        args.rowsum_out = nullptr;  // the caller sums the rows itself
+    }
+}
 
 int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
     GemmArgs args = args_in;
@@ -63,34 +158,38 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
                 args.nseg, kGemmMaxSeg);
     CNT_REQUIRE(args.nprob >= 1 && args.nprob <= kGemmMaxProb, "gemm: %d problems, supported 1..%d",
                 args.nprob, kGemmMaxProb);
-    CNT_REQUIRE(args.splitk >= 0 && (args.splitk == 1 || args.epilogue == EPI_ATOMIC),
+    CNT_REQUIRE(args.splitk >= 0 && (args.splitk == 1 || args.epilogue == EPI_ATOMIC || args.epilogue == EPI_PARTIAL),
                 "gemm: split-K needs the atomic epilogue");
+    CNT_REQUIRE(args.epilogue != EPI_PARTIAL || (args.splitk >= 1 && args.partial_stride > 0),
+                "gemm: the partial-product epilogue is chosen by gemm_plan only");
     for (int p = 0; p < args.nprob; ++p) {
         CNT_REQUIRE(args.prob[p].C != nullptr, "gemm: null output");
         for (int s = 0; s < args.nseg; ++s)
             CNT_REQUIRE(args.prob[p].A[s] && args.prob[p].B[s], "gemm: null operand");
     }
     const int va = pick_vec(args, true), vb = pick_vec(args, false);
-    if (args.splitk == 0) {
-        // Long-K products with a small output (weight gradients): cut K so that the launch has about
-        // `target` workgroups of 64 x 64 tiles, but leave every workgroup at least eight k-iterations -- each
-        // one ends with an atomic add of its whole tile, and those, not the products, dominate short ranges.
-        static const int target = [] { const char *e = std::getenv("CNT_GEMM_SPLIT_TARGET"); return e ? std::atoi(e) : 512; }();
-        const long tiles = (long)((args.m + 63) / 64) * ((args.n + 63) / 64) * args.nprob;
-        const long kt = ((long)args.k + BK - 1) / BK * args.nseg;
-        long s = (target + tiles - 1) / tiles;
-        s = std::min(s, std::max(1L, kt / 8));
-        args.splitk = (int)std::max(1L, s);
-    }
+    gemm_plan(args);
+    if (args.epilogue != EPI_PARTIAL) args.rowsum_out = nullptr;
     const int tile = pick_tile(args);
     const int tiles = ((args.m + tile - 1) / tile) * ((args.n + tile - 1) / tile);
     dim3 grid(tiles, args.splitk, args.nprob);
     ProfileScope prof(stream, args.label ? args.label : "gemm");
+    std::unique_lock<std::mutex> split_lock(g_split_mu, std::defer_lock);
+    if (args.epilogue == EPI_PARTIAL) {
+        split_lock.lock();
+        args.partial = split_scratch(stream);
+        CNT_REQUIRE(args.partial != nullptr, "gemm: no memory for the split-K scratch buffer");
+    }
     if (va == 4) gemm_dispatch_va4(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
     else if (va == 2) gemm_dispatch_va2(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
     else if (args.a_kcontig) gemm_dispatch_va1k(args, grid, stream, vb, args.b_kcontig, tile);
     else gemm_dispatch_va1r(args, grid, stream, vb, args.b_kcontig, tile);
     CNT_HIP(hipGetLastError());
+    if (args.epilogue == EPI_PARTIAL) {
+        const size_t total = args.partial_stride;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, stream, args);
+        CNT_HIP(hipGetLastError());
+    }
     return CNT_OK;
 }
 

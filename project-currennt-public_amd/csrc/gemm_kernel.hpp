@@ -200,6 +200,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
                 args.b_time_on_k != 0);
     };
 
+    // sum of the B operand over this split's k range, per row (dense bias gradient); kept by the waves with wm == 0
+    const bool rowsum = args.rowsum_out != nullptr;
+    float rs[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) rs[j] = 0.0f;
+
     fetch(it_begin, sa0, sb0);
     fetch(min(it_begin + 1, it_end - 1), sa1, sb1);
     sa0.store(lds_a[0], tid);
@@ -233,6 +239,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][kk], fa[i][kk], acc[i][j], 0, 0, 0);
             }
         }
+        if (rowsum) {
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+#pragma unroll
+                for (int kk = 0; kk < FK; ++kk) rs[j] += fb[j][kk];
+        }
 
         if (it + 1 < it_end) {
             held_a.store(lds_a[cur ^ 1], tid);
@@ -248,6 +260,35 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     // epilogue: lane%32 runs along m (contiguous), the 16 accumulators along n
     float *__restrict__ C = pb.C;
     const int half = lane >> 5;
+    if (args.epilogue == EPI_PARTIAL) {
+        // this split's partial product, m x n column-major without padding, after those of the problems before it
+        float *__restrict__ P = args.partial + (size_t)blockIdx.y * args.partial_stride +
+                                (size_t)blockIdx.z * args.m * args.n;
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            const int m = m0 + wm * WT + i * 32 + frag_row;
+            if (m >= args.m) continue;
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int n = n0 + wn * WT + j * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    if (n < args.n) P[(size_t)n * args.m + m] = acc[i][j][r];
+                }
+            }
+        }
+        if (rowsum && wm == 0 && m0 == 0) {
+            float *__restrict__ R = args.partial + (size_t)blockIdx.y * args.partial_stride +
+                                    (size_t)args.nprob * args.m * args.n;
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const float s = rs[j] + __shfl_xor(rs[j], 32);
+                const int n = n0 + wn * WT + j * 32 + frag_row;
+                if (half == 0 && n < args.n) R[n] = s;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
         const int m = m0 + wm * WT + i * 32 + frag_row;

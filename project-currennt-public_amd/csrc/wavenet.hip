@@ -458,7 +458,6 @@ int cnt_wavnetc_backward_weights(void *stream_, int D, int C, int N, const float
     if (C == 0) return CNT_OK;
     CNT_REQUIRE(ctx && ctx_tanh && weight_updates, "wavnetc_backward_weights: null argument");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    CNT_TRY(fill_zero(stream, weight_updates, (size_t)C * 2 * D));
     GemmArgs ga = {};
     ga.m = C; ga.n = 2 * D; ga.k = N;
     ga.a_kcontig = 0; ga.lda = C;
@@ -468,6 +467,9 @@ int cnt_wavnetc_backward_weights(void *stream_, int D, int C, int N, const float
     ga.splitk = 0;  // chosen by the launcher
     ga.prob[0].A[0] = ctx; ga.prob[0].B[0] = ctx_tanh; ga.prob[0].C = weight_updates;
     ga.label = "gemm:wavnetc_dW";
+    ga.overwrite_ok = 1;  // the product covers all C x 2D weights
+    gemm_plan(ga);
+    if (ga.epilogue != EPI_PARTIAL) CNT_TRY(fill_zero(stream, weight_updates, (size_t)C * 2 * D));
     return gemm_launch(stream, ga);
 }
 
