@@ -334,6 +334,7 @@ int cnt_cnn_backward_weights(cnt_cnn *h, void *stream_, const char *patTypes, in
         }
         ga.nprob = pr;
         ga.splitk = 0;  // chosen by the launcher
+        ga.overwrite_ok = 1;  // every tap's P x (d1 - d0) block is written whole; the rest stays as cleared above
         ga.label = "gemm:cnn_dW";
         CNT_TRY(gemm_launch(stream, ga));
     }
