@@ -89,28 +89,35 @@ float *split_scratch(hipStream_t stream) {
     return buf;
 }
 
-// 64 consecutive outputs per block, the splits dealt to four groups of 64 threads whose sums meet in LDS
+// 32 consecutive outputs per block, the splits dealt to eight groups of 32 threads whose sums meet in LDS; four
+// loads in flight per thread
+constexpr int kReduceOutputs = 32;
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs args) {
-    __shared__ float part[4][64];
-    const int tx = threadIdx.x & 63, g = threadIdx.x >> 6;
+    constexpr int G = 256 / kReduceOutputs;
+    __shared__ float part[G][kReduceOutputs];
+    const int tx = threadIdx.x % kReduceOutputs, g = threadIdx.x / kReduceOutputs;
     const size_t mn = (size_t)args.m * args.n;
     const size_t products = mn * args.nprob;
     const size_t total = products + (args.rowsum_out ? (size_t)args.n : 0);
-    const size_t e = (size_t)blockIdx.x * 64 + tx;
-    float a0 = 0.0f, a1 = 0.0f;
+    const size_t e = (size_t)blockIdx.x * kReduceOutputs + tx;
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
     if (e < total) {
         const float *__restrict__ p = args.partial + e;
+        const size_t st = args.partial_stride;
         int s = g;
-        for (; s + 4 < args.splitk; s += 8) {
-            a0 += p[(size_t)s * args.partial_stride];
-            a1 += p[(size_t)(s + 4) * args.partial_stride];
+        for (; s + 3 * G < args.splitk; s += 4 * G) {
+            const float x0 = p[(size_t)s * st], x1 = p[(size_t)(s + G) * st];
+            const float x2 = p[(size_t)(s + 2 * G) * st], x3 = p[(size_t)(s + 3 * G) * st];
+            a0 += x0; a1 += x1; a2 += x2; a3 += x3;
         }
-        if (s < args.splitk) a0 += p[(size_t)s * args.partial_stride];
+        for (; s < args.splitk; s += G) a0 += p[(size_t)s * st];
     }
-    part[g][tx] = a0 + a1;
+    part[g][tx] = (a0 + a1) + (a2 + a3);
     __syncthreads();
     if (g == 0 && e < total) {
-        const float v = (part[0][tx] + part[1][tx]) + (part[2][tx] + part[3][tx]);
+        float v = 0.0f;
+#pragma unroll
+        for (int q = 0; q < G; ++q) v += part[q][tx];
         if (e < products) {
             const size_t z = e / mn, r = e % mn;
             args.prob[z].C[(r / args.m) * args.ldc + r % args.m] = v;
@@ -187,7 +194,8 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
     CNT_HIP(hipGetLastError());
     if (args.epilogue == EPI_PARTIAL) {
         const size_t total = args.partial_stride;
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, stream, args);
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total + kReduceOutputs - 1) / kReduceOutputs)), dim3(256),
+                           0, stream, args);
         CNT_HIP(hipGetLastError());
     }
     return CNT_OK;
