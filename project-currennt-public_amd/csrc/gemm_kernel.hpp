@@ -57,12 +57,18 @@ struct TileStage {
                     const int rc = min(row, rows_total - 1), kc = (k0 + kq) < k_total ? k0 + kq : 0;
                     v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)rc * ld + kc);
                     if (!inside) v = typename VecT<VEC>::type{};
+                } else if (!time_on_k) {
+                    // the row is the time slot, so the whole vector is kept or dropped: as above, the load always
+                    // executes on a clamped address, next to the two pattern bytes instead of after them
+                    const bool inside = row < rows_total && (k0 + kq) < k_total;
+                    const int rc = min(row, rows_total - 1), kc = (k0 + kq) < k_total ? k0 + kq : 0;
+                    const int src = rc + shift;
+                    const int sc = min(max(src, 0), n_slots - 1);
+                    v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)sc * ld + kc);
+                    const char p_own = pat[rc], p_src = pat[sc];
+                    if (!(inside && src == sc && p_own != 0 && p_src != 0)) v = typename VecT<VEC>::type{};
                 } else if (row < rows_total && (k0 + kq) < k_total) {
-                    if (!time_on_k) {
-                        const int src = row + shift;
-                        if (pat[row] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
-                            v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)src * ld + k0 + kq);
-                    } else {
+                    {
                         // vector along k = consecutive time slots: element-wise masking
                         float *e = reinterpret_cast<float *>(&v);
 #pragma unroll
@@ -89,12 +95,17 @@ struct TileStage {
                     const int kc = min(k, k_total - 1), rc = (row0 + rq) < rows_total ? row0 + rq : 0;
                     v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)kc * ld + rc);
                     if (!inside) v = typename VecT<VEC>::type{};
+                } else if (time_on_k) {
+                    // the k line is the time slot: branch-free as above
+                    const bool inside = k < k_total && (row0 + rq) < rows_total;
+                    const int kc = min(k, k_total - 1), rc = (row0 + rq) < rows_total ? row0 + rq : 0;
+                    const int src = kc + shift;
+                    const int sc = min(max(src, 0), n_slots - 1);
+                    v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)sc * ld + rc);
+                    const char p_own = pat[kc], p_src = pat[sc];
+                    if (!(inside && src == sc && p_own != 0 && p_src != 0)) v = typename VecT<VEC>::type{};
                 } else if (k < k_total && (row0 + rq) < rows_total) {
-                    if (time_on_k) {
-                        const int src = k + shift;
-                        if (pat[k] != 0 && src >= 0 && src < n_slots && pat[src] != 0)
-                            v = *reinterpret_cast<const typename VecT<VEC>::type *>(base + (size_t)src * ld + row0 + rq);
-                    } else {
+                    {
                         float *e = reinterpret_cast<float *>(&v);
 #pragma unroll
                         for (int j = 0; j < VEC; ++j) {
