@@ -165,6 +165,9 @@ struct GemmArgs {
 // before gemm_launch and looks at args.epilogue; gemm_launch calls it for everyone else.
 void gemm_plan(GemmArgs &args);
 int gemm_launch(hipStream_t stream, const GemmArgs &args);
+// Frees the split-K scratch buffer that the launcher keeps for `stream` (for owners of a stream about to destroy
+// it; the stream must be idle).  Buffers of streams never released stay until the process ends.
+void gemm_release_stream(hipStream_t stream);
 
 // Convenience: single problem, BLAS-like transposes on column-major matrices.
 int gemm_simple(hipStream_t stream, float *C, int m, int n, int k, const float *A, bool transA,

@@ -129,6 +129,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs args)
 
 }  // namespace
 
+void gemm_release_stream(hipStream_t stream) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    std::lock_guard<std::mutex> lock(g_split_mu);
+    for (size_t i = 0; i < g_split_scratch.size(); ++i)
+        if (g_split_scratch[i].device == dev && g_split_scratch[i].stream == stream) {
+            (void)hipFree(g_split_scratch[i].buf);
+            g_split_scratch.erase(g_split_scratch.begin() + (long)i);
+            return;
+        }
+}
+
 void gemm_plan(GemmArgs &args) {
     if (args.splitk != 0) return;
     // Long-K products with a small output (weight gradients): cut K so that the launch has about

@@ -987,7 +987,12 @@ int cnt_network_destroy(cnt_network *net) {
     }
     for (void *p : net->allocations) (void)hipFree(p);
     for (int k = 0; k < cnt_network::kMaxSide; ++k) {
-        if (net->side[k]) (void)hipStreamDestroy(net->side[k]);
+        if (net->side[k]) {
+            // the product launcher keeps a scratch buffer per stream it has seen
+            (void)hipStreamSynchronize(net->side[k]);
+            cnt::gemm_release_stream(net->side[k]);
+            (void)hipStreamDestroy(net->side[k]);
+        }
         if (net->ev_side[k]) (void)hipEventDestroy(net->ev_side[k]);
     }
     if (net->ev_main) (void)hipEventDestroy(net->ev_main);
