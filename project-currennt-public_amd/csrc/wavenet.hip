@@ -85,34 +85,85 @@ __global__ void core_copy_kernel(int D2, size_t count, const char *__restrict__ 
 // core is conditioned -- the gradient through tanh(X_c) written over ctx_tanh in the same pass.
 // prev_out (optional): outputs of a preceding layer with tanh output; its delta tanh'(y) * error is then written
 // instead of the error.
+template <int V> struct Pack;
+template <> struct Pack<1> { typedef float type; };
+template <> struct Pack<4> { typedef float4 type; };
+
+// VEC consecutive channels per thread (VEC = 4: 16-byte accesses, for D % 4 == 0 and 16-byte aligned buffers)
+template <int VEC>
 __global__ void gated_backward_kernel(int D, size_t count, const char *__restrict__ pat, const float *__restrict__ pre,
                                       const float *__restrict__ err, float *__restrict__ prev_err,
                                       float *__restrict__ ctx_tanh, const float *__restrict__ prev_out) {
+    typedef typename Pack<VEC>::type V;
+    const size_t groups = count / VEC;
+    const size_t per_slot = (size_t)D / VEC;
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; i < count; i += stride) {
-        const size_t t = i / D, d = i % D;
+    for (; i < groups; i += stride) {
+        const size_t t = i / per_slot, d = (i % per_slot) * VEC;
         const size_t i1 = t * 2 * D + d, i2 = i1 + D;
-        float g1 = 0.0f, g2 = 0.0f;
+        float g1[VEC], g2[VEC];
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) g1[q] = g2[q] = 0.0f;
         if (pat[t] != 0) {
-            const float th = tanh_act(pre[i1]);
-            const float sg = logistic(pre[i2]);
-            const float e = err[i];
-            g1 = (1.0f - th * th) * sg * e;
-            g2 = th * (sg * (1.0f - sg)) * e;
+            const V p1 = *reinterpret_cast<const V *>(pre + i1), p2 = *reinterpret_cast<const V *>(pre + i2);
+            const V ev = *reinterpret_cast<const V *>(err + t * D + d);
+            const float *a1 = reinterpret_cast<const float *>(&p1), *a2 = reinterpret_cast<const float *>(&p2);
+            const float *e = reinterpret_cast<const float *>(&ev);
+#pragma unroll
+            for (int q = 0; q < VEC; ++q) {
+                const float th = tanh_act(a1[q]);
+                const float sg = logistic(a2[q]);
+                g1[q] = (1.0f - th * th) * sg * e[q];
+                g2[q] = th * (sg * (1.0f - sg)) * e[q];
+            }
         }
+        V o1, o2;
+        float *w1 = reinterpret_cast<float *>(&o1), *w2 = reinterpret_cast<float *>(&o2);
         if (prev_out) {
-            prev_err[i1] = tanh_deriv(prev_out[i1]) * g1;
-            prev_err[i2] = tanh_deriv(prev_out[i2]) * g2;
+            const V y1 = *reinterpret_cast<const V *>(prev_out + i1), y2 = *reinterpret_cast<const V *>(prev_out + i2);
+            const float *b1 = reinterpret_cast<const float *>(&y1), *b2 = reinterpret_cast<const float *>(&y2);
+#pragma unroll
+            for (int q = 0; q < VEC; ++q) {
+                w1[q] = tanh_deriv(b1[q]) * g1[q];
+                w2[q] = tanh_deriv(b2[q]) * g2[q];
+            }
         } else {
-            prev_err[i1] = g1;
-            prev_err[i2] = g2;
+#pragma unroll
+            for (int q = 0; q < VEC; ++q) {
+                w1[q] = g1[q];
+                w2[q] = g2[q];
+            }
         }
+        *reinterpret_cast<V *>(prev_err + i1) = o1;
+        *reinterpret_cast<V *>(prev_err + i2) = o2;
         if (ctx_tanh) {
-            ctx_tanh[i1] = tanh_deriv(ctx_tanh[i1]) * g1;
-            ctx_tanh[i2] = tanh_deriv(ctx_tanh[i2]) * g2;
+            const V c1 = *reinterpret_cast<const V *>(ctx_tanh + i1), c2 = *reinterpret_cast<const V *>(ctx_tanh + i2);
+            const float *b1 = reinterpret_cast<const float *>(&c1), *b2 = reinterpret_cast<const float *>(&c2);
+#pragma unroll
+            for (int q = 0; q < VEC; ++q) {
+                w1[q] = tanh_deriv(b1[q]) * g1[q];
+                w2[q] = tanh_deriv(b2[q]) * g2[q];
+            }
+            *reinterpret_cast<V *>(ctx_tanh + i1) = o1;
+            *reinterpret_cast<V *>(ctx_tanh + i2) = o2;
         }
     }
+}
+
+int launch_gated_backward(hipStream_t stream, int D, size_t count, const char *pat, const float *pre, const float *err,
+                          float *prev_err, float *ctx_tanh, const float *prev_out) {
+    auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    const bool vec4 = D % 4 == 0 && aligned(pre) && aligned(err) && aligned(prev_err) && aligned(ctx_tanh) &&
+                      aligned(prev_out);
+    if (vec4)
+        hipLaunchKernelGGL(gated_backward_kernel<4>, dim3(stream_blocks(count / 4)), dim3(256), 0, stream, D, count, pat,
+                           pre, err, prev_err, ctx_tanh, prev_out);
+    else
+        hipLaunchKernelGGL(gated_backward_kernel<1>, dim3(stream_blocks(count)), dim3(256), 0, stream, D, count, pat, pre,
+                           err, prev_err, ctx_tanh, prev_out);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
 }
 
 __global__ void sum_context_grad_kernel(int C, int S, int resolution, size_t count, int N,
@@ -385,11 +436,8 @@ int cnt_gatedact_backward(void *stream_, int D, int N, const char *patTypes, con
     CNT_REQUIRE(D > 0 && N > 0, "gatedact_backward: non-positive size");
     const size_t count = (size_t)D * N;
     ProfileScope prof(static_cast<hipStream_t>(stream_), "gated_backward");
-    hipLaunchKernelGGL(gated_backward_kernel, dim3(stream_blocks(count)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream_), D, count, patTypes, pre, output_errors, prev_errors,
-                       static_cast<float *>(nullptr), static_cast<const float *>(nullptr));
-    CNT_HIP(hipGetLastError());
-    return CNT_OK;
+    return launch_gated_backward(static_cast<hipStream_t>(stream_), D, count, patTypes, pre, output_errors, prev_errors,
+                                 nullptr, nullptr);
 }
 
 int cnt_wavnetc_forward(void *stream_, int D, int C, int N, const char *patTypes, const float *weights, const float *ctx,
@@ -433,10 +481,8 @@ int cnt_wavnetc_backward_errors(void *stream_, int D, int C, int N, const char *
     const size_t count = (size_t)D * N;
     {
         ProfileScope prof(stream, "gated_backward");
-        hipLaunchKernelGGL(gated_backward_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, D, count, patTypes,
-                           core_buf, output_errors, prev_errors, C > 0 ? ctx_tanh : static_cast<float *>(nullptr),
-                           prev_tanh_outputs);
-        CNT_HIP(hipGetLastError());
+        CNT_TRY(launch_gated_backward(stream, D, count, patTypes, core_buf, output_errors, prev_errors,
+                                      C > 0 ? ctx_tanh : nullptr, prev_tanh_outputs));
     }
     if (C > 0 && ctx_grad) {
         GemmArgs ga = {};

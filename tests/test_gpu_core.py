@@ -39,6 +39,17 @@ def test_dense(P, D, N, act):
     assert PC.run_dense_case(P, D, N, act, 1.0, seed=P + D) < TOL
 
 
+@pytest.mark.parametrize("P,D,N,bias", [
+    # narrow layers over long inputs take the split-K path that sums partial products and carries the bias
+    # gradient (row sums of the errors, times the layer's bias value) along; 300 x 300 is too large an output for it and
+    # takes the atomic path with its separate column sum
+    (64, 128, 3000, 0.5), (64, 64, 5000, 2.0), (100, 96, 2500, 0.25), (300, 300, 2500, 0.5),
+])
+def test_dense_bias_value_scales_the_bias_gradient(P, D, N, bias):
+    print("dense bias case", P, D, N, bias, flush=True)
+    assert PC.run_dense_case(P, D, N, 0, bias, seed=P + D + N) < TOL
+
+
 def test_sse():
     print("sse case", flush=True)
     assert PC.run_sse_case(187, [40, 33, 40, 12], seed=2) < 1e-5
