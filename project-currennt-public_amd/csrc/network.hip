@@ -223,6 +223,7 @@ struct NetLayer {
     const float **in_ptrs = nullptr;         // skip layers: device tables
     float **tgt_ptrs = nullptr;
     int *tgt_is_skip = nullptr;
+    bool ptrs_aligned = false;               // every buffer the skip kernels touch for this layer is 16-byte aligned
     long weight_count() const { return n_in + n_bias + n_int; }
 };
 
@@ -232,32 +233,39 @@ inline int blocks_for(size_t count) {
     return (int)(b < 1 ? 1 : b);
 }
 
+// The skip kernels move V = float or float4 (16-byte accesses: count % 4 == 0 and every buffer 16-byte aligned);
+// `count` is in units of V.
+__device__ __forceinline__ float vadd(float a, float b) { return a + b; }
+__device__ __forceinline__ float4 vadd(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+
+template <typename V>
 __global__ void skip_sum_kernel(size_t count, int n, const float *const *__restrict__ in, float *__restrict__ out) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (; i < count; i += stride) {
-        float acc = 0.0f;
-        for (int k = 0; k < n; ++k) acc += in[k][i];
-        out[i] = acc;
+        V acc = reinterpret_cast<const V *>(in[0])[i];
+        for (int k = 1; k < n; ++k) acc = vadd(acc, reinterpret_cast<const V *>(in[k])[i]);
+        reinterpret_cast<V *>(out)[i] = acc;
     }
 }
 
 // errors += errors_from_skip, then to every linked source in reverse order: added to a skip layer's side buffer,
 // written over any other layer's error buffer (layers/SkipAddLayer.cu:305-346)
 // errors_from_skip == NULL: nothing to add, `errors` is only read
+template <typename V>
 __global__ void skip_fan_kernel(size_t count, int n, float *const *__restrict__ target, const int *__restrict__ is_skip,
                                 float *errors, const float *__restrict__ errors_from_skip) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (; i < count; i += stride) {
-        float e = errors[i];
+        V e = reinterpret_cast<const V *>(errors)[i];
         if (errors_from_skip) {
-            e = errors_from_skip[i] + e;
-            errors[i] = e;
+            e = vadd(reinterpret_cast<const V *>(errors_from_skip)[i], e);
+            reinterpret_cast<V *>(errors)[i] = e;
         }
         for (int k = 0; k < n; ++k) {
-            float *t = target[k];
-            t[i] = is_skip[k] ? e + t[i] : e;
+            V *t = reinterpret_cast<V *>(target[k]);
+            t[i] = is_skip[k] ? vadd(e, t[i]) : e;
         }
     }
 }
@@ -911,6 +919,13 @@ int finish_build(cnt_network *net, const json::Value *weights) {
         CNT_HIP(hipMemcpy(L.in_ptrs, in.data(), n * sizeof(float *), hipMemcpyHostToDevice));
         std::vector<float *> &t = tgt[(size_t)i];
         L.live_targets = (int)t.size();
+        {
+            auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+            bool ok = aligned(L.out) && aligned(L.total) && aligned(L.eskip);
+            for (const float *p : in) ok = ok && aligned(p);
+            for (const float *p : t) ok = ok && aligned(p);
+            L.ptrs_aligned = ok;
+        }
         if (t.empty()) continue;
         CNT_TRY(device_alloc(net, (void **)&L.tgt_ptrs, t.size() * sizeof(float *), false));
         CNT_TRY(device_alloc(net, (void **)&L.tgt_is_skip, t.size() * sizeof(int), false));
@@ -1168,8 +1183,12 @@ int cnt_network_forward(cnt_network *net, void *stream_) {
             case K_SKIPADD:
                 if (L.pre.size() > 1) {
                     ProfileScope prof(stream, "skip_sum");
-                    hipLaunchKernelGGL(skip_sum_kernel, dim3(blocks_for(count)), dim3(256), 0, stream, count,
-                                       (int)L.pre.size(), L.in_ptrs, L.out);
+                    if (L.ptrs_aligned && count % 4 == 0)
+                        hipLaunchKernelGGL(skip_sum_kernel<float4>, dim3(blocks_for(count / 4)), dim3(256), 0, stream,
+                                           count / 4, (int)L.pre.size(), L.in_ptrs, L.out);
+                    else
+                        hipLaunchKernelGGL(skip_sum_kernel<float>, dim3(blocks_for(count)), dim3(256), 0, stream, count,
+                                           (int)L.pre.size(), L.in_ptrs, L.out);
                     CNT_HIP(hipGetLastError());
                 }
                 break;
@@ -1361,9 +1380,13 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
             case K_SKIPADD: {
                 if (!L.needs_sum && L.live_targets == 0) break;
                 ProfileScope prof(stream, "skip_fan");
-                hipLaunchKernelGGL(skip_fan_kernel, dim3(blocks_for(count)), dim3(256), 0, stream, count,
-                                   L.live_targets, L.tgt_ptrs, L.tgt_is_skip, const_cast<float *>(L.total),
-                                   L.needs_sum ? L.eskip : static_cast<const float *>(nullptr));
+                const float *from_skip = L.needs_sum ? L.eskip : static_cast<const float *>(nullptr);
+                if (L.ptrs_aligned && count % 4 == 0)
+                    hipLaunchKernelGGL(skip_fan_kernel<float4>, dim3(blocks_for(count / 4)), dim3(256), 0, stream, count / 4,
+                                       L.live_targets, L.tgt_ptrs, L.tgt_is_skip, const_cast<float *>(L.total), from_skip);
+                else
+                    hipLaunchKernelGGL(skip_fan_kernel<float>, dim3(blocks_for(count)), dim3(256), 0, stream, count,
+                                       L.live_targets, L.tgt_ptrs, L.tgt_is_skip, const_cast<float *>(L.total), from_skip);
                 CNT_HIP(hipGetLastError());
                 break;
             }
