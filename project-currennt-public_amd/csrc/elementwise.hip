@@ -9,10 +9,13 @@
 namespace cnt {
 namespace {
 
-__global__ void fill_zero_kernel(float *__restrict__ p, size_t count) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+// the first n4 groups of four floats as 16-byte stores (n4 = 0 for a buffer that is not 16-byte aligned), the rest
+// one by one
+__global__ void fill_zero_kernel(float *__restrict__ p, size_t count, size_t n4) {
+    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; i < count; i += stride) p[i] = 0.0f;
+    for (size_t i = first; i < n4; i += stride) reinterpret_cast<float4 *>(p)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (size_t i = 4 * n4 + first; i < count; i += stride) p[i] = 0.0f;
 }
 
 __global__ void fill_zero_pair_kernel(float *__restrict__ p, size_t count, float *__restrict__ q, size_t count_q) {
@@ -31,10 +34,20 @@ __global__ void fill_words_kernel(unsigned *__restrict__ p, size_t count, unsign
 }
 
 // delta = act'(y) * err in place, on every slot (the reference does not mask padding here)
-__global__ void dense_delta_kernel(float *__restrict__ err, const float *__restrict__ y, size_t count, int act) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+// (as above: n4 groups of four floats through 16-byte accesses, the rest one by one)
+__global__ void dense_delta_kernel(float *__restrict__ err, const float *__restrict__ y, size_t count, int act, size_t n4) {
+    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; i < count; i += stride) err[i] = act_deriv(act, y[i]) * err[i];
+    for (size_t i = first; i < n4; i += stride) {
+        const float4 yv = reinterpret_cast<const float4 *>(y)[i];
+        float4 e = reinterpret_cast<float4 *>(err)[i];
+        e.x = act_deriv(act, yv.x) * e.x;
+        e.y = act_deriv(act, yv.y) * e.y;
+        e.z = act_deriv(act, yv.z) * e.z;
+        e.w = act_deriv(act, yv.w) * e.w;
+        reinterpret_cast<float4 *>(err)[i] = e;
+    }
+    for (size_t i = 4 * n4 + first; i < count; i += stride) err[i] = act_deriv(act, y[i]) * err[i];
 }
 
 // out[d] += scale * sum_i v[d + i*D]; out is zeroed by the caller.  A block is 64 rows x 4 column lanes (one
@@ -99,7 +112,8 @@ inline int stream_blocks(size_t count) {
 
 int fill_zero(hipStream_t stream, float *p, size_t count) {
     if (count == 0) return CNT_OK;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, p, count);
+    const size_t n4 = (reinterpret_cast<uintptr_t>(p) & 15) == 0 ? count / 4 : 0;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(stream_blocks(n4 ? n4 + 3 : count)), dim3(256), 0, stream, p, count, n4);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
@@ -162,7 +176,9 @@ int cnt_dense_backward_errors(void *stream_, int P, int D, int N, int act, const
     const size_t count = (size_t)D * N;
     if (act != ACT_IDENTITY) {
         ProfileScope prof(stream, "dense_delta");
-        hipLaunchKernelGGL(dense_delta_kernel, dim3(stream_blocks(count)), dim3(256), 0, stream, err, y, count, act);
+        const size_t n4 = ((reinterpret_cast<uintptr_t>(err) | reinterpret_cast<uintptr_t>(y)) & 15) == 0 ? count / 4 : 0;
+        hipLaunchKernelGGL(dense_delta_kernel, dim3(stream_blocks(n4 ? n4 + 3 : count)), dim3(256), 0, stream, err, y, count,
+                           act, n4);
         CNT_HIP(hipGetLastError());
     }
     if (prev_err) {

@@ -250,6 +250,9 @@ __global__ void mixture_error_kernel(UnitGeom g, const char *__restrict__ pat, c
     }
 }
 
+// VEC4: the mean / std part moves 16 bytes per lane (D, M, Lp, Lt and both start columns multiples of four and all
+// buffers 16-byte aligned, so that four consecutive dimensions of one mixture component sit in one aligned vector)
+template <bool VEC4>
 __global__ void mixture_backward_kernel(UnitGeom g, const char *__restrict__ pat, const float *__restrict__ target,
                                         const float *__restrict__ para, const float *__restrict__ tmp,
                                         float *__restrict__ errors) {
@@ -285,6 +288,26 @@ __global__ void mixture_backward_kernel(UnitGeom g, const char *__restrict__ pat
     const float *t = target + (size_t)f * g.Lt + g.startDOut;
     const float *mean = para + (size_t)g.F * M + (size_t)f * MD;
     const float *sd = para + (size_t)g.F * M * (1 + D) + (size_t)f * MD;
+    if (VEC4) {
+        for (int i = 4 * lane; i < MD; i += 256) {
+            const int m = i / D, d = i - m * D;
+            const float post = safe_exp(tmp[(size_t)f * M + m] - lsum);
+            const float4 mu4 = *reinterpret_cast<const float4 *>(mean + i);
+            const float4 s4 = *reinterpret_cast<const float4 *>(sd + i);
+            const float4 t4 = *reinterpret_cast<const float4 *>(t + d);
+            const float mu[4] = {mu4.x, mu4.y, mu4.z, mu4.w}, sv[4] = {s4.x, s4.y, s4.z, s4.w};
+            const float tv[4] = {t4.x, t4.y, t4.z, t4.w};
+            float em[4], es[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                em[q] = post * (mu[q] - tv[q]) / sv[q] / sv[q];
+                es[q] = (sv[q] > g.var_floor) ? post - em[q] * (mu[q] - tv[q]) : 0.0f;
+            }
+            *reinterpret_cast<float4 *>(e + M + i) = make_float4(em[0], em[1], em[2], em[3]);
+            *reinterpret_cast<float4 *>(e + M + MD + i) = make_float4(es[0], es[1], es[2], es[3]);
+        }
+        return;
+    }
     for (int i = lane; i < MD; i += 64) {
         const int m = i / D, d = i - m * D;
         const float post = safe_exp(tmp[(size_t)f * M + m] - lsum);
@@ -520,8 +543,15 @@ int cnt_mdn_backward(cnt_mdn *h, void *stream_, const float *targets, float *pre
                                prev_errors);
         } else {
             ProfileScope prof(stream, "mdn_mixture_backward");
-            hipLaunchKernelGGL(mixture_backward_kernel, grid, block, 0, stream, g, h->pat, targets, u.para, u.tmp,
-                               prev_errors);
+            auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+            const bool vec4 = g.D % 4 == 0 && g.M % 4 == 0 && g.Lp % 4 == 0 && g.Lt % 4 == 0 && g.startD % 4 == 0 &&
+                              g.startDOut % 4 == 0 && aligned(targets) && aligned(u.para) && aligned(prev_errors);
+            if (vec4)
+                hipLaunchKernelGGL(mixture_backward_kernel<true>, grid, block, 0, stream, g, h->pat, targets, u.para,
+                                   u.tmp, prev_errors);
+            else
+                hipLaunchKernelGGL(mixture_backward_kernel<false>, grid, block, 0, stream, g, h->pat, targets, u.para,
+                                   u.tmp, prev_errors);
         }
         CNT_HIP(hipGetLastError());
     }
