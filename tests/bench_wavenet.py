@@ -31,7 +31,11 @@ def run(args, pkg):
     lengths = [16000, 16000]
     S, T = 2, 16000
     pat, onehot, ctx, target, N = WD.make(lengths, Q, C, upsample=80, seed=4)
-    net = capi.Network(json.dumps(WD.network_json(nb, Q, R, K, C, 1, 10)), S, T, mdn_config=[1, 0, Q, 0, 1, -1])
+    topology = WD.network_json(nb, Q, R, K, C, 1, 10)
+    net = capi.Network(json.dumps(topology), S, T, mdn_config=[1, 0, Q, 0, 1, -1])
+    # rows a dense layer's weight-gradient launch reads per sample: its input and its output errors
+    dense_rows = [prev["size"] + cur["size"] for prev, cur in zip(topology["layers"], topology["layers"][1:])
+                  if cur["type"].startswith("feedforward")]
     shapes = {L["name"]: L["weight_count"] for L in net.layers if L["weight_count"]}
     for k, w in WD.init_weights(shapes, seed=5).items():
         net.layer(k)["weights"].copy_(torch.from_numpy(w))
@@ -70,6 +74,9 @@ def run(args, pkg):
         nbytes = 2 * (R + 2 * R) * 4.0 * N
     elif dom == "gemm:cnn_prev_errors":
         nbytes = (2 * 2 * R + R) * 4.0 * N
+    elif dom == "gemm:dense_dW":
+        # average over the stack's dense layers (30 x 64->64, 30 x 64->128, the 1024->64 embedding, 128->128, 128->1024)
+        nbytes = sum(dense_rows) / len(dense_rows) * 4.0 * N
     else:
         nbytes = 155e3 * N / max(1, sum(v["launches"] for v in kernels.values()))
     roof["achieved"] = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
