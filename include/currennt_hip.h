@@ -64,7 +64,7 @@ int cnt_dense_backward(void *stream, int P, int D, int N, int act, float bias, c
  * Device memory: the weight half of a narrow layer over a long input (P*D up to 64 K floats, N in the thousands)
  * sums split partial products through a scratch buffer of 16 MB per stream, which the library allocates the first
  * time such a product runs on a stream and keeps; the same holds for cnt_cnn_backward_weights and
- * cnt_wavnetc_backward_weights.  Nothing else outside the *_create calls allocates. */
+ * cnt_wavnetc_backward_weights.  Apart from that, only the *_create calls allocate. */
 int cnt_dense_backward_errors(void *stream, int P, int D, int N, int act, const float *weights, const float *y,
                               float *err, float *prev_err);
 int cnt_dense_backward_weights(void *stream, int P, int D, int N, float bias, const float *x, const float *err,
