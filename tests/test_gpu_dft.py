@@ -15,6 +15,9 @@ TOL = 1e-4
     ([(512, 512, 80), (128, 128, 40), (2048, 2048, 640)], 16000, [16000, 9000]),  # benchmark config 5 resolutions
     ([(1024, 800, 200), (4096, 4096, 1024)], 6000, [6000, 5000, 4097]),
     ([(128, 128, 40)], 300, [60]),                           # waveform shorter than one frame
+    # eight waveforms of very different lengths, a long and a short transform: workgroups of the short one make
+    # several passes of sixteen frames, and how many depends on the waveform
+    ([(2048, 2048, 512), (64, 64, 16)], 6000, [6000, 130, 2500, 64, 5999, 1000, 300, 2049]),
 ])
 def test_dft_loss(res, max_len, lengths):
     print("dft case", res, max_len, lengths, flush=True)
