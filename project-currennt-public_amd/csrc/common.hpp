@@ -119,8 +119,11 @@ enum GemmEpilogue {
     EPI_BIAS_ACT = 3,       // C = act(acc + bias_scale * bias_vec[row])
     EPI_BIAS_ACT_SKIP = 4,  // as above, but columns whose pattern type is "none" are left untouched
     EPI_CONTEXT = 5,        // th = tanh(acc); aux_out = th; C = aux_in + th; both 0 on "none" columns
-    EPI_PARTIAL = 6         // split-K without atomics: every split stores its m x n partial product into the
+    EPI_PARTIAL = 6,        // split-K without atomics: every split stores its m x n partial product into the
                             // launcher's scratch, and a second kernel sums the splits into C (set by gemm_plan)
+    EPI_FAN = 7             // a skip layer's backward step in the epilogue of the product that writes the layer's
+                            // errors: e = aux_in + acc (aux_in may be NULL), C = e, and e goes on to fan_n buffers of
+                            // C's layout -- added to those flagged in fan_is_skip, stored over the others
 };
 
 struct GemmProblem {
@@ -131,6 +134,8 @@ struct GemmProblem {
     const float *bias_vec;
     const float *aux_in;  // EPI_CONTEXT, same layout as C
     float *aux_out;       // EPI_CONTEXT, may be NULL
+    float *rowsum_out;    // GemmArgs::rowsum: receives rowsum_scale * sum_k B(j, k), j < n
+    float rowsum_scale;
 };
 
 // Masked mode (dilated convolutions without a materialised column buffer): one index of the B operand is a
@@ -150,20 +155,25 @@ struct GemmArgs {
     GemmProblem prob[kGemmMaxProb];
     const char *label;  // name under which the launch is timed when profiling is on (may be NULL)
     // Split-K products with a small output (EPI_ATOMIC, splitk = 0): `overwrite_ok` allows gemm_plan to choose
-    // EPI_PARTIAL, which overwrites C instead of adding to a cleared C.  With `rowsum_out` (one problem, one operand
-    // pair, unmasked) the same pass also sums the B operand over k: rowsum_out[j] = rowsum_scale * sum_k B(j, k),
-    // the bias gradient of a dense layer, for which the atomic path needs a separate column-sum launch.
+    // EPI_PARTIAL, which overwrites C instead of adding to a cleared C.  With `rowsum` (one operand pair, unmasked)
+    // the same pass also sums every problem's B operand over k into that problem's rowsum_out -- the bias gradient
+    // of a dense layer, for which the atomic path needs a separate column-sum launch.  gemm_plan clears `rowsum`
+    // where it does not choose EPI_PARTIAL.
     int overwrite_ok;
-    float *rowsum_out;
-    float rowsum_scale;
+    int rowsum;
+    int fan_n;                   // EPI_FAN: device tables of fan_n targets and their flags
+    float *const *fan_targets;
+    const int *fan_is_skip;
     float *partial;        // set by the launcher: scratch of splitk * partial_stride floats
-    size_t partial_stride;  // floats per split: nprob * m * n (+ n with rowsum_out)
+    size_t partial_stride;  // floats per split: nprob * m * n (+ nprob * n with rowsum)
 };
 
 // Resolves splitk = 0 (chosen by the launcher) and, where the arguments allow it and it pays, switches an
 // EPI_ATOMIC product to EPI_PARTIAL.  A caller that needs to know whether C must be cleared first calls this
 // before gemm_launch and looks at args.epilogue; gemm_launch calls it for everyone else.
 void gemm_plan(GemmArgs &args);
+// whether a product with these operands can take the EPI_FAN epilogue (operand kinds, alignment)
+bool gemm_fan_supported(const GemmArgs &args);
 int gemm_launch(hipStream_t stream, const GemmArgs &args);
 // Frees the split-K scratch buffer that the launcher keeps for `stream` (for owners of a stream about to destroy
 // it; the stream must be idle).  Buffers of streams never released stay until the process ends.
@@ -172,6 +182,34 @@ void gemm_release_stream(hipStream_t stream);
 // Convenience: single problem, BLAS-like transposes on column-major matrices.
 int gemm_simple(hipStream_t stream, float *C, int m, int n, int k, const float *A, bool transA,
                 const float *B, bool transB, bool accumulate);
+
+// ----- error halves that also do the backward step of the skip layer in front of them ----------------
+// A skip layer adds what its linkers left in its side buffer to the errors its following layer wrote, and hands the
+// sum on (layers/SkipAddLayer.cu:305-346).  When that following layer is a dense or convolution layer, the sum and
+// the hand-over happen in the epilogue of the product that computes those errors, instead of in a launch of their
+// own.  `targets` / `is_skip` are device tables of `n` entries; `from_skip` is the side buffer or NULL.
+struct FanOut {
+    int n;
+    float *const *targets;
+    const int *is_skip;
+    const float *from_skip;
+};
+// *fused tells whether the step was done (operands that the fan epilogue does not exist for, or a convolution
+// with several filter groups, leave it to the caller).
+int dense_backward_errors_fan(hipStream_t stream, int P, int D, int N, int act, const float *weights, const float *y,
+                              float *err, float *prev_err, const FanOut *fan, bool *fused);
+int cnn_backward_errors_fan(cnt_cnn *h, hipStream_t stream, const char *patTypes, int curT, const float *weights,
+                            const float *outputs, float *output_errors, float *prev_errors, int delta_applied,
+                            const FanOut *fan, bool *fused);
+
+// ----- weight-gradient halves of several layers of one shape in one launch --------------------------
+// For the network sequencer: `count` (<= kGemmMaxProb) dense layers with the same P, D, N, or wavnetc layers with the
+// same D, C, N and one context buffer, as the problems of one product.  Same results as `count` calls of
+// cnt_dense_backward_weights / cnt_wavnetc_backward_weights.
+int dense_backward_weights_batch(hipStream_t stream, int P, int D, int N, int count, const float *bias,
+                                 const float *const *x, const float *const *err, float *const *weight_updates);
+int wavnetc_backward_weights_batch(hipStream_t stream, int D, int C, int N, int count, const float *ctx,
+                                   const float *const *ctx_tanh, float *const *weight_updates);
 
 // ----- small streaming kernels (elementwise.hip) ----------------------------------------------------
 int fill_zero(hipStream_t stream, float *p, size_t count);

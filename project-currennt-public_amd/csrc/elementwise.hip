@@ -166,13 +166,19 @@ int cnt_dense_forward(void *stream_, int P, int D, int N, int act, float bias, c
     return gemm_launch(static_cast<hipStream_t>(stream_), ga);
 }
 
-int cnt_dense_backward_errors(void *stream_, int P, int D, int N, int act, const float *weights, const float *y,
+int cnt_dense_backward_errors(void *stream, int P, int D, int N, int act, const float *weights, const float *y,
                               float *err, float *prev_err) {
-    using namespace cnt;
+    return cnt::dense_backward_errors_fan(static_cast<hipStream_t>(stream), P, D, N, act, weights, y, err, prev_err, nullptr,
+                                          nullptr);
+}
+
+extern "C++" int cnt::dense_backward_errors_fan(hipStream_t stream, int P, int D, int N, int act, const float *weights,
+                                                const float *y, float *err, float *prev_err, const FanOut *fan,
+                                                bool *fused) {
+    if (fused) *fused = false;
     CNT_REQUIRE(weights && y && err, "dense_backward_errors: null argument");
     CNT_REQUIRE(P > 0 && D > 0 && N > 0, "dense_backward_errors: non-positive size");
     CNT_REQUIRE(act >= 0 && act <= 3, "dense_backward_errors: unknown activation %d", act);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
     const size_t count = (size_t)D * N;
     if (act != ACT_IDENTITY) {
         ProfileScope prof(stream, "dense_delta");
@@ -189,37 +195,56 @@ int cnt_dense_backward_errors(void *stream_, int P, int D, int N, int act, const
         ga.ldc = P;
         ga.nseg = 1; ga.nprob = 1; ga.splitk = 1; ga.epilogue = EPI_STORE;
         ga.prob[0].A[0] = weights; ga.prob[0].B[0] = err; ga.prob[0].C = prev_err;
+        if (fan && fused && gemm_fan_supported(ga)) {
+            ga.epilogue = EPI_FAN;
+            ga.fan_n = fan->n; ga.fan_targets = fan->targets; ga.fan_is_skip = fan->is_skip;
+            ga.prob[0].aux_in = fan->from_skip;
+            *fused = true;
+        }
         ga.label = "gemm:dense_prev_errors";
         CNT_TRY(gemm_launch(stream, ga));
     }
     return CNT_OK;
 }
 
-int cnt_dense_backward_weights(void *stream_, int P, int D, int N, float bias, const float *x, const float *err,
+int cnt_dense_backward_weights(void *stream, int P, int D, int N, float bias, const float *x, const float *err,
                                float *weight_updates) {
-    using namespace cnt;
-    CNT_REQUIRE(x && err && weight_updates, "dense_backward_weights: null argument");
+    return cnt::dense_backward_weights_batch(static_cast<hipStream_t>(stream), P, D, N, 1, &bias, &x, &err,
+                                             &weight_updates);
+}
+
+extern "C++" int cnt::dense_backward_weights_batch(hipStream_t stream, int P, int D, int N, int count, const float *bias,
+                                                   const float *const *x, const float *const *err,
+                                                   float *const *weight_updates) {
+    CNT_REQUIRE(count >= 1 && count <= kGemmMaxProb, "dense_backward_weights: %d layers in one launch, supported 1..%d",
+                count, kGemmMaxProb);
+    CNT_REQUIRE(bias && x && err && weight_updates, "dense_backward_weights: null argument");
     CNT_REQUIRE(P > 0 && D > 0 && N > 0, "dense_backward_weights: non-positive size");
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
     GemmArgs ga = {};
     ga.m = P; ga.n = D; ga.k = N;
     ga.a_kcontig = 0; ga.lda = P;
     ga.b_kcontig = 0; ga.ldb = D;
     ga.ldc = P;
-    ga.nseg = 1; ga.nprob = 1; ga.epilogue = EPI_ATOMIC;
+    ga.nseg = 1; ga.nprob = count; ga.epilogue = EPI_ATOMIC;
     ga.splitk = 0;  // chosen by the launcher
-    ga.prob[0].A[0] = x; ga.prob[0].B[0] = err; ga.prob[0].C = weight_updates;
+    for (int z = 0; z < count; ++z) {
+        CNT_REQUIRE(x[z] && err[z] && weight_updates[z], "dense_backward_weights: null argument");
+        ga.prob[z].A[0] = x[z]; ga.prob[z].B[0] = err[z]; ga.prob[z].C = weight_updates[z];
+        ga.prob[z].rowsum_out = weight_updates[z] + (size_t)P * D;
+        ga.prob[z].rowsum_scale = bias[z];
+    }
     ga.label = "gemm:dense_dW";
     // narrow layers: the launcher sums partial products instead of adding atomically, which overwrites the
     // weight part and brings the bias part (row sums of the errors) along
     ga.overwrite_ok = 1;
-    ga.rowsum_out = weight_updates + (size_t)P * D;
-    ga.rowsum_scale = bias;
+    ga.rowsum = 1;
     gemm_plan(ga);
     if (ga.epilogue == EPI_PARTIAL) return gemm_launch(stream, ga);
-    CNT_TRY(fill_zero(stream, weight_updates, (size_t)P * D + D));
+    for (int z = 0; z < count; ++z) CNT_TRY(fill_zero(stream, weight_updates[z], (size_t)P * D + D));
     CNT_TRY(gemm_launch(stream, ga));
-    return column_sum(stream, err, D, N, bias, weight_updates + (size_t)P * D);
+    for (int z = 0; z < count; ++z)
+        CNT_TRY(column_sum(stream, err[z], D, N, bias[z], weight_updates[z] + (size_t)P * D));
+    return CNT_OK;
 }
 
 int cnt_dense_backward(void *stream, int P, int D, int N, int act, float bias, const float *weights, const float *x,

@@ -63,7 +63,7 @@ int pick_tile(const GemmArgs &a) {
 // small kernel sums the splits into C.  That also replaces the clearing launch in front of the atomic path and,
 // for dense layers, the separate column sum for the bias gradient (the splits carry the row sums of B along).
 constexpr size_t kSplitScratchFloats = (size_t)4 << 20;  // 16 MB per (device, stream)
-constexpr long kPartialMaxOutput = 64 << 10;             // floats of output (all problems) up to which it pays
+constexpr long kPartialMaxOutput = 128 << 10;            // floats of output (all problems) up to which it pays
 
 struct SplitScratch {
     int device;
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs args)
     const int tx = threadIdx.x % kReduceOutputs, g = threadIdx.x / kReduceOutputs;
     const size_t mn = (size_t)args.m * args.n;
     const size_t products = mn * args.nprob;
-    const size_t total = products + (args.rowsum_out ? (size_t)args.n : 0);
+    const size_t total = products + (args.rowsum ? (size_t)args.n * args.nprob : 0);
     const size_t e = (size_t)blockIdx.x * kReduceOutputs + tx;
     float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
     if (e < total) {
@@ -122,12 +122,17 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs args)
             const size_t z = e / mn, r = e % mn;
             args.prob[z].C[(r / args.m) * args.ldc + r % args.m] = v;
         } else {
-            args.rowsum_out[e - products] = args.rowsum_scale * v;
+            const size_t z = (e - products) / args.n, j = (e - products) % args.n;
+            args.prob[z].rowsum_out[j] = args.prob[z].rowsum_scale * v;
         }
     }
 }
 
 }  // namespace
+
+bool gemm_fan_supported(const GemmArgs &a) {
+    return !a.a_kcontig && a.b_kcontig && a.nprob == 1 && pick_vec(a, true) == 4 && pick_vec(a, false) == 4;
+}
 
 void gemm_release_stream(hipStream_t stream) {
     int dev = 0;
@@ -158,14 +163,14 @@ void gemm_plan(GemmArgs &args) {
     args.splitk = (int)s;
     static const bool partial_on = [] { const char *e = std::getenv("CNT_GEMM_PARTIAL"); return !e || std::atoi(e) != 0; }();
     const long out = (long)args.m * args.n * args.nprob;
-    const size_t stride = (size_t)out + (args.rowsum_out ? (size_t)args.n : 0);
-    const bool rowsum_ok = !args.rowsum_out || (args.nprob == 1 && args.nseg == 1 && !args.masked);
+    const size_t stride = (size_t)out + (args.rowsum ? (size_t)args.n * args.nprob : 0);
+    const bool rowsum_ok = !args.rowsum || (args.nseg == 1 && !args.masked);
     if (partial_on && args.epilogue == EPI_ATOMIC && args.overwrite_ok && rowsum_ok && s >= 8 &&
         out <= kPartialMaxOutput && stride * (size_t)s <= kSplitScratchFloats) {
         args.epilogue = EPI_PARTIAL;
         args.partial_stride = stride;
     } else {
-        args.rowsum_out = nullptr;  // the caller sums the rows itself
+        args.rowsum = 0;  // the caller sums the rows itself
     }
 }
 
@@ -179,6 +184,8 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
                 args.nprob, kGemmMaxProb);
     CNT_REQUIRE(args.splitk >= 0 && (args.splitk == 1 || args.epilogue == EPI_ATOMIC || args.epilogue == EPI_PARTIAL),
                 "gemm: split-K needs the atomic epilogue");
+    CNT_REQUIRE(args.epilogue != EPI_FAN || (gemm_fan_supported(args) && args.splitk == 1),
+                "gemm: the fan epilogue exists for one unsplit problem with 16-byte row-contiguous A and k-contiguous B");
     CNT_REQUIRE(args.epilogue != EPI_PARTIAL || (args.splitk >= 1 && args.partial_stride > 0),
                 "gemm: the partial-product epilogue is chosen by gemm_plan only");
     for (int p = 0; p < args.nprob; ++p) {
@@ -188,7 +195,7 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
     }
     const int va = pick_vec(args, true), vb = pick_vec(args, false);
     gemm_plan(args);
-    if (args.epilogue != EPI_PARTIAL) args.rowsum_out = nullptr;
+    if (args.epilogue != EPI_PARTIAL) args.rowsum = 0;
     const int tile = pick_tile(args);
     const int tiles = ((args.m + tile - 1) / tile) * ((args.n + tile - 1) / tile);
     dim3 grid(tiles, args.splitk, args.nprob);

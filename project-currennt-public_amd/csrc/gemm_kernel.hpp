@@ -160,7 +160,9 @@ struct TileStage {
 // MASKED selects the time-shifted, padding-masked B loader at compile time: its per-element predication is a lot
 // of code, and four copies of it (two prologue fetches, two in the unrolled loop) inside the plain kernels would
 // push their hot loop out of the instruction cache.
-template <int VA, bool AK, int VB, bool BK_, bool MASKED, int TILE>
+// FAN: the EPI_FAN epilogue, a kernel of its own (instantiated for 16-byte row-contiguous A and k-contiguous B only,
+// the shapes of the error products that use it) so that its registers and code stay out of every other product.
+template <int VA, bool AK, int VB, bool BK_, bool MASKED, int TILE, bool FAN = false>
 __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args) {
     constexpr int BM = TILE, BN = TILE;
     constexpr int WT = TILE / 2;   // edge of a wave's block (waves are arranged 2 x 2)
@@ -212,7 +214,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     };
 
     // sum of the B operand over this split's k range, per row (dense bias gradient); kept by the waves with wm == 0
-    const bool rowsum = args.rowsum_out != nullptr;
+    const bool rowsum = args.rowsum != 0;
     float rs[NB];
 #pragma unroll
     for (int j = 0; j < NB; ++j) rs[j] = 0.0f;
@@ -290,12 +292,53 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
         }
         if (rowsum && wm == 0 && m0 == 0) {
             float *__restrict__ R = args.partial + (size_t)blockIdx.y * args.partial_stride +
-                                    (size_t)args.nprob * args.m * args.n;
+                                    (size_t)args.nprob * args.m * args.n + (size_t)blockIdx.z * args.n;
 #pragma unroll
             for (int j = 0; j < NB; ++j) {
                 const float s = rs[j] + __shfl_xor(rs[j], 32);
                 const int n = n0 + wn * WT + j * 32 + frag_row;
                 if (half == 0 && n < args.n) R[n] = s;
+            }
+        }
+        return;
+    }
+    if (FAN) {
+        // All loads of a 32 x 32 tile's sixteen values per lane are issued before anything is stored: the compiler
+        // cannot know that the buffers do not overlap and would otherwise wait for memory once per value.
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            const int m = m0 + wm * WT + i * 32 + frag_row;
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                size_t idx[16];
+                bool ok[16];
+                float e[16], old[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int n = n0 + wn * WT + j * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    ok[r] = m < args.m && n < args.n;
+                    idx[r] = ok[r] ? (size_t)n * args.ldc + m : 0;
+                    old[r] = (ok[r] && pb.aux_in) ? pb.aux_in[idx[r]] : 0.0f;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    e[r] = pb.aux_in ? old[r] + acc[i][j][r] : acc[i][j][r];
+                    if (ok[r]) C[idx[r]] = e[r];
+                }
+                for (int q = 0; q < args.fan_n; ++q) {
+                    float *__restrict__ t = args.fan_targets[q];
+                    if (args.fan_is_skip[q]) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) old[r] = ok[r] ? t[idx[r]] : 0.0f;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            if (ok[r]) t[idx[r]] = e[r] + old[r];
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            if (ok[r]) t[idx[r]] = e[r];
+                    }
+                }
             }
         }
         return;
@@ -320,6 +363,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
                     case EPI_STORE: *dst = v; break;
                     case EPI_ADD: *dst = *dst + v; break;
                     case EPI_ATOMIC: atomicAdd(dst, v); break;
+
                     case EPI_BIAS_ACT: *dst = act_fn(args.act, v + bterm); break;
                     case EPI_BIAS_ACT_SKIP:
                         if (args.pat[n] != 0) *dst = act_fn(args.act, v + bterm);
@@ -338,6 +382,16 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
 
 template <int VA, bool AK, int VB, bool BK_, int TILE>
 void launch_m(const GemmArgs &a, dim3 grid, hipStream_t s) {
+    if (a.epilogue == EPI_FAN) {
+        // gemm_launch has checked that the operands are of the one kind this exists for
+        if constexpr (VA == 4 && !AK && VB == 4 && BK_) {
+            if (a.masked)
+                hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, true, TILE, true>), grid, dim3(NTHREADS), 0, s, a);
+            else
+                hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, false, TILE, true>), grid, dim3(NTHREADS), 0, s, a);
+        }
+        return;
+    }
     if (a.masked) hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, true, TILE>), grid, dim3(NTHREADS), 0, s, a);
     else hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, false, TILE>), grid, dim3(NTHREADS), 0, s, a);
 }

@@ -1287,6 +1287,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     // after the layer's error half.  Handing work to another stream costs the host two event calls; a network of
     // many small layers cannot afford them per layer (the host's enqueue rate then bounds its backward pass), so the
     // weight halves of small layers are collected and handed over a few at a time, those of large layers at once.
+    std::vector<char> fan_done(net->layers.size(), 0);
     std::vector<size_t> pending;
     auto weight_half = [&](size_t i, hipStream_t ws) -> int {
         NetLayer &L = net->layers[i];
@@ -1298,15 +1299,64 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
         if (L.kind == K_CNN) return cnt_cnn_backward_weights(L.cnn, ws, L.pat, L.T, prev.out, L.err, dW);
         return cnt_wavnetc_backward_weights(ws, L.size, L.ctx_dim, L.N, net->ctx, L.cth, dW);
     };
-    auto hand_over = [&]() -> int {
-        if (pending.empty()) return CNT_OK;
-        hipStream_t ws = net->side[next_side];
+    auto next_side_stream = [&](hipStream_t *ws) -> int {
+        *ws = net->side[next_side];
         CNT_HIP(hipEventRecord(net->ev_main, stream));
-        CNT_HIP(hipStreamWaitEvent(ws, net->ev_main, 0));
+        CNT_HIP(hipStreamWaitEvent(*ws, net->ev_main, 0));
         side_used[next_side] = true;
         next_side = (next_side + 1) % net->n_side;
+        return CNT_OK;
+    };
+    auto hand_over = [&]() -> int {
+        if (pending.empty()) return CNT_OK;
+        hipStream_t ws;
+        CNT_TRY(next_side_stream(&ws));
         for (size_t i : pending) CNT_TRY(weight_half(i, ws));
         pending.clear();
+        return CNT_OK;
+    };
+    // Small dense and wavnetc layers of one shape (the 1x1 layers and the conditioning projections of a stack of
+    // identical blocks) wait for each other: eight of them are the problems of ONE product launch, which gives each
+    // workgroup a k range eight times as long as a launch per layer would.  A layer's deltas, its input and its
+    // tanh(context) buffer are final once its error half has run and stay untouched until the next pass, so the
+    // weight half can wait for as long as the pass lasts.
+    struct ShapeGroup {
+        int kind, a, b, n;
+        std::vector<size_t> layers;
+    };
+    std::vector<ShapeGroup> groups;
+    auto hand_over_group = [&](ShapeGroup &g) -> int {
+        if (g.layers.empty()) return CNT_OK;
+        hipStream_t ws;
+        CNT_TRY(next_side_stream(&ws));
+        const int count = (int)g.layers.size();
+        const float *in0[kGemmMaxProb], *in1[kGemmMaxProb];
+        float *dW[kGemmMaxProb], bias[kGemmMaxProb];
+        for (int z = 0; z < count; ++z) {
+            NetLayer &L = net->layers[g.layers[(size_t)z]];
+            NetLayer &prev = net->layers[g.layers[(size_t)z] - 1];
+            dW[z] = net->updates + L.w_off;
+            bias[z] = L.bias;
+            in0[z] = g.kind == K_DENSE ? prev.out : L.cth;
+            in1[z] = L.err;
+        }
+        g.layers.clear();
+        if (g.kind == K_DENSE) return dense_backward_weights_batch(ws, g.a, g.b, g.n, count, bias, in0, in1, dW);
+        return wavnetc_backward_weights_batch(ws, g.a, g.b, g.n, count, net->ctx, in0, dW);
+    };
+    auto join_group = [&](size_t i) -> int {
+        NetLayer &L = net->layers[i];
+        const int a = L.kind == K_DENSE ? net->layers[i - 1].size : L.size;
+        const int b = L.kind == K_DENSE ? L.size : L.ctx_dim;
+        ShapeGroup *g = nullptr;
+        for (ShapeGroup &c : groups)
+            if (c.kind == L.kind && c.a == a && c.b == b && c.n == L.N) g = &c;
+        if (!g) {
+            groups.push_back({L.kind, a, b, L.N, {}});
+            g = &groups.back();
+        }
+        g->layers.push_back(i);
+        if ((int)g->layers.size() == kGemmMaxProb) CNT_TRY(hand_over_group(*g));
         return CNT_OK;
     };
     for (size_t i = net->layers.size() - 1; i >= 1; --i) {
@@ -1343,13 +1393,28 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
             case K_LSTM:
             case K_CNN:
             case K_WAVNETC:
-                if (L.kind == K_DENSE)
-                    CNT_TRY(cnt_dense_backward_errors(stream, prev.size, L.size, N, L.act, W, L.out, L.err, prev_err));
-                else if (L.kind == K_LSTM)
+                if (L.kind == K_DENSE || L.kind == K_CNN) {
+                    // a skip layer in front, whose errors this layer's product writes: its backward step (add the side
+                    // buffer, hand the sum on) rides in the product's epilogue, and its own launch below is left out
+                    FanOut fan = {};
+                    const bool wanted = is_sum_skip(prev.kind) && prev_err && prev_err == prev.total && prev.N == N &&
+                                        (prev.needs_sum || prev.live_targets > 0);
+                    if (wanted) {
+                        fan.n = prev.live_targets;
+                        fan.targets = prev.tgt_ptrs;
+                        fan.is_skip = prev.tgt_is_skip;
+                        fan.from_skip = prev.needs_sum ? prev.eskip : nullptr;
+                    }
+                    bool fused = false;
+                    if (L.kind == K_DENSE)
+                        CNT_TRY(dense_backward_errors_fan(stream, prev.size, L.size, N, L.act, W, L.out, L.err, prev_err,
+                                                          wanted ? &fan : nullptr, &fused));
+                    else
+                        CNT_TRY(cnn_backward_errors_fan(L.cnn, stream, L.pat, L.T, W, L.out, L.err, prev_err,
+                                                        L.delta_fused ? 1 : 0, wanted ? &fan : nullptr, &fused));
+                    fan_done[i - 1] = fused ? 1 : 0;
+                } else if (L.kind == K_LSTM)
                     CNT_TRY(cnt_lstm_backward_errors(L.lstm, stream, W, L.err, prev_err));
-                else if (L.kind == K_CNN)
-                    CNT_TRY(cnt_cnn_backward_errors(L.cnn, stream, L.pat, L.T, W, L.out, L.err, prev_err,
-                                                    L.delta_fused ? 1 : 0));
                 else {
                     CNT_TRY(cnt_wavnetc_backward_errors(stream, L.size, L.ctx_dim, N, L.pat, W, L.core, L.cth, L.err,
                                                         prev.err, net->flagged >= 0 ? net->ctx_grad : nullptr,
@@ -1367,6 +1432,10 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                     CNT_TRY(weight_half(i, stream));
                     break;
                 }
+                if ((L.kind == K_DENSE || L.kind == K_WAVNETC) && (double)prev.size * L.size * N < 4e8) {
+                    CNT_TRY(join_group(i));
+                    break;
+                }
                 pending.push_back(i);
                 {
                     // small: below 4e8 multiply-adds (a WaveNet block's 64..128-wide layers over 32 000 samples are
@@ -1379,6 +1448,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
             case K_SKIPINI:
             case K_SKIPADD: {
                 if (!L.needs_sum && L.live_targets == 0) break;
+                if (fan_done[i]) break;  // done in the epilogue of the following layer's product
                 ProfileScope prof(stream, "skip_fan");
                 const float *from_skip = L.needs_sum ? L.eskip : static_cast<const float *>(nullptr);
                 if (L.ptrs_aligned && count % 4 == 0)
@@ -1426,6 +1496,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
         }
     }
     CNT_TRY(hand_over());
+    for (ShapeGroup &g : groups) CNT_TRY(hand_over_group(g));
     for (int k = 0; k < net->n_side; ++k) {
         if (!side_used[k]) continue;
         CNT_HIP(hipEventRecord(net->ev_side[k], net->side[k]));

@@ -309,12 +309,18 @@ int cnt_cnn_forward(cnt_cnn *h, void *stream_, const char *patTypes, int curT, c
     return CNT_OK;
 }
 
-int cnt_cnn_backward_errors(cnt_cnn *h, void *stream_, const char *patTypes, int curT, const float *weights,
+int cnt_cnn_backward_errors(cnt_cnn *h, void *stream, const char *patTypes, int curT, const float *weights,
                             const float *outputs, float *output_errors, float *prev_errors, int delta_applied) {
-    using namespace cnt;
+    return cnt::cnn_backward_errors_fan(h, static_cast<hipStream_t>(stream), patTypes, curT, weights, outputs, output_errors,
+                                        prev_errors, delta_applied, nullptr, nullptr);
+}
+
+extern "C++" int cnt::cnn_backward_errors_fan(cnt_cnn *h, hipStream_t stream, const char *patTypes, int curT,
+                                              const float *weights, const float *outputs, float *output_errors,
+                                              float *prev_errors, int delta_applied, const FanOut *fan, bool *fused) {
+    if (fused) *fused = false;
     CNT_REQUIRE(h && patTypes && weights && outputs && output_errors, "cnn_backward_errors: null argument");
     CNT_REQUIRE(curT >= 1 && curT <= h->desc.maxT, "cnn_backward_errors: curT %d outside 1..%d", curT, h->desc.maxT);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
     const cnt_cnn_desc &d = h->desc;
     const int P = d.P, D = d.D, S = d.S, N = curT * S;
     const size_t count = (size_t)D * N;
@@ -349,6 +355,12 @@ int cnt_cnn_backward_errors(cnt_cnn *h, void *stream_, const char *patTypes, int
             }
             ga.nseg = seg;
             ga.prob[0].C = prev_errors;
+            if (fan && fused && h->groups.size() == 1 && gemm_fan_supported(ga)) {
+                ga.epilogue = EPI_FAN;
+                ga.fan_n = fan->n; ga.fan_targets = fan->targets; ga.fan_is_skip = fan->is_skip;
+                ga.prob[0].aux_in = fan->from_skip;
+                *fused = true;
+            }
             ga.label = "gemm:cnn_prev_errors";
             CNT_TRY(gemm_launch(stream, ga));
             first = false;
@@ -498,25 +510,34 @@ int cnt_wavnetc_backward_errors(void *stream_, int D, int C, int N, const char *
     return CNT_OK;
 }
 
-int cnt_wavnetc_backward_weights(void *stream_, int D, int C, int N, const float *ctx, const float *ctx_tanh,
+int cnt_wavnetc_backward_weights(void *stream, int D, int C, int N, const float *ctx, const float *ctx_tanh,
                                  float *weight_updates) {
-    using namespace cnt;
+    return cnt::wavnetc_backward_weights_batch(static_cast<hipStream_t>(stream), D, C, N, 1, ctx, &ctx_tanh, &weight_updates);
+}
+
+extern "C++" int cnt::wavnetc_backward_weights_batch(hipStream_t stream, int D, int C, int N, int count, const float *ctx,
+                                                     const float *const *ctx_tanh, float *const *weight_updates) {
+    CNT_REQUIRE(count >= 1 && count <= kGemmMaxProb, "wavnetc_backward_weights: %d layers in one launch, supported 1..%d",
+                count, kGemmMaxProb);
     CNT_REQUIRE(D > 0 && N > 0 && C >= 0, "wavnetc_backward_weights: bad size");
     if (C == 0) return CNT_OK;
     CNT_REQUIRE(ctx && ctx_tanh && weight_updates, "wavnetc_backward_weights: null argument");
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
     GemmArgs ga = {};
     ga.m = C; ga.n = 2 * D; ga.k = N;
     ga.a_kcontig = 0; ga.lda = C;
     ga.b_kcontig = 0; ga.ldb = 2 * D;
     ga.ldc = C;
-    ga.nseg = 1; ga.nprob = 1; ga.epilogue = EPI_ATOMIC;
+    ga.nseg = 1; ga.nprob = count; ga.epilogue = EPI_ATOMIC;
     ga.splitk = 0;  // chosen by the launcher
-    ga.prob[0].A[0] = ctx; ga.prob[0].B[0] = ctx_tanh; ga.prob[0].C = weight_updates;
+    for (int z = 0; z < count; ++z) {
+        CNT_REQUIRE(ctx_tanh[z] && weight_updates[z], "wavnetc_backward_weights: null argument");
+        ga.prob[z].A[0] = ctx; ga.prob[z].B[0] = ctx_tanh[z]; ga.prob[z].C = weight_updates[z];
+    }
     ga.label = "gemm:wavnetc_dW";
     ga.overwrite_ok = 1;  // the product covers all C x 2D weights
     gemm_plan(ga);
-    if (ga.epilogue != EPI_PARTIAL) CNT_TRY(fill_zero(stream, weight_updates, (size_t)C * 2 * D));
+    if (ga.epilogue != EPI_PARTIAL)
+        for (int z = 0; z < count; ++z) CNT_TRY(fill_zero(stream, weight_updates[z], (size_t)C * 2 * D));
     return gemm_launch(stream, ga);
 }
 
