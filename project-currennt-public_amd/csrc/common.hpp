@@ -210,6 +210,13 @@ int dense_backward_weights_batch(hipStream_t stream, int P, int D, int N, int co
                                  const float *const *x, const float *const *err, float *const *weight_updates);
 int wavnetc_backward_weights_batch(hipStream_t stream, int D, int C, int N, int count, const float *ctx,
                                    const float *const *ctx_tanh, float *const *weight_updates);
+// Convolution layers with one filter group each and the same sizes, window and causality (dilations may differ):
+// cnn_batch_taps gives the live taps of such a layer (0: not batchable, several filter groups), and `count` layers
+// with count * taps <= kGemmMaxProb go into one product.
+int cnn_batch_taps(const cnt_cnn *h);
+bool cnn_batch_compatible(const cnt_cnn *a, const cnt_cnn *b);
+int cnn_backward_weights_batch(cnt_cnn *const *h, int count, hipStream_t stream, const char *patTypes, int curT,
+                               const float *const *x, const float *const *output_errors, float *const *weight_updates);
 
 // ----- small streaming kernels (elementwise.hip) ----------------------------------------------------
 int fill_zero(hipStream_t stream, float *p, size_t count);

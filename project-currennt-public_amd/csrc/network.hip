@@ -1321,7 +1321,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     // tanh(context) buffer are final once its error half has run and stay untouched until the next pass, so the
     // weight half can wait for as long as the pass lasts.
     struct ShapeGroup {
-        int kind, a, b, n;
+        int kind, a, b, n, cap;
         std::vector<size_t> layers;
     };
     std::vector<ShapeGroup> groups;
@@ -1332,16 +1332,20 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
         const int count = (int)g.layers.size();
         const float *in0[kGemmMaxProb], *in1[kGemmMaxProb];
         float *dW[kGemmMaxProb], bias[kGemmMaxProb];
+        cnt_cnn *cnn[kGemmMaxProb];
+        const NetLayer &first = net->layers[g.layers[0]];
         for (int z = 0; z < count; ++z) {
             NetLayer &L = net->layers[g.layers[(size_t)z]];
             NetLayer &prev = net->layers[g.layers[(size_t)z] - 1];
             dW[z] = net->updates + L.w_off;
             bias[z] = L.bias;
-            in0[z] = g.kind == K_DENSE ? prev.out : L.cth;
+            in0[z] = g.kind == K_WAVNETC ? L.cth : prev.out;
             in1[z] = L.err;
+            cnn[z] = L.cnn;
         }
         g.layers.clear();
         if (g.kind == K_DENSE) return dense_backward_weights_batch(ws, g.a, g.b, g.n, count, bias, in0, in1, dW);
+        if (g.kind == K_CNN) return cnn_backward_weights_batch(cnn, count, ws, first.pat, first.T, in0, in1, dW);
         return wavnetc_backward_weights_batch(ws, g.a, g.b, g.n, count, net->ctx, in0, dW);
     };
     auto join_group = [&](size_t i) -> int {
@@ -1349,14 +1353,22 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
         const int a = L.kind == K_DENSE ? net->layers[i - 1].size : L.size;
         const int b = L.kind == K_DENSE ? L.size : L.ctx_dim;
         ShapeGroup *g = nullptr;
-        for (ShapeGroup &c : groups)
-            if (c.kind == L.kind && c.a == a && c.b == b && c.n == L.N) g = &c;
+        for (ShapeGroup &c : groups) {
+            if (c.kind != L.kind || c.a != a || c.b != b || c.n != L.N) continue;
+            if (L.kind == K_CNN && !c.layers.empty()) {
+                // same time base and pattern types, same window: only the dilation may differ
+                const NetLayer &o = net->layers[c.layers[0]];
+                if (o.pat != L.pat || o.T != L.T || !cnn_batch_compatible(o.cnn, L.cnn)) continue;
+            }
+            g = &c;
+        }
         if (!g) {
-            groups.push_back({L.kind, a, b, L.N, {}});
+            const int cap = L.kind == K_CNN ? kGemmMaxProb / cnn_batch_taps(L.cnn) : kGemmMaxProb;
+            groups.push_back({L.kind, a, b, L.N, cap, {}});
             g = &groups.back();
         }
         g->layers.push_back(i);
-        if ((int)g->layers.size() == kGemmMaxProb) CNT_TRY(hand_over_group(*g));
+        if ((int)g->layers.size() >= g->cap) CNT_TRY(hand_over_group(*g));
         return CNT_OK;
     };
     for (size_t i = net->layers.size() - 1; i >= 1; --i) {
@@ -1432,7 +1444,9 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                     CNT_TRY(weight_half(i, stream));
                     break;
                 }
-                if ((L.kind == K_DENSE || L.kind == K_WAVNETC) && (double)prev.size * L.size * N < 4e8) {
+                if ((L.kind == K_DENSE || L.kind == K_WAVNETC ||
+                     (L.kind == K_CNN && cnn_batch_taps(L.cnn) > 0 && cnn_batch_taps(L.cnn) <= kGemmMaxProb / 2)) &&
+                    (double)prev.size * L.size * N < 4e8) {
                     CNT_TRY(join_group(i));
                     break;
                 }

@@ -369,6 +369,65 @@ extern "C++" int cnt::cnn_backward_errors_fan(cnt_cnn *h, hipStream_t stream, co
     return CNT_OK;
 }
 
+extern "C++" int cnt::cnn_batch_taps(const cnt_cnn *h) {
+    if (!h || h->groups.size() != 1) return 0;
+    const cnt_cnn_group &g = h->groups[0];
+    return h->desc.causal > 0 ? g.hw + 1 : 2 * g.hw + 1;
+}
+
+extern "C++" bool cnt::cnn_batch_compatible(const cnt_cnn *a, const cnt_cnn *b) {
+    if (cnn_batch_taps(a) == 0 || cnn_batch_taps(a) != cnn_batch_taps(b)) return false;
+    const cnt_cnn_group &ga = a->groups[0], &gb = b->groups[0];
+    return a->desc.P == b->desc.P && a->desc.D == b->desc.D && a->desc.S == b->desc.S && a->Lw == b->Lw &&
+           (a->desc.causal > 0) == (b->desc.causal > 0) && ga.hw == gb.hw && ga.d0 == gb.d0 && ga.d1 == gb.d1 &&
+           ga.col0 == gb.col0;
+}
+
+extern "C++" int cnt::cnn_backward_weights_batch(cnt_cnn *const *h, int count, hipStream_t stream, const char *patTypes,
+                                                 int curT, const float *const *x, const float *const *output_errors,
+                                                 float *const *weight_updates) {
+    CNT_REQUIRE(h && patTypes && x && output_errors && weight_updates && count >= 1, "cnn_backward_weights: null argument");
+    const int taps = cnn_batch_taps(h[0]);
+    CNT_REQUIRE(taps > 0 && count * taps <= kGemmMaxProb, "cnn_backward_weights: %d layers of %d taps in one launch", count,
+                taps);
+    for (int z = 0; z < count; ++z) {
+        CNT_REQUIRE(cnn_batch_compatible(h[0], h[z]), "cnn_backward_weights: layers of different shapes in one launch");
+        CNT_REQUIRE(x[z] && output_errors[z] && weight_updates[z], "cnn_backward_weights: null argument");
+        CNT_REQUIRE(curT >= 1 && curT <= h[z]->desc.maxT, "cnn_backward_weights: curT %d outside 1..%d", curT,
+                    h[z]->desc.maxT);
+    }
+    const cnt_cnn_desc &d = h[0]->desc;
+    const cnt_cnn_group &g0 = h[0]->groups[0];
+    const int P = d.P, D = d.D, S = d.S, N = curT * S;
+    for (int z = 0; z < count; ++z) CNT_TRY(fill_zero(stream, weight_updates[z], (size_t)P * h[z]->Lw + D));
+    GemmArgs ga = {};
+    ga.m = P; ga.n = g0.d1 - g0.d0; ga.k = N;
+    ga.a_kcontig = 0; ga.lda = P;
+    ga.b_kcontig = 0; ga.ldb = D;
+    ga.ldc = (2 * g0.hw + 1) * P;
+    ga.nseg = 1;
+    ga.epilogue = EPI_ATOMIC;
+    ga.masked = 1; ga.b_time_on_k = 1; ga.n_slots = N; ga.pat = patTypes;
+    int pr = 0;
+    for (int z = 0; z < count; ++z) {
+        const cnt_cnn_group &g = h[z]->groups[0];
+        for (int shift = -g.hw; shift <= (d.causal > 0 ? 0 : g.hw); ++shift, ++pr) {
+            ga.prob[pr].A[0] = x[z];
+            ga.prob[pr].B[0] = output_errors[z] + g.d0;
+            ga.prob[pr].b_shift[0] = -shift * g.dil * S;
+            ga.prob[pr].C = weight_updates[z] + (size_t)(g.col0 + g.hw + shift) * P;
+        }
+    }
+    ga.nprob = pr;
+    ga.splitk = 0;  // chosen by the launcher
+    ga.overwrite_ok = 1;
+    ga.label = "gemm:cnn_dW";
+    CNT_TRY(gemm_launch(stream, ga));
+    for (int z = 0; z < count; ++z)
+        CNT_TRY(column_sum(stream, output_errors[z], D, N, h[z]->desc.bias, weight_updates[z] + (size_t)P * h[z]->Lw));
+    return CNT_OK;
+}
+
 int cnt_cnn_backward_weights(cnt_cnn *h, void *stream_, const char *patTypes, int curT, const float *x,
                              const float *output_errors, float *weight_updates) {
     using namespace cnt;
