@@ -466,7 +466,7 @@ struct cnt_network {
     static constexpr int kMaxSide = 4;
     hipStream_t side[kMaxSide] = {};
     hipEvent_t ev_main = nullptr, ev_side[kMaxSide] = {};
-    int n_side = 2;
+    int n_side = 3;
     int overlap = 1;
     // optimizer state (allocated by the first update)
     float *cur_updates = nullptr, *deltas = nullptr, *stats = nullptr;
@@ -1299,18 +1299,26 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
         if (L.kind == K_CNN) return cnt_cnn_backward_weights(L.cnn, ws, L.pat, L.T, prev.out, L.err, dW);
         return cnt_wavnetc_backward_weights(ws, L.size, L.ctx_dim, L.N, net->ctx, L.cth, dW);
     };
-    auto next_side_stream = [&](hipStream_t *ws) -> int {
-        *ws = net->side[next_side];
+    // Large layers' weight halves go round-robin over all side streams, the collected small ones over the first two:
+    // measured on MI355X, a third stream gains 1% on the acoustic model (its last recurrent layer's and the dense
+    // layers' weight gradients end the pass side by side) and loses 2% on the WaveNet stack (three batched products
+    // at once crowd the error chain on the main stream).
+    int next_small = 0;
+    auto next_side_stream = [&](hipStream_t *ws, bool large) -> int {
+        int &cursor = large ? next_side : next_small;
+        const int span = large ? net->n_side : std::min(net->n_side, 2);
+        cursor %= span;
+        *ws = net->side[cursor];
         CNT_HIP(hipEventRecord(net->ev_main, stream));
         CNT_HIP(hipStreamWaitEvent(*ws, net->ev_main, 0));
-        side_used[next_side] = true;
-        next_side = (next_side + 1) % net->n_side;
+        side_used[cursor] = true;
+        cursor = (cursor + 1) % span;
         return CNT_OK;
     };
-    auto hand_over = [&]() -> int {
+    auto hand_over = [&](bool large) -> int {
         if (pending.empty()) return CNT_OK;
         hipStream_t ws;
-        CNT_TRY(next_side_stream(&ws));
+        CNT_TRY(next_side_stream(&ws, large));
         for (size_t i : pending) CNT_TRY(weight_half(i, ws));
         pending.clear();
         return CNT_OK;
@@ -1328,7 +1336,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     auto hand_over_group = [&](ShapeGroup &g) -> int {
         if (g.layers.empty()) return CNT_OK;
         hipStream_t ws;
-        CNT_TRY(next_side_stream(&ws));
+        CNT_TRY(next_side_stream(&ws, false));
         const int count = (int)g.layers.size();
         const float *in0[kGemmMaxProb], *in1[kGemmMaxProb];
         float *dW[kGemmMaxProb], bias[kGemmMaxProb];
@@ -1456,7 +1464,8 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                     // 1.6-2.6e8, the acoustic model's dense layers over 5 880 frames 5.6e8 and more); four at a time
                     // measured best on the 30-block WaveNet stack (5.36 -> 5.23 ms; two: no gain, eight: 5.31 ms)
                     const double macs = (double)prev.size * L.size * N;
-                    if (L.kind == K_LSTM || macs >= 4e8 || pending.size() >= 4) CNT_TRY(hand_over());
+                    const bool large = L.kind == K_LSTM || macs >= 4e8;
+                    if (large || pending.size() >= 4) CNT_TRY(hand_over(large));
                 }
                 break;
             case K_SKIPINI:
@@ -1509,7 +1518,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 break;
         }
     }
-    CNT_TRY(hand_over());
+    CNT_TRY(hand_over(false));
     for (ShapeGroup &g : groups) CNT_TRY(hand_over_group(g));
     for (int k = 0; k < net->n_side; ++k) {
         if (!side_used[k]) continue;
