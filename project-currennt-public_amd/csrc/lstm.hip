@@ -174,9 +174,6 @@ __global__ __launch_bounds__(fwd_threads(JB, NT)) void lstm_forward_chain(const 
 
     int dir, me;
     if (!map_block(p, G, dir, me)) return;
-    // The recursion is the critical path of a backward (forward) pass, and other streams' products share its compute
-    // units meanwhile: its waves go first wherever they compete for an issue slot.
-    __builtin_amdgcn_s_setprio(3);
     const DirPtrs &D = p.d[dir];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int S = p.S, T = p.T;
@@ -472,9 +469,6 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
 
     int dir, me;
     if (!map_block(p, G, dir, me)) return;
-    // The recursion is the critical path of a backward (forward) pass, and other streams' products share its compute
-    // units meanwhile: its waves go first wherever they compete for an issue slot.
-    __builtin_amdgcn_s_setprio(3);
     const DirPtrs &D = p.d[dir];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int S = p.S, T = p.T;
