@@ -74,9 +74,12 @@ def run(args, pkg):
         nbytes = 2 * (R + 2 * R) * 4.0 * N
     elif dom == "gemm:cnn_prev_errors":
         nbytes = (2 * 2 * R + R) * 4.0 * N
-    elif dom == "gemm:dense_dW":
-        # average over the stack's dense layers (30 x 64->64, 30 x 64->128, the 1024->64 embedding, 128->128, 128->1024)
-        nbytes = sum(dense_rows) / len(dense_rows) * 4.0 * N
+    elif dom in ("gemm:dense_dW", "gemm:dense_prev_errors"):
+        # average over the stack's dense layers (30 x 64->64, 30 x 64->128, the 1024->64 embedding, 128->128, 128->1024):
+        # the weight gradient reads a layer's input and deltas, the error product reads the deltas and writes the
+        # preceding layer's errors (the skip layer's step in its epilogue is not counted), over the launches made
+        # (weight gradients: eight layers per launch)
+        nbytes = sum(dense_rows) * 4.0 * N / kernels[dom]["launches"]
     else:
         nbytes = 155e3 * N / max(1, sum(v["launches"] for v in kernels.values()))
     roof["achieved"] = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
