@@ -334,7 +334,7 @@ typedef struct {
     const float *mdn_config; /* content of the --mdn_config file (see cnt_mdn_create); NULL without an mdn layer */
     int mdn_config_len;
     int tie_variance;        /* --tieVariance; only 0 is supported                                               */
-    int no_overlap;          /* != 0: weight gradients on the caller's stream instead of a second stream         */
+    int no_overlap;          /* != 0: weight gradients on the caller's stream instead of streams of the network's */
 } cnt_network_options;
 typedef struct {
     char name[64];
@@ -379,9 +379,10 @@ int cnt_network_load_sequences(cnt_network *net, void *stream, int T, int Tmin, 
 int cnt_network_forward(cnt_network *net, void *stream);
 /* NeuralNetwork::calculateError (NeuralNetwork.cpp:2897-2990): the post-output layer's error into *loss_dev. */
 int cnt_network_calculate_error(cnt_network *net, void *stream, float *loss_dev);
-/* NeuralNetwork::computeBackwardPass (NeuralNetwork.cpp:2744-2800, :2864-2895): layers in reverse order; on
- * return the caller's stream has been made to wait for the second stream, so weight updates are complete in
- * stream order. */
+/* NeuralNetwork::computeBackwardPass (NeuralNetwork.cpp:2744-2800, :2864-2895): layers in reverse order.  The
+ * layers' weight gradients run on streams of the network's own (same priority as any other stream), ordered after
+ * the error computations they depend on; small layers of one shape share a launch.  On return the caller's stream
+ * has been made to wait for those streams, so weight updates are complete in stream order. */
 int cnt_network_backward(cnt_network *net, void *stream);
 /* cnt_lstm_check for every LSTM layer. */
 int cnt_network_check(cnt_network *net, void *stream);
