@@ -1377,6 +1377,11 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
         }
         g->layers.push_back(i);
         if ((int)g->layers.size() >= g->cap) CNT_TRY(hand_over_group(*g));
+        // a network of many small layers that do not share shapes: do not let all of them wait for the pass's end
+        size_t waiting = 0;
+        for (const ShapeGroup &c : groups) waiting += c.layers.size();
+        if (waiting >= 32)
+            for (ShapeGroup &c : groups) CNT_TRY(hand_over_group(c));
         return CNT_OK;
     };
     for (size_t i = net->layers.size() - 1; i >= 1; --i) {
