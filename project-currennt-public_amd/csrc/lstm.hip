@@ -99,11 +99,10 @@ __device__ __forceinline__ bool map_block(const ChainParams &p, int G, int &dir,
 //   * a word that holds kEmpty (an all-ones NaN pattern no product can yield) has not been written yet;
 //     a sender stores the JB values of one (receiver, sequence) pair as 16-byte vectors, a receiver polls
 //     its contiguous G*S*JB words with 16-byte loads and validates every word on its own;
-//   * after reading, the receiver puts kEmpty back.  Three slots rotate (step % 3): the reset of a slot is
-//     issued in step k+1, the receiver's next wait (step k+2) drains all of its outstanding stores before
-//     it can finish, and the sender writes the slot again only in step k+3, after it has seen what the
-//     receiver published at the end of step k+2 -- so the reset is always ordered before the rewrite.
-// The host fills the mailbox with kEmpty before every launch.
+//   * after reading, the receiving workgroup puts kEmpty back.  Four slots rotate (step % 4); the ordering
+//     argument for the reset of a slot against its next use is given with the kernel's wave roles below.
+// A launch that runs to its end leaves every word empty, so the host fills the mailbox with kEmpty once and
+// again only after a launch that gave up.
 // ---------------------------------------------------------------------------------------------------
 constexpr unsigned kEmpty = 0xFFFFFFFFu;
 constexpr int kMailSlots = 4;

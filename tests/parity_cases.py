@@ -135,6 +135,57 @@ def run_lstm_case(P, L, bidir, lengths, seed, wscale=0.1, escale=0.1, bias=1.0, 
     return worst
 
 
+def run_lstm_two_recursions(P, L, bidir, lengths, seed, wscale=0.1, escale=0.1, bias=1.0):
+    """Both GPU implementations of the recursion on the same inputs: the persistent kernels and the step-by-step
+    schedule (a handle created while CNT_LSTM_STEPWISE is set).  No oracle run, so full-size fractions finish in
+    a second.  Returns the worst L2-normalised difference over outputs, errors, weight updates and state."""
+    import torch
+
+    capi = pkg().capi
+    S, T = len(lengths), max(lengths)
+    nd = 2 if bidir else 1
+    N = T * S
+    W, x, outerr = lstm_inputs(P, L, bidir, S, T, lengths, seed, wscale, escale)
+    pat = make_pat_types(lengths, T)
+    Wd, xd, pd = dev(W), dev(x), dev(pat)
+    results = []
+    for stepwise in (False, True):
+        if stepwise:
+            os.environ["CNT_LSTM_STEPWISE"] = "1"
+        try:
+            layer = capi.Lstm(P, L, bidir, S, T, bias)
+        finally:
+            os.environ.pop("CNT_LSTM_STEPWISE", None)
+        out_d = torch.zeros(L * N, dtype=torch.float32, device="cuda")
+        err_d = dev(outerr)
+        ex_d = torch.full((P * N,), 7.0, dtype=torch.float32, device="cuda")
+        dW_d = torch.full((len(W),), 7.0, dtype=torch.float32, device="cuda")
+        layer.load_sequences(pd, T, min(lengths))
+        layer.forward(Wd, xd, out_d)
+        layer.check()
+        layer.backward(Wd, xd, out_d, err_d, ex_d, dW_d)
+        layer.check()
+        torch.cuda.synchronize()
+        r = {"outputs": out_d.cpu().numpy(), "prev_errors": ex_d.cpu().numpy(), "dW": dW_d.cpu().numpy()}
+        for d in range(nd):
+            for k in ("h", "dni", "dig", "dfg", "dog", "cerr"):
+                r["dir%d.%s" % (d, k)] = layer.state(d, k).cpu().numpy()
+        layer.close()
+        results.append(r)
+    dummy = (pat == 0)
+    if dummy.any():
+        for r in results:
+            assert not r["outputs"].reshape(N, L)[dummy].any()
+            assert not r["prev_errors"].reshape(N, P)[dummy].any()
+    worst = 0.0
+    for k in results[0]:
+        e = relerr(results[0][k], results[1][k])
+        if e > 1e-5:
+            print("   %-26s %.3e" % (k, e))
+        worst = max(worst, e)
+    return worst
+
+
 def run_gemm_case(m, n, k, tA, tB, accumulate, seed):
     import torch
 

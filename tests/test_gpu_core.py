@@ -149,6 +149,20 @@ def test_lstm_step_by_step_recursion_equals_the_persistent_kernels(monkeypatch):
     assert PC.run_lstm_case(30, 256, False, [12, 12, 7], seed=6) < TOL
 
 
+def test_lstm_config2_layer_full_length_two_recursions():
+    """A BLSTM layer of benchmark config 2 at its full size (512 inputs, 256 cells per direction, T=600, S=10,
+    lengths drawn from 300..600): the persistent recursion kernels against the step-by-step schedule.  The CPU
+    oracle needs two minutes for this fraction, so the full-length check is the agreement of two independent
+    implementations, each of which the shorter cases above compare with the oracle."""
+    print("lstm config 2 layer, full length, persistent vs stepwise", flush=True)
+    import numpy as np
+
+    rng = np.random.default_rng(2)
+    lengths = [int(v) for v in rng.integers(300, 601, size=10)]
+    lengths[3] = 600
+    assert PC.run_lstm_two_recursions(512, 512, True, lengths, seed=12, wscale=0.08) < TOL
+
+
 def test_lstm_invalid_geometry_is_an_error():
     capi = PC.pkg().capi
     with pytest.raises(RuntimeError):
