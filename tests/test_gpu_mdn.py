@@ -14,6 +14,7 @@ TOL = 1e-4
     ([6, 3, 6], 2, 2, 0),          # Lp=10: padding frames collide with valid mixture-weight slots
     ([9, 4, 7, 9], 3, 5, 7),       # unit does not start at column 0, leading columns stay zero
     ([40, 25, 33, 40, 12, 40, 40, 31, 40, 20], 16, 60, 0),  # benchmark config 3 geometry, shortened
+    ([600, 431, 377, 512, 300, 598, 465, 349, 553, 420], 16, 60, 0),  # benchmark config 3 at full size
     ([12, 7, 12], 8, 12, 4),       # every size a multiple of four behind four leading columns: the 16-byte path
     ([12, 7, 12], 8, 12, 2),       # the same unit two columns further on: not aligned, scalar path
 ])

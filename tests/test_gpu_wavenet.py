@@ -15,6 +15,7 @@ TOL = 1e-4
     (3, [1, 1], [16, 16], [10, 6], 1, 1),                      # dilation longer than the sequences
     (64, [1] * 128, [1] * 128, [300, 220], 1, 1),              # WaveNet block geometry (64 -> 128), dilation 1
     (64, [1] * 128, [512] * 128, [700, 650], 1, 0),            # largest dilation of the stack, no tanh
+    (64, [1] * 128, [512] * 128, [16000, 15100], 1, 1),        # benchmark config 4: one layer at full length
     (382, [2] * 40 + [1] * 30, [1] * 40 + [2] * 30, [33, 40, 21], 0, 1),
     (32, [1] * 24 + [0] * 40, [3] * 24 + [1] * 40, [400, 333, 150], 1, 1),   # two filter groups, ragged lengths
     (16, [0] * 32, [1] * 32, [200, 90], 0, 0),                              # width-1 filters (one tap), not causal
