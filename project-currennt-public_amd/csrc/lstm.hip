@@ -818,6 +818,65 @@ __global__ void lstm_small_grads(const SmallGradParams p) {
     atomicAdd(p.g_peep + 2 * L + u, q_og);
 }
 
+// The same sums for layers whose cell count per direction is a multiple of four: a thread owns four neighbouring
+// cells (16-byte loads), a wave walks whole rows of the state arrays, a workgroup's waves share a chunk of patterns
+// and add up in LDS first, so that a gradient element takes one global atomic per chunk -- atomics to one address
+// serialise, and with a short chunk they, not the loads, set the kernel's time.  blockIdx.z is the direction.
+struct SmallGradDirs {
+    int H, L, S, N, chunk;
+    float bias;
+    const float *dni[2], *dig[2], *dfg[2], *dog[2], *c[2];
+    float *g_bias;  // + g*L + dir*H + u
+    float *g_peep;  // + k*L + dir*H + u
+};
+
+__global__ __launch_bounds__(256) void lstm_small_grads_quads(const SmallGradDirs p) {
+    __shared__ float acc[7][256];
+    const int dir = blockIdx.z;
+    const int quads = p.H / 4;
+    const int qpb = min(quads, 64);     // quads per workgroup
+    const int rows = 256 / qpb;         // pattern rows walked side by side
+    const int tid = threadIdx.x;
+    for (int k = 0; k < 7; ++k) acc[k][tid] = 0.0f;
+    __syncthreads();
+    const int ql = tid % qpb, r = tid / qpb;
+    const int q = blockIdx.x * qpb + ql;
+    if (r < rows && q < quads) {
+        const int i0 = blockIdx.y * p.chunk, i1 = min(p.N, i0 + p.chunk);
+        const int H = p.H, S = p.S;
+        const f32x4 *dni = reinterpret_cast<const f32x4 *>(p.dni[dir]), *dig = reinterpret_cast<const f32x4 *>(p.dig[dir]);
+        const f32x4 *dfg = reinterpret_cast<const f32x4 *>(p.dfg[dir]), *dog = reinterpret_cast<const f32x4 *>(p.dog[dir]);
+        const f32x4 *c = reinterpret_cast<const f32x4 *>(p.c[dir]);
+        f32x4 b0 = {0, 0, 0, 0}, b1 = b0, b2 = b0, b3 = b0, q_ig = b0, q_fg = b0, q_og = b0;
+#pragma unroll 4
+        for (int i = i0 + r; i < i1; i += rows) {
+            const size_t o = ((size_t)i * H) / 4 + q;
+            const f32x4 d_ni = dni[o], d_ig = dig[o], d_fg = dfg[o], d_og = dog[o];
+            b0 += d_ni; b1 += d_ig; b2 += d_fg; b3 += d_og;
+            q_og += c[o] * d_og;
+            // input/forget peepholes look at the cell state one step earlier in processing order
+            const int ie = dir ? i + S : i - S;
+            if (ie >= 0 && ie < p.N) {
+                const f32x4 ce = c[((size_t)ie * H) / 4 + q];
+                q_ig += ce * d_ig;
+                q_fg += ce * d_fg;
+            }
+        }
+        const f32x4 v[7] = {b0 * p.bias, b1 * p.bias, b2 * p.bias, b3 * p.bias, q_ig, q_fg, q_og};
+#pragma unroll
+        for (int k = 0; k < 7; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) atomicAdd(&acc[k][4 * ql + e], v[k][e]);
+    }
+    __syncthreads();
+    const int u = blockIdx.x * qpb * 4 + tid;
+    if (tid < 4 * qpb && u < p.H) {
+        float *gb = p.g_bias + dir * p.H + u, *gp = p.g_peep + dir * p.H + u;
+        for (int k = 0; k < 4; ++k) atomicAdd(gb + k * p.L, acc[k][tid]);
+        for (int k = 0; k < 3; ++k) atomicAdd(gp + k * p.L, acc[4 + k][tid]);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Step-by-step recursion for geometries the persistent kernels do not cover (cells per direction other than 64,
 // 128, 256, 512, or more than 32 parallel sequences): per time step one batched recurrent product through the
@@ -1377,6 +1436,24 @@ int cnt_lstm_backward_weights(cnt_lstm *h, void *stream_, const float *x, float 
             }
         ga.label = "gemm:lstm_dW_internal";
         CNT_TRY(gemm_launch(stream, ga));
+    }
+    if (H % 4 == 0) {
+        SmallGradDirs sp;
+        sp.H = H; sp.L = L; sp.S = S; sp.N = N; sp.bias = d.bias;
+        sp.chunk = 64;
+        for (int dir = 0; dir < 2; ++dir) {
+            const int sd = dir < h->ndir ? dir : 0;
+            sp.dni[dir] = h->state[sd][7]; sp.dig[dir] = h->state[sd][8]; sp.dfg[dir] = h->state[sd][9];
+            sp.dog[dir] = h->state[sd][10]; sp.c[dir] = h->state[sd][4];
+        }
+        sp.g_bias = weight_updates + off_bias;
+        sp.g_peep = weight_updates + off_peep;
+        const int quads = H / 4, qpb = quads < 64 ? quads : 64;
+        dim3 grid((quads + qpb - 1) / qpb, (N + sp.chunk - 1) / sp.chunk, h->ndir);
+        ProfileScope prof(stream, "lstm_small_grads");
+        hipLaunchKernelGGL(lstm_small_grads_quads, grid, dim3(256), 0, stream, sp);
+        CNT_HIP(hipGetLastError());
+        return CNT_OK;
     }
     for (int dir = 0; dir < h->ndir; ++dir) {
         SmallGradParams sp;
