@@ -752,7 +752,10 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
             }
             dl[0 * JB + cj][cs] = s_ni; dl[1 * JB + cj][cs] = s_ig;
             dl[2 * JB + cj][cs] = s_fg; dl[3 * JB + cj][cs] = s_og;
-            res[0][tid] = e; res[1][tid] = ce;
+            // a padding slot receives nothing but the phase bits of partial errors that are zero: its summed error is
+            // the caller's own value, as in the reference
+            res[0][tid] = coef[C_DUMMY][tid] == 0.0f ? e : coef[C_E][tid];
+            res[1][tid] = ce;
             fg_later = fg; cerr_later = ce; dig_later = s_ig; dfg_later = s_fg;
         }
         lds_barrier();  // B
@@ -1187,8 +1190,8 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     if (const char *e = std::getenv("CNT_LSTM_XCD_PACK")) h->xcd_pack = std::atoi(e) != 0;
     // Backward recursion: pause before the first poll of a step, in units of 64 clocks -- roughly the time the
     // senders need for their products (32 clocks per MFMA, (H/64)*JB*NT of them per wave) plus the time a store
-    // takes to become visible.  Measured optimum on MI355X for H=256, JB=4, S=10: 28.
-    h->poll_delay = 20 + (H / 64) * JB * NT / 2;
+    // takes to become visible.  Measured optimum on MI355X for H=256, JB=4, S=10: 30.
+    h->poll_delay = 22 + (H / 64) * JB * NT / 2;
     if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY")) h->poll_delay = std::atoi(e);
     // forward recursion: the senders' cell update (a few hundred clocks) plus store visibility
     h->poll_delay_fwd = 34;  // measured optimum on MI355X at H=256, S=10
