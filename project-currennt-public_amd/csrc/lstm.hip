@@ -13,11 +13,9 @@
 //   backward: each workgroup multiplies its own 4*JB gate deltas with its weight slice and
 //             scatters partial output errors to the owners of the receiving cells (H x S words per
 //             workgroup instead of the 4H x S a gather of the deltas would need).
-// Mailbox words are plain 4-byte floats that validate themselves, so neither tags nor fences sit on the critical
-// path: in the forward mailbox a reserved NaN pattern means "not written yet" and a word is handed back as empty
-// after use, in the backward mailbox the lowest mantissa bit carries the phase of the slot's use and nothing is
-// handed back.  Words are moved 16 bytes at a time and polled with loads that bypass the non-coherent caches; four
-// slots rotate.  Every
+// Mailbox words are plain 4-byte floats; a reserved NaN pattern means "not written yet", so a word validates
+// itself and neither tags nor fences sit on the critical path.  Words are moved 16 bytes at a time, polled with
+// loads that bypass the non-coherent caches, and handed back as empty after use; four slots rotate.  Every
 // poll loop is bounded: when the bound is hit the workgroup raises a device flag and every workgroup drains
 // out.  Inside a workgroup, waves specialise (polling waves that never store, product / cell waves that never
 // wait for a store, one memory wave for all ordinary loads and stores), see the kernels' comments.
@@ -66,7 +64,6 @@ struct ChainParams {
     long long *phase_ticks;  // optional diagnostic: per workgroup accumulated phase durations (100 MHz ticks)
     int poll_delay, poll_gap;  // s_sleep units before the first poll of a step / between polls
     int poll_delay_fwd;
-    unsigned step_base;   // backward mailbox: number of the launch's first step in the slot rotation (mod 8)
 };
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
@@ -98,18 +95,14 @@ __device__ __forceinline__ bool map_block(const ChainParams &p, int G, int &dir,
 // Backward (error) recursion.
 //
 // The partial output errors travel through a mailbox of plain 4-byte words, laid out
-// [slot][receiving workgroup][sending workgroup][sequence][cell of the receiver].  A sender stores the JB values of
-// one (receiver, sequence) pair as 16-byte vectors, a receiver polls its contiguous G*S*JB words with 16-byte loads
-// and validates every word on its own: the lowest mantissa bit of a word is not data but the PHASE of this use of
-// its slot.  Steps are numbered through all launches of a handle (g = step_base + step), slot = g % 4,
-// phase = (g / 4) & 1.  Every word of a slot is rewritten on every use of the slot, so a word that still holds the
-// value of the slot's previous use carries the opposite phase and one that holds this use's value the expected
-// one; nothing has to be handed back or cleared, which takes a third of the mailbox traffic (and every store but
-// the publication itself) out of a step.  A partial error loses its last mantissa bit (6e-8 relative).
-// A slot is rewritten four steps after a use; by then its reader has published three more times, each time after
-// it had consumed the step before, and the writer has seen those publications.
-// The host fills the mailbox with the all-ones pattern (phase 1, which the first use of every slot does not
-// expect) once, and again (restarting the step numbering) after a launch that gave up.
+// [slot][receiving workgroup][sending workgroup][sequence][cell of the receiver]:
+//   * a word that holds kEmpty (an all-ones NaN pattern no product can yield) has not been written yet;
+//     a sender stores the JB values of one (receiver, sequence) pair as 16-byte vectors, a receiver polls
+//     its contiguous G*S*JB words with 16-byte loads and validates every word on its own;
+//   * after reading, the receiving workgroup puts kEmpty back.  Four slots rotate (step % 4); the ordering
+//     argument for the reset of a slot against its next use is given with the kernel's wave roles below.
+// A launch that runs to its end leaves every word empty, so the host fills the mailbox with kEmpty once and
+// again only after a launch that gave up.
 // ---------------------------------------------------------------------------------------------------
 constexpr unsigned kEmpty = 0xFFFFFFFFu;
 constexpr int kMailSlots = 4;
@@ -445,13 +438,16 @@ __global__ __launch_bounds__(fwd_threads(JB, NT)) void lstm_forward_chain(const 
 //                      and leave the gate deltas in LDS (barrier B).  They issue no stores at all, so the only
 //                      memory operations their wait counter ever covers are their own polls.
 //   product waves (4)  hold the recurrent weight slice as MFMA operands; after barrier B they multiply it with
-//                      the deltas and publish the partial errors.
+//                      the deltas and publish the partial errors.  They never wait for a store.
 //   memory wave (1)    owns every other global access: two steps ahead it loads what the cell update needs,
 //                      one step ahead it folds everything that does not depend on the recursion into five
 //                      coefficients per cell (LDS), one step behind it writes the cell update's results to the
 //                      state arrays.
-// Mailbox slots rotate over four steps (see the protocol above).  The product waves drain their stores once per
-// step, right after barrier A, when only the publication of the previous step can still be in flight.
+// Mailbox slots rotate over four steps.  The product waves also hand the words their workgroup consumed in a
+// step back as empty, and drain all of their stores once per step (right after barrier A, when only stores of
+// the previous step can still be in flight), so the reset of the words consumed in step k is complete before
+// this workgroup publishes in step k+1; a sender rewrites those words only in step k+3, after it has seen
+// that publication.
 constexpr int kBwdThreads = 2 * kThreads + 64;
 
 template <int HT, int JB, int NT>
@@ -598,6 +594,11 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
                 for (int mt = 0; mt < MT; ++mt) wA[mt][ks] = wg[pw * (H / 4) + mt * 16 + i];
             }
         }
+        // reset role: the same words this workgroup's receive waves poll (sequence ps, senders pg, pg + PG, ...)
+        const int ptid = tid - kThreads;
+        const int ps = ptid % NS, pg = ptid / NS;
+        const unsigned poll_off = ((unsigned)(pg * S + ps) * JB) * 4u;
+        const unsigned poll_stride = (unsigned)PG * pair_words * 4u;
         wait_all_vmem();
         lds_barrier();  // start of the recursion
         const bool timing = p.phase_ticks != nullptr;
@@ -606,17 +607,15 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
             if (step > 0) {
                 lds_barrier();  // A
                 if (wait_failed) return;
-                // everything this wave stored in the previous step is complete before it publishes again;
-                // the wait hides behind the cell update of the receive waves
+                // everything this wave stored in the previous step (partial errors, resets) is complete
+                // before it publishes again; the wait hides behind the cell update of the receive waves
                 wait_all_vmem();
             }
             lds_barrier();  // B: the deltas of this step are in LDS
             const long long tp0 = timing ? wall_clock64() : 0;
             if (step < T - 1) {
                 // partial output errors of every receiving cell from this workgroup's deltas
-                const unsigned gstep = p.step_base + (unsigned)step;
-                const unsigned slot_off = (unsigned)((size_t)(gstep % kMailSlots) * slot_words * 4u);
-                const unsigned phase = (gstep / kMailSlots) & 1u;
+                const unsigned slot_off = (unsigned)((size_t)(step % kMailSlots) * slot_words * 4u);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     const int s = nt * 16 + (lane & 15);
@@ -642,13 +641,25 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
                                 const int from = pw * (H / 4) + (m0 + u) * 16 + 4 * (lane >> 4);
                                 const int dst = from / JB, jd = from % JB;
                                 u32x4 v = __builtin_bit_cast(u32x4, acc[u]);
-                                // the lowest mantissa bit carries the phase of this use of the slot
-                                v = (v & 0xFFFFFFFEu) | phase;
+                                // a NaN that happens to look like the empty marker is sent as the default NaN
+                                v.x = v.x == kEmpty ? 0x7FC00000u : v.x; v.y = v.y == kEmpty ? 0x7FC00000u : v.y;
+                                v.z = v.z == kEmpty ? 0x7FC00000u : v.z; v.w = v.w == kEmpty ? 0x7FC00000u : v.w;
                                 store128_device(mail, slot_off + ((unsigned)dst * recv_words + (unsigned)(me * S + s) * JB + jd) * 4u, v);
                             }
                         }
                     }
                 }
+            }
+            if (step > 0 && ps < S) {
+                // the words the receive waves consumed in this step (before barrier A) are empty again
+                const u32x4 empty = {kEmpty, kEmpty, kEmpty, kEmpty};
+                const unsigned mine_off =
+                    (unsigned)(((size_t)((step - 1) % kMailSlots) * slot_words + (size_t)me * recv_words) * 4u);
+#pragma unroll
+                for (int jv = 0; jv < JV; ++jv)
+#pragma unroll
+                    for (int q = 0; q < NPOLL; ++q)
+                        store128_device(mail, mine_off + poll_off + 16u * jv + (unsigned)q * poll_stride, empty);
             }
             // `dl` is rewritten only after the next barrier A, which this wave reaches after its LDS reads
             if (timing) busy += wall_clock64() - tp0;
@@ -683,9 +694,7 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
         const bool first = (step == 0), last = (step == T - 1);
 
         if (!first) {
-            const unsigned gprev = p.step_base + (unsigned)step - 1u;
-            const float *mine = D.bmail + (size_t)(gprev % kMailSlots) * slot_words + (size_t)me * recv_words;
-            const unsigned want = (gprev / kMailSlots) & 1u;
+            const float *mine = D.bmail + (size_t)((step - 1) % kMailSlots) * slot_words + (size_t)me * recv_words;
             bool ok = true;
             if (polls) {
                 u32x4 w[JV][NPOLL];
@@ -694,17 +703,16 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
                 // incomplete costs a whole memory round trip, a poll that starts a little late only the delay
                 for (int d = 0; d < p.poll_delay; ++d) __builtin_amdgcn_s_sleep(1);
                 for (;;) {
-                    // bit 0 of `stale` is set if any word still carries the phase of the slot's use before this one
-                    unsigned stale = 0;
+                    unsigned worst = 0;
 #pragma unroll
                     for (int jv = 0; jv < JV; ++jv) {
                         poll_load<NPOLL>(mine, poll_off + 16u * jv, poll_stride, w[jv]);
 #pragma unroll
                         for (int q = 0; q < NPOLL; ++q)
-                            stale |= (w[jv][q].x ^ want) | (w[jv][q].y ^ want) | (w[jv][q].z ^ want) | (w[jv][q].w ^ want);
+                            worst = max(max(worst, w[jv][q].x), max(max(w[jv][q].y, w[jv][q].z), w[jv][q].w));
                     }
                     if (timing) ++poll_rounds;
-                    if ((stale & 1u) == 0u) break;
+                    if (worst != kEmpty) break;
                     if (++spins > p.spin_limit) { ok = false; break; }
                     if ((spins & 255u) == 0u &&
                         __hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
@@ -752,10 +760,7 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
             }
             dl[0 * JB + cj][cs] = s_ni; dl[1 * JB + cj][cs] = s_ig;
             dl[2 * JB + cj][cs] = s_fg; dl[3 * JB + cj][cs] = s_og;
-            // a padding slot receives nothing but the phase bits of partial errors that are zero: its summed error is
-            // the caller's own value, as in the reference
-            res[0][tid] = coef[C_DUMMY][tid] == 0.0f ? e : coef[C_E][tid];
-            res[1][tid] = ce;
+            res[0][tid] = e; res[1][tid] = ce;
             fg_later = fg; cerr_later = ce; dig_later = s_ig; dfg_later = s_fg;
         }
         lds_barrier();  // B
@@ -995,7 +1000,6 @@ struct cnt_lstm {
     int poll_delay, poll_gap, poll_delay_fwd;
     int last_was_forward;  // which recursion the diagnostic buffer describes
     int bmail_dirty;       // the backward mailbox may hold words that are not empty
-    unsigned bmail_step;   // backward mailbox: where the next launch continues the slot rotation (mod 8)
     int stepwise;          // no persistent recursion kernel for this geometry: one product + one cell kernel per step
 };
 
@@ -1064,12 +1068,7 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
         if (fwd) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->fmail[dir]), h->fmail_words, kEmpty));
         else if (h->bmail_dirty) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->bmail[dir]), h->bmail_words, kEmpty));
     }
-    if (!fwd) {
-        if (h->bmail_dirty) h->bmail_step = 0;
-        h->bmail_dirty = 0;
-        p.step_base = h->bmail_step;
-        if (h->T > 1) h->bmail_step = (h->bmail_step + (unsigned)(h->T - 1)) % (2u * kMailSlots);
-    }
+    if (!fwd) h->bmail_dirty = 0;
     const int G = h->H / h->JB;
     p.xcd_pack = fwd ? h->xcd_pack : 0;
     const int blocks = p.xcd_pack ? 8 * G : h->ndir * G;
@@ -1183,15 +1182,14 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     h->desc = *desc; h->ndir = ndir; h->H = H; h->JB = JB; h->NT = NT;
     h->stepwise = stepwise ? 1 : 0;
     h->bmail_dirty = 1;
-    h->bmail_step = 0;
     h->spin_limit = 1u << 22;
     if (const char *e = std::getenv("CNT_LSTM_SPIN_LIMIT")) h->spin_limit = (unsigned)std::strtoul(e, nullptr, 10);
     h->xcd_pack = 0;
     if (const char *e = std::getenv("CNT_LSTM_XCD_PACK")) h->xcd_pack = std::atoi(e) != 0;
     // Backward recursion: pause before the first poll of a step, in units of 64 clocks -- roughly the time the
     // senders need for their products (32 clocks per MFMA, (H/64)*JB*NT of them per wave) plus the time a store
-    // takes to become visible.  Measured optimum on MI355X for H=256, JB=4, S=10: 30.
-    h->poll_delay = 22 + (H / 64) * JB * NT / 2;
+    // takes to become visible.  Measured optimum on MI355X for H=256, JB=4, S=10: 28.
+    h->poll_delay = 20 + (H / 64) * JB * NT / 2;
     if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY")) h->poll_delay = std::atoi(e);
     // forward recursion: the senders' cell update (a few hundred clocks) plus store visibility
     h->poll_delay_fwd = 34;  // measured optimum on MI355X at H=256, S=10
