@@ -1244,8 +1244,9 @@ int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int
     CNT_REQUIRE(curMinT >= 0 && curMinT <= curMaxT, "lstm_load_sequences: curMinT %d outside 0..%d", curMinT, curMaxT);
     h->T = curMaxT; h->Tmin = curMinT; h->pat = patTypes;
     const size_t nstate = (size_t)h->H * h->desc.maxT * h->desc.S;
-    for (int dir = 0; dir < h->ndir; ++dir)
-        CNT_TRY(fill_zero(static_cast<hipStream_t>(stream), h->state[dir][10], nstate));
+    // stored output-gate deltas of both directions, one launch
+    if (h->ndir == 2) CNT_TRY(fill_zero_pair(static_cast<hipStream_t>(stream), h->state[0][10], nstate, h->state[1][10], nstate));
+    else CNT_TRY(fill_zero(static_cast<hipStream_t>(stream), h->state[0][10], nstate));
     return CNT_OK;
 }
 
