@@ -744,8 +744,20 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
         if (cell_valid) {
             float e = coef[C_E][tid];
             if (!first) {
+                // pairwise sum of the sender groups' partial errors: log2(PG) dependent additions instead of PG
+                float part[PG];
 #pragma unroll
-                for (int q = 0; q < PG; ++q) e += psum[q][tid];
+                for (int q = 0; q < PG; ++q) part[q] = psum[q][tid];
+#pragma unroll
+                for (int q = 0; q < PG / 2; ++q) part[q] += part[q + PG / 2];
+#pragma unroll
+                for (int q = 0; q < PG / 4; ++q) part[q] += part[q + PG / 4];
+#pragma unroll
+                for (int q = 0; q < PG / 8; ++q) part[q] += part[q + PG / 8];
+#pragma unroll
+                for (int q = 0; q < PG / 16; ++q) part[q] += part[q + PG / 16];
+                static_assert(PG == 8 || PG == 16, "pairwise sum written for 8 or 16 sender groups");
+                e += part[0];
             }
             const float fg = coef[C_FGACT][tid];
             float s_ni = 0, s_ig = 0, s_fg = 0, s_og = 0, ce = 0;
