@@ -1198,10 +1198,18 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     if (const char *e = std::getenv("CNT_LSTM_SPIN_LIMIT")) h->spin_limit = (unsigned)std::strtoul(e, nullptr, 10);
     h->xcd_pack = 0;
     if (const char *e = std::getenv("CNT_LSTM_XCD_PACK")) h->xcd_pack = std::atoi(e) != 0;
-    // Backward recursion: pause before the first poll of a step, in units of 64 clocks -- roughly the time the
-    // senders need for their products (32 clocks per MFMA, (H/64)*JB*NT of them per wave) plus the time a store
-    // takes to become visible.  Measured optimum on MI355X for H=256, JB=4, S=10: 28.
-    h->poll_delay = 20 + (H / 64) * JB * NT / 2;
+    // Backward recursion: pause before the first poll of a step, in units of 64 clocks -- the time the senders need
+    // for their products (32 clocks per MFMA, (H/64)*JB*NT of them per wave), the time a store takes to become
+    // visible, and a share that grows with the words all workgroups publish per step (ndir * G * H * S).  Fitted to
+    // the measured optima on MI355X: 14 at 64 cells (S=8, two directions), 16-18 at 128 cells, 22-24 at 256 cells
+    // with 4 or 10 sequences, 28 at 256 cells with 16 sequences and for the two-layer acoustic model, whose
+    // recursions share the machine with other streams' products; 512 cells are flat between 18 and 40.
+    {
+        const double mfma = (H / 64) * JB * NT / 2.0;
+        const double words = (double)ndir * (H / JB) * H * desc->S;
+        int pause = (int)(14.0 + 1.25 * mfma + words / 90000.0 + 0.5);
+        h->poll_delay = pause > 40 ? 40 : pause;
+    }
     if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY")) h->poll_delay = std::atoi(e);
     // forward recursion: the senders' cell update (a few hundred clocks) plus store visibility
     h->poll_delay_fwd = 34;  // measured optimum on MI355X at H=256, S=10
