@@ -29,6 +29,10 @@ typedef struct {
 } orc_lstm_dir;
 
 /* scalar helpers (for unit tests of the scalar semantics) */
+// Worker threads for the large loops (default 1).  Outputs are shared out whole, so results do not change.
+void orc_set_threads(int n);
+int orc_get_threads(void);
+
 float orc_logistic(float x);
 float orc_tanh(float x);
 float orc_safe_exp(float x);

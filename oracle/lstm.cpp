@@ -14,6 +14,11 @@
 
 #include <cstring>
 
+static int g_threads = 1;
+namespace orc {
+int threads() { return g_threads; }
+}  // namespace orc
+
 namespace {
 
 struct Geometry {
@@ -156,6 +161,7 @@ void weight_updates(const Geometry &G, const float *x, orc_lstm_dir *const dirs[
         for (int g = 0; g < 4; ++g) {
             const float *dl = delta[g];
             // input weights
+#pragma omp parallel for collapse(2) schedule(static) num_threads(orc::threads()) if (orc::threads() > 1)
             for (int u = 0; u < H; ++u)
                 for (int p = 0; p < P; ++p) {
                     float wu = 0.0f;
@@ -169,6 +175,7 @@ void weight_updates(const Geometry &G, const float *x, orc_lstm_dir *const dirs[
                 dW[G.off_bias + (size_t)g * L + dir * H + u] = wu;
             }
             // recurrent weights: source is the block output of the step the forward pass came from
+#pragma omp parallel for collapse(2) schedule(static) num_threads(orc::threads()) if (orc::threads() > 1)
             for (int u = 0; u < H; ++u)
                 for (int src = 0; src < H; ++src) {
                     float wu = 0.0f;
@@ -251,6 +258,9 @@ void orc_lstm_backward(const orc_lstm_desc *d, const float *weights, const char 
     }
     weight_updates(G, x, dirs, weightUpdates);
 }
+
+void orc_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
+int orc_get_threads() { return g_threads; }
 
 float orc_logistic(float x) { return orc::logistic(x); }
 float orc_tanh(float x) { return orc::tanh_act(x); }

@@ -68,12 +68,19 @@ static inline float log_add(float x, float y) {
     return (float)((double)hi + std::log(1.0 + (double)std::exp(lo - hi)));
 }
 
+// Worker threads the oracle may use (orc_set_threads; 1 unless a caller asks for more).  Threads only ever
+// share out whole output elements: every output is still one sequential, k-ordered sum formed by one thread,
+// so results do not depend on the thread count.
+int threads();
+
 // Column-major products with the reference's summation order: every output is a
 // k-ordered dot product formed from zero, then (optionally) added to the old value.
 //   C (m x n, ldc=m);  tA=false: A is m x k (lda=m)  tA=true: A is k x m (lda=k)
 //                      tB=false: B is k x n (ldb=k)  tB=true: B is n x k (ldb=n)
 static inline void mat_product(float *C, int m, int n, int k, const float *A, bool tA, const float *B,
                                bool tB, bool accumulate) {
+    const int nthr = ((long long)m * n * k >= 200000) ? threads() : 1;
+#pragma omp parallel for collapse(2) schedule(static) num_threads(nthr) if (nthr > 1)
     for (int j = 0; j < n; ++j) {
         for (int i = 0; i < m; ++i) {
             float x = 0.0f;

@@ -78,6 +78,20 @@ def lib():
     return _lib
 
 
+def set_threads(n):
+    """Worker threads of the oracle's large loops; results do not depend on it (whole outputs are shared out)."""
+    lib().orc_set_threads(int(n))
+
+
+def use_all_cores(limit=16):
+    """For the full-size parity cases: as many threads as this process may run on, at most `limit`."""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    set_threads(max(1, min(limit, n)))
+
+
 class LstmState:
     """Host buffers of one direction: every field is an H x (T*S) column-major matrix."""
 

@@ -163,6 +163,23 @@ def test_lstm_config2_layer_full_length_two_recursions():
     assert PC.run_lstm_two_recursions(512, 512, True, lengths, seed=12, wscale=0.08) < TOL
 
 
+def test_lstm_config2_layer_full_length_against_oracle():
+    """The same full-size BLSTM layer (512 inputs, 256 cells per direction, T=600, S=10, lengths drawn from
+    300..600) against the CPU oracle: outputs, error to the preceding layer, every weight-gradient class and
+    every state array, 1e-4 L2-normalised; exact zeros on padding slots.  The oracle shares its outputs out
+    over the host's cores for this one (the sums themselves stay sequential)."""
+    print("lstm config 2 layer, full length, against the oracle", flush=True)
+    import numpy as np
+
+    import oracle_lib as O
+
+    O.use_all_cores()
+    rng = np.random.default_rng(2)
+    lengths = [int(v) for v in rng.integers(300, 601, size=10)]
+    lengths[3] = 600
+    assert PC.run_lstm_case(512, 512, True, lengths, seed=12, wscale=0.08) < TOL
+
+
 def test_lstm_invalid_geometry_is_an_error():
     capi = PC.pkg().capi
     with pytest.raises(RuntimeError):

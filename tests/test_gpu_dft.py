@@ -24,6 +24,14 @@ def test_dft_loss(res, max_len, lengths):
     assert PC.run_dft_case(res, max_len, lengths, seed=len(res) + max_len, gamma=0.8) < TOL
 
 
+def test_dft_loss_config5_full_size():
+    """benchmark config 5 at its size: 8 waveforms x 16000 samples (two of them shorter), the three resolutions."""
+    print("dft config 5 full size", flush=True)
+    res = [(512, 512, 80), (128, 128, 40), (2048, 2048, 640)]
+    lengths = [16000, 16000, 12345, 16000, 16000, 16000, 8000, 16000]
+    assert PC.run_dft_case(res, 16000, lengths, seed=55, gamma=1.0) < TOL
+
+
 @pytest.mark.parametrize("dis_type", [1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("res,max_len,lengths", [
     ([(64, 40, 10)], 333, [333, 120]),

@@ -103,18 +103,24 @@ def test_stacked_network_trains_like_the_oracle(option, momentum, overlap):
 
 # the last case has channel counts that are not multiples of four: no 16-byte accesses anywhere, and the skip layers'
 # backward steps run as launches of their own instead of in the epilogue of the following layer's product
-@pytest.mark.parametrize("nb,cnn_tanh,R,K", [(4, 1, 32, 64), (11, 0, 32, 64), (3, 1, 30, 50)])
-def test_wavenet_network_file_against_oracle_graph(nb, cnn_tanh, R, K):
+# The fifth case is a stack with benchmark config 4's layer sizes (64 residual / 128 skip channels, 80 conditioning
+# dimensions up-sampled 80 times) and one full cycle of its dilations, 1 ... 512, over waveforms long enough that
+# every dilation reaches valid history and the sequences' ragged ends, against the oracle's graph.
+@pytest.mark.parametrize("nb,cnn_tanh,R,K,Q,C,lengths,cycle,upsample", [
+    (4, 1, 32, 64, 64, 20, [120, 90], 3, 20), (11, 0, 32, 64, 64, 20, [120, 90], 3, 20),
+    (3, 1, 30, 50, 64, 20, [120, 90], 3, 20),
+    (10, 1, 64, 128, 256, 80, [4000, 3300], 10, 80),
+])
+def test_wavenet_network_file_against_oracle_graph(nb, cnn_tanh, R, K, Q, C, lengths, cycle, upsample):
     import torch
 
-    print("wavenet network file", nb, cnn_tanh, R, K, flush=True)
+    print("wavenet network file", nb, cnn_tanh, R, K, Q, C, lengths, cycle, flush=True)
     pkg = PC.pkg()
     capi, networks = pkg.capi, pkg.networks
-    Q, C = 64, 20
-    lengths = [120, 90]
+    O.use_all_cores()
     S, T = len(lengths), max(lengths)
-    pat, onehot, ctx, target, N = WD.make(lengths, Q, C, upsample=20, seed=2)
-    ref = networks.WaveNet(OM.OracleBackend(), nb, S, T, Q=Q, R=R, K=K, C=C, cnn_tanh=cnn_tanh, dilation_cycle=3)
+    pat, onehot, ctx, target, N = WD.make(lengths, Q, C, upsample=upsample, seed=2)
+    ref = networks.WaveNet(OM.OracleBackend(), nb, S, T, Q=Q, R=R, K=K, C=C, cnn_tanh=cnn_tanh, dilation_cycle=cycle)
     shapes = {k: len(ref.buf[k]["W"]) for k in ref.weight_names()}
     W = WD.init_weights(shapes, seed=3)
     for k, w in W.items():
@@ -124,7 +130,7 @@ def test_wavenet_network_file_against_oracle_graph(nb, cnn_tanh, R, K):
     ref.calculate_error()
     ref.backward()
 
-    doc = WD.network_json(nb, Q, R, K, C, cnn_tanh, 3)
+    doc = WD.network_json(nb, Q, R, K, C, cnn_tanh, cycle)
     net = capi.Network(json.dumps(doc), S, T + 7, mdn_config=[1, 0, Q, 0, 1, -1])   # buffers longer than the fraction
     names = [L["name"] for L in net.layers if L["weight_count"]]
     assert sorted(names) == sorted(W)

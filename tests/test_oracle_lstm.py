@@ -186,3 +186,29 @@ def test_mat_product_matches_numpy():
         Bm = B.T if not tB else B  # k x n
         want = 1 + (Am.astype(np.float64) @ Bm.astype(np.float64))
         assert relerr(Cm.reshape(n, m).T, want) < 1e-6
+
+
+def test_oracle_thread_count_does_not_change_results():
+    """Threads share out whole output elements; every sum stays sequential, so results are bit-identical."""
+    P, L, lengths = 40, 128, [30, 22, 30, 9]
+    S, T = len(lengths), max(lengths)
+    H, N = L // 2, T * S
+    rng = np.random.default_rng(9)
+    W = rng.uniform(-0.1, 0.1, O.lib().orc_lstm_weight_count(P, L, 1)).astype(np.float32)
+    x = rng.standard_normal(T * S * P).astype(np.float32)
+    outerr = (0.1 * rng.standard_normal(T * S * L)).astype(np.float32)
+    pat = make_pat_types(lengths, T)
+    results = []
+    for threads in (1, 4):
+        O.set_threads(threads)
+        desc = O.LstmDesc(P, L, 1, S, T, min(lengths), 1.0)
+        fw, bw = O.LstmState(H, N), O.LstmState(H, N)
+        out = np.zeros(L * N, dtype=np.float32)
+        O.lstm_forward(desc, W, pat, x, fw, bw, out)
+        ex = np.zeros(P * N, dtype=np.float32)
+        dW = np.zeros_like(W)
+        O.lstm_backward(desc, W, pat, x, outerr, fw, bw, ex, dW)
+        results.append((out, ex, dW))
+    O.set_threads(1)
+    for a, b in zip(*results):
+        assert np.array_equal(a, b)
