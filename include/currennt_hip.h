@@ -69,7 +69,12 @@ int cnt_dense_backward_errors(void *stream, int P, int D, int N, int act, const 
                               float *err, float *prev_err);
 int cnt_dense_backward_weights(void *stream, int P, int D, int N, float bias, const float *x, const float *err,
                                float *weight_updates);
-
+/* The scratch buffer of `stream` for those split products (16 MB of device memory), allocated now instead of
+ * inside the first product that wants it, and freed again (the stream must be idle).  No counterpart in the
+ * reference, whose cuBLAS handle owns its workspace.  A product that finds no buffer and cannot get one (out of
+ * memory, a stream under capture) adds its splits atomically instead. */
+int cnt_gemm_reserve(void *stream);
+int cnt_gemm_release(void *stream);
 /* ---- SSE post-output layer ---------------------------------------------------------------------
  * SsePostOutputLayer::computeBackwardPass (layers/SsePostOutputLayer.cu:224-267):
  * err = y - target, exactly 0 on padding slots. */

@@ -67,6 +67,8 @@ _SIGNATURES = {
     "cnt_dense_backward": (I, [VP, I, I, I, I, F, VP, VP, VP, VP, VP, VP]),
     "cnt_dense_backward_errors": (I, [VP, I, I, I, I, VP, VP, VP, VP]),
     "cnt_dense_backward_weights": (I, [VP, I, I, I, F, VP, VP, VP]),
+    "cnt_gemm_reserve": (I, [VP]),
+    "cnt_gemm_release": (I, [VP]),
     "cnt_sse_backward": (I, [VP, I, I, VP, VP, VP, VP]),
     "cnt_sse_error": (I, [VP, I, I, VP, VP, VP, VP]),
     "cnt_dataset_open": (I, [C.c_char_p, C.POINTER(DatasetDesc), C.POINTER(VP)]),
@@ -217,6 +219,14 @@ def dense_backward_errors(P, D, N, act, W, y, err, prev_err, stream=None):
 
 def dense_backward_weights(P, D, N, bias, x, err, dW, stream=None):
     check(lib().cnt_dense_backward_weights(stream_ptr(stream), P, D, N, bias, ptr(x), ptr(err), ptr(dW)))
+
+
+def gemm_reserve(stream=None):
+    check(lib().cnt_gemm_reserve(stream_ptr(stream)))
+
+
+def gemm_release(stream=None):
+    check(lib().cnt_gemm_release(stream_ptr(stream)))
 
 
 def sse_backward(D, N, pat, y, tgt, err, stream=None):

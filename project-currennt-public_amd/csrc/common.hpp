@@ -164,20 +164,22 @@ struct GemmArgs {
     int fan_n;                   // EPI_FAN: device tables of fan_n targets and their flags
     float *const *fan_targets;
     const int *fan_is_skip;
-    float *partial;        // set by the launcher: scratch of splitk * partial_stride floats
+    float *partial;        // scratch of splitk * partial_stride floats: the stream's buffer (set by gemm_plan) or the caller's
     size_t partial_stride;  // floats per split: nprob * m * n (+ nprob * n with rowsum)
 };
 
 // Resolves splitk = 0 (chosen by the launcher) and, where the arguments allow it and it pays, switches an
 // EPI_ATOMIC product to EPI_PARTIAL.  A caller that needs to know whether C must be cleared first calls this
 // before gemm_launch and looks at args.epilogue; gemm_launch calls it for everyone else.
-void gemm_plan(GemmArgs &args);
+void gemm_plan(GemmArgs &args, hipStream_t stream);
 // whether a product with these operands can take the EPI_FAN epilogue (operand kinds, alignment)
 bool gemm_fan_supported(const GemmArgs &args);
 int gemm_launch(hipStream_t stream, const GemmArgs &args);
 // Frees the split-K scratch buffer that the launcher keeps for `stream` (for owners of a stream about to destroy
 // it; the stream must be idle).  Buffers of streams never released stay until the process ends.
 void gemm_release_stream(hipStream_t stream);
+// Allocates the split-K scratch buffer of `stream` now instead of inside the first product that wants it.
+int gemm_reserve_stream(hipStream_t stream);
 
 // Convenience: single problem, BLAS-like transposes on column-major matrices.
 int gemm_simple(hipStream_t stream, float *C, int m, int n, int k, const float *A, bool transA,

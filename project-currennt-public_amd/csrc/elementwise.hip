@@ -238,12 +238,19 @@ extern "C++" int cnt::dense_backward_weights_batch(hipStream_t stream, int P, in
     // weight part and brings the bias part (row sums of the errors) along
     ga.overwrite_ok = 1;
     ga.rowsum = 1;
-    gemm_plan(ga);
+    gemm_plan(ga, stream);
     if (ga.epilogue == EPI_PARTIAL) return gemm_launch(stream, ga);
     for (int z = 0; z < count; ++z) CNT_TRY(fill_zero(stream, weight_updates[z], (size_t)P * D + D));
     CNT_TRY(gemm_launch(stream, ga));
     for (int z = 0; z < count; ++z)
         CNT_TRY(column_sum(stream, err[z], D, N, bias[z], weight_updates[z] + (size_t)P * D));
+    return CNT_OK;
+}
+
+int cnt_gemm_reserve(void *stream) { return cnt::gemm_reserve_stream(static_cast<hipStream_t>(stream)); }
+
+int cnt_gemm_release(void *stream) {
+    cnt::gemm_release_stream(static_cast<hipStream_t>(stream));
     return CNT_OK;
 }
 

@@ -74,12 +74,21 @@ std::mutex g_split_mu;  // held while a product and its reduction are enqueued, 
 std::vector<SplitScratch> g_split_scratch;
 
 // One scratch buffer per stream: launches on a stream execute in order, so the next product on the same stream
-// cannot overwrite partial sums that a reduction has yet to read.  Never freed.
-float *split_scratch(hipStream_t stream) {
+// cannot overwrite partial sums that a reduction has yet to read.  Kept until gemm_release_stream.
+float *split_scratch_find(hipStream_t stream) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     for (const SplitScratch &e : g_split_scratch)
         if (e.device == dev && e.stream == stream) return e.buf;
+    return nullptr;
+}
+
+// the stream's buffer, allocated now if the stream has none; NULL when the allocation is refused (out of memory,
+// a stream under capture): the caller then takes the atomic path
+float *split_scratch(hipStream_t stream) {
+    if (float *buf = split_scratch_find(stream)) return buf;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     float *buf = nullptr;
     if (hipMalloc(reinterpret_cast<void **>(&buf), kSplitScratchFloats * sizeof(float)) != hipSuccess) {
         (void)hipGetLastError();
@@ -146,7 +155,13 @@ void gemm_release_stream(hipStream_t stream) {
         }
 }
 
-void gemm_plan(GemmArgs &args) {
+int gemm_reserve_stream(hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_split_mu);
+    CNT_REQUIRE(split_scratch(stream) != nullptr, "gemm: no memory for the split-K scratch buffer");
+    return CNT_OK;
+}
+
+void gemm_plan(GemmArgs &args, hipStream_t stream) {
     if (args.splitk != 0) return;
     // Long-K products with a small output (weight gradients): cut K so that the launch has about
     // `target` workgroups of 64 x 64 tiles, but leave every workgroup at least eight k-iterations -- each
@@ -165,8 +180,16 @@ void gemm_plan(GemmArgs &args) {
     const long out = (long)args.m * args.n * args.nprob;
     const size_t stride = (size_t)out + (args.rowsum ? (size_t)args.n * args.nprob : 0);
     const bool rowsum_ok = !args.rowsum || (args.nseg == 1 && !args.masked);
-    if (partial_on && args.epilogue == EPI_ATOMIC && args.overwrite_ok && rowsum_ok && s >= 8 &&
-        out <= kPartialMaxOutput && stride * (size_t)s <= kSplitScratchFloats) {
+    bool partial = partial_on && args.epilogue == EPI_ATOMIC && args.overwrite_ok && rowsum_ok && s >= 8 &&
+                   out <= kPartialMaxOutput && stride * (size_t)s <= kSplitScratchFloats;
+    if (partial && !args.partial) {
+        // the stream's scratch buffer: reserved by its owner, else allocated on first use; without one (allocation
+        // refused) the product adds atomically
+        std::lock_guard<std::mutex> lock(g_split_mu);
+        args.partial = split_scratch(stream);
+        partial = args.partial != nullptr;
+    }
+    if (partial) {
         args.epilogue = EPI_PARTIAL;
         args.partial_stride = stride;
     } else {
@@ -186,7 +209,7 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
                 "gemm: split-K needs the atomic epilogue");
     CNT_REQUIRE(args.epilogue != EPI_FAN || (gemm_fan_supported(args) && args.splitk == 1),
                 "gemm: the fan epilogue exists for one unsplit problem with 16-byte row-contiguous A and k-contiguous B");
-    CNT_REQUIRE(args.epilogue != EPI_PARTIAL || (args.splitk >= 1 && args.partial_stride > 0),
+    CNT_REQUIRE(args.epilogue != EPI_PARTIAL || (args.splitk >= 1 && args.partial_stride > 0 && args.partial),
                 "gemm: the partial-product epilogue is chosen by gemm_plan only");
     for (int p = 0; p < args.nprob; ++p) {
         CNT_REQUIRE(args.prob[p].C != nullptr, "gemm: null output");
@@ -194,18 +217,15 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
             CNT_REQUIRE(args.prob[p].A[s] && args.prob[p].B[s], "gemm: null operand");
     }
     const int va = pick_vec(args, true), vb = pick_vec(args, false);
-    gemm_plan(args);
+    gemm_plan(args, stream);
     if (args.epilogue != EPI_PARTIAL) args.rowsum = 0;
     const int tile = pick_tile(args);
     const int tiles = ((args.m + tile - 1) / tile) * ((args.n + tile - 1) / tile);
     dim3 grid(tiles, args.splitk, args.nprob);
     ProfileScope prof(stream, args.label ? args.label : "gemm");
     std::unique_lock<std::mutex> split_lock(g_split_mu, std::defer_lock);
-    if (args.epilogue == EPI_PARTIAL) {
-        split_lock.lock();
-        args.partial = split_scratch(stream);
-        CNT_REQUIRE(args.partial != nullptr, "gemm: no memory for the split-K scratch buffer");
-    }
+    // a product and its reduction stay adjacent on the stream
+    if (args.epilogue == EPI_PARTIAL) split_lock.lock();
     if (va == 4) gemm_dispatch_va4(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
     else if (va == 2) gemm_dispatch_va2(args, grid, stream, args.a_kcontig, vb, args.b_kcontig, tile);
     else if (args.a_kcontig) gemm_dispatch_va1k(args, grid, stream, vb, args.b_kcontig, tile);

@@ -983,6 +983,7 @@ int finish_build(cnt_network *net, const json::Value *weights) {
     for (int k = 0; k < net->n_side; ++k) {
         CNT_HIP(hipStreamCreateWithFlags(&net->side[k], hipStreamNonBlocking));
         CNT_HIP(hipEventCreateWithFlags(&net->ev_side[k], hipEventDisableTiming));
+        CNT_TRY(cnt::gemm_reserve_stream(net->side[k]));  // the weight halves' split-K scratch, not inside a pass
     }
     return CNT_OK;
 }

@@ -594,7 +594,7 @@ extern "C++" int cnt::wavnetc_backward_weights_batch(hipStream_t stream, int D, 
     }
     ga.label = "gemm:wavnetc_dW";
     ga.overwrite_ok = 1;  // the product covers all C x 2D weights
-    gemm_plan(ga);
+    gemm_plan(ga, stream);
     if (ga.epilogue != EPI_PARTIAL)
         for (int z = 0; z < count; ++z) CNT_TRY(fill_zero(stream, weight_updates[z], (size_t)C * 2 * D));
     return gemm_launch(stream, ga);
