@@ -75,6 +75,15 @@ int cnt_dense_backward_weights(void *stream, int P, int D, int N, float bias, co
  * memory, a stream under capture) adds its splits atomically instead. */
 int cnt_gemm_reserve(void *stream);
 int cnt_gemm_release(void *stream);
+/* cnt_dense_backward_weights for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): same arguments, same result, but the split partial products go
+ * through an 8 MB array that is part of the library's code object (one copy per GPU, held until the process ends),
+ * so the call allocates nothing.  No counterpart in the reference.  Limit: P*D + D <= 2 097 152 floats, larger
+ * layers are refused with CNT_ERR_ARG.  All calls on one GPU share that array: calls that overlap in time on one
+ * GPU (different streams or threads) race; calls on one stream are ordered and safe. */
+int cnt_dense_backward_weights_static(void *stream, int P, int D, int N, float bias, const float *x, const float *err,
+                                      float *weight_updates);
+
 /* ---- SSE post-output layer ---------------------------------------------------------------------
  * SsePostOutputLayer::computeBackwardPass (layers/SsePostOutputLayer.cu:224-267):
  * err = y - target, exactly 0 on padding slots. */

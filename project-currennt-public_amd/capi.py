@@ -67,6 +67,7 @@ _SIGNATURES = {
     "cnt_dense_backward": (I, [VP, I, I, I, I, F, VP, VP, VP, VP, VP, VP]),
     "cnt_dense_backward_errors": (I, [VP, I, I, I, I, VP, VP, VP, VP]),
     "cnt_dense_backward_weights": (I, [VP, I, I, I, F, VP, VP, VP]),
+    "cnt_dense_backward_weights_static": (I, [VP, I, I, I, F, VP, VP, VP]),
     "cnt_gemm_reserve": (I, [VP]),
     "cnt_gemm_release": (I, [VP]),
     "cnt_sse_backward": (I, [VP, I, I, VP, VP, VP, VP]),
@@ -219,6 +220,10 @@ def dense_backward_errors(P, D, N, act, W, y, err, prev_err, stream=None):
 
 def dense_backward_weights(P, D, N, bias, x, err, dW, stream=None):
     check(lib().cnt_dense_backward_weights(stream_ptr(stream), P, D, N, bias, ptr(x), ptr(err), ptr(dW)))
+
+
+def dense_backward_weights_static(P, D, N, bias, x, err, dW, stream=None):
+    check(lib().cnt_dense_backward_weights_static(stream_ptr(stream), P, D, N, bias, ptr(x), ptr(err), ptr(dW)))
 
 
 def gemm_reserve(stream=None):

@@ -180,6 +180,9 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args);
 void gemm_release_stream(hipStream_t stream);
 // Allocates the split-K scratch buffer of `stream` now instead of inside the first product that wants it.
 int gemm_reserve_stream(hipStream_t stream);
+// cnt_dense_backward_weights with the partial products in a scratch array that is part of the code object
+int gemm_dense_weights_static(hipStream_t stream, int P, int D, int N, float bias, const float *x, const float *err,
+                              float *weight_updates);
 
 // Convenience: single problem, BLAS-like transposes on column-major matrices.
 int gemm_simple(hipStream_t stream, float *C, int m, int n, int k, const float *A, bool transA,

@@ -247,6 +247,14 @@ extern "C++" int cnt::dense_backward_weights_batch(hipStream_t stream, int P, in
     return CNT_OK;
 }
 
+int cnt_dense_backward_weights_static(void *stream, int P, int D, int N, float bias, const float *x, const float *err,
+                                      float *weight_updates) {
+    using namespace cnt;
+    CNT_REQUIRE(x && err && weight_updates, "dense_backward_weights_static: null argument");
+    CNT_REQUIRE(P > 0 && D > 0 && N > 0, "dense_backward_weights_static: non-positive size");
+    return gemm_dense_weights_static(static_cast<hipStream_t>(stream), P, D, N, bias, x, err, weight_updates);
+}
+
 int cnt_gemm_reserve(void *stream) { return cnt::gemm_reserve_stream(static_cast<hipStream_t>(stream)); }
 
 int cnt_gemm_release(void *stream) {

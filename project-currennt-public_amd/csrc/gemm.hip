@@ -98,6 +98,35 @@ float *split_scratch(hipStream_t stream) {
     return buf;
 }
 
+// ----- scratch that is part of the loaded code object, for callers that must not allocate ---------------------
+// Every device the library runs on holds its own copy of this array at its own address until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress: the address a kernel may use is looked
+// up once per device and kept in g_static_ptr.
+constexpr size_t kStaticScratchFloats = (size_t)2 << 20;  // 8 MB
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+float *g_static_ptr[kMaxDevices];
+
+// device address of the current device's copy of `scratch` (NULL with the error text set on failure)
+float *static_scratch() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("static scratch: no current device");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_split_mu);
+    if (!g_static_ptr[dev]) {
+        void *ptr = nullptr;
+        const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !ptr) {
+            set_error("static scratch: hipGetSymbolAddress: %s", hipGetErrorString(err));
+            return nullptr;
+        }
+        g_static_ptr[dev] = static_cast<float *>(ptr);
+    }
+    return g_static_ptr[dev];
+}
+
 // 32 consecutive outputs per block, the splits dealt to eight groups of 32 threads whose sums meet in LDS; four
 // loads in flight per thread
 constexpr int kReduceOutputs = 32;
@@ -238,6 +267,42 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
         CNT_HIP(hipGetLastError());
     }
     return CNT_OK;
+}
+
+// A dense layer's weight gradient (dW = x * delta^T, P x D, plus the bias part: bias * row sums of delta) as a
+// split-K product whose partial products go through the code object's own scratch array: no allocation at all.
+int gemm_dense_weights_static(hipStream_t stream, int P, int D, int N, float bias, const float *x, const float *err,
+                              float *weight_updates) {
+    const size_t stride = (size_t)P * D + D;
+    CNT_REQUIRE(stride <= kStaticScratchFloats,
+                "dense_backward_weights_static: %d x %d weights + %d biases = %zu floats exceed the static scratch of %zu "
+                "floats; use cnt_dense_backward_weights", P, D, D, stride, kStaticScratchFloats);
+    float *buf = static_scratch();
+    if (!buf) return CNT_ERR_HIP;
+    GemmArgs ga = {};
+    ga.m = P; ga.n = D; ga.k = N;
+    ga.a_kcontig = 0; ga.lda = P;
+    ga.b_kcontig = 0; ga.ldb = D;
+    ga.ldc = P;
+    ga.nseg = 1; ga.nprob = 1;
+    ga.prob[0].A[0] = x; ga.prob[0].B[0] = err; ga.prob[0].C = weight_updates;
+    ga.prob[0].rowsum_out = weight_updates + (size_t)P * D;
+    ga.prob[0].rowsum_scale = bias;
+    ga.label = "gemm:dense_dW_static";
+    ga.rowsum = 1;
+    // as many splits as the usual plan takes, as far as their partial products fit into the array
+    GemmArgs probe = ga;
+    probe.epilogue = EPI_ATOMIC; probe.splitk = 0; probe.overwrite_ok = 0;
+    gemm_plan(probe, stream);
+    size_t splits = (size_t)probe.splitk;
+    if (splits * stride > kStaticScratchFloats) splits = kStaticScratchFloats / stride;
+    const long kt = ((long)N + BK - 1) / BK;
+    while (splits > 1 && ((long)splits - 1) * ((kt + (long)splits - 1) / (long)splits) >= kt) --splits;  // no empty split
+    ga.splitk = (int)splits;
+    ga.epilogue = EPI_PARTIAL;
+    ga.partial = buf;
+    ga.partial_stride = stride;
+    return gemm_launch(stream, ga);
 }
 
 int gemm_simple(hipStream_t stream, float *C, int m, int n, int k, const float *A, bool transA,
