@@ -188,6 +188,18 @@ int gemm_dense_weights_static(hipStream_t stream, int P, int D, int N, float bia
 int gemm_simple(hipStream_t stream, float *C, int m, int n, int k, const float *A, bool transA,
                 const float *B, bool transB, bool accumulate);
 
+// cnt_opt_step with a device flag in front of it: when *veto is non-zero at the time the kernel runs (a recursion of
+// the pass that produced the gradients gave up), the step changes nothing.
+int opt_step_guarded(hipStream_t stream, int option, long n, float *weights, const float *layer_updates, float *cur_updates,
+                     float *stats, float *weight_deltas, const float *mask, float frac_length, float beta1_accum,
+                     float beta2_accum, float learning_rate, float momentum, const int *veto);
+// LSTM handles of a network share one such flag: a recursion that gives up also sets *veto (until the owner clears it).
+void lstm_set_veto(cnt_lstm *h, int *veto);
+// non-zero if a recursion of this handle has given up since the last report (no synchronisation: it only sees
+// launches that have already ended); the report clears the mark
+int lstm_take_failure(cnt_lstm *h);
+int report_failure(cnt_network *net);
+
 // ----- error halves that also do the backward step of the skip layer in front of them ----------------
 // A skip layer adds what its linkers left in its side buffer to the errors its following layer wrote, and hands the
 // sum on (layers/SkipAddLayer.cu:305-346).  When that following layer is a dense or convolution layer, the sum and

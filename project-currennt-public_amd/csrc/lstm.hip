@@ -29,6 +29,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <new>
+#include <type_traits>
 #include <vector>
 
 namespace cnt {
@@ -64,7 +65,22 @@ struct ChainParams {
     long long *phase_ticks;  // optional diagnostic: per workgroup accumulated phase durations (100 MHz ticks)
     int poll_delay, poll_gap;  // s_sleep units before the first poll of a step / between polls
     int poll_delay_fwd;
+    int *latch;  // host-visible mark "a recursion of this handle gave up" (pinned host memory), never cleared by kernels
+    int *veto;   // optional device flag shared by a network's handles, set together with the latch
+    // XCD-local backward recursion: jobs = (direction, group of sequences), see lstm_local.hpp
+    int njobs;
+    struct { int dir, seq0, nseq; } job[8];
+    unsigned *ctl;   // placement counters, zero at launch
+    float *lmail;    // one mailbox per job
 };
+
+// A workgroup that gives up: every workgroup of the launch sees the device flag and drains; the host sees the latch
+// at its next call into the handle, the optimizer step of a network sees the veto flag.
+__device__ __forceinline__ void raise_abort(const ChainParams &p) {
+    __hip_atomic_store(p.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(p.latch, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (p.veto) __hip_atomic_store(p.veto, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
 // global load and store of the wave, which would put the HBM latency of the look-ahead loads and the
@@ -420,7 +436,7 @@ __global__ __launch_bounds__(fwd_threads(JB, NT)) void lstm_forward_chain(const 
         if (!ok) wait_failed = 1;
         lds_barrier();
         if (wait_failed) {
-            if (tid == 0) __hip_atomic_store(p.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (tid == 0) raise_abort(p);
             return;
         }
         if (timing) ph0 += wall_clock64() - tk0;
@@ -735,7 +751,7 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
             if (!ok) wait_failed = 1;
             lds_barrier();  // A
             if (wait_failed) {
-                if (tid == 0) __hip_atomic_store(p.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (tid == 0) raise_abort(p);
                 return;
             }
         }
@@ -787,6 +803,29 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
         long long *o = p.phase_ticks + (size_t)blockIdx.x * 6;
         o[0] = ph0; o[1] = ph1; o[3] = ph3; o[4] = poll_rounds;
     }
+}
+
+#include "lstm_local.hpp"
+
+// Runs in front of every recursion launch (one workgroup).  If the launch before gave up, the device flag is still
+// set and mailbox words may be left over: refill the mailboxes and clear the flag, so that a handle heals without
+// its owner's help.  Always: zero the placement counters of the XCD-local recursion.
+struct GuardParams {
+    int *abort_flag;
+    unsigned *ctl;
+    int nctl;
+    unsigned *mail[3];
+    size_t words[3];
+};
+__global__ __launch_bounds__(1024) void chain_guard(const GuardParams g) {
+    const bool heal = __hip_atomic_load(g.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+    if (heal) {
+        for (int m = 0; m < 3; ++m)
+            for (size_t i = threadIdx.x; i < g.words[m]; i += blockDim.x) g.mail[m][i] = kEmpty;
+    }
+    for (int i = threadIdx.x; i < g.nctl; i += blockDim.x) g.ctl[i] = 0u;
+    __syncthreads();
+    if (heal && threadIdx.x == 0) __hip_atomic_store(g.abort_flag, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -1013,6 +1052,16 @@ struct cnt_lstm {
     int last_was_forward;  // which recursion the diagnostic buffer describes
     int bmail_dirty;       // the backward mailbox may hold words that are not empty
     int stepwise;          // no persistent recursion kernel for this geometry: one product + one cell kernel per step
+    int *latch_host, *latch_dev;  // pinned host word a kernel that gives up sets; read by the host without a sync
+    int *veto;             // a network's shared flag (device), or NULL
+    // XCD-local backward recursion
+    int local;             // 1: lstm_backward_local runs the error recursion
+    int njobs;
+    struct { int dir, seq0, nseq; } job[8];
+    unsigned *ctl;
+    float *lmail;
+    size_t lmail_words;
+    int last_blocks;       // workgroups of the last recursion launch
 };
 
 namespace cnt {
@@ -1066,26 +1115,63 @@ void fill_chain_params(const cnt_lstm *h, const float *weights, ChainParams &p) 
     }
     p.spin_limit = h->spin_limit;
     p.abort_flag = h->abort_flag;
+    p.latch = h->latch_dev;
+    p.veto = h->veto;
+    p.njobs = h->njobs;
+    for (int j = 0; j < h->njobs; ++j) { p.job[j].dir = h->job[j].dir; p.job[j].seq0 = h->job[j].seq0; p.job[j].nseq = h->job[j].nseq; }
+    p.ctl = h->ctl;
+    p.lmail = h->lmail;
     p.phase_ticks = h->phase_ticks;
     p.poll_delay = h->poll_delay; p.poll_gap = h->poll_gap; p.poll_delay_fwd = h->poll_delay_fwd;
 }
 
+chain_kernel_t pick_local_kernel(int H, int &JB) {
+    if (H == 256) { JB = 8; return (chain_kernel_t)lstm_backward_local<256, 8>; }
+    if (H == 128) { JB = 4; return (chain_kernel_t)lstm_backward_local<128, 4>; }
+    if (H == 64) { JB = 4; return (chain_kernel_t)lstm_backward_local<64, 4>; }
+    return nullptr;
+}
+
 int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
-    chain_kernel_t k = pick_kernel(fwd, h->H, h->JB, h->NT);
+    const bool local = !fwd && h->local;
+    int local_jb = 0;
+    chain_kernel_t k = local ? pick_local_kernel(h->H, local_jb) : pick_kernel(fwd, h->H, h->JB, h->NT);
     CNT_REQUIRE(k != nullptr, "lstm: no recursion kernel for H=%d JB=%d S=%d", h->H, h->JB, h->desc.S);
-    // Every word of the mailbox starts out empty.  The forward recursion leaves its last outputs behind; the
-    // backward recursion hands every word back, so its mailbox only needs the fill once and again after a
-    // recursion that gave up (cnt_lstm_check marks it dirty).
+    {
+        // heals the handle after a launch that gave up, zeroes the placement counters
+        GuardParams g = {};
+        g.abort_flag = h->abort_flag;
+        g.ctl = h->ctl; g.nctl = h->ctl ? kCtlWords : 0;
+        g.mail[0] = reinterpret_cast<unsigned *>(h->bmail[0]); g.words[0] = h->bmail[0] ? h->bmail_words : 0;
+        g.mail[1] = reinterpret_cast<unsigned *>(h->bmail[1]); g.words[1] = h->bmail[1] ? h->bmail_words : 0;
+        g.mail[2] = reinterpret_cast<unsigned *>(h->lmail); g.words[2] = h->lmail ? h->lmail_words : 0;
+        hipLaunchKernelGGL(chain_guard, dim3(1), dim3(1024), 0, stream, g);
+        CNT_HIP(hipGetLastError());
+    }
+    // Every word of a mailbox starts out empty.  The forward recursion leaves its last outputs behind; the
+    // backward recursions hand every word back, so their mailboxes need the fill once (and the guard above refills
+    // them after a recursion that gave up).
     for (int dir = 0; dir < h->ndir; ++dir) {
         if (fwd) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->fmail[dir]), h->fmail_words, kEmpty));
-        else if (h->bmail_dirty) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->bmail[dir]), h->bmail_words, kEmpty));
+        else if (h->bmail_dirty && h->bmail[dir]) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->bmail[dir]), h->bmail_words, kEmpty));
     }
+    if (!fwd && h->bmail_dirty && h->lmail) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->lmail), h->lmail_words, kEmpty));
     if (!fwd) h->bmail_dirty = 0;
+    h->last_was_forward = fwd ? 1 : 0;
+    ProfileScope prof(stream, fwd ? "lstm_forward_chain" : "lstm_backward_chain");
+    if (local) {
+        // enough workgroups that njobs complete teams form on any spread over the XCDs
+        const int G = h->H / local_jb;
+        const int blocks = (h->njobs * G + 8 * (G - 1) + 7) / 8 * 8;
+        h->last_blocks = blocks;
+        hipLaunchKernelGGL(k, dim3(blocks), dim3(local_threads(h->H)), 0, stream, p);
+        CNT_HIP(hipGetLastError());
+        return CNT_OK;
+    }
     const int G = h->H / h->JB;
     p.xcd_pack = fwd ? h->xcd_pack : 0;
     const int blocks = p.xcd_pack ? 8 * G : h->ndir * G;
-    h->last_was_forward = fwd ? 1 : 0;
-    ProfileScope prof(stream, fwd ? "lstm_forward_chain" : "lstm_backward_chain");
+    h->last_blocks = blocks;
     hipLaunchKernelGGL(k, dim3(blocks), dim3(fwd ? kThreads + 64 * ((h->JB * 16 * h->NT + 63) / 64) + 64 : kBwdThreads), 0, stream, p);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
@@ -1229,10 +1315,42 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
         if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->fmail[dir]), h->fmail_words * sizeof(float));
         if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->bmail[dir]), h->bmail_words * sizeof(float));
     }
+    // XCD-local error recursion: 64, 128 or 256 cells per direction and sequence groups of at most four
+    {
+        int local_jb = 0;
+        const int max_jobs = kLocalMaxJobs / ndir;  // per direction
+        const int groups = desc->S < max_jobs ? desc->S : max_jobs;
+        const bool fits = !stepwise && pick_local_kernel(H, local_jb) != nullptr && (desc->S + groups - 1) / groups <= kLocalSeqs;
+        const char *e = std::getenv("CNT_LSTM_LOCAL");
+        h->local = fits && (!e || std::atoi(e) != 0);
+        if (h->local) {
+            // sequences dealt to the groups as evenly as possible, in order
+            for (int dir = 0; dir < ndir; ++dir) {
+                int seq = 0;
+                for (int q = 0; q < groups; ++q) {
+                    const int cnt = desc->S / groups + (q < desc->S % groups ? 1 : 0);
+                    h->job[h->njobs].dir = dir; h->job[h->njobs].seq0 = seq; h->job[h->njobs].nseq = cnt;
+                    ++h->njobs;
+                    seq += cnt;
+                }
+            }
+            h->lmail_words = (size_t)h->njobs * (size_t)kMailSlots * (H / local_jb) * (H / local_jb) * kLocalSeqs * local_jb;
+            if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->lmail), h->lmail_words * sizeof(float));
+            if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->ctl), kCtlWords * sizeof(unsigned));
+            if (err == hipSuccess) err = hipMemset(h->ctl, 0, kCtlWords * sizeof(unsigned));
+        }
+    }
     if (err == hipSuccess && std::getenv("CNT_LSTM_TIMING"))
         err = hipMalloc(reinterpret_cast<void **>(&h->phase_ticks), 8 * 512 * 6 * sizeof(long long));
+    if (err == hipSuccess && h->phase_ticks) err = hipMemset(h->phase_ticks, 0, 8 * 512 * 6 * sizeof(long long));
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->abort_flag), sizeof(int));
     if (err == hipSuccess) err = hipMemset(h->abort_flag, 0, sizeof(int));
+    // the word a kernel that gives up sets for the host: pinned, mapped, coherent host memory
+    if (err == hipSuccess) err = hipHostMalloc(reinterpret_cast<void **>(&h->latch_host), sizeof(int), hipHostMallocMapped);
+    if (err == hipSuccess) {
+        *h->latch_host = 0;
+        err = hipHostGetDevicePointer(reinterpret_cast<void **>(&h->latch_dev), h->latch_host, 0);
+    }
     if (err != hipSuccess) {
         set_error("lstm_create: %s", hipGetErrorString(err));
         cnt_lstm_destroy(h);
@@ -1252,6 +1370,9 @@ int cnt_lstm_destroy(cnt_lstm *h) {
     }
     if (h->abort_flag) (void)hipFree(h->abort_flag);
     if (h->phase_ticks) (void)hipFree(h->phase_ticks);
+    if (h->lmail) (void)hipFree(h->lmail);
+    if (h->ctl) (void)hipFree(h->ctl);
+    if (h->latch_host) (void)hipHostFree(h->latch_host);
     delete h;
     return CNT_OK;
 }
@@ -1286,15 +1407,39 @@ float *cnt_lstm_state(cnt_lstm *h, int dir, int which) {
     return h->state[dir][which];
 }
 
+static const char *kGaveUp = "lstm: a recursion kernel gave up waiting for a neighbouring workgroup; results are invalid";
+
+extern "C++" void cnt::lstm_set_veto(cnt_lstm *h, int *veto) {
+    if (h) h->veto = veto;
+}
+
+extern "C++" int cnt::lstm_take_failure(cnt_lstm *h) {
+    if (!h || !h->latch_host) return 0;
+    volatile int *latch = h->latch_host;
+    if (*latch == 0) return 0;
+    *latch = 0;
+    return 1;
+}
+
+// Every entry point that launches or consumes a recursion starts with this: a recursion that gave up in an EARLIER
+// call (and has ended by now) turns the current call into CNT_ERR_DEVICE, also for callers that never call
+// cnt_lstm_check.  The handle itself is healed by the guard kernel in front of its next launch.  A handle that belongs to
+// a network (it carries the network's veto flag) leaves the report to the network's entry points.
+#define CNT_LSTM_REPORT_FAILURE(h)              \
+    do {                                        \
+        if (!(h)->veto && cnt::lstm_take_failure(h)) { \
+            cnt::set_error("%s", kGaveUp);      \
+            return CNT_ERR_DEVICE;              \
+        }                                       \
+    } while (0)
+
 int cnt_lstm_check(cnt_lstm *h, void *stream) {
     using namespace cnt;
     CNT_REQUIRE(h, "lstm_check: null handle");
-    int flag = 0;
     CNT_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
-    CNT_HIP(hipMemcpy(&flag, h->abort_flag, sizeof(int), hipMemcpyDeviceToHost));
     if (h->phase_ticks) {
-        // diagnostic: mean phase durations of the last backward recursion over the workgroups that took part
-        const int blocks = h->ndir * (h->H / h->JB);
+        // diagnostic: mean phase durations of the last recursion over the workgroups that took part
+        const int blocks = h->last_blocks;
         std::vector<long long> t((size_t)blocks * 6);
         CNT_HIP(hipMemcpy(t.data(), h->phase_ticks, t.size() * sizeof(long long), hipMemcpyDeviceToHost));
         CNT_HIP(hipMemset(h->phase_ticks, 0, t.size() * sizeof(long long)));
@@ -1311,13 +1456,12 @@ int cnt_lstm_check(cnt_lstm *h, void *stream) {
                          "(T=%d, %d workgroups)\n", m[0] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, h->T, active);
         else
             std::fprintf(stderr, "lstm backward per step [us]: receive waves wait %.3f cell %.3f loop %.3f poll rounds %.2f | "
-                         "product waves busy %.3f | memory wave busy after B %.3f (T=%d, %d workgroups)\n",
-                         m[0] * us, m[1] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, m[2] * us, m[5] * us, h->T, active);
+                         "product waves busy %.3f | memory wave busy after B %.3f (T=%d, %d workgroups%s)\n",
+                         m[0] * us, m[1] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, m[2] * us, m[5] * us, h->T, active,
+                         h->local ? ", XCD-local" : "");
     }
-    if (flag != 0) {
-        h->bmail_dirty = 1;
-        CNT_HIP(hipMemset(h->abort_flag, 0, sizeof(int)));
-        set_error("lstm: a recursion kernel gave up waiting for a neighbouring workgroup; results are invalid");
+    if (lstm_take_failure(h)) {
+        set_error("%s", kGaveUp);
         return CNT_ERR_DEVICE;
     }
     return CNT_OK;
@@ -1327,6 +1471,7 @@ int cnt_lstm_forward(cnt_lstm *h, void *stream_, const float *weights, const flo
     using namespace cnt;
     CNT_REQUIRE(h && weights && x && outputs, "lstm_forward: null argument");
     CNT_REQUIRE(h->T > 0, "lstm_forward: load_sequences has not been called");
+    CNT_LSTM_REPORT_FAILURE(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const cnt_lstm_desc &d = h->desc;
     const int P = d.P, L = d.L, H = h->H, N = h->T * d.S;
@@ -1362,6 +1507,7 @@ int cnt_lstm_backward_errors(cnt_lstm *h, void *stream_, const float *weights, f
     using namespace cnt;
     CNT_REQUIRE(h && weights && output_errors, "lstm_backward_errors: null argument");
     CNT_REQUIRE(h->T > 0, "lstm_backward_errors: load_sequences has not been called");
+    CNT_LSTM_REPORT_FAILURE(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
 
     // 1. error recursion (splits the interleaved output errors on the fly)
@@ -1381,6 +1527,7 @@ int cnt_lstm_backward_prev_errors(cnt_lstm *h, void *stream_, const float *weigh
     using namespace cnt;
     CNT_REQUIRE(h && weights && prev_errors, "lstm_backward_prev_errors: null argument");
     CNT_REQUIRE(h->T > 0, "lstm_backward_prev_errors: load_sequences has not been called");
+    CNT_LSTM_REPORT_FAILURE(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const cnt_lstm_desc &d = h->desc;
     const int P = d.P, L = d.L, H = h->H, S = d.S, N = h->T * S;
@@ -1408,6 +1555,7 @@ int cnt_lstm_backward_weights(cnt_lstm *h, void *stream_, const float *x, float 
     using namespace cnt;
     CNT_REQUIRE(h && x && weight_updates, "lstm_backward_weights: null argument");
     CNT_REQUIRE(h->T > 0, "lstm_backward_weights: load_sequences has not been called");
+    CNT_LSTM_REPORT_FAILURE(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const cnt_lstm_desc &d = h->desc;
     const int P = d.P, L = d.L, H = h->H, S = d.S, N = h->T * S;

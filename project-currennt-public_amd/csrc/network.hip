@@ -473,6 +473,8 @@ struct cnt_network {
     int stats_option = -1;
     float beta1_accum = 1.0f, beta2_accum = 1.0f;
     int mdn_target_start = 0, mdn_classes = 0;
+    // set on the device by an LSTM recursion that gives up; the optimizer step looks at it and leaves the weights alone
+    int *veto = nullptr;
 };
 
 namespace cnt {
@@ -558,6 +560,8 @@ int build_layer_into(cnt_network *net, NetLayer &L, const json::Value &obj, cons
         L.bidir = t == "blstm";
         cnt_lstm_desc d = {P, L.size, L.bidir, net->S, L.maxTr, L.bias};
         CNT_TRY(cnt_lstm_create(&d, &L.lstm));
+        if (!net->veto) CNT_TRY(device_alloc(net, (void **)&net->veto, sizeof(int), true));
+        cnt::lstm_set_veto(L.lstm, net->veto);
     } else if (t == "skipini" || t == "skipadd") {
         // NeuralNetwork.cpp:470-530 offers every earlier skip layer plus the layer right before; SkipAddLayer.cu:
         // 96-138 keeps those named by preSkipLayer, or by default the last two of the offer (a skipini, and the
@@ -1127,6 +1131,7 @@ int cnt_network_load_sequences(cnt_network *net, void *stream_, int T, int Tmin,
                                const float *inputs, const float *targets) {
     using namespace cnt;
     CNT_REQUIRE(net && patTypes, "network_load_sequences: null argument");
+    CNT_TRY(report_failure(net));
     CNT_REQUIRE(T >= 1 && T <= net->maxT && Tmin >= 1 && Tmin <= T, "network_load_sequences: lengths %d / %d outside "
                 "1..%d", T, Tmin, net->maxT);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -1164,6 +1169,7 @@ int cnt_network_load_sequences(cnt_network *net, void *stream_, int T, int Tmin,
 int cnt_network_forward(cnt_network *net, void *stream_) {
     using namespace cnt;
     CNT_REQUIRE(net && net->T > 0, "network_forward: no fraction loaded");
+    CNT_TRY(report_failure(net));
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     // what the skip layers' forward passes clear (layers/SkipAddLayer.cu:195-205)
     if (net->skip_error_count) CNT_TRY(fill_zero(stream, net->skip_errors, net->skip_error_count));
@@ -1280,6 +1286,7 @@ int cnt_network_calculate_error(cnt_network *net, void *stream_, float *loss_dev
 int cnt_network_backward(cnt_network *net, void *stream_) {
     using namespace cnt;
     CNT_REQUIRE(net && net->T > 0, "network_backward: no fraction loaded");
+    CNT_TRY(report_failure(net));
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     int next_side = 0;
     bool side_used[cnt_network::kMaxSide] = {};
@@ -1534,18 +1541,42 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     return CNT_OK;
 }
 
+// CNT_ERR_DEVICE if a recursion of one of the network's LSTM layers has given up (and ended) since the last report;
+// clears every layer's mark and the device flag that holds the optimizer step back.
+extern "C++" int cnt::report_failure(cnt_network *net) {
+    bool failed = false;
+    for (auto &L : net->layers)
+        if (L.lstm && cnt::lstm_take_failure(L.lstm)) failed = true;
+    if (!failed) return CNT_OK;
+    if (net->veto) CNT_HIP(hipMemset(net->veto, 0, sizeof(int)));
+    set_error("network: an LSTM recursion gave up waiting for a neighbouring workgroup; the results of that pass are "
+              "invalid and a weight update that followed it was skipped");
+    return CNT_ERR_DEVICE;
+}
+
 int cnt_network_check(cnt_network *net, void *stream) {
     using namespace cnt;
     CNT_REQUIRE(net, "network_check: null handle");
+    // every recurrent layer is looked at (each report clears that layer's mark), the first failure is returned
+    int status = CNT_OK;
     for (auto &L : net->layers)
-        if (L.lstm) CNT_TRY(cnt_lstm_check(L.lstm, stream));
-    return CNT_OK;
+        if (L.lstm) {
+            const int s = cnt_lstm_check(L.lstm, stream);
+            if (s != CNT_OK && status == CNT_OK) status = s;
+        }
+    if (status != CNT_OK && net->veto) CNT_HIP(hipMemset(net->veto, 0, sizeof(int)));
+    if (status == CNT_OK) status = report_failure(net);  // a layer whose launch ended on another stream
+    return status;
 }
 
 int cnt_network_update(cnt_network *net, void *stream_, int option, float learning_rate, float momentum,
                        float frac_length) {
     using namespace cnt;
     CNT_REQUIRE(net, "network_update: null handle");
+    // A pass whose recursion gave up must not reach the weights.  Two nets: launches that have already ended are
+    // seen here, on the host; one that ends later sets the device flag the optimizer kernel looks at, and the next
+    // call into the network reports it.
+    CNT_TRY(report_failure(net));
     const size_t n = (size_t)net->n_weights;
     if (!net->cur_updates) {
         CNT_TRY(device_alloc(net, (void **)&net->cur_updates, n * sizeof(float), true));
@@ -1568,8 +1599,9 @@ int cnt_network_update(cnt_network *net, void *stream_, int option, float learni
     bool own_rates = false;
     for (const auto &L : net->layers) own_rates = own_rates || (L.weight_count() > 0 && L.learning_rate > -0.5f);
     if (!own_rates)
-        return cnt_opt_step(stream_, option, (long)n, net->weights, net->updates, net->cur_updates, net->stats, net->deltas,
-                            nullptr, frac_length, net->beta1_accum, net->beta2_accum, learning_rate, momentum);
+        return opt_step_guarded(static_cast<hipStream_t>(stream_), option, (long)n, net->weights, net->updates, net->cur_updates,
+                                net->stats, net->deltas, nullptr, frac_length, net->beta1_accum, net->beta2_accum, learning_rate,
+                                momentum, net->veto);
     // a layer's own "learningRate" replaces the optimizer's (optimizers/SteepestDescentOptimizer.cu:402-403, :425-426): one
     // launch per trainable layer
     for (const auto &L : net->layers) {
@@ -1577,9 +1609,10 @@ int cnt_network_update(cnt_network *net, void *stream_, int option, float learni
         if (c == 0) continue;
         const long o = L.w_off;
         float *st = net->stats ? net->stats + (adam ? 2 * o : o) : nullptr;
-        CNT_TRY(cnt_opt_step(stream_, option, c, net->weights + o, net->updates + o, net->cur_updates + o, st,
-                             net->deltas + o, nullptr, frac_length, net->beta1_accum, net->beta2_accum,
-                             L.learning_rate > -0.5f ? L.learning_rate : learning_rate, momentum));
+        CNT_TRY(opt_step_guarded(static_cast<hipStream_t>(stream_), option, c, net->weights + o, net->updates + o,
+                                 net->cur_updates + o, st, net->deltas + o, nullptr, frac_length, net->beta1_accum,
+                                 net->beta2_accum, L.learning_rate > -0.5f ? L.learning_rate : learning_rate, momentum,
+                                 net->veto));
     }
     return CNT_OK;
 }

@@ -30,6 +30,7 @@ struct OptArgs {
     int option;                  // 0 plain, 1 AdaGrad, 2 averaged, 3 stochastic AdaGrad, 5 Adam
     int add;                     // accumulate: add to cur instead of overwriting it
     float frac_length, beta1_accum, beta2_accum, learning_rate, momentum;
+    const int *veto;             // optional device flag: non-zero means the gradients are invalid, nothing is touched
 };
 
 __device__ __forceinline__ bool bad(float g) { return isnan(g) || isinf(g); }
@@ -68,6 +69,7 @@ template <int MODE>
 __global__ __launch_bounds__(256) void optimizer_kernel(const OptArgs a) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
+    if (a.veto && *a.veto != 0) return;
     for (; i < a.n; i += stride) {
         float g;
         if (MODE == 0 || MODE == 3) g = a.add ? a.layer_updates[i] + a.cur[i] : a.layer_updates[i];
@@ -138,6 +140,14 @@ int cnt_opt_update_weights(void *stream, long n, float *weights, float *cur_upda
 int cnt_opt_step(void *stream, int option, long n, float *weights, const float *layer_updates, float *cur_updates,
                  float *stats, float *weight_deltas, const float *mask, float frac_length, float beta1_accum,
                  float beta2_accum, float learning_rate, float momentum) {
+    return cnt::opt_step_guarded(static_cast<hipStream_t>(stream), option, n, weights, layer_updates, cur_updates, stats,
+                                 weight_deltas, mask, frac_length, beta1_accum, beta2_accum, learning_rate, momentum, nullptr);
+}
+
+extern "C++" int cnt::opt_step_guarded(hipStream_t stream, int option, long n, float *weights, const float *layer_updates,
+                                       float *cur_updates, float *stats, float *weight_deltas, const float *mask,
+                                       float frac_length, float beta1_accum, float beta2_accum, float learning_rate,
+                                       float momentum, const int *veto) {
     using namespace cnt;
     CNT_REQUIRE(n >= 0 && (n == 0 || (weights && layer_updates && cur_updates && weight_deltas)), "opt_step: bad argument");
     CNT_REQUIRE(known_option(option), "opt_step: unknown optimizer option %d", option);
@@ -149,8 +159,9 @@ int cnt_opt_step(void *stream, int option, long n, float *weights, const float *
     a.weights = weights; a.mask = mask; a.option = option == 4 ? 0 : option;
     a.frac_length = frac_length; a.beta1_accum = beta1_accum; a.beta2_accum = beta2_accum;
     a.learning_rate = learning_rate; a.momentum = momentum;
-    ProfileScope prof(static_cast<hipStream_t>(stream), "opt_step");
-    hipLaunchKernelGGL(optimizer_kernel<3>, dim3(blocks_for(a.n)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+    a.veto = veto;
+    ProfileScope prof(stream, "opt_step");
+    hipLaunchKernelGGL(optimizer_kernel<3>, dim3(blocks_for(a.n)), dim3(256), 0, stream, a);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
