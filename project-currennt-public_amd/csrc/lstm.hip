@@ -1062,6 +1062,7 @@ struct cnt_lstm {
     float *lmail;
     size_t lmail_words;
     int last_blocks;       // workgroups of the last recursion launch
+    int poll_delay_local;  // pause before the first poll of a step in the XCD-local recursion, units of 64 clocks
 };
 
 namespace cnt {
@@ -1164,6 +1165,7 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
         const int G = h->H / local_jb;
         const int blocks = (h->njobs * G + 8 * (G - 1) + 7) / 8 * 8;
         h->last_blocks = blocks;
+        p.poll_delay = h->poll_delay_local;
         hipLaunchKernelGGL(k, dim3(blocks), dim3(local_threads(h->H)), 0, stream, p);
         CNT_HIP(hipGetLastError());
         return CNT_OK;
@@ -1296,7 +1298,10 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
         int pause = (int)(14.0 + 1.25 * mfma + words / 90000.0 + 0.5);
         h->poll_delay = pause > 40 ? 40 : pause;
     }
-    if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY")) h->poll_delay = std::atoi(e);
+    // XCD-local recursion: product (about 0.3 us) and one hop through the L2 (about 0.45 us) pass between a step's
+    // barrier and the arrival of the next partial errors
+    h->poll_delay_local = 8;
+    if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY")) h->poll_delay = h->poll_delay_local = std::atoi(e);
     // forward recursion: the senders' cell update (a few hundred clocks) plus store visibility
     h->poll_delay_fwd = 34;  // measured optimum on MI355X at H=256, S=10
     if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY_FWD")) h->poll_delay_fwd = std::atoi(e);
@@ -1398,6 +1403,7 @@ int cnt_lstm_set_wait_bounds(cnt_lstm *h, unsigned spin_limit, int poll_delay_ba
                 poll_delay_forward <= 4096, "lstm_set_wait_bounds: poll delays must be within 0..4096");
     h->spin_limit = spin_limit;
     h->poll_delay = poll_delay_backward;
+    h->poll_delay_local = poll_delay_backward < 8 ? poll_delay_backward : 8;
     h->poll_delay_fwd = poll_delay_forward;
     return CNT_OK;
 }
@@ -1440,25 +1446,42 @@ int cnt_lstm_check(cnt_lstm *h, void *stream) {
     if (h->phase_ticks) {
         // diagnostic: mean phase durations of the last recursion over the workgroups that took part
         const int blocks = h->last_blocks;
-        std::vector<long long> t((size_t)blocks * 6);
+        const bool local = h->local && !h->last_was_forward;
+        const int stride = local ? 8 : 6;
+        std::vector<long long> t((size_t)blocks * stride);
         CNT_HIP(hipMemcpy(t.data(), h->phase_ticks, t.size() * sizeof(long long), hipMemcpyDeviceToHost));
-        CNT_HIP(hipMemset(h->phase_ticks, 0, t.size() * sizeof(long long)));
-        double m[6] = {0, 0, 0, 0, 0, 0};
+        double m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         int active = 0;
         for (int b = 0; b < blocks; ++b) {
-            if (t[(size_t)b * 6 + 3] == 0) continue;
+            if (t[(size_t)b * stride + 3] == 0) continue;
             ++active;
-            for (int q = 0; q < 6; ++q) m[q] += (double)t[(size_t)b * 6 + q];
+            for (int q = 0; q < stride; ++q) m[q] += (double)t[(size_t)b * stride + q];
         }
+        if (local && std::getenv("CNT_LSTM_TRACE")) {
+            std::vector<long long> tr((size_t)blocks * kTraceStride);
+            CNT_HIP(hipMemcpy(tr.data(), h->phase_ticks + kTraceBase, tr.size() * sizeof(long long), hipMemcpyDeviceToHost));
+            for (int b = 0; b < blocks; ++b) {
+                if (t[(size_t)b * stride + 3] == 0) continue;
+                const long long *r = &tr[(size_t)b * kTraceStride];
+                std::fprintf(stderr, "trace block %d job %lld member %lld xcd %lld:", b, r[0], r[1], r[2]);
+                for (int q = 0; q < 5 * kTraceSteps; ++q) std::fprintf(stderr, " %lld", r[4 + q]);
+                std::fprintf(stderr, "\n");
+            }
+        }
+        CNT_HIP(hipMemset(h->phase_ticks, 0, 8 * 512 * 6 * sizeof(long long)));
         const double us = active ? 0.01 / active / h->T : 0.0;
         if (h->last_was_forward)
             std::fprintf(stderr, "lstm forward per step [us]: gather waves wait+product %.3f loop %.3f poll rounds %.2f "
                          "(T=%d, %d workgroups)\n", m[0] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, h->T, active);
+        else if (local)
+            std::fprintf(stderr, "lstm backward per step [us], XCD-local: cell wave wait+poll %.3f (lane 0's polls %.3f in %.2f rounds) "
+                         "update+barrier %.3f loop %.3f | product waves busy %.3f (store acknowledgement %.3f) | memory wave busy "
+                         "%.3f (T=%d, %d workgroups)\n", m[0] * us, m[6] * us, active ? m[4] / active / h->T : 0.0, m[1] * us,
+                         m[3] * us, m[2] * us, m[7] * us, m[5] * us, h->T, active);
         else
             std::fprintf(stderr, "lstm backward per step [us]: receive waves wait %.3f cell %.3f loop %.3f poll rounds %.2f | "
-                         "product waves busy %.3f | memory wave busy after B %.3f (T=%d, %d workgroups%s)\n",
-                         m[0] * us, m[1] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, m[2] * us, m[5] * us, h->T, active,
-                         h->local ? ", XCD-local" : "");
+                         "product waves busy %.3f | memory wave busy after B %.3f (T=%d, %d workgroups)\n",
+                         m[0] * us, m[1] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, m[2] * us, m[5] * us, h->T, active);
     }
     if (lstm_take_failure(h)) {
         set_error("%s", kGaveUp);
