@@ -1475,9 +1475,9 @@ int cnt_lstm_check(cnt_lstm *h, void *stream) {
                          "(T=%d, %d workgroups)\n", m[0] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, h->T, active);
         else if (local)
             std::fprintf(stderr, "lstm backward per step [us], XCD-local: cell wave wait+poll %.3f (lane 0's polls %.3f in %.2f rounds) "
-                         "update+barrier %.3f loop %.3f | product waves busy %.3f (store acknowledgement %.3f) | memory wave busy "
-                         "%.3f (T=%d, %d workgroups)\n", m[0] * us, m[6] * us, active ? m[4] / active / h->T : 0.0, m[1] * us,
-                         m[3] * us, m[2] * us, m[7] * us, m[5] * us, h->T, active);
+                         "update+barrier %.3f loop %.3f | product waves busy %.3f | memory wave busy %.3f (T=%d, %d workgroups)\n",
+                         m[0] * us, m[6] * us, active ? m[4] / active / h->T : 0.0, m[1] * us, m[3] * us, m[2] * us, m[5] * us,
+                         h->T, active);
         else
             std::fprintf(stderr, "lstm backward per step [us]: receive waves wait %.3f cell %.3f loop %.3f poll rounds %.2f | "
                          "product waves busy %.3f | memory wave busy after B %.3f (T=%d, %d workgroups)\n",

@@ -206,7 +206,7 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
         load_step(1, in); wait_all_vmem(); put_coef(1, in);
         load_step(2, in);
         const bool mtiming = p.phase_ticks != nullptr;
-        long long mbusy = 0, mwait = 0;
+        long long mbusy = 0;
         lds_barrier();  // start of the recursion
         for (int step = 0; step < T; ++step) {
             const int t = slot_of(step), b = step & 1;
@@ -214,7 +214,6 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
             if (wait_failed) return;
             const long long tm0 = mtiming ? wall_clock64() : 0;
             wait_all_vmem();  // inputs requested a step ago are there, state stores of the step before are done
-            const long long tm1 = mtiming ? wall_clock64() : 0;
             put_coef(step + 2, in);
             load_step(step + 3, in);
             if (valid) {
@@ -225,11 +224,10 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
                 if (p.herr_out) p.herr_out[gi] = res[b][0][lane];
                 else D.herr[gi] = res[b][0][lane];
             }
-            if (mtiming) { mwait += tm1 - tm0; mbusy += wall_clock64() - tm0; }
+            if (mtiming) mbusy += wall_clock64() - tm0;
         }
         if (mtiming && lane == 0) {
             p.phase_ticks[(size_t)blockIdx.x * 8 + 5] = mbusy;
-            (void)mwait;
         }
         return;
     }
@@ -253,7 +251,7 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
         wait_all_vmem();
         lds_barrier();  // start of the recursion
         const bool timing = p.phase_ticks != nullptr;
-        long long busy = 0, ack = 0;
+        long long busy = 0;
         for (int step = 0; step < T; ++step) {
             lds_barrier();  // the deltas of this step are in LDS
             // looked at only at the end of the step: the read is in flight behind the barrier together with the
@@ -289,14 +287,9 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
             if (failed) return;
             if (timing) {
                 busy += wall_clock64() - tp0;
-                if (p.poll_gap == 77) {  // diagnosis only: how long the stores of a step take to be acknowledged
-                    const long long ta = wall_clock64();
-                    wait_all_vmem();
-                    ack += wall_clock64() - ta;
-                }
             }
         }
-        if (timing && tid == 64) { p.phase_ticks[(size_t)blockIdx.x * 8 + 2] = busy; p.phase_ticks[(size_t)blockIdx.x * 8 + 7] = ack; }
+        if (timing && tid == 64) p.phase_ticks[(size_t)blockIdx.x * 8 + 2] = busy;
         return;
     }
 
