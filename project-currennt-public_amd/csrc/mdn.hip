@@ -250,6 +250,86 @@ __global__ void mixture_error_kernel(UnitGeom g, const char *__restrict__ pat, c
     }
 }
 
+// The same error pass for units whose data can be moved 16 bytes at a time (the condition of the VEC4 backward
+// kernel below).  Four lanes share a mixture component: lane (m, p) reads the 16-byte vectors p, p+4, ... of the
+// component's means and deviations, so one load instruction of the wave covers 64 contiguous bytes of sixteen
+// components; the four partial sums meet through two DPP steps instead of one six-step wave reduction per component.
+// The log-sum over the components is max + log(sum exp(. - max)) over the wave (the reference's running log_add in
+// another order: terms below e^-69 of the largest drop out either way).  A wave takes several frames in turn and a
+// workgroup adds its frames' log-sums in LDS, so the single result word receives one atomic per 8 frames -- 6000
+// atomics on one address, which serialise, were what the previous kernel's time went to.
+constexpr int kErrFramesPerWave = 2;
+__global__ __launch_bounds__(256) void mixture_error_vec_kernel(UnitGeom g, const char *__restrict__ pat,
+                                                                const float *__restrict__ target,
+                                                                const float *__restrict__ para, float *__restrict__ tmp,
+                                                                float *__restrict__ result) {
+    __shared__ float lp_sh[4][64];
+    __shared__ float block_sum[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int M = g.M, D = g.D, MD = M * D, DV = D / 4;
+    const int p = lane & 3, ml = lane >> 2;  // lane (ml, p): component ml of the pass, quarter p
+    const float gauss_const = (float)(D * log(2 * 3.141215) / 2.0);  // the reference's own value of pi
+    float wave_total = 0.0f;
+    for (int i = 0; i < kErrFramesPerWave; ++i) {
+        const int f = (blockIdx.x * 4 + wave) * kErrFramesPerWave + i;
+        if (f >= g.F) break;
+        if (pat[f] == 0) {
+            for (int m = lane; m < M; m += 64) tmp[(size_t)f * M + m] = 0.0f;  // distance pass writes 0, the rest skips
+            continue;
+        }
+        const float4 *t4 = reinterpret_cast<const float4 *>(target + (size_t)f * g.Lt + g.startDOut);
+        const float4 *mean4 = reinterpret_cast<const float4 *>(para + (size_t)g.F * M + (size_t)f * MD);
+        const float4 *sd4 = reinterpret_cast<const float4 *>(para + (size_t)g.F * M * (1 + D) + (size_t)f * MD);
+        float mx = lim::kLogZero;
+        float lp_mine[4];  // component lane + 64*pass, held by lanes below M - 64*pass after the exchange
+        int npass = 0;
+        for (int m0 = 0; m0 < M; m0 += 16, ++npass) {
+            const int m = m0 + ml;
+            float dist = 0.0f, logsd = 0.0f;
+            if (m < M) {
+                for (int v = p; v < DV; v += 4) {
+                    const float4 s = sd4[m * DV + v], mu = mean4[m * DV + v], tv = t4[v];
+                    const float d0 = tv.x - mu.x, d1 = tv.y - mu.y, d2 = tv.z - mu.z, d3 = tv.w - mu.w;
+                    dist += d0 * d0 / (s.x * s.x) * 0.5f; dist += d1 * d1 / (s.y * s.y) * 0.5f;
+                    dist += d2 * d2 / (s.z * s.z) * 0.5f; dist += d3 * d3 / (s.w * s.w) * 0.5f;
+                    logsd += safe_log(s.x) + safe_log(s.y) + safe_log(s.z) + safe_log(s.w);
+                }
+            }
+            // the four quarters of a component sit in one quad
+            dist += __shfl_xor(dist, 1); logsd += __shfl_xor(logsd, 1);
+            dist += __shfl_xor(dist, 2); logsd += __shfl_xor(logsd, 2);
+            if (m < M && p == 0) {
+                float lp = logf(para[(size_t)f * M + m]) - dist - gauss_const - logsd;
+                if (lp < lim::kLSmall) lp = lim::kLSmall;
+                tmp[(size_t)f * M + m] = lp;
+                lp_sh[wave][ml] = lp;
+            }
+            // one component per lane for the log-sum (lanes 0..15 of this pass); same wave, so no barrier
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            const float lp = (lane < 16 && m0 + lane < M) ? lp_sh[wave][lane] : lim::kLogZero;
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (npass < 4) lp_mine[npass] = lp;
+            mx = fmaxf(mx, lp);
+        }
+        mx = wave_max(mx);
+        float se = 0.0f;
+        for (int q = 0; q < npass && q < 4; ++q)
+            if (lane < 16 && 16 * q + lane < M) se += expf(lp_mine[q] - mx);
+        se = wave_sum(se);
+        const float lsum = mx + logf(se);
+        if (lane == 0) {
+            tmp[(size_t)g.F * M + f] = lsum;
+            wave_total -= lsum;
+        }
+    }
+    if (lane == 0) block_sum[wave] = wave_total;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float v = (block_sum[0] + block_sum[1]) + (block_sum[2] + block_sum[3]);
+        if (v != 0.0f) atomicAdd(result, v);
+    }
+}
+
 // VEC4: the mean / std part moves 16 bytes per lane (D, M, Lp, Lt and both start columns multiples of four and all
 // buffers 16-byte aligned, so that four consecutive dimensions of one mixture component sit in one aligned vector)
 template <bool VEC4>
@@ -509,9 +589,18 @@ int cnt_mdn_calculate_error(cnt_mdn *h, void *stream_, const float *targets, flo
                                u.para, result_dev);
         } else {
             ProfileScope prof(stream, "mdn_mixture_error");
-            const dim3 grid((g.F + kFramesPerBlock - 1) / kFramesPerBlock), block(64 * kFramesPerBlock);
-            hipLaunchKernelGGL(mixture_error_kernel, grid, block, 0, stream, g, h->pat, targets, u.para, u.tmp,
-                               result_dev);
+            auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+            const bool vec4 = g.D % 4 == 0 && g.M % 4 == 0 && g.M <= 64 && g.Lt % 4 == 0 && g.startDOut % 4 == 0 &&
+                              aligned(targets) && aligned(u.para);
+            if (vec4) {
+                const int per_block = 4 * kErrFramesPerWave;
+                hipLaunchKernelGGL(mixture_error_vec_kernel, dim3((g.F + per_block - 1) / per_block), dim3(256), 0, stream, g,
+                                   h->pat, targets, u.para, u.tmp, result_dev);
+            } else {
+                const dim3 grid((g.F + kFramesPerBlock - 1) / kFramesPerBlock), block(64 * kFramesPerBlock);
+                hipLaunchKernelGGL(mixture_error_kernel, grid, block, 0, stream, g, h->pat, targets, u.para, u.tmp,
+                                   result_dev);
+            }
         }
         CNT_HIP(hipGetLastError());
     }

@@ -128,12 +128,17 @@ def mdn_c3(args, pkg):
     layer.calculate_error(td, res)
 
     def step():
+        # the gradient needs the posteriors the error pass leaves behind (MDNUnit.cu:6037-6193 before :6222), so a
+        # step is both
+        layer.calculate_error(td, res)
         layer.backward(td, err)
 
     sec = _timed(step, args.steps, args.warmup)
     kernels = _profile(capi, step, args.steps)
-    dom = "mdn_mixture_backward"
-    nbytes = F * (Lp * 4 + (M + 1) * 4 + D * 4 + Lp * 4)
+    dom = max(("mdn_mixture_backward", "mdn_mixture_error"), key=lambda k: kernels[k]["avg_ms"])
+    # error pass: weights, means, deviations and targets in, M + 1 log-likelihood terms out;
+    # gradient pass: the same in plus those terms, Lp errors out
+    nbytes = F * ((Lp + D + M + 1) * 4 if dom == "mdn_mixture_error" else (Lp + M + 1 + D + Lp) * 4)
     ach = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
     roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None,
             "kernel": dom}
