@@ -12,6 +12,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libcurrennt_hip.so")
 BIN_DIR = os.path.join(HERE, "bin")
 HOST_DRIVER = os.path.join(BIN_DIR, "run_stack")
+HOST_DRIVERS = ["run_stack", "run_graph"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -57,14 +58,15 @@ def build_library(verbose=True):
 
 
 def build_host_driver():
-    """C++ layer shells (host/layers.hpp) + the stack driver, linked against the C-ABI library."""
+    """C++ layer shells (host/layers.hpp) + the drivers that run them, linked against the C-ABI library."""
     os.makedirs(BIN_DIR, exist_ok=True)
-    cmd = [HIPCC, "-O2", "-std=c++17", "-Wall", "-x", "c++", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
-           os.path.join(HERE, "host", "run_stack.cpp"), "-o", HOST_DRIVER, "-L" + LIB_DIR, "-lcurrennt_hip",
-           "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN/../lib", "-Wl,-rpath,/opt/rocm/lib"]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("host driver build failed:\n" + r.stdout + r.stderr)
+    for name in HOST_DRIVERS:
+        cmd = [HIPCC, "-O2", "-std=c++17", "-Wall", "-x", "c++", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
+               os.path.join(HERE, "host", name + ".cpp"), "-o", os.path.join(BIN_DIR, name), "-L" + LIB_DIR,
+               "-lcurrennt_hip", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN/../lib", "-Wl,-rpath,/opt/rocm/lib"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("host driver build failed:\n" + r.stdout + r.stderr)
     return HOST_DRIVER
 
 

@@ -79,3 +79,143 @@ def test_cpp_driver_reports_errors_like_the_reference(tmp_path):
     r = subprocess.run([driver, str(job), str(tmp_path / "o.bin")], capture_output=True, text=True, timeout=100)
     assert r.returncode == 2
     assert "FAILED in running CURENNT" in r.stderr and "odd layer size" in r.stderr
+
+
+# ---- every layer type of the path through its C++ shell (run_graph) --------------------------------------------------
+
+def _graph_driver():
+    capi = PC.pkg().capi
+    driver = os.path.join(os.path.dirname(capi.LIB_PATH), "..", "bin", "run_graph")
+    assert os.path.exists(driver), "host driver not built"
+    return driver
+
+
+def _run_graph(tmp_path, statements, files):
+    with open(tmp_path / "job.txt", "w") as f:
+        f.write("\n".join(statements) + "\n")
+    for name, arr in files.items():
+        np.ascontiguousarray(arr).tofile(tmp_path / name)
+    r = subprocess.run([_graph_driver(), str(tmp_path)], capture_output=True, text=True, timeout=100)
+    print(r.stdout, r.stderr, flush=True)
+    assert r.returncode == 0
+    return float(open(tmp_path / "loss.txt").read())
+
+
+def _result(tmp_path, name, kind):
+    return np.fromfile(tmp_path / ("%s.%s.bin" % (name, kind)), dtype=np.float32)
+
+
+def test_cpp_shells_wavenet_blocks_match_oracle(tmp_path):
+    """Three WaveNet blocks (cnn -> wavnetc -> 1x1 -> skipadd / skipini fan) with a softmax mdn output through the
+    CNNLayer, WavNetCore, SkipAddLayer, FeedForwardLayer and MDNLayer shells against the oracle's graph walk."""
+    import wavenet_data as WD
+
+    print("c++ shells: wavenet blocks", flush=True)
+    networks = PC.pkg().networks
+    nb, Q, R, K, C = 3, 32, 16, 32, 8
+    lengths = [60, 45]
+    S, T = len(lengths), max(lengths)
+    pat, onehot, ctx, target, N = WD.make(lengths, Q, C, upsample=10, seed=5)
+    ref = networks.WaveNet(OM.OracleBackend(), nb, S, T, Q=Q, R=R, K=K, C=C, cnn_tanh=1, dilation_cycle=3)
+    W = WD.init_weights({k: len(ref.buf[k]["W"]) for k in ref.weight_names()}, seed=6)
+    for k, w in W.items():
+        ref.buf[k]["W"][:] = w
+    ref.set_inputs(pat, onehot, ctx, target)
+    ref.forward()
+    ref.calculate_error()
+    ref.backward()
+
+    st = ["geometry %d %d %d" % (S, T, min(lengths)), "input %d" % Q, "ff emb 0 %d 1.0" % R, "skipini causalSkip %d" % R]
+    res = "causalSkip"
+    for l in range(nb):
+        st += ["cnn cnn%d %d 1.0 1 1 1 %d" % (l, 2 * R, 2 ** (l % 3)), "wavnetc wav%d %d %d" % (l, R, C),
+               "ff out%d 0 %d 1.0" % (l, R), "skipadd sadd%d %d %s,out%d" % (l, R, res, l), "skipini temp%d %d" % (l, R),
+               "ff sot%d 0 %d 1.0" % (l, K), "skipini skip%d %d" % (l, K), "skipadd temp2_%d %d temp%d" % (l, R, l)]
+        res = "temp2_%d" % l
+    st += ["skipadd postAdd %d %s" % (K, ",".join("skip%d" % l for l in range(nb))), "ff postL1 1 %d 1.0" % K,
+           "ff output 0 %d 1.0" % Q, "post mdn 1 6 1 0 %d 0 1 -1" % Q]
+    files = {"pat.bin": pat, "input.bin": onehot, "targets.bin": target, "context.bin": ctx}
+    files.update({k + ".W.bin": w for k, w in W.items()})
+    loss = _run_graph(tmp_path, st, files)
+    ref_loss = float(ref.loss[0])
+    assert abs(loss - ref_loss) <= 1e-4 * abs(ref_loss)
+    for k in ref.weight_names():
+        assert PC.relerr(_result(tmp_path, k, "dW"), ref.buf[k]["dW"]) < 1e-4, k
+    assert PC.relerr(_result(tmp_path, "postAdd", "out"), ref.buf["postAdd"]["out"]) < 1e-4
+
+
+def test_cpp_shells_mixture_density_stack_matches_oracle(tmp_path):
+    """feedforward_tanh -> feedforward_identity -> mdn with one mixture unit through the MDNLayer shell."""
+    import oracle_lib as O
+
+    print("c++ shells: mixture density stack", flush=True)
+    rng = np.random.default_rng(31)
+    P, Hd, M, D = 5, 8, 4, 4
+    Lp = M + 2 * M * D
+    lengths = [14, 9, 14, 11]
+    S, T = len(lengths), max(lengths)
+    N = S * T
+    pat = make_pat_types(lengths, T)
+    valid = pat != 0
+    x = rng.standard_normal((N, P)).astype(np.float32); x[~valid] = 0
+    tgt = rng.standard_normal((N, D)).astype(np.float32); tgt[~valid] = 0
+    w1 = rng.uniform(-0.5, 0.5, P * Hd + Hd).astype(np.float32)
+    w2 = rng.uniform(-0.5, 0.5, Hd * Lp + Lp).astype(np.float32)
+    h1, y = np.zeros(Hd * N, np.float32), np.zeros(Lp * N, np.float32)
+    O.dense_forward(P, Hd, N, 1, 1.0, w1, x.reshape(-1), h1)
+    O.dense_forward(Hd, Lp, N, 0, 1.0, w2, h1, y)
+    para, tmp = np.zeros(N * M * (1 + 2 * D), np.float32), np.zeros(N * M + N, np.float32)
+    O.mdn_mixture_forward(N, Lp, 0, M, D, 0.0, pat, y, para)
+    ref_loss = O.mdn_mixture_error(N, D, 0, M, D, pat, tgt.reshape(-1), para, tmp)
+    ey = np.zeros(Lp * N, np.float32)
+    O.mdn_mixture_backward(N, Lp, D, 0, 0, M, D, 0.0, pat, tgt.reshape(-1), para, tmp, ey)
+    eh1, dw1, dw2 = np.zeros(Hd * N, np.float32), np.zeros_like(w1), np.zeros_like(w2)
+    O.dense_backward(Hd, Lp, N, 0, 1.0, w2, h1, y, ey.copy(), eh1, dw2)
+    O.dense_backward(P, Hd, N, 1, 1.0, w1, x.reshape(-1), h1, eh1, None, dw1)
+    st = ["geometry %d %d %d" % (S, T, min(lengths)), "input %d" % P, "ff h 1 %d 1.0" % Hd, "ff out 0 %d 1.0" % Lp,
+          "post mdn %d 6 1 0 %d 0 %d %d" % (D, Lp, D, M)]
+    loss = _run_graph(tmp_path, st, {"pat.bin": pat, "input.bin": x, "targets.bin": tgt, "h.W.bin": w1, "out.W.bin": w2})
+    assert abs(loss - ref_loss) <= 1e-4 * abs(ref_loss)
+    assert PC.relerr(_result(tmp_path, "h", "dW"), dw1) < 1e-4
+    assert PC.relerr(_result(tmp_path, "out", "dW"), dw2) < 1e-4
+
+
+def test_cpp_shells_gatedact_and_dft_stack_matches_oracle(tmp_path):
+    """feedforward -> gatedact -> feedforward (one output) -> dft with two resolutions and the phase term through the
+    GatedActLayer and DFTPostoutputLayer shells."""
+    import oracle_lib as O
+
+    print("c++ shells: gatedact + dft stack", flush=True)
+    rng = np.random.default_rng(41)
+    P, D, T = 4, 8, 900
+    pat = make_pat_types([T], T)
+    x = rng.standard_normal((T, P)).astype(np.float32)
+    tgt = (0.3 * rng.standard_normal(T)).astype(np.float32)
+    w1 = rng.uniform(-0.5, 0.5, P * 2 * D + 2 * D).astype(np.float32)
+    w2 = rng.uniform(-0.5, 0.5, D + 1).astype(np.float32)
+    h1, g, y = np.zeros(2 * D * T, np.float32), np.zeros(D * T, np.float32), np.zeros(T, np.float32)
+    O.dense_forward(P, 2 * D, T, 0, 1.0, w1, x.reshape(-1), h1)
+    O.gated_forward(D, T, pat, h1, g)
+    O.dense_forward(D, 1, T, 0, 1.0, w2, g, y)
+    res = [(128, 100, 25), (64, 64, 16)]
+    gamma, zeta, dis = 0.7, 0.4, 1
+    ey, ref_loss = np.zeros(T, np.float64), 0.0
+    for (Nf, Nw, Hs) in res:
+        gbuf = np.zeros(T, np.float32)
+        ref_loss += O.dft_spectral_loss(dis, Nf, Nw, Hs, 0, T, T, gamma, 1e-5, y.copy(), tgt.copy(), gbuf)
+        ey += gbuf
+        ref_loss += O.dft_phase_loss(Nf, Nw, Hs, 0, T, T, zeta, y.copy(), tgt.copy(), gbuf)
+        ey += gbuf
+    ey = ey.astype(np.float32)
+    eg, eh1, dw1, dw2 = np.zeros(D * T, np.float32), np.zeros(2 * D * T, np.float32), np.zeros_like(w1), np.zeros_like(w2)
+    O.dense_backward(D, 1, T, 0, 1.0, w2, g, y, ey.copy(), eg, dw2)
+    O.gated_backward(D, T, pat, h1, eg, eh1)
+    O.dense_backward(P, 2 * D, T, 0, 1.0, w1, x.reshape(-1), h1, eh1, None, dw1)
+    st = ["geometry 1 %d %d" % (T, T), "input %d" % P, "ff pre 0 %d 1.0" % (2 * D), "gatedact gate %d" % D, "ff wave 0 1 1.0",
+          "post dft %g %d %g %d %s" % (gamma, dis, zeta, len(res), " ".join("%d %d %d" % r for r in res))]
+    loss = _run_graph(tmp_path, st, {"pat.bin": pat, "input.bin": x, "targets.bin": tgt, "pre.W.bin": w1, "wave.W.bin": w2})
+    assert abs(loss - ref_loss) <= 1e-4 * abs(ref_loss)
+    assert PC.relerr(_result(tmp_path, "gate", "out"), g) < 1e-4
+    assert PC.relerr(_result(tmp_path, "wave", "err"), ey) < 1e-4
+    assert PC.relerr(_result(tmp_path, "pre", "dW"), dw1) < 1e-4
+    assert PC.relerr(_result(tmp_path, "wave", "dW"), dw2) < 1e-4
