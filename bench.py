@@ -25,13 +25,17 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "bench"))   # the secondary workloads and the synthetic-data generators
+sys.path.insert(0, os.path.join(ROOT, "oracle"))  # the CPU checker: imported only by the cpu_baseline legs
 
 import numpy as np  # noqa: E402
 
-# HBM bytes one launch of lstm_backward_chain moves on this workload (T=588, S=10, H=256, two directions), from
-# two rocprofv3 --pmc runs scaled by a copy of known size: 1070 MiB read + 1605 MiB written
-# (profiles/acoustic_backward_hbm_traffic.md).  Algorithmic bytes of the same launch: 120 MB.
-CHAIN_TRAFFIC_BYTES = int((1070.0 + 1605.3) * 2 ** 20)
+# HBM bytes one launch of the backward recursion kernel moves on this workload (T=588, S=10, H=256, two directions),
+# from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a copy of known size; the figure and the command
+# that made it are in the profile named here.  Algorithmic bytes of the same launch: 120 MB.  None = not measured
+# for the kernel this tree runs.
+CHAIN_TRAFFIC_BYTES = None
+CHAIN_TRAFFIC_SOURCE = "profiles/acoustic_backward_hbm_traffic.md"
 
 METRIC = "BLSTM backward frames/sec at 1 MI355X; % HBM/MFMA roofline vs host CPU"
 PEAK_FP32_MFMA_TFLOPS = 157.3
@@ -72,8 +76,7 @@ def backward_flops_per_slot(input_size, specs):
 
 def cpu_baseline(input_size, specs, S, seed, sample_T):
     """Times the oracle's backward on a short fraction of the same network (one core, sequential)."""
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import oracle_models as OM
+    import oracle_models as OM  # the checker, only for this reported baseline
 
     lengths, T, x, tgt, pat = make_fraction(seed, S, sample_T, max(1, sample_T // 2), input_size, specs[-1]["size"])
     weights = OM.init_weights(input_size, specs, seed + 1, 0.08)
@@ -101,6 +104,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--workload", default="acoustic", choices=["acoustic", "lstm_c1", "mdn_c3", "dft_c5", "wavenet_c4", "opt_step", "nc_fraction"],
                     help="acoustic = benchmark configs[1] (the headline metric); the others are the remaining configs")
+    ap.add_argument("--via-layer-calls", action="store_true",
+                    help="also time the same backward pass through one C-ABI call per layer on one stream (the binding "
+                         "INTEGRATION.md shows for the reference's Layer classes) and print it as `via_layer_calls`")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters)")
@@ -118,7 +124,7 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
     pkg = load_package()
-    capi, networks = pkg.capi, pkg.networks
+    capi = pkg.capi
     if args.calibrate_copy:
         a = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
         b = torch.empty_like(a)
@@ -127,14 +133,13 @@ def main():
         torch.cuda.synchronize()
         del a, b
     if args.workload != "acoustic":
-        sys.path.insert(0, os.path.join(ROOT, "tests"))
-        import bench_workloads
+        import workloads
 
-        print(json.dumps(bench_workloads.run(args.workload, args, pkg)))
+        print(json.dumps(workloads.run(args.workload, args, pkg)))
         return
 
     S, Tmax, seed = 10, 600, 20240
-    input_size, specs = networks.acoustic_model_spec()
+    input_size, specs = pkg.specs.acoustic_model_spec()
     lengths, T, x, tgt, pat = make_fraction(seed, S, Tmax, 300, input_size, 187)
     frames = sum(lengths)
 
@@ -198,13 +203,23 @@ def main():
         # one launch = both directions of one BLSTM layer over all T*S slots; the only dense work on the
         # recursion is the recurrent product, 8*H^2 flops per slot and direction
         flops = 2 * 8.0 * H * H * slots
+        # What bounds a recursion of T dependent steps is not the matrix pipe but the hop every step ends with: the
+        # library's probe measures one hop between two workgroups of an XCD with a step's arithmetic in between.
+        hop_us = capi.probe_hop_latency(same_xcd=True, with_compute=True, rounds=2000)
+        hop_bare_us = capi.probe_hop_latency(same_xcd=True, with_compute=False, rounds=2000)
+        hop_far_us = capi.probe_hop_latency(same_xcd=False, with_compute=False, rounds=2000)
+        us_per_step = 1e3 * kernels[dom]["avg_ms"] / T
         roof = {"bound": "mfma", "achieved": flops / dom_avg_s / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "traffic": CHAIN_TRAFFIC_BYTES,
+                "unit": "TFLOP/s", "traffic": CHAIN_TRAFFIC_BYTES, "traffic_source": CHAIN_TRAFFIC_SOURCE,
                 "kernel": dom,
-                "note": "latency-bound recursion: T sequential steps, each a 256x1024x%d product spread over "
-                        "64 workgroups per direction plus one mailbox round trip; traffic = HBM bytes per launch "
-                        "from rocprofv3 FETCH_SIZE/WRITE_SIZE (profiles/acoustic_backward_hbm_traffic.md), mostly "
-                        "mailbox write-through and polls" % S}
+                "us_per_step": us_per_step,
+                "latency_floor_us_per_step": hop_us,
+                "frac_of_latency_floor": hop_us / us_per_step,
+                "hop_us": {"same_xcd": hop_bare_us, "same_xcd_with_step_arithmetic": hop_us, "across_xcds": hop_far_us},
+                "note": "latency-bound recursion: T sequential steps, each a 256x1024x%d product cut into (direction, "
+                        "sequence group) jobs of 32 workgroups per XCD plus one exchange through that XCD's L2; `frac` is "
+                        "against the fp32 MFMA peak as the metric asks, `frac_of_latency_floor` against T x (one measured "
+                        "hop + a step's arithmetic), the bound that applies" % S}
     elif dom.startswith("gemm"):
         flops = backward_flops_per_slot(input_size, specs) * slots / max(1, len([k for k in kernels if k.startswith("gemm")]))
         roof = {"bound": "mfma", "achieved": flops / dom_avg_s / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS,
@@ -215,7 +230,9 @@ def main():
                 "traffic": None, "kernel": dom}
     roof["frac"] = roof["achieved"] / roof["peak"]
 
-    step_flops = backward_flops_per_slot(input_size, specs) * slots
+    # useful work: the valid frames (padding slots do no useful work); the padded-slot figure is kept beside it
+    step_flops = backward_flops_per_slot(input_size, specs) * frames
+    step_flops_padded = backward_flops_per_slot(input_size, specs) * slots
     out = {
         "metric": METRIC, "value": value, "unit": "frames/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
@@ -227,13 +244,39 @@ def main():
         "step_roofline": {"bound": "mfma", "achieved": step_flops / (ms_per_step * 1e-3) / 1e12,
                           "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                           "frac": step_flops / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
-                          "flops_per_slot": backward_flops_per_slot(input_size, specs)},
+                          "flops_per_frame": backward_flops_per_slot(input_size, specs),
+                          "counted": "valid frames (%d of %d slots)" % (frames, slots),
+                          "frac_over_padded_slots": step_flops_padded / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS},
         "forward_backward_ms": fb_ms,
         "kernels": kernels,
     }
+    net.close()
+    if args.via_layer_calls:
+        import layer_calls
+
+        model = layer_calls.LayerCallModel(capi, input_size, specs, S, T, np.random.default_rng(seed + 1), 0.08)
+        model.load_sequences(pat_d, T, min(lengths), torch.from_numpy(x).cuda(), torch.from_numpy(tgt).cuda())
+        model.forward()
+        model.check()
+
+        def layer_step():
+            model.load_sequences(pat_d, T, min(lengths))
+            model.backward()
+
+        for _ in range(args.warmup):
+            layer_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            layer_step()
+        torch.cuda.synchronize()
+        dt2 = time.perf_counter() - t0
+        model.check()
+        model.close()
+        out["via_layer_calls"] = {"value": frames * args.steps / dt2, "unit": "frames/s", "ms_per_step": 1e3 * dt2 / args.steps,
+                                  "note": "same model and fraction, one C-ABI call per layer on one stream (no side streams)"}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(input_size, specs, S, seed, args.cpu_sample_T)
-    net.close()
     print(json.dumps(out))
 
 

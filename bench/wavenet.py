@@ -9,8 +9,7 @@ import time
 
 import numpy as np
 
-import oracle_models as OM
-import wavenet_data as WD
+import synth as WD
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
@@ -24,14 +23,14 @@ def flops_per_sample(nb, Q, R, K, C):
 def run(args, pkg):
     import torch
 
-    import bench_workloads as BW
+    import workloads as BW
 
-    capi, networks = pkg.capi, pkg.networks
+    capi = pkg.capi
     nb, Q, R, K, C = 30, 1024, 64, 128, 80
     lengths = [16000, 16000]
     S, T = 2, 16000
     pat, onehot, ctx, target, N = WD.make(lengths, Q, C, upsample=80, seed=4)
-    topology = WD.network_json(nb, Q, R, K, C, 1, 10)
+    topology = pkg.specs.wavenet_network_doc(nb, Q, R, K, C, 1, 10)
     net = capi.Network(json.dumps(topology), S, T, mdn_config=[1, 0, Q, 0, 1, -1])
     # rows a dense layer's weight-gradient launch reads per sample: its input and its output errors
     dense_rows = [prev["size"] + cur["size"] for prev, cur in zip(topology["layers"], topology["layers"][1:])
@@ -89,10 +88,12 @@ def run(args, pkg):
                                "frac": 155e3 * N / sec / 1e9 / PEAK_HBM_GBS, "bytes_per_sample": 155e3,
                                "mfma_tflops": step_flops / sec / 1e12}}
     if not args.no_cpu:
+        import oracle_models as OM  # the checker, only for this reported baseline
+
         # one block-sized slice of the same stack on the oracle: 2 blocks, 2 x 600 samples, scaled per sample and block
         nb_s, T_s = 2, 600
         p2, o2, c2, t2, N2 = WD.make([T_s, T_s], Q, C, upsample=80, seed=4)
-        ref = networks.WaveNet(OM.OracleBackend(), nb_s, S, T_s, Q=Q, R=R, K=K, C=C, cnn_tanh=1)
+        ref = OM.WaveNet(OM.OracleBackend(), nb_s, S, T_s, Q=Q, R=R, K=K, C=C, cnn_tanh=1)
         sh = {k: len(ref.buf[k]["W"]) for k in ref.weight_names()}
         for k, w in WD.init_weights(sh, seed=5).items():
             ref.buf[k]["W"][:] = w

@@ -6,8 +6,7 @@ import time
 
 import numpy as np
 
-import oracle_lib as O
-from torch_models import make_pat_types
+from synth import make_pat_types
 
 METRIC = "BLSTM backward frames/sec at 1 MI355X; % HBM/MFMA roofline vs host CPU"
 PEAK_FP32_MFMA_TFLOPS = 157.3
@@ -60,7 +59,7 @@ def lstm_c1(args, pkg):
     P, H, S, lengths = 382, 256, 4, [200, 200, 200, 150]
     T, N = 200, 800
     rng = np.random.default_rng(1)
-    nW = O.lib().orc_lstm_weight_count(P, H, 0)
+    nW = capi.lib().cnt_lstm_weight_count(P, H, 0)
     W = rng.uniform(-0.1, 0.1, nW).astype(np.float32)
     x = rng.standard_normal((T, S, P)).astype(np.float32)
     err = (0.1 * rng.standard_normal((T, S, H))).astype(np.float32)
@@ -93,6 +92,8 @@ def lstm_c1(args, pkg):
             "traffic": None, "kernel": dom, "note": "latency-bound recursion (T sequential steps)"}
     extra = {"roofline": roof, "kernels": kernels}
     if not args.no_cpu:
+        import oracle_lib as O  # the checker, only for this reported baseline
+
         desc = O.LstmDesc(P, H, 0, S, T, 150, 1.0)
         fw = O.LstmState(H, N)
         o = np.zeros(H * N, dtype=np.float32)
@@ -151,6 +152,8 @@ def mdn_c3(args, pkg):
     sec_full = _timed(full, args.steps, 1)
     extra = {"roofline": roof, "kernels": kernels, "forward_error_backward_ms": 1e3 * sec_full}
     if not args.no_cpu:
+        import oracle_lib as O  # the checker, only for this reported baseline
+
         para = np.zeros(F * M * (1 + 2 * D), dtype=np.float32)
         tmp = np.zeros(F * M + F, dtype=np.float32)
         eo = np.zeros(F * Lp, dtype=np.float32)
@@ -194,6 +197,8 @@ def dft_c5(args, pkg):
             "kernel": dom, "note": "4.6 MB and 0.17 GFLOP in total: launch- and latency-bound, far from either roof"}
     extra = {"roofline": roof, "kernels": kernels}
     if not args.no_cpu:
+        import oracle_lib as O  # the checker, only for this reported baseline
+
         g = np.zeros(n, dtype=np.float32)
         t0 = time.perf_counter()
         for (N, Nw, Hs) in res:
@@ -214,8 +219,8 @@ def opt_step(args, pkg):
 
     import torch
 
-    capi, networks = pkg.capi, pkg.networks
-    input_size, specs = networks.acoustic_model_spec()
+    capi = pkg.capi
+    input_size, specs = pkg.specs.acoustic_model_spec()
     layers = [{"size": input_size, "name": "input", "type": "input"}]
     layers += [dict(sp, name="l%d" % i) for i, sp in enumerate(specs)]
     net = capi.Network(json.dumps({"layers": layers}), 10, 16)
@@ -238,6 +243,8 @@ def opt_step(args, pkg):
                     "find in the 256 MB last-level cache: the figure is not a pure HBM rate"}
     extra = {"roofline": roof, "kernels": kernels}
     if not args.no_cpu:
+        import oracle_lib as O  # the checker, only for this reported baseline
+
         hw = [np.zeros(n, np.float32) for n in sizes]
         t0 = time.perf_counter()
         reps = 5
@@ -296,6 +303,8 @@ def nc_fraction(args, pkg):
                           "note": "host-side reader: the figure is file bytes delivered per second by one CPU core; the "
                                   "HBM peak is listed only because the field is mandatory"}}
     if not args.no_cpu:
+        import oracle_lib as O  # the checker, only for this reported baseline
+
         spec = importlib.util.spec_from_file_location("nc_fraction", os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "nc_fraction.py"))
         NF = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(NF)
@@ -315,7 +324,7 @@ def nc_fraction(args, pkg):
 
 def run(name, args, pkg):
     if name == "wavenet_c4":
-        import bench_wavenet
+        import wavenet
 
-        return bench_wavenet.run(args, pkg)
+        return wavenet.run(args, pkg)
     return {"lstm_c1": lstm_c1, "mdn_c3": mdn_c3, "dft_c5": dft_c5, "opt_step": opt_step, "nc_fraction": nc_fraction}[name](args, pkg)

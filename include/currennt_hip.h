@@ -35,6 +35,12 @@ const char *cnt_last_error(void);
  * label (order of first use), its launch count and summed duration in ms, or CNT_ERR_ARG past the end. */
 int cnt_profile_enable(int on);
 int cnt_profile_get(int index, char *label, int label_cap, int *launches, float *total_ms);
+/* Measurement hook without a counterpart in the reference: the time of one hop of a word between two workgroups the
+ * way the recursion kernels exchange data -- a store and a polling load that bypasses the per-CU cache -- on the
+ * same XCD (through its L2) or on two XCDs (through the memory side), with (with_compute) or without the arithmetic
+ * a recursion step does between receiving and sending.  T times this is the floor of a T-step recursion spread
+ * over compute units.  Synchronous; *hop_us (host memory) receives microseconds per hop. */
+int cnt_probe_hop_latency(void *stream, int same_xcd, int with_compute, int rounds, float *hop_us);
 
 /* ---- helpers::Matrix product seam -------------------------------------------------------------
  * Replaces helpers::Matrix<Gpu>::assignProduct / addProduct (helpers/Matrix.cu:353-377, which call

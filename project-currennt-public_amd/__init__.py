@@ -6,4 +6,4 @@ benchmark can drive it with device buffers owned by PyTorch; it contains no comp
 refuses to work when the library is missing.
 """
 from . import capi  # noqa: F401
-from . import networks  # noqa: F401
+from . import specs  # noqa: F401

@@ -68,6 +68,7 @@ _SIGNATURES = {
     "cnt_dense_backward_errors": (I, [VP, I, I, I, I, VP, VP, VP, VP]),
     "cnt_dense_backward_weights": (I, [VP, I, I, I, F, VP, VP, VP]),
     "cnt_dense_backward_weights_static": (I, [VP, I, I, I, F, VP, VP, VP]),
+    "cnt_probe_hop_latency": (I, [VP, I, I, I, C.POINTER(F)]),
     "cnt_gemm_reserve": (I, [VP]),
     "cnt_gemm_release": (I, [VP]),
     "cnt_sse_backward": (I, [VP, I, I, VP, VP, VP, VP]),
@@ -224,6 +225,13 @@ def dense_backward_weights(P, D, N, bias, x, err, dW, stream=None):
 
 def dense_backward_weights_static(P, D, N, bias, x, err, dW, stream=None):
     check(lib().cnt_dense_backward_weights_static(stream_ptr(stream), P, D, N, bias, ptr(x), ptr(err), ptr(dW)))
+
+
+def probe_hop_latency(same_xcd=True, with_compute=True, rounds=2000, stream=None):
+    """Microseconds per hop of a word between two workgroups (see cnt_probe_hop_latency)."""
+    out = F(0.0)
+    check(lib().cnt_probe_hop_latency(stream_ptr(stream), int(same_xcd), int(with_compute), int(rounds), C.byref(out)))
+    return float(out.value)
 
 
 def gemm_reserve(stream=None):

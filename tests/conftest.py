@@ -6,8 +6,9 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
-if os.path.dirname(os.path.abspath(__file__)) not in sys.path:
-    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+for _d in (os.path.dirname(os.path.abspath(__file__)), os.path.join(ROOT, "oracle"), os.path.join(ROOT, "bench")):
+    if _d not in sys.path:
+        sys.path.insert(0, _d)
 
 
 def pytest_configure(config):

@@ -12,7 +12,10 @@ import sys
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.dirname(HERE))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+for _d in (os.path.dirname(HERE), os.path.join(ROOT, "oracle"), os.path.join(ROOT, "bench")):
+    if _d not in sys.path:
+        sys.path.insert(0, _d)
 
 import oracle_lib as O  # noqa: E402
 from torch_models import make_pat_types  # noqa: E402

@@ -1,4 +1,4 @@
-"""Layer-by-layer sequencing of the HIP library for stacked networks (the role of
+"""Test harness: layer-by-layer sequencing of the HIP library for stacked networks (the role of
 NeuralNetwork::__computeForward_LayerByLayer / __computeBackward_LayerByLayer,
 NeuralNetwork.cpp:1419-1471 and :2743-2800 of the reference).  Buffers are torch CUDA tensors,
 every computation is a C-ABI call; nothing here computes on the host.
@@ -9,7 +9,9 @@ feedforward_relu, lstm, blstm, and a final sse post-output layer.
 """
 import torch
 
-from . import capi
+from __graft_entry__ import load_package
+
+capi = load_package().capi
 
 _FF_ACT = {"feedforward_identity": 0, "feedforward_tanh": 1, "feedforward_logistic": 2, "feedforward_relu": 3}
 
@@ -269,29 +271,6 @@ class Trainer:
         return loss
 
 
-def acoustic_model_spec():
-    """benchmark config 2: 382 -> 2 x feedforward_tanh 512 -> 2 x blstm 512 -> feedforward_identity 187 -> sse."""
-    return 382, [
-        {"type": "feedforward_tanh", "size": 512, "bias": 1.0},
-        {"type": "feedforward_tanh", "size": 512, "bias": 1.0},
-        {"type": "blstm", "size": 512, "bias": 1.0},
-        {"type": "blstm", "size": 512, "bias": 1.0},
-        {"type": "feedforward_identity", "size": 187, "bias": 1.0},
-        {"type": "sse", "size": 187},
-    ]
-
-
-# ---------------------------------------------------------------------------------------------------------
-# WaveNet-style stack (benchmark config 4), topology of the reference's example network
-# obsolete/scripts/EXAMPLE/MODEL_WAVENET/network.jsn: embedding of the fed-back one-hot sample, then per block
-#   cnn (causal, dilated, 2R filters) -> wavnetc (gate, conditioned) -> out (R->R) -> skipadd(residual, out)
-#   -> temp (skipini) -> skipouttrans (R->K) -> skip (skipini) ; temp2 = skipadd(temp) feeds the next block,
-# then skipadd over all skip layers -> feedforward_tanh -> feedforward_identity (Q classes) -> mdn softmax.
-# The graph walk below is shared by the HIP backend (this file) and the CPU-oracle backend of the tests; a
-# backend supplies buffers and the layer primitives.  Error routing follows SkipAddLayer.cu:305-346: a skip
-# layer adds its side buffer to its error buffer, accumulates into skip predecessors' side buffers and
-# overwrites plain predecessors' error buffers.
-# ---------------------------------------------------------------------------------------------------------
 class HipBackend:
     """Layer primitives on the HIP library; buffers are torch CUDA tensors."""
 
@@ -346,113 +325,4 @@ class HipBackend:
             h.close()
 
 
-class WaveNet:
-    def __init__(self, backend, n_blocks, S, T, Q=1024, R=64, K=128, C=80, cnn_tanh=1, dilation_cycle=10):
-        self.b, self.nb, self.S, self.T = backend, n_blocks, S, T
-        self.Q, self.R, self.K, self.C, self.cnn_tanh = Q, R, K, C, cnn_tanh
-        self.N = S * T
-        self.dils = [2 ** (l % dilation_cycle) for l in range(n_blocks)]
-        N, z = self.N, backend.zeros
-        self.buf = {}
-
-        def layer(name, size, nW=0, skip=False):
-            d = {"out": z(size * N), "err": z(size * N), "size": size}
-            if nW:
-                d["W"], d["dW"] = z(nW), z(nW)
-            if skip:
-                d["eskip"] = z(size * N)
-            self.buf[name] = d
-            return d
-
-        layer("emb", R, Q * R + R)
-        layer("causalSkip", R, skip=True)
-        for l in range(n_blocks):
-            layer("cnn%d" % l, 2 * R, R * 3 * 2 * R + 2 * R)
-            w = layer("wav%d" % l, R, C * 2 * R)
-            w["core"], w["cth"] = z(2 * R * N), z(2 * R * N)
-            layer("out%d" % l, R, R * R + R)
-            layer("sadd%d" % l, R, skip=True)
-            layer("temp%d" % l, R, skip=True)
-            layer("sot%d" % l, K, R * K + K)
-            layer("skip%d" % l, K, skip=True)
-            layer("temp2_%d" % l, R, skip=True)
-        layer("postAdd", K, skip=True)
-        layer("postL1", K, K * K + K)
-        layer("output", Q, K * Q + Q)
-        self.zeroK = z(K * N)
-        self.softmax = backend.softmax_make(Q, S, T)
-        self.loss = z(1)
-
-    def weight_names(self):
-        return [k for k, v in self.buf.items() if "W" in v]
-
-    def set_inputs(self, pat, onehot, ctx, target):
-        self.pat, self.x0, self.ctx, self.target = pat, onehot, ctx, target
-        self.softmax.load_sequences(pat, self.T)
-
-    def _res(self, l):
-        return self.buf["causalSkip"] if l == 0 else self.buf["temp2_%d" % (l - 1)]
-
-    def forward(self):
-        B, b, N, R, K, Q, C = self.buf, self.b, self.N, self.R, self.K, self.Q, self.C
-        b.dense_forward(Q, R, N, 0, B["emb"]["W"], self.x0, B["emb"]["out"])
-        cs = B["causalSkip"]
-        b.skipadd_forward([B["emb"]["out"]], cs["out"], cs["err"], cs["eskip"])
-        for l in range(self.nb):
-            res, cnn, wav, out = self._res(l), B["cnn%d" % l], B["wav%d" % l], B["out%d" % l]
-            sadd, temp, sot, skip, temp2 = B["sadd%d" % l], B["temp%d" % l], B["sot%d" % l], B["skip%d" % l], B["temp2_%d" % l]
-            b.cnn_forward(l, R, 2 * R, self.S, self.T, self.dils[l], self.cnn_tanh, self.pat, cnn["W"], res["out"], cnn["out"])
-            b.wavnetc_forward(R, C, N, self.pat, wav["W"], self.ctx, cnn["out"], wav["core"], wav["cth"], wav["out"])
-            b.dense_forward(R, R, N, 0, out["W"], wav["out"], out["out"])
-            b.skipadd_forward([res["out"], out["out"]], sadd["out"], sadd["err"], sadd["eskip"])
-            b.skipadd_forward([sadd["out"]], temp["out"], temp["err"], temp["eskip"])
-            b.dense_forward(R, K, N, 0, sot["W"], temp["out"], sot["out"])
-            b.skipadd_forward([sot["out"]], skip["out"], skip["err"], skip["eskip"])
-            b.skipadd_forward([temp["out"]], temp2["out"], temp2["err"], temp2["eskip"])
-        pa = B["postAdd"]
-        b.skipadd_forward([B["skip%d" % l]["out"] for l in range(self.nb)], pa["out"], pa["err"], pa["eskip"])
-        b.dense_forward(K, K, N, 1, B["postL1"]["W"], pa["out"], B["postL1"]["out"])
-        b.dense_forward(K, Q, N, 0, B["output"]["W"], B["postL1"]["out"], B["output"]["out"])
-        self.softmax.forward(B["output"]["out"])
-
-    def calculate_error(self):
-        self.softmax.calculate_error(self.target, self.loss)
-        return self.loss
-
-    def reset_skip_errors(self):
-        """What the skip layers' forward pass clears (SkipAddLayer.cu:195-205); needed before a backward pass is
-        repeated without a forward pass in between."""
-        for v in self.buf.values():
-            if "eskip" in v:
-                v["err"].zero_()
-                v["eskip"].zero_()
-
-    def backward(self):
-        B, b, N, R, K, Q, C = self.buf, self.b, self.N, self.R, self.K, self.Q, self.C
-        self.softmax.backward(self.target, B["output"]["err"])
-        b.dense_backward(K, Q, N, 0, B["output"]["W"], B["postL1"]["out"], B["output"]["out"], B["output"]["err"],
-                         B["postL1"]["err"], B["output"]["dW"])
-        pa = B["postAdd"]
-        b.dense_backward(K, K, N, 1, B["postL1"]["W"], pa["out"], B["postL1"]["out"], B["postL1"]["err"], pa["err"],
-                         B["postL1"]["dW"])
-        b.skipadd_backward(pa["err"], pa["eskip"], [B["skip%d" % l]["eskip"] for l in range(self.nb)], [1] * self.nb,
-                           self.zeroK)
-        for l in range(self.nb - 1, -1, -1):
-            res, cnn, wav, out = self._res(l), B["cnn%d" % l], B["wav%d" % l], B["out%d" % l]
-            sadd, temp, sot, skip, temp2 = B["sadd%d" % l], B["temp%d" % l], B["sot%d" % l], B["skip%d" % l], B["temp2_%d" % l]
-            b.skipadd_backward(temp2["err"], temp2["eskip"], [temp["eskip"]], [1], None)
-            b.skipadd_backward(skip["err"], skip["eskip"], [sot["err"]], [0], None)
-            b.dense_backward(R, K, N, 0, sot["W"], temp["out"], sot["out"], sot["err"], temp["err"], sot["dW"])
-            b.skipadd_backward(temp["err"], temp["eskip"], [sadd["eskip"]], [1], None)
-            b.skipadd_backward(sadd["err"], sadd["eskip"], [res["eskip"], out["err"]], [1, 0], None)
-            b.dense_backward(R, R, N, 0, out["W"], wav["out"], out["out"], out["err"], wav["err"], out["dW"])
-            b.wavnetc_backward(R, C, N, self.pat, wav["W"], self.ctx, wav["core"], wav["cth"], wav["err"], cnn["err"], wav["dW"])
-            b.cnn_backward(l, R, 2 * R, self.S, self.T, self.dils[l], self.cnn_tanh, self.pat, cnn["W"], res["out"], cnn["out"],
-                           cnn["err"], res["err"], cnn["dW"])
-        cs = B["causalSkip"]
-        b.skipadd_backward(cs["err"], cs["eskip"], [B["emb"]["err"]], [0], None)
-        b.dense_backward(Q, R, N, 0, B["emb"]["W"], self.x0, B["emb"]["out"], B["emb"]["err"], None, B["emb"]["dW"])
-
-    def close(self):
-        self.softmax.close()
-        self.b.close()
+from oracle_models import WaveNet  # noqa: E402,F401  (the graph walk itself is backend-neutral and lives beside the oracle)

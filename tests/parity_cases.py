@@ -8,7 +8,9 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+for _d in (os.path.dirname(os.path.abspath(__file__)), os.path.join(ROOT, "oracle"), os.path.join(ROOT, "bench")):
+    if _d not in sys.path:
+        sys.path.insert(0, _d)
 
 import oracle_lib as O  # noqa: E402
 from torch_models import make_pat_types  # noqa: E402
@@ -18,6 +20,13 @@ def pkg():
     from __graft_entry__ import load_package
 
     return load_package()
+
+
+def networks():
+    """The tests' layer-by-layer walks over the C ABI (tests/networks.py)."""
+    import networks as N
+
+    return N
 
 
 def relerr(a, b):

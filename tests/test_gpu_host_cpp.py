@@ -108,10 +108,10 @@ def _result(tmp_path, name, kind):
 def test_cpp_shells_wavenet_blocks_match_oracle(tmp_path):
     """Three WaveNet blocks (cnn -> wavnetc -> 1x1 -> skipadd / skipini fan) with a softmax mdn output through the
     CNNLayer, WavNetCore, SkipAddLayer, FeedForwardLayer and MDNLayer shells against the oracle's graph walk."""
-    import wavenet_data as WD
+    import synth as WD
 
     print("c++ shells: wavenet blocks", flush=True)
-    networks = PC.pkg().networks
+    networks = PC.networks()
     nb, Q, R, K, C = 3, 32, 16, 32, 8
     lengths = [60, 45]
     S, T = len(lengths), max(lengths)

@@ -29,8 +29,8 @@ def test_acoustic_model_forward_backward():
     import torch
 
     print("acoustic model parity", flush=True)
-    networks = PC.pkg().networks
-    input_size, specs = networks.acoustic_model_spec()
+    networks = PC.networks()
+    input_size, specs = PC.pkg().specs.acoustic_model_spec()
     S = 10
     lengths, T, x, tgt, pat = make_fraction(7, S, 20, 10, input_size, 187)
     weights = OM.init_weights(input_size, specs, 8, 0.08)

@@ -10,7 +10,7 @@ import pytest
 import oracle_lib as O
 import oracle_models as OM
 import parity_cases as PC
-import wavenet_data as WD
+import synth as WD
 from torch_models import make_pat_types
 
 pytestmark = pytest.mark.gpu
@@ -28,7 +28,7 @@ def test_stacked_network_trains_like_the_oracle(option, momentum, overlap):
 
     print("network case", option, momentum, overlap, flush=True)
     pkg = PC.pkg()
-    capi, networks = pkg.capi, pkg.networks
+    capi, networks = pkg.capi, PC.networks()
     P, Q, S = 20, 6, 4
     specs = [{"name": "ff1", "type": "feedforward_tanh", "size": 32, "bias": 1.0},
              {"name": "bl1", "type": "blstm", "size": 128, "bias": 1.0},
@@ -116,7 +116,7 @@ def test_wavenet_network_file_against_oracle_graph(nb, cnn_tanh, R, K, Q, C, len
 
     print("wavenet network file", nb, cnn_tanh, R, K, Q, C, lengths, cycle, flush=True)
     pkg = PC.pkg()
-    capi, networks = pkg.capi, pkg.networks
+    capi, networks = pkg.capi, PC.networks()
     O.use_all_cores()
     S, T = len(lengths), max(lengths)
     pat, onehot, ctx, target, N = WD.make(lengths, Q, C, upsample=upsample, seed=2)
@@ -130,7 +130,7 @@ def test_wavenet_network_file_against_oracle_graph(nb, cnn_tanh, R, K, Q, C, len
     ref.calculate_error()
     ref.backward()
 
-    doc = WD.network_json(nb, Q, R, K, C, cnn_tanh, cycle)
+    doc = PC.pkg().specs.wavenet_network_doc(nb, Q, R, K, C, cnn_tanh, cycle)
     net = capi.Network(json.dumps(doc), S, T + 7, mdn_config=[1, 0, Q, 0, 1, -1])   # buffers longer than the fraction
     names = [L["name"] for L in net.layers if L["weight_count"]]
     assert sorted(names) == sorted(W)
@@ -249,7 +249,7 @@ def test_wavenet_with_frame_rate_conditioning_network():
 
     print("wavenet network file with conditioning sub-network", flush=True)
     pkg = PC.pkg()
-    capi, networks = pkg.capi, pkg.networks
+    capi, networks = pkg.capi, PC.networks()
     nb, Q, R, K = 3, 64, 32, 64
     E, HB, DC, C, RES = 12, 128, 10, 11, 4
     lengths = [120, 90]
@@ -315,7 +315,7 @@ def test_wavenet_with_frame_rate_conditioning_network():
     dW_ref["exL2"], dW_ref["exL3"] = dw_lstm, dw_cnn
 
     # ---- the library, from the network file ---------------------------------------------------------------------
-    doc = WD.network_json(nb, Q, R, K, C, 1, 3)
+    doc = PC.pkg().specs.wavenet_network_doc(nb, Q, R, K, C, 1, 3)
     cond = [{"size": E, "name": "exL1", "type": "externalloader", "bias": 1.0, "resolution": RES},
             {"size": E, "name": "exSkip", "bias": 1.0, "type": "skipini", "resolution": RES},
             {"size": HB, "name": "exL2", "bias": 1.0, "type": "blstm", "resolution": RES},
@@ -367,9 +367,9 @@ def test_full_size_acoustic_backward_is_affine_in_the_targets():
 
     print("full-size acoustic linearity", flush=True)
     pkg = PC.pkg()
-    capi, networks = pkg.capi, pkg.networks
+    capi, networks = pkg.capi, PC.networks()
     S, Tmax = 10, 600
-    input_size, specs = networks.acoustic_model_spec()
+    input_size, specs = PC.pkg().specs.acoustic_model_spec()
     rng = np.random.default_rng(77)
     lengths = [int(v) for v in rng.integers(300, Tmax + 1, size=S)]
     T = max(lengths)
@@ -416,7 +416,7 @@ def test_full_size_wavenet_sequencer_matches_layer_by_layer_walk():
 
     print("full-size wavenet sequencer vs walk", flush=True)
     pkg = PC.pkg()
-    capi, networks = pkg.capi, pkg.networks
+    capi, networks = pkg.capi, PC.networks()
     nb, Q, R, K, C = 30, 1024, 64, 128, 80
     lengths = [16000, 15000]
     S, T = 2, 16000
@@ -430,7 +430,7 @@ def test_full_size_wavenet_sequencer_matches_layer_by_layer_walk():
     walk.forward()
     walk.calculate_error()
     walk.backward()
-    net = capi.Network(json.dumps(WD.network_json(nb, Q, R, K, C, 1, 10)), S, T, mdn_config=[1, 0, Q, 0, 1, -1])
+    net = capi.Network(json.dumps(PC.pkg().specs.wavenet_network_doc(nb, Q, R, K, C, 1, 10)), S, T, mdn_config=[1, 0, Q, 0, 1, -1])
     for L in net.layers:
         if L["weight_count"]:
             L["weights"].copy_(torch.from_numpy(W[L["name"]]))

@@ -38,7 +38,7 @@ def test_train_fractions_from_json_and_nc(tmp_path, option, momentum):
 
     print("training case", option, momentum, flush=True)
     pkg = PC.pkg()
-    capi, networks = pkg.capi, pkg.networks
+    capi, networks = pkg.capi, PC.networks()
     P, Q, S = 20, 6, 4
     specs = [{"name": "ff1", "type": "feedforward_tanh", "size": 32, "bias": 1.0},
              {"name": "bl1", "type": "blstm", "size": 128, "bias": 1.0},
@@ -111,7 +111,7 @@ def test_train_fractions_from_json_and_nc(tmp_path, option, momentum):
 
 
 def test_network_json_errors(tmp_path):
-    networks = PC.pkg().networks
+    networks = PC.networks()
     p = str(tmp_path / "n.jsn")
     json.dump({"layers": [{"size": 3, "name": "input", "type": "input"}, {"size": 4, "name": "c", "type": "cnn"},
                           {"size": 4, "name": "post", "type": "sse"}]}, open(p, "w"))

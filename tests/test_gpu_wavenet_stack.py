@@ -5,7 +5,7 @@ import pytest
 
 import oracle_models as OM
 import parity_cases as PC
-import wavenet_data as WD
+import synth as WD
 
 pytestmark = pytest.mark.gpu
 
@@ -15,7 +15,7 @@ def test_wavenet_stack(cnn_tanh):
     import torch
 
     print("wavenet stack", cnn_tanh, flush=True)
-    networks = PC.pkg().networks
+    networks = PC.networks()
     nb, Q, R, K, C = 4, 64, 64, 128, 80
     lengths = [120, 90]
     S, T = len(lengths), max(lengths)

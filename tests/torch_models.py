@@ -4,15 +4,7 @@ import numpy as np
 import torch
 
 
-def make_pat_types(lengths, T):
-    """patTypes[t*S+s]: 0 none, 1 first, 2 normal, 3 last (sequences left-aligned)."""
-    S = len(lengths)
-    pat = np.zeros((T, S), dtype=np.int8)
-    for s, n in enumerate(lengths):
-        pat[:n, s] = 2
-        pat[0, s] = 1
-        pat[n - 1, s] = 3
-    return pat.reshape(-1)
+from synth import make_pat_types  # noqa: E402,F401  (one definition, shared with the benchmark)
 
 
 def split_lstm_weights(W, P, L, bidir):
