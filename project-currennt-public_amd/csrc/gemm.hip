@@ -6,7 +6,7 @@
 // products of a BLSTM become one pass), several independent problems per launch, split-K for the
 // long-K weight-gradient shapes, and a fused bias + activation epilogue for the dense forward.
 //
-// Tiling: T x T x 16 per workgroup with T = 128 or 64, four 64-lane waves in a 2 x 2 arrangement, each wave
+// Tiling: T x T x 32 per workgroup with T = 128 or 64, four 64-lane waves in a 2 x 2 arrangement, each wave
 // owning a T/2 x T/2 block as tiles of v_mfma_f32_32x32x2_f32.  An operand tile sits in LDS in the
 // orientation it has in memory, so that staging never transposes: k-contiguous operands as [row][k] with
 // a (BK+4)-float pitch (16-byte fragment reads, conflict free), row-contiguous operands as [k][row]
