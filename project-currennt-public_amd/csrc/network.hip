@@ -1296,6 +1296,25 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     // many small layers cannot afford them per layer (the host's enqueue rate then bounds its backward pass), so the
     // weight halves of small layers are collected and handed over a few at a time, those of large layers at once.
     std::vector<char> fan_done(net->layers.size(), 0);
+    std::vector<char> errors_done(net->layers.size(), 0);  // error step done by the block launch of a later layer
+    static const bool fuse_blocks = [] { const char *e = std::getenv("CNT_NET_FUSE_BLOCKS"); return !e || std::atoi(e) != 0; }();
+    // WaveNet residual block seen from its skip 1x1 layer i: [cnn 2R][wavnetc R][dense R, identity][skipadd, shares
+    // the following sum][skipini][dense K, identity (i)]
+    auto block_at = [&](size_t i) {
+        if (!fuse_blocks || i < 5) return false;
+        const NetLayer &sk = net->layers[i], &ini = net->layers[i - 1], &add = net->layers[i - 2], &out = net->layers[i - 3];
+        const NetLayer &wav = net->layers[i - 4], &cnn = net->layers[i - 5];
+        const int R = ini.size;
+        auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+        return sk.kind == K_DENSE && sk.act == ACT_IDENTITY && ini.kind == K_SKIPINI && ini.err && ini.err == ini.total &&
+               is_sum_skip(add.kind) && add.total == ini.total && !add.needs_sum && add.live_targets == 0 && add.size == R &&
+               out.kind == K_DENSE && out.act == ACT_IDENTITY && out.err == ini.total && out.size == R &&
+               wav.kind == K_WAVNETC && wav.size == R && wav.core && (wav.ctx_dim == 0 || wav.cth) &&
+               cnn.kind == K_CNN && cnn.size == 2 * R && cnn.err &&
+               sk.N == ini.N && sk.N == out.N && sk.N == wav.N && sk.N == cnn.N &&
+               wavenet_block_errors_supported(R, sk.size) && aligned(sk.err) && aligned(ini.total) && aligned(ini.eskip) &&
+               aligned(wav.core) && aligned(wav.cth) && aligned(cnn.out) && aligned(cnn.err);
+    };
     std::vector<size_t> pending;
     auto weight_half = [&](size_t i, hipStream_t ws) -> int {
         NetLayer &L = net->layers[i];
@@ -1439,7 +1458,20 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                         fan.from_skip = prev.needs_sum ? prev.eskip : nullptr;
                     }
                     bool fused = false;
+                    if (errors_done[i]) {
+                        // its errors went on inside the block launch of the skip 1x1 layer
+                    } else if (block_at(i)) {
+                        const NetLayer &out = net->layers[i - 3], &wav = net->layers[i - 4], &cnn = net->layers[i - 5];
+                        CNT_TRY(wavenet_block_errors(stream, prev.size, L.size, N, L.pat, W, net->weights + out.w_off, L.err,
+                                                     prev_err, wanted ? &fan : nullptr, wav.core,
+                                                     wav.ctx_dim > 0 ? wav.cth : nullptr, cnn.delta_fused ? cnn.out : nullptr,
+                                                     cnn.err));
+                        fan_done[i - 1] = 1;
+                        errors_done[i - 3] = errors_done[i - 4] = 1;
+                        goto weight_half_of_layer;
+                    }
                     static const bool early = [] { const char *e = std::getenv("CNT_NET_EARLY_WEIGHTS"); return !e || std::atoi(e) != 0; }();
+                    if (errors_done[i]) goto weight_half_of_layer;
                     if (L.kind == K_DENSE && early && net->overlap && prev_err && (double)prev.size * L.size * N >= 4e8) {
                         // a large dense layer: deltas first, then its weight half starts on a side stream next to the
                         // product for the preceding layer's errors instead of after it
@@ -1474,9 +1506,14 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                     }
                     CNT_TRY(cnt_lstm_backward_errors(L.lstm, stream, W, L.err, prev_err));
                 } else {
-                    CNT_TRY(cnt_wavnetc_backward_errors(stream, L.size, L.ctx_dim, N, L.pat, W, L.core, L.cth, L.err,
-                                                        prev.err, net->flagged >= 0 ? net->ctx_grad : nullptr,
-                                                        prev.delta_fused ? prev.out : nullptr));
+                    if (errors_done[i]) {
+                        if (L.ctx_dim > 0 && net->flagged >= 0)
+                            CNT_TRY(wavnetc_context_grad(stream, L.size, L.ctx_dim, N, W, L.cth, net->ctx_grad));
+                    } else {
+                        CNT_TRY(cnt_wavnetc_backward_errors(stream, L.size, L.ctx_dim, N, L.pat, W, L.core, L.cth, L.err,
+                                                            prev.err, net->flagged >= 0 ? net->ctx_grad : nullptr,
+                                                            prev.delta_fused ? prev.out : nullptr));
+                    }
                     if ((int)i == net->first_wavnetc && net->flagged >= 0) {
                         // every wavnetc layer has added its share; hand the sum per frame to the layer that feeds them
                         // (layers/wavNetCore.cu:895-913)
@@ -1485,6 +1522,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                                                              net->ctx_grad, f.err));
                     }
                 }
+            weight_half_of_layer:
                 if (L.kind == K_WAVNETC && L.ctx_dim == 0) break;
                 if (!net->overlap) {
                     CNT_TRY(weight_half(i, stream));

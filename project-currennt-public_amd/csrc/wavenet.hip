@@ -166,6 +166,201 @@ int launch_gated_backward(hipStream_t stream, int D, size_t count, const char *p
     return CNT_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Error path of one residual block in one launch: the 1x1 layer that feeds the skip sum (R -> K), the skip layer in
+// front of it (adds what later layers handed to it and hands the sum on), the 1x1 layer behind the gated unit
+// (R -> R) and the gated unit itself.  Run layer by layer this is a product that writes R x N errors, a second
+// product that reads them and writes R x N, and an elementwise pass that reads those; here the R x N intermediates
+// stay in registers.
+//
+// A wave owns 16 samples.  Both products are computed transposed, D[channel][sample] = sum_k W[k][channel] *
+// E[sample][k], with v_mfma_f32_16x16x4f32: a lane then holds, for ITS sample (lane % 16), four consecutive channels
+// per accumulator (channel = 16*tile + 4*(lane/16) + v), i.e. 16-byte pieces of the sample-major buffers, and the sum
+// over k may run in any order: instruction (j, i) takes k = 16j + 4*(lane/16) + i from both operands.  With that order
+// the B operand of the first product is K/16 16-byte loads per lane straight from the error buffer (64 contiguous
+// bytes per sample and load), and the accumulators of the first product ARE the B operand of the second (register i
+// of tile j).  The weights sit in LDS in the order the A operand wants them, one 16-byte read per four instructions.
+struct BlockErrArgs {
+    int N;
+    const char *pat;
+    const float *w_skip;     // [K][R]: weights of the R -> K layer (element (k, r) at k*R + r)
+    const float *w_out;      // [R][R]: weights of the R -> R layer
+    const float *e_skip;     // K x N: errors at the outputs of the R -> K layer
+    const float *from_skip;  // R x N or null: what later layers handed to the skip layer
+    float *total;            // R x N: the skip layer's summed errors (= the R -> R layer's output errors)
+    int fan_n;
+    float *const *fan_targets;
+    const int *fan_is_skip;
+    const float *pre;        // 2R x N: pre-activations of the gated unit
+    const float *conv_tanh;  // 2R x N or null: outputs of a convolution layer with tanh output
+    float *ctx_tanh;         // 2R x N or null: tanh of the conditioning part, overwritten with its gradient
+    float *deltas;           // 2R x N: errors (or deltas) of the convolution layer
+};
+
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+template <int R, int K>
+__global__ __launch_bounds__(256, 2) void wavenet_block_errors_kernel(const BlockErrArgs a) {
+    static_assert(R % 16 == 0 && K % 16 == 0 && R <= 128, "block geometry");
+    constexpr int RT = R / 16;  // channel tiles
+    constexpr int KJ = K / 16, RJ = R / 16;
+    // A operands: [tile][j][lane = 16*quarter + channel in tile][i] = W[16j + 4*quarter + i][16*tile + channel]
+    __shared__ __attribute__((aligned(16))) float w1[RT * KJ * 64 * 4];
+    __shared__ __attribute__((aligned(16))) float w2[RT * RJ * 64 * 4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int quarter = lane >> 4, col = lane & 15;
+    const int n_raw = (blockIdx.x * 4 + wave) * 16 + col;
+    const bool ok = n_raw < a.N;
+    const size_t n = ok ? n_raw : a.N - 1;  // lanes past the end compute on the last sample and store nothing
+
+    // every global read that does not depend on a product is requested up front
+    constexpr int F1 = K * R / 4 / 256, F2 = R * R / 4 / 256;
+    static_assert((K * R) % 1024 == 0 && (R * R) % 1024 == 0, "weights are staged in 16-byte pieces by 256 threads");
+    float4 s1[F1], s2[F2];
+#pragma unroll
+    for (int q = 0; q < F1; ++q) s1[q] = reinterpret_cast<const float4 *>(a.w_skip)[q * 256 + tid];
+#pragma unroll
+    for (int q = 0; q < F2; ++q) s2[q] = reinterpret_cast<const float4 *>(a.w_out)[q * 256 + tid];
+    float4 b1[KJ];
+    {
+        const float4 *src = reinterpret_cast<const float4 *>(a.e_skip + n * K + 4 * quarter);
+#pragma unroll
+        for (int j = 0; j < KJ; ++j) b1[j] = src[4 * j];
+    }
+    float4 side[RT];
+    if (a.from_skip) {
+#pragma unroll
+        for (int t = 0; t < RT; ++t) side[t] = *reinterpret_cast<const float4 *>(a.from_skip + n * R + 16 * t + 4 * quarter);
+    }
+    const bool live = a.pat[n] != 0;
+    auto stage = [](float *w, int J, int idx4, const float4 &v) {
+        // element (k, ch .. ch+3): same k, four neighbouring channels of one tile
+        const int k = idx4 * 4 / R, ch = idx4 * 4 % R;
+        float *dst = w + ((((ch / 16) * J + k / 16) * 4 + ((k >> 2) & 3)) * 16 + ch % 16) * 4 + (k & 3);
+        dst[0] = v.x; dst[4] = v.y; dst[8] = v.z; dst[12] = v.w;
+    };
+#pragma unroll
+    for (int q = 0; q < F1; ++q) stage(w1, KJ, q * 256 + tid, s1[q]);
+#pragma unroll
+    for (int q = 0; q < F2; ++q) stage(w2, RJ, q * 256 + tid, s2[q]);
+    __syncthreads();
+
+    f32x4v e[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        f32x4v acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < KJ; ++j) {
+            const float4 w = *reinterpret_cast<const float4 *>(&w1[((t * KJ + j) * 64 + lane) * 4]);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, b1[j].x, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, b1[j].y, acc1, 0, 0, 0);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, b1[j].z, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.w, b1[j].w, acc1, 0, 0, 0);
+        }
+        e[t] = acc0 + acc1;
+    }
+    // the skip layer's step: add the side buffer, keep the sum, hand it on
+    if (a.from_skip) {
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            e[t][0] += side[t].x; e[t][1] += side[t].y; e[t][2] += side[t].z; e[t][3] += side[t].w;
+        }
+    }
+    // gate operands requested before the second product starts
+    float4 p1[RT], p2[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        const size_t at = n * 2 * R + 16 * t + 4 * quarter;
+        p1[t] = *reinterpret_cast<const float4 *>(a.pre + at);
+        p2[t] = *reinterpret_cast<const float4 *>(a.pre + at + R);
+    }
+    if (ok) {
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+            *reinterpret_cast<float4 *>(a.total + n * R + 16 * t + 4 * quarter) = float4{e[t][0], e[t][1], e[t][2], e[t][3]};
+        for (int q = 0; q < a.fan_n; ++q) {
+            float *tgt = a.fan_targets[q];
+            if (a.fan_is_skip[q]) {
+                float4 old[RT];
+#pragma unroll
+                for (int t = 0; t < RT; ++t) old[t] = *reinterpret_cast<const float4 *>(tgt + n * R + 16 * t + 4 * quarter);
+#pragma unroll
+                for (int t = 0; t < RT; ++t)
+                    *reinterpret_cast<float4 *>(tgt + n * R + 16 * t + 4 * quarter) =
+                        float4{e[t][0] + old[t].x, e[t][1] + old[t].y, e[t][2] + old[t].z, e[t][3] + old[t].w};
+            } else {
+#pragma unroll
+                for (int t = 0; t < RT; ++t)
+                    *reinterpret_cast<float4 *>(tgt + n * R + 16 * t + 4 * quarter) = float4{e[t][0], e[t][1], e[t][2], e[t][3]};
+            }
+        }
+    }
+
+    // second product: errors at the gated unit's outputs
+    f32x4v u[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        f32x4v acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < RJ; ++j) {
+            const float4 w = *reinterpret_cast<const float4 *>(&w2[((t * RJ + j) * 64 + lane) * 4]);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, e[j][0], acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, e[j][1], acc1, 0, 0, 0);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, e[j][2], acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.w, e[j][3], acc1, 0, 0, 0);
+        }
+        u[t] = acc0 + acc1;
+    }
+
+    // the gated unit (see gated_backward_kernel), four channels at a time
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        const size_t at = n * 2 * R + 16 * t + 4 * quarter;
+        const float *a1 = reinterpret_cast<const float *>(&p1[t]), *a2 = reinterpret_cast<const float *>(&p2[t]);
+        float g1[4], g2[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float th = tanh_act(a1[q]);
+            const float sg = logistic(a2[q]);
+            const float ev = u[t][q];
+            g1[q] = live ? (1.0f - th * th) * sg * ev : 0.0f;
+            g2[q] = live ? th * (sg * (1.0f - sg)) * ev : 0.0f;
+        }
+        float4 o1 = {g1[0], g1[1], g1[2], g1[3]}, o2 = {g2[0], g2[1], g2[2], g2[3]};
+        if (a.conv_tanh) {
+            const float4 y1 = *reinterpret_cast<const float4 *>(a.conv_tanh + at);
+            const float4 y2 = *reinterpret_cast<const float4 *>(a.conv_tanh + at + R);
+            o1 = float4{tanh_deriv(y1.x) * g1[0], tanh_deriv(y1.y) * g1[1], tanh_deriv(y1.z) * g1[2], tanh_deriv(y1.w) * g1[3]};
+            o2 = float4{tanh_deriv(y2.x) * g2[0], tanh_deriv(y2.y) * g2[1], tanh_deriv(y2.z) * g2[2], tanh_deriv(y2.w) * g2[3]};
+        }
+        if (ok) {
+            *reinterpret_cast<float4 *>(a.deltas + at) = o1;
+            *reinterpret_cast<float4 *>(a.deltas + at + R) = o2;
+        }
+        if (a.ctx_tanh) {
+            const float4 c1 = *reinterpret_cast<const float4 *>(a.ctx_tanh + at);
+            const float4 c2 = *reinterpret_cast<const float4 *>(a.ctx_tanh + at + R);
+            const float4 q1 = {tanh_deriv(c1.x) * g1[0], tanh_deriv(c1.y) * g1[1], tanh_deriv(c1.z) * g1[2], tanh_deriv(c1.w) * g1[3]};
+            const float4 q2 = {tanh_deriv(c2.x) * g2[0], tanh_deriv(c2.y) * g2[1], tanh_deriv(c2.z) * g2[2], tanh_deriv(c2.w) * g2[3]};
+            if (ok) {
+                *reinterpret_cast<float4 *>(a.ctx_tanh + at) = q1;
+                *reinterpret_cast<float4 *>(a.ctx_tanh + at + R) = q2;
+            }
+        }
+    }
+}
+
+typedef void (*block_err_kernel_t)(const BlockErrArgs);
+block_err_kernel_t pick_block_errors_kernel(int R, int K) {
+    if (R == 64 && K == 128) return wavenet_block_errors_kernel<64, 128>;
+    if (R == 64 && K == 256) return wavenet_block_errors_kernel<64, 256>;
+    if (R == 64 && K == 64) return wavenet_block_errors_kernel<64, 64>;
+    if (R == 32 && K == 128) return wavenet_block_errors_kernel<32, 128>;
+    if (R == 32 && K == 64) return wavenet_block_errors_kernel<32, 64>;
+    if (R == 32 && K == 32) return wavenet_block_errors_kernel<32, 32>;
+    return nullptr;
+}
+
 __global__ void sum_context_grad_kernel(int C, int S, int resolution, size_t count, int N,
                                         const char *__restrict__ pat_frames, const char *__restrict__ pat,
                                         const float *__restrict__ ctx_grad, float *__restrict__ frame_grad) {
@@ -540,6 +735,43 @@ int cnt_wavnetc_forward(void *stream_, int D, int C, int N, const char *patTypes
     return cnt_gatedact_forward(stream_, D, N, patTypes, core_buf, outputs);
 }
 
+extern "C++" bool cnt::wavenet_block_errors_supported(int R, int K) { return pick_block_errors_kernel(R, K) != nullptr; }
+
+extern "C++" int cnt::wavenet_block_errors(hipStream_t stream, int R, int K, int N, const char *patTypes,
+                                           const float *skip_weights, const float *out_weights, const float *skip_errors,
+                                           float *total, const FanOut *fan, const float *core_buf, float *ctx_tanh,
+                                           const float *conv_tanh_outputs, float *conv_errors) {
+    block_err_kernel_t k = pick_block_errors_kernel(R, K);
+    CNT_REQUIRE(k != nullptr, "wavenet_block_errors: no kernel for %d residual and %d skip channels", R, K);
+    CNT_REQUIRE(N > 0 && patTypes && skip_weights && out_weights && skip_errors && total && core_buf && conv_errors,
+                "wavenet_block_errors: null argument");
+    BlockErrArgs a = {};
+    a.N = N; a.pat = patTypes; a.w_skip = skip_weights; a.w_out = out_weights; a.e_skip = skip_errors;
+    a.total = total;
+    if (fan) { a.from_skip = fan->from_skip; a.fan_n = fan->n; a.fan_targets = fan->targets; a.fan_is_skip = fan->is_skip; }
+    a.pre = core_buf; a.conv_tanh = conv_tanh_outputs; a.ctx_tanh = ctx_tanh; a.deltas = conv_errors;
+    auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    CNT_REQUIRE(aligned(skip_errors) && aligned(total) && aligned(a.from_skip) && aligned(core_buf) && aligned(ctx_tanh) &&
+                aligned(conv_tanh_outputs) && aligned(conv_errors), "wavenet_block_errors: buffers must be 16-byte aligned");
+    ProfileScope prof(stream, "wavenet_block_errors");
+    hipLaunchKernelGGL(k, dim3((N + 63) / 64), dim3(256), 0, stream, a);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
+
+extern "C++" int cnt::wavnetc_context_grad(hipStream_t stream, int D, int C, int N, const float *weights,
+                                           const float *ctx_tanh, float *ctx_grad) {
+    GemmArgs ga = {};
+    ga.m = C; ga.n = N; ga.k = 2 * D;
+    ga.a_kcontig = 0; ga.lda = C;
+    ga.b_kcontig = 1; ga.ldb = 2 * D;
+    ga.ldc = C;
+    ga.nseg = 1; ga.nprob = 1; ga.splitk = 1; ga.epilogue = EPI_ADD;
+    ga.prob[0].A[0] = weights; ga.prob[0].B[0] = ctx_tanh; ga.prob[0].C = ctx_grad;
+    ga.label = "gemm:wavnetc_ctx_grad";
+    return gemm_launch(stream, ga);
+}
+
 int cnt_wavnetc_backward_errors(void *stream_, int D, int C, int N, const char *patTypes, const float *weights,
                                 const float *core_buf, float *ctx_tanh, const float *output_errors, float *prev_errors,
                                 float *ctx_grad, const float *prev_tanh_outputs) {
@@ -555,17 +787,7 @@ int cnt_wavnetc_backward_errors(void *stream_, int D, int C, int N, const char *
         CNT_TRY(launch_gated_backward(stream, D, count, patTypes, core_buf, output_errors, prev_errors,
                                       C > 0 ? ctx_tanh : nullptr, prev_tanh_outputs));
     }
-    if (C > 0 && ctx_grad) {
-        GemmArgs ga = {};
-        ga.m = C; ga.n = N; ga.k = 2 * D;
-        ga.a_kcontig = 0; ga.lda = C;
-        ga.b_kcontig = 1; ga.ldb = 2 * D;
-        ga.ldc = C;
-        ga.nseg = 1; ga.nprob = 1; ga.splitk = 1; ga.epilogue = EPI_ADD;
-        ga.prob[0].A[0] = weights; ga.prob[0].B[0] = ctx_tanh; ga.prob[0].C = ctx_grad;
-        ga.label = "gemm:wavnetc_ctx_grad";
-        CNT_TRY(gemm_launch(stream, ga));
-    }
+    if (C > 0 && ctx_grad) CNT_TRY(wavnetc_context_grad(stream, D, C, N, weights, ctx_tanh, ctx_grad));
     return CNT_OK;
 }
 
