@@ -218,9 +218,13 @@ int dense_backward_errors_fan(hipStream_t stream, int P, int D, int N, int act, 
 // Error path of one WaveNet residual block in one launch (skip 1x1 layer, the skip layer in front of it, the 1x1
 // layer behind the gated unit, the gated unit): see wavenet_block_errors_kernel.
 bool wavenet_block_errors_supported(int R, int K);
+// `fold` (optional): the convolution layer above the block, whose error product (two live taps) is added to the
+// block's summed errors inside the same launch instead of being written to the closing skip layer first
+bool cnn_foldable(const cnt_cnn *h, int R);
 int wavenet_block_errors(hipStream_t stream, int R, int K, int N, const char *patTypes, const float *skip_weights,
                          const float *out_weights, const float *skip_errors, float *total, const FanOut *fan,
-                         const float *core_buf, float *ctx_tanh, const float *conv_tanh_outputs, float *conv_errors);
+                         const float *core_buf, float *ctx_tanh, const float *conv_tanh_outputs, float *conv_errors,
+                         const cnt_cnn *fold, const float *fold_weights, const float *fold_deltas);
 int wavnetc_context_grad(hipStream_t stream, int D, int C, int N, const float *weights, const float *ctx_tanh,
                          float *ctx_grad);
 int cnn_backward_errors_fan(cnt_cnn *h, hipStream_t stream, const char *patTypes, int curT, const float *weights,

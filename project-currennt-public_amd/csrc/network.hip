@@ -217,6 +217,7 @@ struct NetLayer {
     int ext_frames = 0, index_load_method = 0;
     int cnn_tanh = 0;                        // cnn: "tanhoutput"
     bool delta_fused = false;                // cnn followed by a wavnetc layer: that layer writes this layer's delta
+    bool fold_ok = false;                    // cnn whose error product can ride in the launch of the block below it
     const float *total = nullptr;            // skip layers: where the summed error stands after the layer's step
     bool needs_sum = false;                  // skip layers: errors += side buffer is not a no-op
     int live_targets = 0;                    // skip layers: sources that receive the sum through a launch
@@ -936,6 +937,26 @@ int finish_build(cnt_network *net, const json::Value *weights) {
         CNT_HIP(hipMemcpy(L.tgt_ptrs, t.data(), t.size() * sizeof(float *), hipMemcpyHostToDevice));
         CNT_HIP(hipMemcpy(L.tgt_is_skip, flag[(size_t)i].data(), t.size() * sizeof(int), hipMemcpyHostToDevice));
     }
+    // A convolution layer i that sits on a block's closing skipadd layer [i-1], behind that block's skip collector
+    // [i-2], skip 1x1 layer [i-3] and skipini layer [i-4]: when the closing layer does nothing but add what the later
+    // block handed to it and hand the sum to the skipini layer, and nothing else writes that layer's side buffer, the
+    // convolution's error product can be added to the block's sum inside the block's own launch (the buffers in between
+    // are then never written).  Checked here on the pointer tables; sizes and alignment when the launch is made.
+    for (int i = 8; i < n_layers; ++i) {
+        NetLayer &C = net->layers[(size_t)i];
+        if (C.kind != K_CNN) continue;
+        const NetLayer &closing = net->layers[(size_t)i - 1], &collector = net->layers[(size_t)i - 2];
+        const NetLayer &ini = net->layers[(size_t)i - 4];
+        if (closing.kind != K_SKIPADD || closing.pre.size() != 1 || closing.pre[0] != i - 4) continue;
+        if (!closing.err || closing.err != closing.total || !closing.needs_sum || !closing.eskip) continue;
+        if (ini.kind != K_SKIPINI || !ini.needs_sum || !ini.eskip) continue;
+        if (tgt[(size_t)i - 1].size() != 1 || tgt[(size_t)i - 1][0] != ini.eskip || !flag[(size_t)i - 1][0]) continue;
+        if (!is_sum_skip(collector.kind) || collector.needs_sum || !tgt[(size_t)i - 2].empty()) continue;
+        int writers = 0;
+        for (int y = 0; y < n_layers; ++y)
+            for (float *t : tgt[(size_t)y]) writers += t == ini.eskip ? 1 : 0;
+        C.fold_ok = writers == 1;
+    }
     // pattern types of the lower time resolutions, one buffer per resolution
     for (auto &L : net->layers) {
         if (L.res == 1) continue;
@@ -1041,6 +1062,7 @@ int cnt_network_create(const char *json_text, int parallel_sequences, int max_se
     net->S = parallel_sequences;
     net->maxT = max_seq_length;
     if (options) net->overlap = options->no_overlap ? 0 : 1;
+    if (const char *e = std::getenv("CNT_NET_OVERLAP")) net->overlap = std::atoi(e) != 0 ? 1 : 0;  // measurements
     int status = CNT_OK;
     for (const auto &obj : layers->arr) {
         if (obj.type != json::Value::OBJ) {
@@ -1300,6 +1322,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     static const bool fuse_blocks = [] { const char *e = std::getenv("CNT_NET_FUSE_BLOCKS"); return !e || std::atoi(e) != 0; }();
     // WaveNet residual block seen from its skip 1x1 layer i: [cnn 2R][wavnetc R][dense R, identity][skipadd, shares
     // the following sum][skipini][dense K, identity (i)]
+    std::vector<int> fold_from(net->layers.size(), -1);  // skip 1x1 layer -> convolution layer folded into its launch
     auto block_at = [&](size_t i) {
         if (!fuse_blocks || i < 5) return false;
         const NetLayer &sk = net->layers[i], &ini = net->layers[i - 1], &add = net->layers[i - 2], &out = net->layers[i - 3];
@@ -1313,7 +1336,15 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                cnn.kind == K_CNN && cnn.size == 2 * R && cnn.err &&
                sk.N == ini.N && sk.N == out.N && sk.N == wav.N && sk.N == cnn.N &&
                wavenet_block_errors_supported(R, sk.size) && aligned(sk.err) && aligned(ini.total) && aligned(ini.eskip) &&
-               aligned(wav.core) && aligned(wav.cth) && aligned(cnn.out) && aligned(cnn.err);
+               aligned(wav.core) && aligned(wav.cth) && aligned(cnn.out) && aligned(cnn.err) &&
+               aligned(net->weights + sk.w_off) && aligned(net->weights + out.w_off);
+    };
+    auto fold_at = [&](size_t i) {
+        if (i < 8) return false;
+        const NetLayer &C = net->layers[i], &closing = net->layers[i - 1], &sk = net->layers[i - 3];
+        auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+        return C.fold_ok && block_at(i - 3) && C.N == sk.N && closing.N == sk.N && cnn_foldable(C.cnn, closing.size) &&
+               (C.delta_fused || !C.cnn_tanh) && aligned(net->weights + C.w_off) && aligned(C.err) && aligned(closing.eskip);
     };
     std::vector<size_t> pending;
     auto weight_half = [&](size_t i, hipStream_t ws) -> int {
@@ -1460,12 +1491,23 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                     bool fused = false;
                     if (errors_done[i]) {
                         // its errors went on inside the block launch of the skip 1x1 layer
+                    } else if (L.kind == K_CNN && fold_at(i)) {
+                        // the block below adds this layer's error product to its own sum
+                        fold_from[i - 3] = (int)i;
+                        fan_done[i - 1] = 1;
+                        goto weight_half_of_layer;
                     } else if (block_at(i)) {
                         const NetLayer &out = net->layers[i - 3], &wav = net->layers[i - 4], &cnn = net->layers[i - 5];
+                        const NetLayer *fold = fold_from[i] >= 0 ? &net->layers[(size_t)fold_from[i]] : nullptr;
+                        FanOut block_fan = fan;
+                        // with a folded convolution, what the later block handed to the closing skipadd layer comes in
+                        // directly (that layer would have added it to the convolution's product and handed the sum on)
+                        if (fold) block_fan.from_skip = net->layers[(size_t)fold_from[i] - 1].eskip;
                         CNT_TRY(wavenet_block_errors(stream, prev.size, L.size, N, L.pat, W, net->weights + out.w_off, L.err,
-                                                     prev_err, wanted ? &fan : nullptr, wav.core,
+                                                     prev_err, (wanted || fold) ? &block_fan : nullptr, wav.core,
                                                      wav.ctx_dim > 0 ? wav.cth : nullptr, cnn.delta_fused ? cnn.out : nullptr,
-                                                     cnn.err));
+                                                     cnn.err, fold ? fold->cnn : nullptr,
+                                                     fold ? net->weights + fold->w_off : nullptr, fold ? fold->err : nullptr));
                         fan_done[i - 1] = 1;
                         errors_done[i - 3] = errors_done[i - 4] = 1;
                         goto weight_half_of_layer;

@@ -195,32 +195,41 @@ struct BlockErrArgs {
     const float *conv_tanh;  // 2R x N or null: outputs of a convolution layer with tanh output
     float *ctx_tanh;         // 2R x N or null: tanh of the conditioning part, overwritten with its gradient
     float *deltas;           // 2R x N: errors (or deltas) of the convolution layer
+    // folded convolution (two live taps, R inputs, 2R filters) whose errors go to the block's closing skip layer:
+    const float *conv_w[2];      // weight of (filter 0, tap q); filter d at + d*conv_ld, input channel p at + p
+    int conv_ld;
+    int conv_shift[2];           // tap q reads the delta of slot n + conv_shift[q]
+    const float *conv_deltas;    // 2R x N deltas of that convolution layer
 };
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
-template <int R, int K>
-__global__ __launch_bounds__(256, 2) void wavenet_block_errors_kernel(const BlockErrArgs a) {
+template <int R, int K, bool CONV>
+__global__ __launch_bounds__(CONV ? 512 : 256, CONV ? 1 : 2) void wavenet_block_errors_kernel(const BlockErrArgs a) {
     static_assert(R % 16 == 0 && K % 16 == 0 && R <= 128, "block geometry");
+    constexpr int NT = CONV ? 512 : 256;  // the folded convolution's weights take 2 x 2R x R words of LDS more
     constexpr int RT = R / 16;  // channel tiles
-    constexpr int KJ = K / 16, RJ = R / 16;
+    constexpr int KJ = K / 16, RJ = R / 16, CJ = 2 * R / 16;
     // A operands: [tile][j][lane = 16*quarter + channel in tile][i] = W[16j + 4*quarter + i][16*tile + channel]
     __shared__ __attribute__((aligned(16))) float w1[RT * KJ * 64 * 4];
     __shared__ __attribute__((aligned(16))) float w2[RT * RJ * 64 * 4];
+    __shared__ __attribute__((aligned(16))) float wc[CONV ? 2 * RT * CJ * 64 * 4 : 4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int quarter = lane >> 4, col = lane & 15;
-    const int n_raw = (blockIdx.x * 4 + wave) * 16 + col;
+    const int n_raw = (blockIdx.x * (NT / 64) + wave) * 16 + col;
     const bool ok = n_raw < a.N;
     const size_t n = ok ? n_raw : a.N - 1;  // lanes past the end compute on the last sample and store nothing
 
     // every global read that does not depend on a product is requested up front
-    constexpr int F1 = K * R / 4 / 256, F2 = R * R / 4 / 256;
-    static_assert((K * R) % 1024 == 0 && (R * R) % 1024 == 0, "weights are staged in 16-byte pieces by 256 threads");
+    constexpr int T1 = K * R / 4, T2 = R * R / 4, TC = 2 * R * R / 4;  // 16-byte pieces
+    constexpr int F1 = (T1 + NT - 1) / NT, F2 = (T2 + NT - 1) / NT, FC = CONV ? (TC + NT - 1) / NT : 0;
     float4 s1[F1], s2[F2];
 #pragma unroll
-    for (int q = 0; q < F1; ++q) s1[q] = reinterpret_cast<const float4 *>(a.w_skip)[q * 256 + tid];
+    for (int q = 0; q < F1; ++q)
+        if (q * NT + tid < T1) s1[q] = reinterpret_cast<const float4 *>(a.w_skip)[q * NT + tid];
 #pragma unroll
-    for (int q = 0; q < F2; ++q) s2[q] = reinterpret_cast<const float4 *>(a.w_out)[q * 256 + tid];
+    for (int q = 0; q < F2; ++q)
+        if (q * NT + tid < T2) s2[q] = reinterpret_cast<const float4 *>(a.w_out)[q * NT + tid];
     float4 b1[KJ];
     {
         const float4 *src = reinterpret_cast<const float4 *>(a.e_skip + n * K + 4 * quarter);
@@ -240,9 +249,59 @@ __global__ __launch_bounds__(256, 2) void wavenet_block_errors_kernel(const Bloc
         dst[0] = v.x; dst[4] = v.y; dst[8] = v.z; dst[12] = v.w;
     };
 #pragma unroll
-    for (int q = 0; q < F1; ++q) stage(w1, KJ, q * 256 + tid, s1[q]);
+    for (int q = 0; q < F1; ++q)
+        if (q * NT + tid < T1) stage(w1, KJ, q * NT + tid, s1[q]);
 #pragma unroll
-    for (int q = 0; q < F2; ++q) stage(w2, RJ, q * 256 + tid, s2[q]);
+    for (int q = 0; q < F2; ++q)
+        if (q * NT + tid < T2) stage(w2, RJ, q * NT + tid, s2[q]);
+    // folded convolution: tap q contributes sum_d Wc[d][tap q][p] * delta[slot n + shift q][d], counted only where both
+    // slots are inside the fraction and not padding (the rule of the convolution layer's own error product)
+    float4 bc[CONV ? 2 : 1][CONV ? CJ : 1];
+    if (CONV) {
+#pragma unroll
+        for (int tap = 0; tap < 2; ++tap) {
+            float4 sc[FC > 0 ? FC : 1];
+#pragma unroll
+            for (int q = 0; q < FC; ++q) {
+                const int idx4 = q * NT + tid;
+                if (idx4 < TC) sc[q] = *reinterpret_cast<const float4 *>(a.conv_w[tap] + (size_t)(idx4 * 4 / R) * a.conv_ld + idx4 * 4 % R);
+            }
+#pragma unroll
+            for (int q = 0; q < FC; ++q)
+                if (q * NT + tid < TC) stage(wc + tap * (RT * CJ * 64 * 4), CJ, q * NT + tid, sc[q]);
+        }
+#pragma unroll
+        for (int tap = 0; tap < 2; ++tap) {
+            const long long src = (long long)n + a.conv_shift[tap];
+            const bool inside = src >= 0 && src < a.N;
+            const size_t sc = inside ? (size_t)src : n;
+            const bool keep = live && inside && a.pat[sc] != 0;
+            const float4 *p = reinterpret_cast<const float4 *>(a.conv_deltas + sc * 2 * R + 4 * quarter);
+#pragma unroll
+            for (int j = 0; j < CJ; ++j) {
+                const float4 v = p[4 * j];
+                bc[tap][j] = keep ? v : float4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
+    }
+    // operands of the later phases are requested before the products start: the products then run while they arrive
+    float4 p1[RT], p2[RT], y1[RT], y2[RT], c1[RT], c2[RT], old0[RT];
+    const bool add_first = ok && a.fan_n > 0 && a.fan_is_skip[0] != 0;
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        const size_t at = n * 2 * R + 16 * t + 4 * quarter;
+        p1[t] = *reinterpret_cast<const float4 *>(a.pre + at);
+        p2[t] = *reinterpret_cast<const float4 *>(a.pre + at + R);
+        if (a.conv_tanh) {
+            y1[t] = *reinterpret_cast<const float4 *>(a.conv_tanh + at);
+            y2[t] = *reinterpret_cast<const float4 *>(a.conv_tanh + at + R);
+        }
+        if (a.ctx_tanh) {
+            c1[t] = *reinterpret_cast<const float4 *>(a.ctx_tanh + at);
+            c2[t] = *reinterpret_cast<const float4 *>(a.ctx_tanh + at + R);
+        }
+        if (add_first) old0[t] = *reinterpret_cast<const float4 *>(a.fan_targets[0] + n * R + 16 * t + 4 * quarter);
+    }
     __syncthreads();
 
     f32x4v e[RT];
@@ -257,6 +316,18 @@ __global__ __launch_bounds__(256, 2) void wavenet_block_errors_kernel(const Bloc
             acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, b1[j].z, acc0, 0, 0, 0);
             acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.w, b1[j].w, acc1, 0, 0, 0);
         }
+        if (CONV) {
+#pragma unroll
+            for (int tap = 0; tap < 2; ++tap)
+#pragma unroll
+                for (int j = 0; j < CJ; ++j) {
+                    const float4 w = *reinterpret_cast<const float4 *>(&wc[(((tap * RT + t) * CJ + j) * 64 + lane) * 4]);
+                    acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, bc[tap][j].x, acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, bc[tap][j].y, acc1, 0, 0, 0);
+                    acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, bc[tap][j].z, acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.w, bc[tap][j].w, acc1, 0, 0, 0);
+                }
+        }
         e[t] = acc0 + acc1;
     }
     // the skip layer's step: add the side buffer, keep the sum, hand it on
@@ -265,14 +336,6 @@ __global__ __launch_bounds__(256, 2) void wavenet_block_errors_kernel(const Bloc
         for (int t = 0; t < RT; ++t) {
             e[t][0] += side[t].x; e[t][1] += side[t].y; e[t][2] += side[t].z; e[t][3] += side[t].w;
         }
-    }
-    // gate operands requested before the second product starts
-    float4 p1[RT], p2[RT];
-#pragma unroll
-    for (int t = 0; t < RT; ++t) {
-        const size_t at = n * 2 * R + 16 * t + 4 * quarter;
-        p1[t] = *reinterpret_cast<const float4 *>(a.pre + at);
-        p2[t] = *reinterpret_cast<const float4 *>(a.pre + at + R);
     }
     if (ok) {
 #pragma unroll
@@ -283,7 +346,8 @@ __global__ __launch_bounds__(256, 2) void wavenet_block_errors_kernel(const Bloc
             if (a.fan_is_skip[q]) {
                 float4 old[RT];
 #pragma unroll
-                for (int t = 0; t < RT; ++t) old[t] = *reinterpret_cast<const float4 *>(tgt + n * R + 16 * t + 4 * quarter);
+                for (int t = 0; t < RT; ++t)
+                    old[t] = q == 0 ? old0[t] : *reinterpret_cast<const float4 *>(tgt + n * R + 16 * t + 4 * quarter);
 #pragma unroll
                 for (int t = 0; t < RT; ++t)
                     *reinterpret_cast<float4 *>(tgt + n * R + 16 * t + 4 * quarter) =
@@ -328,20 +392,16 @@ __global__ __launch_bounds__(256, 2) void wavenet_block_errors_kernel(const Bloc
         }
         float4 o1 = {g1[0], g1[1], g1[2], g1[3]}, o2 = {g2[0], g2[1], g2[2], g2[3]};
         if (a.conv_tanh) {
-            const float4 y1 = *reinterpret_cast<const float4 *>(a.conv_tanh + at);
-            const float4 y2 = *reinterpret_cast<const float4 *>(a.conv_tanh + at + R);
-            o1 = float4{tanh_deriv(y1.x) * g1[0], tanh_deriv(y1.y) * g1[1], tanh_deriv(y1.z) * g1[2], tanh_deriv(y1.w) * g1[3]};
-            o2 = float4{tanh_deriv(y2.x) * g2[0], tanh_deriv(y2.y) * g2[1], tanh_deriv(y2.z) * g2[2], tanh_deriv(y2.w) * g2[3]};
+            o1 = float4{tanh_deriv(y1[t].x) * g1[0], tanh_deriv(y1[t].y) * g1[1], tanh_deriv(y1[t].z) * g1[2], tanh_deriv(y1[t].w) * g1[3]};
+            o2 = float4{tanh_deriv(y2[t].x) * g2[0], tanh_deriv(y2[t].y) * g2[1], tanh_deriv(y2[t].z) * g2[2], tanh_deriv(y2[t].w) * g2[3]};
         }
         if (ok) {
             *reinterpret_cast<float4 *>(a.deltas + at) = o1;
             *reinterpret_cast<float4 *>(a.deltas + at + R) = o2;
         }
         if (a.ctx_tanh) {
-            const float4 c1 = *reinterpret_cast<const float4 *>(a.ctx_tanh + at);
-            const float4 c2 = *reinterpret_cast<const float4 *>(a.ctx_tanh + at + R);
-            const float4 q1 = {tanh_deriv(c1.x) * g1[0], tanh_deriv(c1.y) * g1[1], tanh_deriv(c1.z) * g1[2], tanh_deriv(c1.w) * g1[3]};
-            const float4 q2 = {tanh_deriv(c2.x) * g2[0], tanh_deriv(c2.y) * g2[1], tanh_deriv(c2.z) * g2[2], tanh_deriv(c2.w) * g2[3]};
+            const float4 q1 = {tanh_deriv(c1[t].x) * g1[0], tanh_deriv(c1[t].y) * g1[1], tanh_deriv(c1[t].z) * g1[2], tanh_deriv(c1[t].w) * g1[3]};
+            const float4 q2 = {tanh_deriv(c2[t].x) * g2[0], tanh_deriv(c2[t].y) * g2[1], tanh_deriv(c2[t].z) * g2[2], tanh_deriv(c2[t].w) * g2[3]};
             if (ok) {
                 *reinterpret_cast<float4 *>(a.ctx_tanh + at) = q1;
                 *reinterpret_cast<float4 *>(a.ctx_tanh + at + R) = q2;
@@ -351,13 +411,16 @@ __global__ __launch_bounds__(256, 2) void wavenet_block_errors_kernel(const Bloc
 }
 
 typedef void (*block_err_kernel_t)(const BlockErrArgs);
-block_err_kernel_t pick_block_errors_kernel(int R, int K) {
-    if (R == 64 && K == 128) return wavenet_block_errors_kernel<64, 128>;
-    if (R == 64 && K == 256) return wavenet_block_errors_kernel<64, 256>;
-    if (R == 64 && K == 64) return wavenet_block_errors_kernel<64, 64>;
-    if (R == 32 && K == 128) return wavenet_block_errors_kernel<32, 128>;
-    if (R == 32 && K == 64) return wavenet_block_errors_kernel<32, 64>;
-    if (R == 32 && K == 32) return wavenet_block_errors_kernel<32, 32>;
+block_err_kernel_t pick_block_errors_kernel(int R, int K, bool conv) {
+#define CNT_BLOCK_KERNEL(r, k) \
+    if (R == r && K == k) return conv ? wavenet_block_errors_kernel<r, k, true> : wavenet_block_errors_kernel<r, k, false>;
+    CNT_BLOCK_KERNEL(64, 128)
+    CNT_BLOCK_KERNEL(64, 256)
+    CNT_BLOCK_KERNEL(64, 64)
+    CNT_BLOCK_KERNEL(32, 128)
+    CNT_BLOCK_KERNEL(32, 64)
+    CNT_BLOCK_KERNEL(32, 32)
+#undef CNT_BLOCK_KERNEL
     return nullptr;
 }
 
@@ -735,13 +798,20 @@ int cnt_wavnetc_forward(void *stream_, int D, int C, int N, const char *patTypes
     return cnt_gatedact_forward(stream_, D, N, patTypes, core_buf, outputs);
 }
 
-extern "C++" bool cnt::wavenet_block_errors_supported(int R, int K) { return pick_block_errors_kernel(R, K) != nullptr; }
+extern "C++" bool cnt::wavenet_block_errors_supported(int R, int K) { return pick_block_errors_kernel(R, K, false) != nullptr; }
+
+extern "C++" bool cnt::cnn_foldable(const cnt_cnn *h, int R) {
+    // one run of filters, causal, two live taps, R inputs and 2R filters
+    return h && h->groups.size() == 1 && h->desc.causal > 0 && h->groups[0].hw == 1 && h->groups[0].d0 == 0 &&
+           h->groups[0].d1 == h->desc.D && h->desc.P == R && h->desc.D == 2 * R;
+}
 
 extern "C++" int cnt::wavenet_block_errors(hipStream_t stream, int R, int K, int N, const char *patTypes,
                                            const float *skip_weights, const float *out_weights, const float *skip_errors,
                                            float *total, const FanOut *fan, const float *core_buf, float *ctx_tanh,
-                                           const float *conv_tanh_outputs, float *conv_errors) {
-    block_err_kernel_t k = pick_block_errors_kernel(R, K);
+                                           const float *conv_tanh_outputs, float *conv_errors, const cnt_cnn *fold,
+                                           const float *fold_weights, const float *fold_deltas) {
+    block_err_kernel_t k = pick_block_errors_kernel(R, K, fold != nullptr);
     CNT_REQUIRE(k != nullptr, "wavenet_block_errors: no kernel for %d residual and %d skip channels", R, K);
     CNT_REQUIRE(N > 0 && patTypes && skip_weights && out_weights && skip_errors && total && core_buf && conv_errors,
                 "wavenet_block_errors: null argument");
@@ -751,10 +821,25 @@ extern "C++" int cnt::wavenet_block_errors(hipStream_t stream, int R, int K, int
     if (fan) { a.from_skip = fan->from_skip; a.fan_n = fan->n; a.fan_targets = fan->targets; a.fan_is_skip = fan->is_skip; }
     a.pre = core_buf; a.conv_tanh = conv_tanh_outputs; a.ctx_tanh = ctx_tanh; a.deltas = conv_errors;
     auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-    CNT_REQUIRE(aligned(skip_errors) && aligned(total) && aligned(a.from_skip) && aligned(core_buf) && aligned(ctx_tanh) &&
-                aligned(conv_tanh_outputs) && aligned(conv_errors), "wavenet_block_errors: buffers must be 16-byte aligned");
-    ProfileScope prof(stream, "wavenet_block_errors");
-    hipLaunchKernelGGL(k, dim3((N + 63) / 64), dim3(256), 0, stream, a);
+    if (fold) {
+        CNT_REQUIRE(cnn_foldable(fold, R) && fold_weights && fold_deltas && aligned(fold_weights) && aligned(fold_deltas),
+                    "wavenet_block_errors: this convolution layer cannot be folded into the block");
+        const cnt_cnn_group &g = fold->groups[0];
+        const int P = fold->desc.P;
+        a.conv_ld = (2 * g.hw + 1) * P;
+        for (int tap = 0; tap < 2; ++tap) {
+            const int shift = -tap;  // taps at shift 0 and -1 (cnn_backward_errors_fan)
+            a.conv_w[tap] = fold_weights + (size_t)(g.col0 + g.hw + shift) * P;
+            a.conv_shift[tap] = -shift * g.dil * fold->desc.S;
+        }
+        a.conv_deltas = fold_deltas;
+    }
+    CNT_REQUIRE(aligned(skip_weights) && aligned(out_weights) && aligned(skip_errors) && aligned(total) &&
+                aligned(a.from_skip) && aligned(core_buf) && aligned(ctx_tanh) && aligned(conv_tanh_outputs) &&
+                aligned(conv_errors), "wavenet_block_errors: buffers must be 16-byte aligned");
+    ProfileScope prof(stream, fold ? "wavenet_block_errors+cnn" : "wavenet_block_errors");
+    if (fold) hipLaunchKernelGGL(k, dim3((N + 127) / 128), dim3(512), 0, stream, a);
+    else hipLaunchKernelGGL(k, dim3((N + 63) / 64), dim3(256), 0, stream, a);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
