@@ -406,6 +406,11 @@ int cnt_network_calculate_error(cnt_network *net, void *stream, float *loss_dev)
 int cnt_network_backward(cnt_network *net, void *stream);
 /* cnt_lstm_check for every LSTM layer. */
 int cnt_network_check(cnt_network *net, void *stream);
+/* cnt_lstm_set_wait_bounds for the LSTM layer at `layer_index` of the network (CNT_ERR_ARG for any other layer).  No
+ * counterpart in the reference; like that call it exists so that a test can force one layer's recursion to give up
+ * without any kernel hanging. */
+int cnt_network_set_wait_bounds(cnt_network *net, int layer_index, unsigned spin_limit, int poll_delay_backward,
+                                int poll_delay_forward);
 /* One optimizer step over all weights in a single launch (see cnt_opt_step; the network keeps the optimizer's
  * current updates, deltas, statistics and Adam's accumulated betas).  If a layer of the network file carries its
  * own "learningRate" (layers/TrainableLayer.cu:110-111), the step is one launch per trainable layer instead. */

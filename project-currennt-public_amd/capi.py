@@ -94,6 +94,7 @@ _SIGNATURES = {
     "cnt_lstm_backward_weights": (I, [VP, VP, VP, VP]),
     "cnt_lstm_backward_prev_errors": (I, [VP, VP, VP, VP]),
     "cnt_lstm_set_wait_bounds": (I, [VP, C.c_uint, I, I]),
+    "cnt_network_set_wait_bounds": (I, [VP, I, C.c_uint, I, I]),
     "cnt_lstm_state": (VP, [VP, I, I]),
     "cnt_lstm_weight_count": (C.c_long, [I, I, I]),
     "cnt_lstm_check": (I, [VP, VP]),
@@ -543,6 +544,10 @@ class Network:
 
     def check(self, stream=None):
         check(lib().cnt_network_check(self.handle, stream_ptr(stream)))
+
+    def set_wait_bounds(self, layer_index, spin_limit, poll_delay_backward, poll_delay_forward):
+        check(lib().cnt_network_set_wait_bounds(self.handle, layer_index, spin_limit, poll_delay_backward,
+                                                poll_delay_forward))
 
     def update(self, option, learning_rate, momentum, frac_length, stream=None):
         check(lib().cnt_network_update(self.handle, stream_ptr(stream), option, learning_rate, momentum, frac_length))

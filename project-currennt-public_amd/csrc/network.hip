@@ -1674,6 +1674,15 @@ int cnt_network_check(cnt_network *net, void *stream) {
     return status;
 }
 
+int cnt_network_set_wait_bounds(cnt_network *net, int layer_index, unsigned spin_limit, int poll_delay_backward,
+                                int poll_delay_forward) {
+    using namespace cnt;
+    CNT_REQUIRE(net, "network_set_wait_bounds: null handle");
+    CNT_REQUIRE(layer_index >= 0 && (size_t)layer_index < net->layers.size() && net->layers[(size_t)layer_index].lstm,
+                "network_set_wait_bounds: layer %d is not an LSTM layer", layer_index);
+    return cnt_lstm_set_wait_bounds(net->layers[(size_t)layer_index].lstm, spin_limit, poll_delay_backward, poll_delay_forward);
+}
+
 int cnt_network_update(cnt_network *net, void *stream_, int option, float learning_rate, float momentum,
                        float frac_length) {
     using namespace cnt;

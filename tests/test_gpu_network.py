@@ -101,6 +101,68 @@ def test_stacked_network_trains_like_the_oracle(option, momentum, overlap):
     net.close()
 
 
+def test_network_reports_a_later_lstm_layer_that_gave_up_and_keeps_the_weights():
+    """Failure handling at network level, forced from the host: the SECOND recurrent layer's recursions get a spin
+    limit of zero, the first layer's stay as they are.  Every kernel still ends normally; the failure is reported by
+    cnt_network_check (which looks at every recurrent layer) or by the call into the network that follows the failed
+    launch, the optimizer step of that pass does not touch the weights, and with the bounds restored the same network
+    handle trains on."""
+    import torch
+
+    print("network give-up case", flush=True)
+    capi = PC.pkg().capi
+    P, Q, S, T = 16, 5, 6, 40
+    specs = [{"name": "bl1", "type": "blstm", "size": 128, "bias": 1.0},
+             {"name": "bl2", "type": "blstm", "size": 512, "bias": 1.0},
+             {"name": "out", "type": "feedforward_identity", "size": Q, "bias": 1.0},
+             {"name": "postoutput", "type": "sse", "size": Q}]
+    doc = {"layers": [{"size": P, "name": "input", "type": "input"}] + specs}
+    net = capi.Network(json.dumps(doc), S, T)
+    rng = np.random.default_rng(8)
+    net.weights.copy_(torch.from_numpy(rng.uniform(-0.1, 0.1, net.n_weights).astype(np.float32)))
+    pat = torch.full((T * S,), 2, dtype=torch.int8, device="cuda")
+    x = PC.dev(rng.standard_normal(T * S * P).astype(np.float32))
+    tgt = PC.dev(rng.standard_normal(T * S * Q).astype(np.float32))
+
+    def one_pass():
+        net.load_sequences(pat, T, T, x, tgt)
+        net.forward()
+        net.backward()
+        net.update(0, 1e-3, 0.0, float(T * S))
+        net.check()
+
+    one_pass()
+    torch.cuda.synchronize()
+    before = net.weights.clone()
+    second = [i for i, L in enumerate(net.layers) if L["type"] == "blstm"][1]
+    with pytest.raises(RuntimeError):
+        net.set_wait_bounds(0, 0, 0, 0)  # the input layer is not a recurrent layer
+    net.set_wait_bounds(second, 0, 0, 0)
+    failures = 0
+    for _ in range(3):  # an attempt only fails if some poll really comes back incomplete
+        try:
+            one_pass()
+        except RuntimeError as e:
+            assert "gave up" in str(e)
+            failures += 1
+            torch.cuda.synchronize()
+            try:
+                net.check()  # a second failed launch of the same attempt may have ended meanwhile
+            except RuntimeError:
+                pass
+            # the pass that failed did not reach the weights
+            assert torch.equal(net.weights, before)
+            break
+        before = net.weights.clone()  # a pass in which every poll happened to succeed is an ordinary pass
+    assert failures >= 1
+    net.set_wait_bounds(second, 1 << 22, 28, 34)
+    one_pass()
+    torch.cuda.synchronize()
+    assert not torch.equal(net.weights, before)
+    assert bool(torch.isfinite(net.weights).all())
+    net.close()
+
+
 # the last case has channel counts that are not multiples of four: no 16-byte accesses anywhere, and the skip layers'
 # backward steps run as launches of their own instead of in the epilogue of the following layer's product
 # The fifth case is a stack with benchmark config 4's layer sizes (64 residual / 128 skip channels, 80 conditioning
