@@ -224,7 +224,9 @@ bool cnn_foldable(const cnt_cnn *h, int R);
 int wavenet_block_errors(hipStream_t stream, int R, int K, int N, const char *patTypes, const float *skip_weights,
                          const float *out_weights, const float *skip_errors, float *total, const FanOut *fan,
                          const float *core_buf, float *ctx_tanh, const float *conv_tanh_outputs, float *conv_errors,
-                         const cnt_cnn *fold, const float *fold_weights, const float *fold_deltas);
+                         const cnt_cnn *fold, const float *fold_weights, const float *fold_deltas, float *colsum_partial);
+// workgroups of that launch = rows of `colsum_partial` ([rows][2R]: per-workgroup sums of conv_errors over the samples)
+int wavenet_block_rows(int N, bool fold);
 int wavnetc_context_grad(hipStream_t stream, int D, int C, int N, const float *weights, const float *ctx_tanh,
                          float *ctx_grad);
 int cnn_backward_errors_fan(cnt_cnn *h, hipStream_t stream, const char *patTypes, int curT, const float *weights,
@@ -245,7 +247,8 @@ int wavnetc_backward_weights_batch(hipStream_t stream, int D, int C, int N, int 
 int cnn_batch_taps(const cnt_cnn *h);
 bool cnn_batch_compatible(const cnt_cnn *a, const cnt_cnn *b);
 int cnn_backward_weights_batch(cnt_cnn *const *h, int count, hipStream_t stream, const char *patTypes, int curT,
-                               const float *const *x, const float *const *output_errors, float *const *weight_updates);
+                               const float *const *x, const float *const *output_errors, float *const *weight_updates,
+                               const float *const *colsum_partial = nullptr, const int *colsum_rows = nullptr);
 
 // ----- small streaming kernels (elementwise.hip) ----------------------------------------------------
 int fill_zero(hipStream_t stream, float *p, size_t count);

@@ -376,7 +376,6 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
         wait_all_vmem();
         const bool failed = __builtin_amdgcn_ballot_w64(!ok) != 0;  // only this wave ever gives up
         if (failed) wait_failed = 1;
-        const long long tk2 = timing ? wall_clock64() : 0;
         lds_barrier();
         if (failed) {
             if (lane == 0) raise_abort(p);

@@ -218,6 +218,8 @@ struct NetLayer {
     int cnn_tanh = 0;                        // cnn: "tanhoutput"
     bool delta_fused = false;                // cnn followed by a wavnetc layer: that layer writes this layer's delta
     bool fold_ok = false;                    // cnn whose error product can ride in the launch of the block below it
+    float *colsum = nullptr;                 // cnn in front of a wavnetc layer: per-workgroup sums of its deltas ([rows][size])
+    int colsum_rows = 0;                     // rows written by this pass's block launch (0: none)
     const float *total = nullptr;            // skip layers: where the summed error stands after the layer's step
     bool needs_sum = false;                  // skip layers: errors += side buffer is not a no-op
     int live_targets = 0;                    // skip layers: sources that receive the sum through a launch
@@ -957,6 +959,14 @@ int finish_build(cnt_network *net, const json::Value *weights) {
             for (float *t : tgt[(size_t)y]) writers += t == ini.eskip ? 1 : 0;
         C.fold_ok = writers == 1;
     }
+    // a block launch leaves the sums of the convolution layer's deltas per workgroup (bias gradient without another
+    // pass over the deltas)
+    for (int i = 1; i + 1 < n_layers; ++i) {
+        NetLayer &C = net->layers[(size_t)i];
+        if (C.kind != K_CNN || net->layers[(size_t)i + 1].kind != K_WAVNETC || C.size != 2 * net->layers[(size_t)i + 1].size) continue;
+        const size_t rows = ((size_t)net->S * C.maxTr + 63) / 64;
+        CNT_TRY(device_alloc(net, (void **)&C.colsum, rows * C.size * sizeof(float), false));
+    }
     // pattern types of the lower time resolutions, one buffer per resolution
     for (auto &L : net->layers) {
         if (L.res == 1) continue;
@@ -1319,6 +1329,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     // weight halves of small layers are collected and handed over a few at a time, those of large layers at once.
     std::vector<char> fan_done(net->layers.size(), 0);
     std::vector<char> errors_done(net->layers.size(), 0);  // error step done by the block launch of a later layer
+    for (auto &L : net->layers) L.colsum_rows = 0;
     static const bool fuse_blocks = [] { const char *e = std::getenv("CNT_NET_FUSE_BLOCKS"); return !e || std::atoi(e) != 0; }();
     // WaveNet residual block seen from its skip 1x1 layer i: [cnn 2R][wavnetc R][dense R, identity][skipadd, shares
     // the following sum][skipini][dense K, identity (i)]
@@ -1399,6 +1410,8 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
         const float *in0[kGemmMaxProb], *in1[kGemmMaxProb];
         float *dW[kGemmMaxProb], bias[kGemmMaxProb];
         cnt_cnn *cnn[kGemmMaxProb];
+        const float *colsum[kGemmMaxProb];
+        int colsum_rows[kGemmMaxProb];
         const NetLayer &first = net->layers[g.layers[0]];
         for (int z = 0; z < count; ++z) {
             NetLayer &L = net->layers[g.layers[(size_t)z]];
@@ -1408,10 +1421,11 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
             in0[z] = g.kind == K_WAVNETC ? L.cth : prev.out;
             in1[z] = L.err;
             cnn[z] = L.cnn;
+            colsum[z] = L.colsum; colsum_rows[z] = L.colsum_rows;
         }
         g.layers.clear();
         if (g.kind == K_DENSE) return dense_backward_weights_batch(ws, g.a, g.b, g.n, count, bias, in0, in1, dW);
-        if (g.kind == K_CNN) return cnn_backward_weights_batch(cnn, count, ws, first.pat, first.T, in0, in1, dW);
+        if (g.kind == K_CNN) return cnn_backward_weights_batch(cnn, count, ws, first.pat, first.T, in0, in1, dW, colsum, colsum_rows);
         return wavnetc_backward_weights_batch(ws, g.a, g.b, g.n, count, net->ctx, in0, dW);
     };
     auto join_group = [&](size_t i) -> int {
@@ -1507,7 +1521,9 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                                                      prev_err, (wanted || fold) ? &block_fan : nullptr, wav.core,
                                                      wav.ctx_dim > 0 ? wav.cth : nullptr, cnn.delta_fused ? cnn.out : nullptr,
                                                      cnn.err, fold ? fold->cnn : nullptr,
-                                                     fold ? net->weights + fold->w_off : nullptr, fold ? fold->err : nullptr));
+                                                     fold ? net->weights + fold->w_off : nullptr, fold ? fold->err : nullptr,
+                                                     cnn.colsum));
+                        if (cnn.colsum) net->layers[i - 5].colsum_rows = wavenet_block_rows(N, fold != nullptr);
                         fan_done[i - 1] = 1;
                         errors_done[i - 3] = errors_done[i - 4] = 1;
                         goto weight_half_of_layer;

@@ -200,12 +200,13 @@ struct BlockErrArgs {
     int conv_ld;
     int conv_shift[2];           // tap q reads the delta of slot n + conv_shift[q]
     const float *conv_deltas;    // 2R x N deltas of that convolution layer
+    float *colsum;               // optional, [workgroups][2R]: this workgroup's sums of `deltas` over its samples
 };
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 template <int R, int K, bool CONV>
-__global__ __launch_bounds__(CONV ? 512 : 256, CONV ? 1 : 2) void wavenet_block_errors_kernel(const BlockErrArgs a) {
+__global__ __launch_bounds__(CONV ? 512 : 256, (CONV || K > 128) ? 1 : 2) void wavenet_block_errors_kernel(const BlockErrArgs a) {
     static_assert(R % 16 == 0 && K % 16 == 0 && R <= 128, "block geometry");
     constexpr int NT = CONV ? 512 : 256;  // the folded convolution's weights take 2 x 2R x R words of LDS more
     constexpr int RT = R / 16;  // channel tiles
@@ -213,7 +214,9 @@ __global__ __launch_bounds__(CONV ? 512 : 256, CONV ? 1 : 2) void wavenet_block_
     // A operands: [tile][j][lane = 16*quarter + channel in tile][i] = W[16j + 4*quarter + i][16*tile + channel]
     __shared__ __attribute__((aligned(16))) float w1[RT * KJ * 64 * 4];
     __shared__ __attribute__((aligned(16))) float w2[RT * RJ * 64 * 4];
-    __shared__ __attribute__((aligned(16))) float wc[CONV ? 2 * RT * CJ * 64 * 4 : 4];
+    // one tap of the folded convolution at a time: with both taps the workgroup would hold 112 KB of the compute unit's
+    // 160 KB and nothing that wants 64 KB (a weight-gradient product on another stream) could run next to it
+    __shared__ __attribute__((aligned(16))) float wc[CONV ? RT * CJ * 64 * 4 : 4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int quarter = lane >> 4, col = lane & 15;
     const int n_raw = (blockIdx.x * (NT / 64) + wave) * 16 + col;
@@ -257,19 +260,21 @@ __global__ __launch_bounds__(CONV ? 512 : 256, CONV ? 1 : 2) void wavenet_block_
     // folded convolution: tap q contributes sum_d Wc[d][tap q][p] * delta[slot n + shift q][d], counted only where both
     // slots are inside the fraction and not padding (the rule of the convolution layer's own error product)
     float4 bc[CONV ? 2 : 1][CONV ? CJ : 1];
+    float4 sc1[FC > 0 ? FC : 1];  // the second tap's weights wait in registers until the first tap's products are done
     if (CONV) {
+        float4 sc0[FC > 0 ? FC : 1];
 #pragma unroll
-        for (int tap = 0; tap < 2; ++tap) {
-            float4 sc[FC > 0 ? FC : 1];
-#pragma unroll
-            for (int q = 0; q < FC; ++q) {
-                const int idx4 = q * NT + tid;
-                if (idx4 < TC) sc[q] = *reinterpret_cast<const float4 *>(a.conv_w[tap] + (size_t)(idx4 * 4 / R) * a.conv_ld + idx4 * 4 % R);
+        for (int q = 0; q < FC; ++q) {
+            const int idx4 = q * NT + tid;
+            if (idx4 < TC) {
+                const size_t at = (size_t)(idx4 * 4 / R) * a.conv_ld + idx4 * 4 % R;
+                sc0[q] = *reinterpret_cast<const float4 *>(a.conv_w[0] + at);
+                sc1[q] = *reinterpret_cast<const float4 *>(a.conv_w[1] + at);
             }
-#pragma unroll
-            for (int q = 0; q < FC; ++q)
-                if (q * NT + tid < TC) stage(wc + tap * (RT * CJ * 64 * 4), CJ, q * NT + tid, sc[q]);
         }
+#pragma unroll
+        for (int q = 0; q < FC; ++q)
+            if (q * NT + tid < TC) stage(wc, CJ, q * NT + tid, sc0[q]);
 #pragma unroll
         for (int tap = 0; tap < 2; ++tap) {
             const long long src = (long long)n + a.conv_shift[tap];
@@ -284,22 +289,14 @@ __global__ __launch_bounds__(CONV ? 512 : 256, CONV ? 1 : 2) void wavenet_block_
             }
         }
     }
-    // operands of the later phases are requested before the products start: the products then run while they arrive
-    float4 p1[RT], p2[RT], y1[RT], y2[RT], c1[RT], c2[RT], old0[RT];
+    // the gate's pre-activations and the first target's old values are requested before the products start
+    float4 p1[RT], p2[RT], old0[RT];
     const bool add_first = ok && a.fan_n > 0 && a.fan_is_skip[0] != 0;
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
         const size_t at = n * 2 * R + 16 * t + 4 * quarter;
         p1[t] = *reinterpret_cast<const float4 *>(a.pre + at);
         p2[t] = *reinterpret_cast<const float4 *>(a.pre + at + R);
-        if (a.conv_tanh) {
-            y1[t] = *reinterpret_cast<const float4 *>(a.conv_tanh + at);
-            y2[t] = *reinterpret_cast<const float4 *>(a.conv_tanh + at + R);
-        }
-        if (a.ctx_tanh) {
-            c1[t] = *reinterpret_cast<const float4 *>(a.ctx_tanh + at);
-            c2[t] = *reinterpret_cast<const float4 *>(a.ctx_tanh + at + R);
-        }
         if (add_first) old0[t] = *reinterpret_cast<const float4 *>(a.fan_targets[0] + n * R + 16 * t + 4 * quarter);
     }
     __syncthreads();
@@ -318,17 +315,35 @@ __global__ __launch_bounds__(CONV ? 512 : 256, CONV ? 1 : 2) void wavenet_block_
         }
         if (CONV) {
 #pragma unroll
-            for (int tap = 0; tap < 2; ++tap)
-#pragma unroll
-                for (int j = 0; j < CJ; ++j) {
-                    const float4 w = *reinterpret_cast<const float4 *>(&wc[(((tap * RT + t) * CJ + j) * 64 + lane) * 4]);
-                    acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, bc[tap][j].x, acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, bc[tap][j].y, acc1, 0, 0, 0);
-                    acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, bc[tap][j].z, acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.w, bc[tap][j].w, acc1, 0, 0, 0);
-                }
+            for (int j = 0; j < CJ; ++j) {
+                const float4 w = *reinterpret_cast<const float4 *>(&wc[((t * CJ + j) * 64 + lane) * 4]);
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, bc[0][j].x, acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, bc[0][j].y, acc1, 0, 0, 0);
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, bc[0][j].z, acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.w, bc[0][j].w, acc1, 0, 0, 0);
+            }
         }
         e[t] = acc0 + acc1;
+    }
+    if (CONV) {
+        __syncthreads();  // every wave is done with the first tap's weights
+#pragma unroll
+        for (int q = 0; q < FC; ++q)
+            if (q * NT + tid < TC) stage(wc, CJ, q * NT + tid, sc1[q]);
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            f32x4v acc0 = e[t], acc1 = {0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < CJ; ++j) {
+                const float4 w = *reinterpret_cast<const float4 *>(&wc[((t * CJ + j) * 64 + lane) * 4]);
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, bc[1][j].x, acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, bc[1][j].y, acc1, 0, 0, 0);
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, bc[1][j].z, acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.w, bc[1][j].w, acc1, 0, 0, 0);
+            }
+            e[t] = acc0 + acc1;
+        }
     }
     // the skip layer's step: add the side buffer, keep the sum, hand it on
     if (a.from_skip) {
@@ -377,6 +392,7 @@ __global__ __launch_bounds__(CONV ? 512 : 256, CONV ? 1 : 2) void wavenet_block_
     }
 
     // the gated unit (see gated_backward_kernel), four channels at a time
+    float4 cs1[RT], cs2[RT];  // what this lane writes to `deltas`, for the bias gradient of the convolution layer
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
         const size_t at = n * 2 * R + 16 * t + 4 * quarter;
@@ -392,22 +408,82 @@ __global__ __launch_bounds__(CONV ? 512 : 256, CONV ? 1 : 2) void wavenet_block_
         }
         float4 o1 = {g1[0], g1[1], g1[2], g1[3]}, o2 = {g2[0], g2[1], g2[2], g2[3]};
         if (a.conv_tanh) {
-            o1 = float4{tanh_deriv(y1[t].x) * g1[0], tanh_deriv(y1[t].y) * g1[1], tanh_deriv(y1[t].z) * g1[2], tanh_deriv(y1[t].w) * g1[3]};
-            o2 = float4{tanh_deriv(y2[t].x) * g2[0], tanh_deriv(y2[t].y) * g2[1], tanh_deriv(y2[t].z) * g2[2], tanh_deriv(y2[t].w) * g2[3]};
+            const float4 y1 = *reinterpret_cast<const float4 *>(a.conv_tanh + at);
+            const float4 y2 = *reinterpret_cast<const float4 *>(a.conv_tanh + at + R);
+            o1 = float4{tanh_deriv(y1.x) * g1[0], tanh_deriv(y1.y) * g1[1], tanh_deriv(y1.z) * g1[2], tanh_deriv(y1.w) * g1[3]};
+            o2 = float4{tanh_deriv(y2.x) * g2[0], tanh_deriv(y2.y) * g2[1], tanh_deriv(y2.z) * g2[2], tanh_deriv(y2.w) * g2[3]};
         }
         if (ok) {
             *reinterpret_cast<float4 *>(a.deltas + at) = o1;
             *reinterpret_cast<float4 *>(a.deltas + at + R) = o2;
         }
+        cs1[t] = ok ? o1 : float4{0.0f, 0.0f, 0.0f, 0.0f};
+        cs2[t] = ok ? o2 : float4{0.0f, 0.0f, 0.0f, 0.0f};
         if (a.ctx_tanh) {
-            const float4 q1 = {tanh_deriv(c1[t].x) * g1[0], tanh_deriv(c1[t].y) * g1[1], tanh_deriv(c1[t].z) * g1[2], tanh_deriv(c1[t].w) * g1[3]};
-            const float4 q2 = {tanh_deriv(c2[t].x) * g2[0], tanh_deriv(c2[t].y) * g2[1], tanh_deriv(c2[t].z) * g2[2], tanh_deriv(c2[t].w) * g2[3]};
+            const float4 c1 = *reinterpret_cast<const float4 *>(a.ctx_tanh + at);
+            const float4 c2 = *reinterpret_cast<const float4 *>(a.ctx_tanh + at + R);
+            const float4 q1 = {tanh_deriv(c1.x) * g1[0], tanh_deriv(c1.y) * g1[1], tanh_deriv(c1.z) * g1[2], tanh_deriv(c1.w) * g1[3]};
+            const float4 q2 = {tanh_deriv(c2.x) * g2[0], tanh_deriv(c2.y) * g2[1], tanh_deriv(c2.z) * g2[2], tanh_deriv(c2.w) * g2[3]};
             if (ok) {
                 *reinterpret_cast<float4 *>(a.ctx_tanh + at) = q1;
                 *reinterpret_cast<float4 *>(a.ctx_tanh + at + R) = q2;
             }
         }
     }
+    if (a.colsum) {
+        // sums over the wave's sixteen samples (lanes that share lane / 16), then over the workgroup's waves
+        __shared__ float csum[NT / 64][2 * R];
+        auto over_samples = [](float v) {
+            v += __shfl_xor(v, 1); v += __shfl_xor(v, 2); v += __shfl_xor(v, 4); v += __shfl_xor(v, 8);
+            return v;
+        };
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            const float4 u1 = {over_samples(cs1[t].x), over_samples(cs1[t].y), over_samples(cs1[t].z), over_samples(cs1[t].w)};
+            const float4 u2 = {over_samples(cs2[t].x), over_samples(cs2[t].y), over_samples(cs2[t].z), over_samples(cs2[t].w)};
+            if (col == 0) {
+                *reinterpret_cast<float4 *>(&csum[wave][16 * t + 4 * quarter]) = u1;
+                *reinterpret_cast<float4 *>(&csum[wave][R + 16 * t + 4 * quarter]) = u2;
+            }
+        }
+        __syncthreads();
+        if (tid < 2 * R) {
+            float v = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NT / 64; ++w) v += csum[w][tid];
+            a.colsum[(size_t)blockIdx.x * 2 * R + tid] = v;
+        }
+    }
+}
+
+// out[d] = scale * sum over rows of partial[row][d] (the second half of a column sum whose first half rode in
+// wavenet_block_errors_kernel); overwrites
+__global__ __launch_bounds__(256) void colsum_finish_kernel(const float *__restrict__ partial, int rows, int D, float scale,
+                                                            float *__restrict__ out) {
+    __shared__ float part[4][64];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int d = blockIdx.x * 64 + tx;
+    float acc0 = 0.0f, acc1 = 0.0f;
+    if (d < D) {
+        int r = ty;
+        for (; r + 4 < rows; r += 8) { acc0 += partial[(size_t)r * D + d]; acc1 += partial[(size_t)(r + 4) * D + d]; }
+        if (r < rows) acc0 += partial[(size_t)r * D + d];
+    }
+    part[ty][tx] = acc0 + acc1;
+    __syncthreads();
+    if (ty == 0 && d < D) out[d] = scale * ((part[0][tx] + part[1][tx]) + (part[2][tx] + part[3][tx]));
+}
+
+struct FillList {
+    float *ptr[kGemmMaxProb];
+    unsigned long long count[kGemmMaxProb];
+    int n;
+};
+// zeroes up to kGemmMaxProb small buffers in one launch (blockIdx.y = buffer)
+__global__ void fill_zero_list_kernel(const FillList f) {
+    float *p = f.ptr[blockIdx.y];
+    const size_t count = f.count[blockIdx.y];
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) p[i] = 0.0f;
 }
 
 typedef void (*block_err_kernel_t)(const BlockErrArgs);
@@ -643,7 +719,8 @@ extern "C++" bool cnt::cnn_batch_compatible(const cnt_cnn *a, const cnt_cnn *b) 
 
 extern "C++" int cnt::cnn_backward_weights_batch(cnt_cnn *const *h, int count, hipStream_t stream, const char *patTypes,
                                                  int curT, const float *const *x, const float *const *output_errors,
-                                                 float *const *weight_updates) {
+                                                 float *const *weight_updates, const float *const *colsum_partial,
+                                                 const int *colsum_rows) {
     CNT_REQUIRE(h && patTypes && x && output_errors && weight_updates && count >= 1, "cnn_backward_weights: null argument");
     const int taps = cnn_batch_taps(h[0]);
     CNT_REQUIRE(taps > 0 && count * taps <= kGemmMaxProb, "cnn_backward_weights: %d layers of %d taps in one launch", count,
@@ -657,7 +734,19 @@ extern "C++" int cnt::cnn_backward_weights_batch(cnt_cnn *const *h, int count, h
     const cnt_cnn_desc &d = h[0]->desc;
     const cnt_cnn_group &g0 = h[0]->groups[0];
     const int P = d.P, D = d.D, S = d.S, N = curT * S;
-    for (int z = 0; z < count; ++z) CNT_TRY(fill_zero(stream, weight_updates[z], (size_t)P * h[z]->Lw + D));
+    {
+        FillList fl = {};
+        size_t most = 0;
+        for (int z = 0; z < count; ++z) {
+            fl.ptr[z] = weight_updates[z];
+            fl.count[z] = (size_t)P * h[z]->Lw + D;
+            most = std::max(most, (size_t)fl.count[z]);
+        }
+        fl.n = count;
+        hipLaunchKernelGGL(fill_zero_list_kernel, dim3((unsigned)std::min<size_t>((most + 255) / 256, 256), count), dim3(256), 0,
+                           stream, fl);
+        CNT_HIP(hipGetLastError());
+    }
     GemmArgs ga = {};
     ga.m = P; ga.n = g0.d1 - g0.d0; ga.k = N;
     ga.a_kcontig = 0; ga.lda = P;
@@ -681,8 +770,17 @@ extern "C++" int cnt::cnn_backward_weights_batch(cnt_cnn *const *h, int count, h
     ga.overwrite_ok = 1;
     ga.label = "gemm:cnn_dW";
     CNT_TRY(gemm_launch(stream, ga));
-    for (int z = 0; z < count; ++z)
-        CNT_TRY(column_sum(stream, output_errors[z], D, N, h[z]->desc.bias, weight_updates[z] + (size_t)P * h[z]->Lw));
+    for (int z = 0; z < count; ++z) {
+        float *bias_grad = weight_updates[z] + (size_t)P * h[z]->Lw;
+        if (colsum_partial && colsum_partial[z] && colsum_rows[z] > 0) {
+            // the launch that wrote these deltas summed them per workgroup
+            hipLaunchKernelGGL(colsum_finish_kernel, dim3((D + 63) / 64), dim3(256), 0, stream, colsum_partial[z],
+                               colsum_rows[z], D, h[z]->desc.bias, bias_grad);
+            CNT_HIP(hipGetLastError());
+        } else {
+            CNT_TRY(column_sum(stream, output_errors[z], D, N, h[z]->desc.bias, bias_grad));
+        }
+    }
     return CNT_OK;
 }
 
@@ -800,6 +898,8 @@ int cnt_wavnetc_forward(void *stream_, int D, int C, int N, const char *patTypes
 
 extern "C++" bool cnt::wavenet_block_errors_supported(int R, int K) { return pick_block_errors_kernel(R, K, false) != nullptr; }
 
+extern "C++" int cnt::wavenet_block_rows(int N, bool fold) { return fold ? (N + 127) / 128 : (N + 63) / 64; }
+
 extern "C++" bool cnt::cnn_foldable(const cnt_cnn *h, int R) {
     // one run of filters, causal, two live taps, R inputs and 2R filters
     return h && h->groups.size() == 1 && h->desc.causal > 0 && h->groups[0].hw == 1 && h->groups[0].d0 == 0 &&
@@ -810,7 +910,7 @@ extern "C++" int cnt::wavenet_block_errors(hipStream_t stream, int R, int K, int
                                            const float *skip_weights, const float *out_weights, const float *skip_errors,
                                            float *total, const FanOut *fan, const float *core_buf, float *ctx_tanh,
                                            const float *conv_tanh_outputs, float *conv_errors, const cnt_cnn *fold,
-                                           const float *fold_weights, const float *fold_deltas) {
+                                           const float *fold_weights, const float *fold_deltas, float *colsum_partial) {
     block_err_kernel_t k = pick_block_errors_kernel(R, K, fold != nullptr);
     CNT_REQUIRE(k != nullptr, "wavenet_block_errors: no kernel for %d residual and %d skip channels", R, K);
     CNT_REQUIRE(N > 0 && patTypes && skip_weights && out_weights && skip_errors && total && core_buf && conv_errors,
@@ -820,6 +920,7 @@ extern "C++" int cnt::wavenet_block_errors(hipStream_t stream, int R, int K, int
     a.total = total;
     if (fan) { a.from_skip = fan->from_skip; a.fan_n = fan->n; a.fan_targets = fan->targets; a.fan_is_skip = fan->is_skip; }
     a.pre = core_buf; a.conv_tanh = conv_tanh_outputs; a.ctx_tanh = ctx_tanh; a.deltas = conv_errors;
+    a.colsum = colsum_partial;
     auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (fold) {
         CNT_REQUIRE(cnn_foldable(fold, R) && fold_weights && fold_deltas && aligned(fold_weights) && aligned(fold_deltas),
@@ -838,8 +939,7 @@ extern "C++" int cnt::wavenet_block_errors(hipStream_t stream, int R, int K, int
                 aligned(a.from_skip) && aligned(core_buf) && aligned(ctx_tanh) && aligned(conv_tanh_outputs) &&
                 aligned(conv_errors), "wavenet_block_errors: buffers must be 16-byte aligned");
     ProfileScope prof(stream, fold ? "wavenet_block_errors+cnn" : "wavenet_block_errors");
-    if (fold) hipLaunchKernelGGL(k, dim3((N + 127) / 128), dim3(512), 0, stream, a);
-    else hipLaunchKernelGGL(k, dim3((N + 63) / 64), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL(k, dim3(wavenet_block_rows(N, fold != nullptr)), dim3(fold ? 512 : 256), 0, stream, a);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
