@@ -34,7 +34,7 @@ import numpy as np  # noqa: E402
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a copy of known size; the figure and the command
 # that made it are in the profile named here.  Algorithmic bytes of the same launch: 120 MB.  None = not measured
 # for the kernel this tree runs.
-CHAIN_TRAFFIC_BYTES = None
+CHAIN_TRAFFIC_BYTES = 173.6e6  # (47 440 KiB x 2.00 fetched + 74 690 KiB written) per launch of lstm_backward_local<256, 8>
 CHAIN_TRAFFIC_SOURCE = "profiles/acoustic_backward_hbm_traffic.md"
 
 METRIC = "BLSTM backward frames/sec at 1 MI355X; % HBM/MFMA roofline vs host CPU"
