@@ -160,7 +160,12 @@ float *cnt_lstm_state(cnt_lstm *h, int dir, int which);
 long cnt_lstm_weight_count(int P, int L, int bidir);
 /* Waits for the stream and reports whether a recursion kernel of this handle gave up waiting for a
  * neighbouring workgroup (CNT_ERR_DEVICE; the results of that pass are invalid).  The reference has
- * no counterpart: its per-step launches cannot stall on each other. */
+ * no counterpart: its per-step launches cannot stall on each other.
+ * Failure contract of the handle: a recursion that gives up ends normally (no kernel hangs or faults) and latches
+ * the failure in host-visible memory.  It is returned, once, by this call or by the NEXT call of any kind into the
+ * same handle after the failed launch has ended (cnt_lstm_load_sequences, _forward, _backward*, ...), so a caller
+ * that never calls cnt_lstm_check still sees CNT_ERR_DEVICE, one call late.  The launch after that heals the
+ * handle's mailboxes; nothing has to be recreated. */
 int cnt_lstm_check(cnt_lstm *h, void *stream);
 
 /* ---- mixture-density post-output layer ----------------------------------------------------------
@@ -404,7 +409,11 @@ int cnt_network_calculate_error(cnt_network *net, void *stream, float *loss_dev)
  * the error computations they depend on; small layers of one shape share a launch.  On return the caller's stream
  * has been made to wait for those streams, so weight updates are complete in stream order. */
 int cnt_network_backward(cnt_network *net, void *stream);
-/* cnt_lstm_check for every LSTM layer. */
+/* cnt_lstm_check for every LSTM layer (all of them are looked at; the first failure is returned).  Failure contract
+ * of the network: a pass in which a recursion gave up cannot reach the weights -- the failed launch sets a device
+ * flag that the optimizer kernel of cnt_network_update reads, so even an update that was enqueued before the host
+ * could see the failure leaves weights and optimizer state untouched -- and CNT_ERR_DEVICE is returned by this call
+ * or by the next cnt_network_load_sequences / _forward / _backward / _update after the failed launch has ended. */
 int cnt_network_check(cnt_network *net, void *stream);
 /* cnt_lstm_set_wait_bounds for the LSTM layer at `layer_index` of the network (CNT_ERR_ARG for any other layer).  No
  * counterpart in the reference; like that call it exists so that a test can force one layer's recursion to give up
