@@ -256,7 +256,9 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
             lds_barrier();  // the deltas of this step are in LDS
             // looked at only at the end of the step: the read is in flight behind the barrier together with the
             // deltas', and what a failed step publishes no longer matters
-            const int failed = *const_cast<volatile int *>(&wait_failed);
+            // read through the LDS address space: a volatile read through a generic pointer becomes a flat load, which
+            // takes the vector-memory path
+            const int failed = *(__attribute__((address_space(3))) volatile int *)&wait_failed;
             if (tid == 64) trace_stamp(p, step, 3);
             const long long tp0 = timing ? wall_clock64() : 0;
             // everything this wave stored in the previous step (partial errors, resets) has reached the L2 before it
