@@ -88,8 +88,13 @@ def lstm_c1(args, pkg):
     dom = "lstm_backward_chain"
     flops = 8.0 * H * H * N
     ach = flops / (kernels[dom]["avg_ms"] * 1e-3) / 1e12
+    us_per_step = kernels[dom]["avg_ms"] * 1e3 / T
+    hop_us = capi.probe_hop_latency(same_xcd=True, with_compute=True, rounds=2000)
     roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_FP32_MFMA_TFLOPS,
-            "traffic": None, "kernel": dom, "note": "latency-bound recursion (T sequential steps)"}
+            "traffic": None, "kernel": dom, "us_per_step": us_per_step, "latency_floor_us_per_step": hop_us,
+            "frac_of_latency_floor": hop_us / us_per_step,
+            "note": "latency-bound recursion (T sequential steps, one job of four sequences on one XCD): `frac` is against the "
+                    "fp32 MFMA peak, `frac_of_latency_floor` against one measured hop inside an XCD plus a step's arithmetic"}
     extra = {"roofline": roof, "kernels": kernels}
     if not args.no_cpu:
         import oracle_lib as O  # the checker, only for this reported baseline

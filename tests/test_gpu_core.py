@@ -88,6 +88,40 @@ def test_lstm_clip_and_repeat_backward():
     assert PC.run_lstm_case(24, 128, True, [10, 6, 10], seed=5, wscale=0.5, escale=20.0, repeat_backward=True) < TOL
 
 
+def test_weight_gradients_spread_between_runs():
+    """The weight gradients are summed with fp32 atomics or per-split partial sums, so their bits may depend on the
+    order in which workgroups finish.  Three passes over the same inputs: the layer's errors must be bit-identical
+    (the recursion and the error products have a fixed summation order), the weight gradients within 1e-5
+    L2-normalised of each other (the parity tolerance against the oracle is 1e-4)."""
+    import numpy as np
+    import torch
+
+    print("lstm run-to-run spread", flush=True)
+    capi = PC.pkg().capi
+    P, L, S, T = 96, 512, 10, 160
+    rng = np.random.default_rng(11)
+    lengths = [int(v) for v in rng.integers(80, T + 1, size=S)]
+    lengths[0] = T
+    W, x, outerr = PC.lstm_inputs(P, L, True, S, T, lengths, 1)
+    pat = PC.make_pat_types(lengths, T)
+    Wd, xd, pd, ed = PC.dev(W), PC.dev(x), PC.dev(pat), PC.dev(outerr)
+    out = torch.zeros(L * T * S, device="cuda")
+    layer = capi.Lstm(P, L, True, S, T)
+    runs = []
+    for _ in range(3):
+        ex = torch.zeros(P * T * S, device="cuda"); dW = torch.zeros_like(Wd)
+        layer.load_sequences(pd, T, min(lengths))
+        layer.forward(Wd, xd, out)
+        layer.backward(Wd, xd, out, ed.clone(), ex, dW)
+        layer.check()
+        torch.cuda.synchronize()
+        runs.append((ex.cpu().numpy().copy(), dW.cpu().numpy().copy()))
+    layer.close()
+    for ex, dW in runs[1:]:
+        assert np.array_equal(ex, runs[0][0])
+        assert PC.relerr(dW, runs[0][1]) < 1e-5
+
+
 def test_lstm_config1_unidirectional():
     """benchmark config 1: P=382, H=256, T=200, S=4 with one sequence of 150 frames."""
     print("lstm config 1", flush=True)
