@@ -197,6 +197,8 @@ int opt_step_guarded(hipStream_t stream, int option, long n, float *weights, con
 void lstm_set_veto(cnt_lstm *h, int *veto);
 // non-zero if a recursion of this handle has given up since the last report (no synchronisation: it only sees
 // launches that have already ended); the report clears the mark
+// cnt_lstm_backward_weights in two parts that write disjoint ranges (1: input weights, 2: the rest)
+int lstm_backward_weights_parts(cnt_lstm *h, hipStream_t stream, const float *x, float *weight_updates, int parts);
 int lstm_take_failure(cnt_lstm *h);
 int report_failure(cnt_network *net);
 

@@ -1618,21 +1618,31 @@ int cnt_lstm_backward_prev_errors(cnt_lstm *h, void *stream_, const float *weigh
     return CNT_OK;
 }
 
-int cnt_lstm_backward_weights(cnt_lstm *h, void *stream_, const float *x, float *weight_updates) {
-    using namespace cnt;
+int cnt_lstm_backward_weights(cnt_lstm *h, void *stream, const float *x, float *weight_updates) {
+    return cnt::lstm_backward_weights_parts(h, static_cast<hipStream_t>(stream), x, weight_updates, 3);
+}
+
+// parts: 1 = input weights, 2 = bias, recurrent and peephole weights; the two parts write disjoint ranges of the
+// weight updates and may run on different streams
+extern "C++" int cnt::lstm_backward_weights_parts(cnt_lstm *h, hipStream_t stream, const float *x, float *weight_updates,
+                                                  int parts) {
     CNT_REQUIRE(h && x && weight_updates, "lstm_backward_weights: null argument");
     CNT_REQUIRE(h->T > 0, "lstm_backward_weights: load_sequences has not been called");
     CNT_LSTM_REPORT_FAILURE(h);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
     const cnt_lstm_desc &d = h->desc;
     const int P = d.P, L = d.L, H = h->H, S = d.S, N = h->T * S;
 
     // 3. weight updates (overwritten every call, as the reference's transform-assign does)
     const size_t nW = weight_count(P, L, d.bidir);
-    CNT_TRY(fill_zero(stream, weight_updates, nW));
     const size_t off_bias = (size_t)4 * P * L, off_int = off_bias + (size_t)4 * L;
     const size_t off_peep = off_int + (size_t)4 * L * H;
-    {
+    if ((parts & 3) == 3) {
+        CNT_TRY(fill_zero(stream, weight_updates, nW));
+    } else {
+        if (parts & 1) CNT_TRY(fill_zero(stream, weight_updates, off_bias));
+        if (parts & 2) CNT_TRY(fill_zero(stream, weight_updates + off_bias, nW - off_bias));
+    }
+    if (parts & 1) {
         // input weights: dW_in[g,dir] (P x H) = x (P x N) * delta^T
         GemmArgs ga = {};
         ga.m = P; ga.n = H; ga.k = N;
@@ -1651,6 +1661,7 @@ int cnt_lstm_backward_weights(cnt_lstm *h, void *stream_, const float *x, float 
         ga.label = "gemm:lstm_dW_input";
         CNT_TRY(gemm_launch(stream, ga));
     }
+    if (!(parts & 2)) return CNT_OK;
     if (h->T > 1) {
         // recurrent weights: dW_int[g,dir][src + to*H] = sum h[src] at the earlier step * delta[to]
         GemmArgs ga = {};
