@@ -817,7 +817,8 @@ struct GuardParams {
     unsigned *mail[3];
     size_t words[3];
 };
-__global__ __launch_bounds__(1024) void chain_guard(const GuardParams g) {
+// the work of one workgroup (any size)
+__device__ __forceinline__ void guard_body(const GuardParams &g) {
     const bool heal = __hip_atomic_load(g.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
     if (heal) {
         for (int m = 0; m < 3; ++m)
@@ -827,6 +828,7 @@ __global__ __launch_bounds__(1024) void chain_guard(const GuardParams g) {
     __syncthreads();
     if (heal && threadIdx.x == 0) __hip_atomic_store(g.abort_flag, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__global__ __launch_bounds__(1024) void chain_guard(const GuardParams g) { guard_body(g); }
 
 // ---------------------------------------------------------------------------------------------------
 // Bias and peephole gradients: per (direction, gate, cell) sums over all patterns
@@ -1138,7 +1140,8 @@ struct WarmParams {
     int count;
 };
 
-__global__ __launch_bounds__(256) void warm_cache(const WarmParams w) {
+__global__ __launch_bounds__(256) void warm_cache(const WarmParams w, const GuardParams g) {
+    if (blockIdx.x == 0) guard_body(g);  // the guard in front of the recursion rides along (a launch less)
     const size_t first = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 16, pitch = (size_t)gridDim.x * blockDim.x * 16;
     for (int a = 0; a < w.count; ++a) {
         const char *base = static_cast<const char *>(w.ptr[a]);
@@ -1149,7 +1152,7 @@ __global__ __launch_bounds__(256) void warm_cache(const WarmParams w) {
     }
 }
 
-int warm_backward_inputs(const cnt_lstm *h, hipStream_t stream, const ChainParams &p) {
+int warm_backward_inputs(const cnt_lstm *h, hipStream_t stream, const ChainParams &p, const GuardParams &g) {
     WarmParams w = {};
     const size_t state_bytes = (size_t)h->T * p.S * p.H * sizeof(float);
     auto add = [&](const void *ptr, size_t bytes) {
@@ -1162,7 +1165,7 @@ int warm_backward_inputs(const cnt_lstm *h, hipStream_t stream, const ChainParam
     }
     add(p.outerr, (size_t)h->T * p.S * p.L * sizeof(float));
     ProfileScope prof(stream, "lstm_warm_states");
-    hipLaunchKernelGGL(warm_cache, dim3(2048), dim3(256), 0, stream, w);
+    hipLaunchKernelGGL(warm_cache, dim3(2048), dim3(256), 0, stream, w, g);
     CNT_HIP(hipGetLastError());
     return CNT_OK;
 }
@@ -1179,14 +1182,16 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     int local_jb = 0;
     chain_kernel_t k = local ? pick_local_kernel(h->H, local_jb) : pick_kernel(fwd, h->H, h->JB, h->NT);
     CNT_REQUIRE(k != nullptr, "lstm: no recursion kernel for H=%d JB=%d S=%d", h->H, h->JB, h->desc.S);
-    {
-        // heals the handle after a launch that gave up, zeroes the placement counters
-        GuardParams g = {};
-        g.abort_flag = h->abort_flag;
-        g.ctl = h->ctl; g.nctl = h->ctl ? kCtlWords : 0;
-        g.mail[0] = reinterpret_cast<unsigned *>(h->bmail[0]); g.words[0] = h->bmail[0] ? h->bmail_words : 0;
-        g.mail[1] = reinterpret_cast<unsigned *>(h->bmail[1]); g.words[1] = h->bmail[1] ? h->bmail_words : 0;
-        g.mail[2] = reinterpret_cast<unsigned *>(h->lmail); g.words[2] = h->lmail ? h->lmail_words : 0;
+    // heals the handle after a launch that gave up, zeroes the placement counters; in front of the XCD-local backward
+    // recursion it is part of the cache-warming launch
+    GuardParams g = {};
+    g.abort_flag = h->abort_flag;
+    g.ctl = h->ctl; g.nctl = h->ctl ? kCtlWords : 0;
+    g.mail[0] = reinterpret_cast<unsigned *>(h->bmail[0]); g.words[0] = h->bmail[0] ? h->bmail_words : 0;
+    g.mail[1] = reinterpret_cast<unsigned *>(h->bmail[1]); g.words[1] = h->bmail[1] ? h->bmail_words : 0;
+    g.mail[2] = reinterpret_cast<unsigned *>(h->lmail); g.words[2] = h->lmail ? h->lmail_words : 0;
+    const bool guard_rides = local && !fwd && h->warm && !(h->bmail_dirty && h->lmail);
+    if (!guard_rides) {
         hipLaunchKernelGGL(chain_guard, dim3(1), dim3(1024), 0, stream, g);
         CNT_HIP(hipGetLastError());
     }
@@ -1200,7 +1205,11 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     if (!fwd && h->bmail_dirty && h->lmail) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->lmail), h->lmail_words, kEmpty));
     if (!fwd) h->bmail_dirty = 0;
     h->last_was_forward = fwd ? 1 : 0;
-    if (local && h->warm) CNT_TRY(warm_backward_inputs(h, stream, p));
+    if (local && h->warm) {
+        GuardParams none = {};
+        none.abort_flag = h->abort_flag;  // with nothing to zero or refill the body only reads the flag
+        CNT_TRY(warm_backward_inputs(h, stream, p, guard_rides ? g : none));
+    }
     ProfileScope prof(stream, fwd ? "lstm_forward_chain" : "lstm_backward_chain");
     if (local) {
         // enough workgroups that njobs complete teams form on any spread over the XCDs
