@@ -71,9 +71,9 @@ def run(args, pkg):
     if dom == "wavenet_block_errors+cnn":
         # one residual block's error path: reads the skip errors (K), what the later block handed on (R), the deltas of
         # the convolution above (2R, both taps from the same array), the gate pre-activations, the convolution's tanh
-        # outputs and the conditioning tanh (2R each); writes the block's summed errors (R), adds them to the earlier
-        # block's side buffer (R read + R write), writes the convolution deltas and the conditioning gradient (2R each)
-        nbytes = ((K + R + 4 * 2 * R) + (R + 2 * R + 2 * 2 * R)) * 4.0 * N
+        # outputs and the conditioning tanh (2R each); writes the block's summed errors (R, which the earlier block's
+        # launch reads where they stand), the convolution deltas and the conditioning gradient (2R each)
+        nbytes = ((K + R + 4 * 2 * R) + (R + 2 * 2 * R)) * 4.0 * N
     elif dom == "gemm:cnn_dW":
         # per launch: read x (R) and the deltas (2R) for each of the two live taps, write nothing of size N
         nbytes = 2 * (R + 2 * R) * 4.0 * N

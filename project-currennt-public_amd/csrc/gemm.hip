@@ -196,7 +196,12 @@ void gemm_plan(GemmArgs &args, hipStream_t stream) {
     // `target` workgroups of 64 x 64 tiles, but leave every workgroup at least eight k-iterations -- each
     // one ends with an atomic add (or a store) of its whole tile, and those, not the products, dominate short
     // ranges.
-    static const int target = [] { const char *e = std::getenv("CNT_GEMM_SPLIT_TARGET"); return e ? std::atoi(e) : 512; }();
+    // Outputs of one or two tiles per problem (the WaveNet layers' 64 x 64 ... 80 x 128 weights) take twice the
+    // workgroups: measured on MI355X next to the error chain of the same pass, 1024 workgroups end the stack's backward
+    // pass 4% sooner than 512, and 1536 or more (where the partial products no longer fit the scratch buffer and the
+    // launch adds atomically) 4-8% later; the acoustic model's wide outputs are best at 512.
+    static const int forced_target = [] { const char *e = std::getenv("CNT_GEMM_SPLIT_TARGET"); return e ? std::atoi(e) : 0; }();
+    const int target = forced_target > 0 ? forced_target : ((long)args.m * args.n <= 16384 ? 1024 : 512);
     const long tiles = (long)((args.m + 63) / 64) * ((args.n + 63) / 64) * args.nprob;
     const long kt = ((long)args.k + BK - 1) / BK * args.nseg;
     long s = (target + tiles - 1) / tiles;

@@ -218,6 +218,7 @@ struct NetLayer {
     int cnn_tanh = 0;                        // cnn: "tanhoutput"
     bool delta_fused = false;                // cnn followed by a wavnetc layer: that layer writes this layer's delta
     bool fold_ok = false;                    // cnn whose error product can ride in the launch of the block below it
+    bool direct_ok = false;                  // ... and the block above hands its sum to nothing but that launch
     float *colsum = nullptr;                 // cnn in front of a wavnetc layer: per-workgroup sums of its deltas ([rows][size])
     int colsum_rows = 0;                     // rows written by this pass's block launch (0: none)
     const float *total = nullptr;            // skip layers: where the summed error stands after the layer's step
@@ -958,6 +959,17 @@ int finish_build(cnt_network *net, const json::Value *weights) {
         for (int y = 0; y < n_layers; ++y)
             for (float *t : tgt[(size_t)y]) writers += t == ini.eskip ? 1 : 0;
         C.fold_ok = writers == 1;
+        // The closing layer's side buffer has one writer too, the skipini layer of the block above (layer i+4), which
+        // hands its sum to nothing else: the block below can then read that sum where it stands, and the copy into the
+        // side buffer is left out.
+        if (!C.fold_ok || i + 4 >= n_layers) continue;
+        const NetLayer &above = net->layers[(size_t)i + 4];
+        if (above.kind != K_SKIPINI || !above.total || above.total != above.err) continue;
+        if (tgt[(size_t)i + 4].size() != 1 || tgt[(size_t)i + 4][0] != closing.eskip || !flag[(size_t)i + 4][0]) continue;
+        writers = 0;
+        for (int y = 0; y < n_layers; ++y)
+            for (float *t : tgt[(size_t)y]) writers += t == closing.eskip ? 1 : 0;
+        C.direct_ok = writers == 1;
     }
     // a block launch leaves the sums of the convolution layer's deltas per workgroup (bias gradient without another
     // pass over the deltas)
@@ -1334,6 +1346,8 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     // WaveNet residual block seen from its skip 1x1 layer i: [cnn 2R][wavnetc R][dense R, identity][skipadd, shares
     // the following sum][skipini][dense K, identity (i)]
     std::vector<int> fold_from(net->layers.size(), -1);  // skip 1x1 layer -> convolution layer folded into its launch
+    std::vector<const float *> direct_from(net->layers.size(), nullptr);  // skip 1x1 layer -> the block above's sum
+    static const bool direct_sums = [] { const char *e = std::getenv("CNT_NET_DIRECT_SUMS"); return !e || std::atoi(e) != 0; }();
     auto block_at = [&](size_t i) {
         if (!fuse_blocks || i < 5) return false;
         const NetLayer &sk = net->layers[i], &ini = net->layers[i - 1], &add = net->layers[i - 2], &out = net->layers[i - 3];
@@ -1529,9 +1543,19 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                         FanOut block_fan = fan;
                         // with a folded convolution, what the later block handed to the closing skipadd layer comes in
                         // directly (that layer would have added it to the convolution's product and handed the sum on)
-                        if (fold) block_fan.from_skip = net->layers[(size_t)fold_from[i] - 1].eskip;
+                        if (fold)
+                            block_fan.from_skip = direct_from[i] ? direct_from[i] : net->layers[(size_t)fold_from[i] - 1].eskip;
+                        // the block below folds this block's convolution in and is this sum's only reader: it reads
+                        // the sum where this launch leaves it, nothing is handed on
+                        if (direct_sums && wanted && cnn.direct_ok && fold_at(i - 5)) {
+                            block_fan.n = 0;
+                            block_fan.targets = nullptr;
+                            block_fan.is_skip = nullptr;
+                            direct_from[i - 8] = prev_err;
+                        }
+                        const bool fan_live = block_fan.n > 0 || block_fan.from_skip;
                         CNT_TRY(wavenet_block_errors(stream, prev.size, L.size, N, L.pat, W, net->weights + out.w_off, L.err,
-                                                     prev_err, (wanted || fold) ? &block_fan : nullptr, wav.core,
+                                                     prev_err, fan_live ? &block_fan : nullptr, wav.core,
                                                      wav.ctx_dim > 0 ? wav.cth : nullptr, cnn.delta_fused ? cnn.out : nullptr,
                                                      cnn.err, fold ? fold->cnn : nullptr,
                                                      fold ? net->weights + fold->w_off : nullptr, fold ? fold->err : nullptr,
