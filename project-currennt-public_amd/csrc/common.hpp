@@ -166,6 +166,7 @@ struct GemmArgs {
     const int *fan_is_skip;
     float *partial;        // scratch of splitk * partial_stride floats: the stream's buffer (set by gemm_plan) or the caller's
     size_t partial_stride;  // floats per split: nprob * m * n (+ nprob * n with rowsum)
+    int xcd_map;            // set by gemm_launch: workgroups pick their tile by XCD (gemm_kernel.hpp)
 };
 
 // Resolves splitk = 0 (chosen by the launcher) and, where the arguments allow it and it pays, switches an

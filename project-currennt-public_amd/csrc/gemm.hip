@@ -256,6 +256,14 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
     const int tile = pick_tile(args);
     const int tiles = ((args.m + tile - 1) / tile) * ((args.n + tile - 1) / tile);
     dim3 grid(tiles, args.splitk, args.nprob);
+    // XCD-aware placement (gemm_kernel.hpp) for launches of several problems: measured with FETCH_SIZE on MI355X it
+    // cuts what the L2s fetch 2.2-2.6x for the WaveNet stack's batched weight gradients (a convolution's two taps and
+    // a stack's conditioning projections share an operand) and ends that pass 0.5% sooner.  For one problem per launch
+    // it cuts the fetches 2-4x as well (the acoustic model's weight gradients: 270 -> 68 MB) and the products run 1%
+    // faster, but that model's pass came out 0.7% slower in every run, so single problems keep the launch order
+    // (CNT_GEMM_XCD_MAP=2 maps them too, 0 maps nothing).
+    static const int xcd_map = [] { const char *e = std::getenv("CNT_GEMM_XCD_MAP"); return e ? std::atoi(e) : 1; }();
+    args.xcd_map = (xcd_map == 2 || (xcd_map == 1 && args.nprob > 1)) && (long)tiles * args.splitk * args.nprob >= 16 ? 1 : 0;
     ProfileScope prof(stream, args.label ? args.label : "gemm");
     std::unique_lock<std::mutex> split_lock(g_split_mu, std::defer_lock);
     // a product and its reduction stay adjacent on the stream

@@ -186,17 +186,36 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     const int wave = tid >> 6;
     const int wm = wave & 1, wn = wave >> 1;
 
+    // Which tile, k range and problem this workgroup takes.  Workgroups go to the eight XCDs in turn, in launch
+    // order, and each XCD has its own L2: the workgroups one XCD receives take CONSECUTIVE positions of the order
+    // (tile, problem, k range), with the tiles of one output walked in bands of eight rows of tiles.  What runs on one XCD
+    // at a time is then a compact block of tiles of one k range (its operand panels are fetched into that L2 once
+    // instead of once per XCD) and, for several problems per launch, the same k range of neighbouring problems
+    // (which share an operand where a layer's taps or a stack's layers read the same input).
     const int tiles_m = (args.m + BM - 1) / BM;
-    const int tile = blockIdx.x;
+    int tile = blockIdx.x, split_id = blockIdx.y, prob_id = blockIdx.z;
+    if (args.xcd_map) {
+        const unsigned total = gridDim.x * gridDim.y * gridDim.z;
+        const unsigned at = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const unsigned per = total / 8, rem = total % 8, xcd = at % 8, slot = at / 8;
+        const unsigned pos = xcd < rem ? xcd * (per + 1) + slot : rem * (per + 1) + (xcd - rem) * per + slot;
+        const unsigned in_output = pos % gridDim.x, rest = pos / gridDim.x;
+        prob_id = (int)(rest % gridDim.z);
+        split_id = (int)(rest / gridDim.z);
+        const int tiles_n = (int)gridDim.x / tiles_m;
+        const int band = (int)in_output / (8 * tiles_n), off = (int)in_output % (8 * tiles_n);
+        const int rows = min(tiles_m - 8 * band, 8);
+        tile = (8 * band + off % rows) + (off / rows) * tiles_m;
+    }
     const int m0 = (tile % tiles_m) * BM;
     const int n0 = (tile / tiles_m) * BN;
-    const GemmProblem &pb = args.prob[blockIdx.z];
+    const GemmProblem &pb = args.prob[prob_id];
 
     // iteration space: segments x k-tiles, cut into splitk contiguous ranges
     const int kt_per_seg = (args.k + BK - 1) / BK;
     const int total_it = kt_per_seg * args.nseg;
     const int per_split = (total_it + args.splitk - 1) / args.splitk;
-    const int it_begin = blockIdx.y * per_split;
+    const int it_begin = split_id * per_split;
     const int it_end = min(total_it, it_begin + per_split);
     if (it_begin >= it_end) return;
 
@@ -286,8 +305,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     const int half = lane >> 5;
     if (args.epilogue == EPI_PARTIAL) {
         // this split's partial product, m x n column-major without padding, after those of the problems before it
-        float *__restrict__ P = args.partial + (size_t)blockIdx.y * args.partial_stride +
-                                (size_t)blockIdx.z * args.m * args.n;
+        float *__restrict__ P = args.partial + (size_t)split_id * args.partial_stride +
+                                (size_t)prob_id * args.m * args.n;
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const int m = m0 + wm * WT + i * 32 + frag_row;
@@ -302,8 +321,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
             }
         }
         if (rowsum && wm == 0 && m0 == 0) {
-            float *__restrict__ R = args.partial + (size_t)blockIdx.y * args.partial_stride +
-                                    (size_t)args.nprob * args.m * args.n + (size_t)blockIdx.z * args.n;
+            float *__restrict__ R = args.partial + (size_t)split_id * args.partial_stride +
+                                    (size_t)args.nprob * args.m * args.n + (size_t)prob_id * args.n;
 #pragma unroll
             for (int j = 0; j < NB; ++j) {
                 const float s = rs[j] + __shfl_xor(rs[j], 32);
