@@ -68,6 +68,11 @@ def run(args, pkg):
     dom = max(kernels, key=lambda k: kernels[k]["ms_per_step"])
     step_flops = flops_per_sample(nb, Q, R, K, C) * N
     roof = {"bound": "hbm", "kernel": dom, "traffic": None, "peak": PEAK_HBM_GBS, "unit": "GB/s"}
+    if dom == "wavenet_block_errors+cnn" and (R, K, N) == (64, 128, 32000):
+        # two rocprofv3 --pmc runs (FETCH_SIZE x 2.00 by a copy of known size, WRITE_SIZE x 1.00) of this workload:
+        # 104.6 MB read + 55.5 MB written per launch of wavenet_block_errors_kernel<64, 128, true>
+        roof["traffic"] = 160.1e6
+        roof["traffic_source"] = "profiles/wavenet_c4_backward_kernel_stats.md"
     if dom == "wavenet_block_errors+cnn":
         # one residual block's error path: reads the skip errors (K), what the later block handed on (R), the deltas of
         # the convolution above (2R, both taps from the same array), the gate pre-activations, the convolution's tanh
