@@ -255,23 +255,25 @@ __global__ void mixture_error_kernel(UnitGeom g, const char *__restrict__ pat, c
 // component's means and deviations, so one load instruction of the wave covers 64 contiguous bytes of sixteen
 // components; the four partial sums meet through two DPP steps instead of one six-step wave reduction per component.
 // The log-sum over the components is max + log(sum exp(. - max)) over the wave (the reference's running log_add in
-// another order: terms below e^-69 of the largest drop out either way).  A wave takes several frames in turn and a
-// workgroup adds its frames' log-sums in LDS, so the single result word receives one atomic per 8 frames -- 6000
-// atomics on one address, which serialise, were what the previous kernel's time went to.
-constexpr int kErrFramesPerWave = 2;
-__global__ __launch_bounds__(256) void mixture_error_vec_kernel(UnitGeom g, const char *__restrict__ pat,
+// another order: terms below e^-69 of the largest drop out either way).  A wave takes one frame (a frame is one chain
+// of loads, reductions and transcendentals; two frames in turn per wave are 1-2 % slower), and the eight
+// waves of a workgroup add their frames' log-sums in LDS, so the single result word receives one atomic per 8
+// frames -- 6000 atomics on one address, which serialise, were what the first kernel's time went to.
+constexpr int kErrFramesPerWave = 1;
+constexpr int kErrWaves = 8;
+__global__ __launch_bounds__(64 * kErrWaves) void mixture_error_vec_kernel(UnitGeom g, const char *__restrict__ pat,
                                                                 const float *__restrict__ target,
                                                                 const float *__restrict__ para, float *__restrict__ tmp,
                                                                 float *__restrict__ result) {
-    __shared__ float lp_sh[4][64];
-    __shared__ float block_sum[4];
+    __shared__ float lp_sh[kErrWaves][64];
+    __shared__ float block_sum[kErrWaves];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int M = g.M, D = g.D, MD = M * D, DV = D / 4;
     const int p = lane & 3, ml = lane >> 2;  // lane (ml, p): component ml of the pass, quarter p
     const float gauss_const = (float)(D * log(2 * 3.141215) / 2.0);  // the reference's own value of pi
     float wave_total = 0.0f;
     for (int i = 0; i < kErrFramesPerWave; ++i) {
-        const int f = (blockIdx.x * 4 + wave) * kErrFramesPerWave + i;
+        const int f = (blockIdx.x * kErrWaves + wave) * kErrFramesPerWave + i;
         if (f >= g.F) break;
         if (pat[f] == 0) {
             for (int m = lane; m < M; m += 64) tmp[(size_t)f * M + m] = 0.0f;  // distance pass writes 0, the rest skips
@@ -287,12 +289,23 @@ __global__ __launch_bounds__(256) void mixture_error_vec_kernel(UnitGeom g, cons
             const int m = m0 + ml;
             float dist = 0.0f, logsd = 0.0f;
             if (m < M) {
-                for (int v = p; v < DV; v += 4) {
-                    const float4 s = sd4[m * DV + v], mu = mean4[m * DV + v], tv = t4[v];
-                    const float d0 = tv.x - mu.x, d1 = tv.y - mu.y, d2 = tv.z - mu.z, d3 = tv.w - mu.w;
-                    dist += d0 * d0 / (s.x * s.x) * 0.5f; dist += d1 * d1 / (s.y * s.y) * 0.5f;
-                    dist += d2 * d2 / (s.z * s.z) * 0.5f; dist += d3 * d3 / (s.w * s.w) * 0.5f;
-                    logsd += safe_log(s.x) + safe_log(s.y) + safe_log(s.z) + safe_log(s.w);
+                // sixteen vectors of a component per round, four per lane, all twelve loads of a lane requested
+                // before the first is used (a loop over v alone waits for memory once per vector)
+                for (int v0 = 0; v0 < DV; v0 += 16) {
+                    float4 s[4], mu[4], tv[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int v = min(v0 + p + 4 * q, DV - 1);
+                        s[q] = sd4[m * DV + v]; mu[q] = mean4[m * DV + v]; tv[q] = t4[v];
+                    }
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (v0 + p + 4 * q >= DV) continue;
+                        const float d0 = tv[q].x - mu[q].x, d1 = tv[q].y - mu[q].y, d2 = tv[q].z - mu[q].z, d3 = tv[q].w - mu[q].w;
+                        dist += d0 * d0 / (s[q].x * s[q].x) * 0.5f; dist += d1 * d1 / (s[q].y * s[q].y) * 0.5f;
+                        dist += d2 * d2 / (s[q].z * s[q].z) * 0.5f; dist += d3 * d3 / (s[q].w * s[q].w) * 0.5f;
+                        logsd += safe_log(s[q].x) + safe_log(s[q].y) + safe_log(s[q].z) + safe_log(s[q].w);
+                    }
                 }
             }
             // the four quarters of a component sit in one quad
@@ -325,7 +338,9 @@ __global__ __launch_bounds__(256) void mixture_error_vec_kernel(UnitGeom g, cons
     if (lane == 0) block_sum[wave] = wave_total;
     __syncthreads();
     if (threadIdx.x == 0) {
-        const float v = (block_sum[0] + block_sum[1]) + (block_sum[2] + block_sum[3]);
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kErrWaves; w += 2) v += block_sum[w] + block_sum[w + 1];
         if (v != 0.0f) atomicAdd(result, v);
     }
 }
@@ -593,8 +608,8 @@ int cnt_mdn_calculate_error(cnt_mdn *h, void *stream_, const float *targets, flo
             const bool vec4 = g.D % 4 == 0 && g.M % 4 == 0 && g.M <= 64 && g.Lt % 4 == 0 && g.startDOut % 4 == 0 &&
                               aligned(targets) && aligned(u.para);
             if (vec4) {
-                const int per_block = 4 * kErrFramesPerWave;
-                hipLaunchKernelGGL(mixture_error_vec_kernel, dim3((g.F + per_block - 1) / per_block), dim3(256), 0, stream, g,
+                const int per_block = kErrWaves * kErrFramesPerWave;
+                hipLaunchKernelGGL(mixture_error_vec_kernel, dim3((g.F + per_block - 1) / per_block), dim3(64 * kErrWaves), 0, stream, g,
                                    h->pat, targets, u.para, u.tmp, result_dev);
             } else {
                 const dim3 grid((g.F + kFramesPerBlock - 1) / kFramesPerBlock), block(64 * kFramesPerBlock);
