@@ -68,6 +68,8 @@ def test_sse():
     (32, 1024, True, [7, 5, 7]),
     (20, 256, False, [5] * 24),            # more than 16 parallel sequences with 256 cells
     (16, 128, True, [1, 1]),               # a single time step, two sequences
+    (24, 256, True, [7, 4, 7] * 6),        # 18 parallel sequences, bidirectional: the recursion that spans the XCDs
+    (24, 128, False, [3, 9, 1, 9, 2]),     # very ragged, one sequence of a single step among longer ones
     # geometries without a persistent recursion kernel: step-by-step recursion
     (12, 64, True, [30, 23]),              # 32 cells per direction (the reference example's conditioning BLSTM)
     (7, 20, False, [9, 4, 9]),             # 20 cells, sizes that are no multiple of anything
