@@ -171,6 +171,9 @@ def test_network_reports_a_later_lstm_layer_that_gave_up_and_keeps_the_weights()
 @pytest.mark.parametrize("nb,cnn_tanh,R,K,Q,C,lengths,cycle,upsample", [
     (4, 1, 32, 64, 64, 20, [120, 90], 3, 20), (11, 0, 32, 64, 64, 20, [120, 90], 3, 20),
     (3, 1, 30, 50, 64, 20, [120, 90], 3, 20),
+    # the other widths the fused block launch is built for
+    (3, 1, 64, 256, 64, 20, [70, 52], 3, 20), (3, 0, 64, 64, 64, 20, [70, 52], 3, 20),
+    (3, 1, 32, 128, 64, 20, [70, 52], 3, 20), (3, 0, 32, 32, 64, 20, [70, 52], 3, 20),
     (10, 1, 64, 128, 256, 80, [4000, 3300], 10, 80),
 ])
 def test_wavenet_network_file_against_oracle_graph(nb, cnn_tanh, R, K, Q, C, lengths, cycle, upsample):
