@@ -147,6 +147,22 @@ int cnt_lstm_backward_weights(cnt_lstm *h, void *stream, const float *x, float *
  * recursion; a caller can then start cnt_lstm_backward_weights on another stream as soon as the recursion is
  * done and compute the preceding layer's errors meanwhile. */
 int cnt_lstm_backward_prev_errors(cnt_lstm *h, void *stream, const float *weights, float *prev_errors);
+/* The same two pieces over a part of the fraction, for callers that overlap the end of a layer's recursion with the
+ * products that follow it (the reference runs the recursion step by step, layers/LstmLayer.cu:2136-2252, and the
+ * product over the whole fraction, :2298-2334; splitting either changes no result).
+ * cnt_lstm_backward_errors_range runs steps [step_begin, step_end) of the curMaxT steps of the recursion; the
+ * ranges of one pass must be launched in order on one stream, the first from step 0, and nothing else may use the
+ * handle in between.  Only where cnt_lstm_backward_can_split returns 1 (layers whose backward recursion runs as one
+ * persistent kernel per group of sequences); elsewhere it is an error.
+ * cnt_lstm_backward_steps_done: the time steps [t_begin, t_end) whose deltas are final once `steps` steps have run
+ * (both directions have passed them), i.e. what cnt_lstm_backward_prev_errors_range may already compute:
+ * prev_errors columns of the time steps [t_begin, t_end) only. */
+int cnt_lstm_backward_can_split(const cnt_lstm *h);
+int cnt_lstm_backward_errors_range(cnt_lstm *h, void *stream, const float *weights, float *output_errors,
+                                   int step_begin, int step_end);
+int cnt_lstm_backward_steps_done(const cnt_lstm *h, int steps, int *t_begin, int *t_end);
+int cnt_lstm_backward_prev_errors_range(cnt_lstm *h, void *stream, const float *weights, float *prev_errors,
+                                        int t_begin, int t_end);
 /* Device pointer to one internal buffer.  dir: 0 forward, 1 backward states.  which:
  * 0 niActs 1 igActs 2 fgActs 3 ogActs 4 cellStates 5 tmpOutputs 6 tmpOutputErrors
  * 7 niDeltas 8 igDeltas 9 fgDeltas 10 ogDeltas 11 cellStateErrors.  NULL if out of range. */

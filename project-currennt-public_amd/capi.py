@@ -93,6 +93,10 @@ _SIGNATURES = {
     "cnt_lstm_backward_errors": (I, [VP, VP, VP, VP, VP]),
     "cnt_lstm_backward_weights": (I, [VP, VP, VP, VP]),
     "cnt_lstm_backward_prev_errors": (I, [VP, VP, VP, VP]),
+    "cnt_lstm_backward_can_split": (I, [VP]),
+    "cnt_lstm_backward_errors_range": (I, [VP, VP, VP, VP, I, I]),
+    "cnt_lstm_backward_steps_done": (I, [VP, I, C.POINTER(I), C.POINTER(I)]),
+    "cnt_lstm_backward_prev_errors_range": (I, [VP, VP, VP, VP, I, I]),
     "cnt_lstm_set_wait_bounds": (I, [VP, C.c_uint, I, I]),
     "cnt_network_set_wait_bounds": (I, [VP, I, C.c_uint, I, I]),
     "cnt_lstm_state": (VP, [VP, I, I]),
@@ -367,6 +371,20 @@ class Lstm:
 
     def backward_prev_errors(self, W, prev_err, stream=None):
         check(lib().cnt_lstm_backward_prev_errors(self.handle, stream_ptr(stream), ptr(W), ptr(prev_err)))
+
+    def backward_can_split(self):
+        return bool(lib().cnt_lstm_backward_can_split(self.handle))
+
+    def backward_errors_range(self, W, outerr, step_begin, step_end, stream=None):
+        check(lib().cnt_lstm_backward_errors_range(self.handle, stream_ptr(stream), ptr(W), ptr(outerr), step_begin, step_end))
+
+    def backward_steps_done(self, steps):
+        a, b = I(0), I(0)
+        check(lib().cnt_lstm_backward_steps_done(self.handle, steps, C.byref(a), C.byref(b)))
+        return a.value, b.value
+
+    def backward_prev_errors_range(self, W, prev_err, t_begin, t_end, stream=None):
+        check(lib().cnt_lstm_backward_prev_errors_range(self.handle, stream_ptr(stream), ptr(W), ptr(prev_err), t_begin, t_end))
 
     def check(self, stream=None):
         check(lib().cnt_lstm_check(self.handle, stream_ptr(stream)))

@@ -72,6 +72,10 @@ struct ChainParams {
     struct { int dir, seq0, nseq; } job[8];
     unsigned *ctl;   // placement counters, zero at launch
     float *lmail;    // one mailbox per job
+    // XCD-local backward recursion over a range of its steps: [step_begin, step_end) of 0 .. T.  A launch that starts
+    // at a later step takes what the step before it left: the carried cell-state terms from the state arrays, the
+    // partial errors from the mailbox (which nothing may touch in between).
+    int step_begin, step_end;
 };
 
 // A workgroup that gives up: every workgroup of the launch sees the device flag and drains; the host sees the latch
@@ -1103,6 +1107,7 @@ void fill_chain_params(const cnt_lstm *h, const float *weights, ChainParams &p) 
     const int P = d.P, L = d.L, H = h->H;
     std::memset(&p, 0, sizeof(p));
     p.H = H; p.L = L; p.S = d.S; p.T = h->T; p.Tmin = h->Tmin; p.ndir = h->ndir; p.bias = d.bias;
+    p.step_begin = 0; p.step_end = h->T;
     p.pat = h->pat;
     const size_t off_bias = (size_t)4 * P * L, off_int = off_bias + (size_t)4 * L;
     const size_t off_peep = off_int + (size_t)4 * L * H;
@@ -1190,7 +1195,13 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     g.mail[0] = reinterpret_cast<unsigned *>(h->bmail[0]); g.words[0] = h->bmail[0] ? h->bmail_words : 0;
     g.mail[1] = reinterpret_cast<unsigned *>(h->bmail[1]); g.words[1] = h->bmail[1] ? h->bmail_words : 0;
     g.mail[2] = reinterpret_cast<unsigned *>(h->lmail); g.words[2] = h->lmail ? h->lmail_words : 0;
-    const bool guard_rides = local && !fwd && h->warm && !(h->bmail_dirty && h->lmail);
+    // a launch that continues a recursion in the middle: the counters are zeroed, nothing is refilled or warmed
+    const bool resumes = local && p.step_begin > 0;
+    CNT_REQUIRE(local || (p.step_begin == 0 && p.step_end == h->T), "lstm: only the XCD-local backward recursion runs a "
+                "range of steps");
+    CNT_REQUIRE(p.step_begin >= 0 && p.step_begin < p.step_end && p.step_end <= h->T, "lstm: steps %d..%d of %d",
+                p.step_begin, p.step_end, h->T);
+    const bool guard_rides = local && !fwd && h->warm && !resumes && !(h->bmail_dirty && h->lmail);
     if (!guard_rides) {
         hipLaunchKernelGGL(chain_guard, dim3(1), dim3(1024), 0, stream, g);
         CNT_HIP(hipGetLastError());
@@ -1205,7 +1216,7 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     if (!fwd && h->bmail_dirty && h->lmail) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->lmail), h->lmail_words, kEmpty));
     if (!fwd) h->bmail_dirty = 0;
     h->last_was_forward = fwd ? 1 : 0;
-    if (local && h->warm) {
+    if (local && h->warm && !resumes) {
         GuardParams none = {};
         none.abort_flag = h->abort_flag;  // with nothing to zero or refill the body only reads the flag
         CNT_TRY(warm_backward_inputs(h, stream, p, guard_rides ? g : none));
@@ -1600,13 +1611,52 @@ int cnt_lstm_backward_errors(cnt_lstm *h, void *stream_, const float *weights, f
 }
 
 int cnt_lstm_backward_prev_errors(cnt_lstm *h, void *stream_, const float *weights, float *prev_errors) {
+    CNT_REQUIRE(h, "lstm_backward_prev_errors: null argument");
+    return cnt_lstm_backward_prev_errors_range(h, stream_, weights, prev_errors, 0, h->T);
+}
+
+int cnt_lstm_backward_steps_done(const cnt_lstm *h, int steps, int *t_begin, int *t_end) {
+    using namespace cnt;
+    CNT_REQUIRE(h && t_begin && t_end, "lstm_backward_steps_done: null argument");
+    CNT_REQUIRE(h->T > 0 && steps >= 0 && steps <= h->T, "lstm_backward_steps_done: %d steps of %d", steps, h->T);
+    // the first direction's recursion runs from the last time step down, the second one's from the first up
+    *t_begin = h->T - steps;
+    *t_end = h->ndir == 2 ? steps : h->T;
+    if (*t_end < *t_begin) *t_end = *t_begin;
+    return CNT_OK;
+}
+
+int cnt_lstm_backward_errors_range(cnt_lstm *h, void *stream_, const float *weights, float *output_errors, int step_begin,
+                                   int step_end) {
+    using namespace cnt;
+    CNT_REQUIRE(h && weights && output_errors, "lstm_backward_errors_range: null argument");
+    CNT_REQUIRE(h->T > 0, "lstm_backward_errors_range: load_sequences has not been called");
+    CNT_REQUIRE(!h->stepwise && h->local, "lstm_backward_errors_range: this layer's recursion cannot run a range of its "
+                "steps (cnt_lstm_backward_can_split)");
+    CNT_LSTM_REPORT_FAILURE(h);
+    ChainParams p;
+    fill_chain_params(h, weights, p);
+    p.outerr = output_errors;
+    p.herr_out = (h->ndir == 1) ? output_errors : nullptr;
+    p.step_begin = step_begin; p.step_end = step_end;
+    return launch_chain(h, static_cast<hipStream_t>(stream_), false, p);
+}
+
+int cnt_lstm_backward_can_split(const cnt_lstm *h) { return h && !h->stepwise && h->local ? 1 : 0; }
+
+int cnt_lstm_backward_prev_errors_range(cnt_lstm *h, void *stream_, const float *weights, float *prev_errors, int t_begin,
+                                        int t_end) {
     using namespace cnt;
     CNT_REQUIRE(h && weights && prev_errors, "lstm_backward_prev_errors: null argument");
     CNT_REQUIRE(h->T > 0, "lstm_backward_prev_errors: load_sequences has not been called");
+    CNT_REQUIRE(t_begin >= 0 && t_begin <= t_end && t_end <= h->T, "lstm_backward_prev_errors: time steps %d..%d of %d",
+                t_begin, t_end, h->T);
     CNT_LSTM_REPORT_FAILURE(h);
+    if (t_begin == t_end) return CNT_OK;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const cnt_lstm_desc &d = h->desc;
-    const int P = d.P, L = d.L, H = h->H, S = d.S, N = h->T * S;
+    const int P = d.P, L = d.L, H = h->H, S = d.S, N = (t_end - t_begin) * S;
+    const size_t first = (size_t)t_begin * S;  // slots are time-major
     // e_x = sum_{dir,g} W_in[g,dir] * delta[g,dir]  (overwrite)
     {
         GemmArgs ga = {};
@@ -1618,9 +1668,9 @@ int cnt_lstm_backward_prev_errors(cnt_lstm *h, void *stream_, const float *weigh
         for (int dir = 0; dir < h->ndir; ++dir)
             for (int g = 0; g < 4; ++g) {
                 ga.prob[0].A[dir * 4 + g] = weights + (size_t)g * P * L + (size_t)dir * P * H;
-                ga.prob[0].B[dir * 4 + g] = h->state[dir][7 + g];
+                ga.prob[0].B[dir * 4 + g] = h->state[dir][7 + g] + first * H;
             }
-        ga.prob[0].C = prev_errors;
+        ga.prob[0].C = prev_errors + first * P;
         ga.label = "gemm:lstm_prev_errors";
         CNT_TRY(gemm_launch(stream, ga));
     }

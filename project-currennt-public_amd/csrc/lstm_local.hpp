@@ -202,13 +202,14 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
             coef[b][C_DUMMY][lane] = ((t >= p.Tmin) && (x.pat == 0)) ? 1.0f : 0.0f;
         };
         StepIn in;
-        load_step(0, in); wait_all_vmem(); put_coef(0, in);
-        load_step(1, in); wait_all_vmem(); put_coef(1, in);
-        load_step(2, in);
+        const int sb = p.step_begin;
+        load_step(sb, in); wait_all_vmem(); put_coef(sb, in);
+        load_step(sb + 1, in); wait_all_vmem(); put_coef(sb + 1, in);
+        load_step(sb + 2, in);
         const bool mtiming = p.phase_ticks != nullptr;
         long long mbusy = 0;
         lds_barrier();  // start of the recursion
-        for (int step = 0; step < T; ++step) {
+        for (int step = sb; step < p.step_end; ++step) {
             const int t = slot_of(step), b = step & 1;
             lds_barrier();  // results of this step are in LDS; the cell wave is done with this parity's coefficients
             if (wait_failed) return;
@@ -252,7 +253,7 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
         lds_barrier();  // start of the recursion
         const bool timing = p.phase_ticks != nullptr;
         long long busy = 0;
-        for (int step = 0; step < T; ++step) {
+        for (int step = p.step_begin; step < p.step_end; ++step) {
             lds_barrier();  // the deltas of this step are in LDS
             // looked at only at the end of the step: the read is in flight behind the barrier together with the
             // deltas', and what a failed step publishes no longer matters
@@ -309,6 +310,11 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
     float p_ig = 0, p_fg = 0, p_og = 0;
     if (cell_lane) { p_ig = D.peep[0][j0 + cc]; p_fg = D.peep[1][j0 + cc]; p_og = D.peep[2][j0 + cc]; }
     float fg_later = 0, cerr_later = 0, dig_later = 0, dfg_later = 0;
+    if (p.step_begin > 0 && cell_lane && cj < nseq) {
+        // a launch that starts in the middle: what the step before carried over stands in the state arrays
+        const size_t gi = (size_t)slot_of(p.step_begin - 1) * n + (size_t)(seq0 + cj) * H + j0 + cc;
+        fg_later = D.fg[gi]; cerr_later = D.cerr[gi]; dig_later = D.dig[gi]; dfg_later = D.dfg[gi];
+    }
     long long ph0 = 0, ph1 = 0, ph3 = 0, ph6 = 0, poll_rounds = 0;
     const bool timing = p.phase_ticks != nullptr;
     const long long tk_begin = timing ? wall_clock64() : 0;
@@ -316,7 +322,7 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
     wait_all_vmem();  // peepholes are in registers before the recursion starts
     lds_barrier();    // start of the recursion: coefficients of steps 0 and 1 are in LDS
 
-    for (int step = 0; step < T; ++step) {
+    for (int step = p.step_begin; step < p.step_end; ++step) {
         const long long tk0 = timing ? wall_clock64() : 0;
         const bool first = (step == 0), last = (step == T - 1);
         const int b = step & 1;

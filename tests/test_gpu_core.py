@@ -124,6 +124,67 @@ def test_weight_gradients_spread_between_runs():
         assert PC.relerr(dW, runs[0][1]) < 1e-5
 
 
+@pytest.mark.parametrize("L,bidir,S,T,cuts", [
+    (512, True, 10, 60, [45]), (512, True, 10, 60, [1, 30, 59]), (256, False, 7, 50, [37]), (128, True, 3, 9, [2, 3]),
+])
+def test_lstm_recursion_in_several_launches_is_the_same_recursion(L, bidir, S, T, cuts):
+    """The backward recursion run as ranges of its steps, and the error product for the preceding layer computed for
+    the time steps that are final early and for the rest afterwards: every state array and every error is
+    bit-identical to the single launch and the single product."""
+    import numpy as np
+    import torch
+
+    print("lstm split recursion", L, bidir, S, T, cuts, flush=True)
+    capi = PC.pkg().capi
+    P = 40
+    rng = np.random.default_rng(L + S)
+    lengths = [int(v) for v in rng.integers(max(1, T // 2), T + 1, size=S)]
+    lengths[0] = T
+    W, x, outerr = PC.lstm_inputs(P, L, bidir, S, T, lengths, 3)
+    pat = PC.make_pat_types(lengths, T)
+    Wd, xd, pd, ed = PC.dev(W), PC.dev(x), PC.dev(pat), PC.dev(outerr)
+    out = torch.zeros(L * T * S, device="cuda")
+    layer = capi.Lstm(P, L, bidir, S, T)
+    assert layer.backward_can_split()
+    names = ["herr", "dni", "dig", "dfg", "dog", "cerr"]
+
+    def snapshot(err, ex):
+        torch.cuda.synchronize()
+        got = {"outerr": err.cpu().numpy().copy(), "ex": ex.cpu().numpy().copy()}
+        for d in range(2 if bidir else 1):
+            for k in names:
+                got["%s%d" % (k, d)] = layer.state(d, k).cpu().numpy().copy()
+        return got
+
+    layer.load_sequences(pd, T, min(lengths))
+    layer.forward(Wd, xd, out)
+    err, ex = ed.clone(), torch.full((P * T * S,), 7.0, device="cuda")
+    layer.backward_errors(Wd, err, ex)
+    layer.check()
+    whole = snapshot(err, ex)
+
+    layer.load_sequences(pd, T, min(lengths))
+    layer.forward(Wd, xd, out)
+    err, ex = ed.clone(), torch.full((P * T * S,), 7.0, device="cuda")
+    edges = [0] + cuts + [T]
+    done_lo, done_hi = T, T  # time steps whose columns of ex are written
+    for a, b in zip(edges, edges[1:]):
+        layer.backward_errors_range(Wd, err, a, b)
+        lo, hi = layer.backward_steps_done(b)
+        if hi > lo and done_lo == done_hi:
+            layer.backward_prev_errors_range(Wd, ex, lo, hi)  # once, as soon as some time steps are final
+            done_lo, done_hi = lo, hi
+    if done_lo == done_hi:
+        done_lo = done_hi = 0
+    layer.backward_prev_errors_range(Wd, ex, 0, done_lo)
+    layer.backward_prev_errors_range(Wd, ex, done_hi, T)
+    layer.check()
+    parts = snapshot(err, ex)
+    layer.close()
+    for k in whole:
+        assert np.array_equal(whole[k], parts[k]), k
+
+
 def test_lstm_config1_unidirectional():
     """benchmark config 1: P=382, H=256, T=200, S=4 with one sequence of 150 frames."""
     print("lstm config 1", flush=True)
