@@ -156,7 +156,9 @@ int cnt_lstm_backward_prev_errors(cnt_lstm *h, void *stream, const float *weight
  * persistent kernel per group of sequences); elsewhere it is an error.
  * cnt_lstm_backward_steps_done: the time steps [t_begin, t_end) whose deltas are final once `steps` steps have run
  * (both directions have passed them), i.e. what cnt_lstm_backward_prev_errors_range may already compute:
- * prev_errors columns of the time steps [t_begin, t_end) only. */
+ * prev_errors columns of the time steps [t_begin, t_end) only.
+ * (The library's own network sequencer does not split: on MI355X the second launch's cold start cost more than the
+ * overlap gained for the benchmark model.) */
 int cnt_lstm_backward_can_split(const cnt_lstm *h);
 int cnt_lstm_backward_errors_range(cnt_lstm *h, void *stream, const float *weights, float *output_errors,
                                    int step_begin, int step_end);
