@@ -148,6 +148,11 @@ def mdn_c3(args, pkg):
     ach = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
     roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None,
             "kernel": dom}
+    if (F, M, D) == (6000, 16, 60):
+        # two rocprofv3 --pmc runs of this workload (FETCH_SIZE x 2.00 by a copy of known size, WRITE_SIZE x 1.00):
+        # error kernel 48.0 MB read + 0.4 MB written, gradient kernel 49.6 MB read + 47.3 MB written per launch
+        roof["traffic"] = 48.4e6 if dom == "mdn_mixture_error" else 96.9e6
+        roof["traffic_source"] = "profiles/mdn_c3_backward_kernel_stats.md"
 
     def full():
         layer.forward(xd)
