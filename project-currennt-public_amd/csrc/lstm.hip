@@ -333,12 +333,12 @@ __global__ __launch_bounds__(fwd_threads(JB, NT)) void lstm_forward_chain(const 
             } else {
                 float x_ni = a_ni + b_ni, x_ig = a_ig + b_ig, x_fg = a_fg + b_fg, x_og = a_og + b_og;
                 if (!first) { x_ig += c_prev * p_ig; x_fg += c_prev * p_fg; }
-                const float ni = tanh_act(x_ni), ig = logistic(x_ig), fg = logistic(x_fg);
+                const float ni = tanh_quick(x_ni), ig = logistic_quick(x_ig), fg = logistic_quick(x_fg);
                 float c = ni * ig;
                 if (!first) c += c_prev * fg;
                 x_og += c * p_og;
-                const float og = logistic(x_og);
-                hval = tanh_act(c) * og;
+                const float og = logistic_quick(x_og);
+                hval = tanh_quick(c) * og;
                 res[b][R_NI][id] = ni; res[b][R_IG][id] = ig; res[b][R_FG][id] = fg; res[b][R_OG][id] = og;
                 res[b][R_C][id] = c;
                 flags = 3;
@@ -1367,7 +1367,7 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     if (const char *e = std::getenv("CNT_LSTM_WARM")) h->warm = std::atoi(e) != 0;
     if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY")) h->poll_delay = h->poll_delay_local = std::atoi(e);
     // forward recursion: the senders' cell update (a few hundred clocks) plus store visibility
-    h->poll_delay_fwd = 34;  // measured optimum on MI355X at H=256, S=10
+    h->poll_delay_fwd = 26;  // measured optimum on MI355X at H=256, S=10 (24-26 for 64 and 128 cells, S=4..8)
     if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY_FWD")) h->poll_delay_fwd = std::atoi(e);
     if (const char *e = std::getenv("CNT_LSTM_POLL_GAP")) h->poll_gap = std::atoi(e);
     hipError_t err = hipGetDevice(&h->device);
