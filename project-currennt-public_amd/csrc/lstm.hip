@@ -1367,7 +1367,9 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     if (const char *e = std::getenv("CNT_LSTM_WARM")) h->warm = std::atoi(e) != 0;
     if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY")) h->poll_delay = h->poll_delay_local = std::atoi(e);
     // forward recursion: the senders' cell update (a few hundred clocks) plus store visibility
-    h->poll_delay_fwd = 26;  // measured optimum on MI355X at H=256, S=10 (24-26 for 64 and 128 cells, S=4..8)
+    // measured optima on MI355X: 26 at H=256 (S=10 and S=4), 25-26 at H=128 (S=8), 24 at H=64 (S=6); two units early
+    // cost a second poll round (+0.2 us per step), every unit late costs its 0.027 us
+    h->poll_delay_fwd = H <= 64 ? 24 : 26;
     if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY_FWD")) h->poll_delay_fwd = std::atoi(e);
     if (const char *e = std::getenv("CNT_LSTM_POLL_GAP")) h->poll_gap = std::atoi(e);
     hipError_t err = hipGetDevice(&h->device);
