@@ -290,3 +290,36 @@ def test_lstm_invalid_geometry_is_an_error():
         capi.Lstm(10, 129, True, 4, 10)      # odd size of a bidirectional layer
     with pytest.raises(RuntimeError):
         capi.Lstm(10, 0, False, 4, 10)
+
+
+def test_lstm_partial_recursion_rejects_what_it_cannot_do():
+    import torch
+
+    capi = PC.pkg().capi
+    T, S = 12, 3
+    pat = PC.dev(PC.make_pat_types([T] * S, T))
+    # 20 cells: step-by-step recursion, which has no partial form
+    small = capi.Lstm(8, 20, False, S, T)
+    small.load_sequences(pat, T, T)
+    assert not small.backward_can_split()
+    W = torch.zeros(int(capi.lib().cnt_lstm_weight_count(8, 20, 0)), device="cuda")
+    err = torch.zeros(20 * T * S, device="cuda")
+    with pytest.raises(RuntimeError, match="cannot run a range"):
+        small.backward_errors_range(W, err, 0, 6)
+    small.close()
+    layer = capi.Lstm(8, 128, True, S, T)
+    layer.load_sequences(pat, T, T)
+    assert layer.backward_can_split()
+    W = torch.zeros(int(capi.lib().cnt_lstm_weight_count(8, 128, 1)), device="cuda")
+    err = torch.zeros(128 * T * S, device="cuda")
+    ex = torch.zeros(8 * T * S, device="cuda")
+    for a, b in ((0, 0), (5, 4), (-1, 3), (0, T + 1)):
+        with pytest.raises(RuntimeError, match="steps"):
+            layer.backward_errors_range(W, err, a, b)
+    with pytest.raises(RuntimeError, match="time steps"):
+        layer.backward_prev_errors_range(W, ex, 3, T + 1)
+    assert layer.backward_steps_done(0) == (T, T)
+    assert layer.backward_steps_done(T) == (0, T)
+    assert layer.backward_steps_done(9) == (3, 9)
+    assert layer.backward_steps_done(4) == (8, 8)   # nothing final yet in a bidirectional layer
+    layer.close()
