@@ -203,8 +203,11 @@ def dft_c5(args, pkg):
     dom = "dft_loss"
     nbytes = 12.0 * W * n  # per launch = one resolution: read source + target, write gradient
     ach = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
-    roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None,
-            "kernel": dom, "note": "4.6 MB and 0.17 GFLOP in total: launch- and latency-bound, far from either roof"}
+    # traffic: two rocprofv3 --pmc runs of this workload (FETCH_SIZE x 2.00 by a copy of known size, WRITE_SIZE x 1.00):
+    # dft_loss_kernel 6.3 MB read (every sample is part of four frames per resolution) + 6.3 MB written (overlap-add)
+    roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
+            "traffic": 12.6e6 if (W, n) == (8, 16000) else None, "traffic_source": "profiles/dft_c5_backward_kernel_stats.md",
+            "kernel": dom, "note": "1.5 MB of samples and gradients, 0.17 GFLOP: launch- and latency-bound, far from either roof"}
     extra = {"roofline": roof, "kernels": kernels}
     if not args.no_cpu:
         import oracle_lib as O  # the checker, only for this reported baseline
@@ -248,7 +251,8 @@ def opt_step(args, pkg):
     nbytes = total * 40.0  # per weight: read g, m, v, delta, w; write cur, m, v, delta, w
     ach = nbytes / (kernels["opt_step"]["ms_per_step"] * 1e-3) / 1e9
     roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
-            "traffic": None, "kernel": "opt_step",
+            # two rocprofv3 --pmc runs of this workload: 74.2 MB fetched by the L2s + 74.2 MB written per launch
+            "traffic": 148.4e6, "traffic_source": "profiles/opt_step_kernel_stats.md", "kernel": "opt_step",
             "note": "one launch over all 3.7 M weights; 40 B per weight = 148 MB per step, which repeated steps "
                     "find in the 256 MB last-level cache: the figure is not a pure HBM rate"}
     extra = {"roofline": roof, "kernels": kernels}
