@@ -91,7 +91,10 @@ def lstm_c1(args, pkg):
     us_per_step = kernels[dom]["avg_ms"] * 1e3 / T
     hop_us = capi.probe_hop_latency(same_xcd=True, with_compute=True, rounds=2000)
     roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_FP32_MFMA_TFLOPS,
-            "traffic": None, "kernel": dom, "us_per_step": us_per_step, "latency_floor_us_per_step": hop_us,
+            # two rocprofv3 --pmc runs of this workload (FETCH_SIZE x 2.00 by a copy of known size, WRITE_SIZE x 1.00):
+            # 12.2 MB read + 7.0 MB written per launch of lstm_backward_local<256, 8>; algorithmic 12.5 MB
+            "traffic": 19.2e6, "traffic_source": "profiles/lstm_c1_backward_kernel_stats.md",
+            "kernel": dom, "us_per_step": us_per_step, "latency_floor_us_per_step": hop_us,
             "frac_of_latency_floor": hop_us / us_per_step,
             "note": "latency-bound recursion (T sequential steps, one job of four sequences on one XCD): `frac` is against the "
                     "fp32 MFMA peak, `frac_of_latency_floor` against one measured hop inside an XCD plus a step's arithmetic"}
