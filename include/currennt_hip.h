@@ -151,8 +151,10 @@ int cnt_lstm_backward_prev_errors(cnt_lstm *h, void *stream, const float *weight
  * products that follow it (the reference runs the recursion step by step, layers/LstmLayer.cu:2136-2252, and the
  * product over the whole fraction, :2298-2334; splitting either changes no result).
  * cnt_lstm_backward_errors_range runs steps [step_begin, step_end) of the curMaxT steps of the recursion; the
- * ranges of one pass must be launched in order on one stream, the first from step 0, and nothing else may use the
- * handle in between.  Only where cnt_lstm_backward_can_split returns 1 (layers whose backward recursion runs as one
+ * ranges of one pass must be launched in order on one stream, the first from step 0.  The handle keeps the step the
+ * pass stands at: a range that starts anywhere else is refused (CNT_ERR_ARG), and a pass that is abandoned half way
+ * -- a range from step 0, cnt_lstm_backward_errors, cnt_lstm_forward or cnt_lstm_load_sequences before step curMaxT
+ * was reached -- is dropped cleanly (the partial errors it left in the mailbox are discarded).  Only where cnt_lstm_backward_can_split returns 1 (layers whose backward recursion runs as one
  * persistent kernel per group of sequences); elsewhere it is an error.
  * cnt_lstm_backward_steps_done: the time steps [t_begin, t_end) whose deltas are final once `steps` steps have run
  * (both directions have passed them), i.e. what cnt_lstm_backward_prev_errors_range may already compute:
@@ -430,8 +432,11 @@ int cnt_network_backward(cnt_network *net, void *stream);
 /* cnt_lstm_check for every LSTM layer (all of them are looked at; the first failure is returned).  Failure contract
  * of the network: a pass in which a recursion gave up cannot reach the weights -- the failed launch sets a device
  * flag that the optimizer kernel of cnt_network_update reads, so even an update that was enqueued before the host
- * could see the failure leaves weights and optimizer state untouched -- and CNT_ERR_DEVICE is returned by this call
- * or by the next cnt_network_load_sequences / _forward / _backward / _update after the failed launch has ended. */
+ * could see the failure leaves weights and optimizer state (momentum, statistics, Adam's bias-correction products,
+ * which live in device memory for that reason) untouched -- and CNT_ERR_DEVICE is returned by this call or by the next
+ * cnt_network_load_sequences / _forward / _backward / _update after the failed launch has ended (the library records
+ * an event behind every recursion launch and reports nothing before that event has passed).  The report clears the
+ * flag in the order of the stream it is made on, so the calls of a pass belong on one stream, of any kind. */
 int cnt_network_check(cnt_network *net, void *stream);
 /* cnt_lstm_set_wait_bounds for the LSTM layer at `layer_index` of the network (CNT_ERR_ARG for any other layer).  No
  * counterpart in the reference; like that call it exists so that a test can force one layer's recursion to give up

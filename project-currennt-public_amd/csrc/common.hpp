@@ -204,7 +204,10 @@ int gemm_simple(hipStream_t stream, float *C, int m, int n, int k, const float *
 // the pass that produced the gradients gave up), the step changes nothing.
 int opt_step_guarded(hipStream_t stream, int option, long n, float *weights, const float *layer_updates, float *cur_updates,
                      float *stats, float *weight_deltas, const float *mask, float frac_length, float beta1_accum,
-                     float beta2_accum, float learning_rate, float momentum, const int *veto);
+                     float beta2_accum, float learning_rate, float momentum, const int *veto, const float *accum_dev);
+// Adam's bias-correction products (two floats in device memory, both 1 before the first step) advanced by one step,
+// unless *veto is non-zero; opt_step_guarded reads them in place of its two float arguments when accum_dev is given.
+int opt_adam_advance(hipStream_t stream, float *accum_dev, const int *veto);
 // LSTM handles of a network share one such flag: a recursion that gives up also sets *veto (until the owner clears it).
 void lstm_set_veto(cnt_lstm *h, int *veto);
 // non-zero if a recursion of this handle has given up since the last report (no synchronisation: it only sees
@@ -212,7 +215,7 @@ void lstm_set_veto(cnt_lstm *h, int *veto);
 // cnt_lstm_backward_weights in two parts that write disjoint ranges (1: input weights, 2: the rest)
 int lstm_backward_weights_parts(cnt_lstm *h, hipStream_t stream, const float *x, float *weight_updates, int parts);
 int lstm_take_failure(cnt_lstm *h);
-int report_failure(cnt_network *net);
+int report_failure(cnt_network *net, hipStream_t stream);
 
 // ----- error halves that also do the backward step of the skip layer in front of them ----------------
 // A skip layer adds what its linkers left in its side buffer to the errors its following layer wrote, and hands the

@@ -1070,6 +1070,12 @@ struct cnt_lstm {
     int last_blocks;       // workgroups of the last recursion launch
     int warm;  // read the recursion's inputs once before the XCD-local backward recursion (CNT_LSTM_WARM=0: off)
     int poll_delay_local;  // pause before the first poll of a step in the XCD-local recursion, units of 64 clocks
+    // recorded behind every recursion launch: the failure latch is taken only once the launch that may have set it has
+    // ended, so that no workgroup of that launch can set it (or the veto) again after the report
+    hipEvent_t launch_done;
+    int launch_pending;
+    // backward recursion run as ranges of steps: the step the next range has to start at (0: a fresh pass)
+    int next_step;
 };
 
 namespace cnt {
@@ -1201,6 +1207,14 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
                 "range of steps");
     CNT_REQUIRE(p.step_begin >= 0 && p.step_begin < p.step_end && p.step_end <= h->T, "lstm: steps %d..%d of %d",
                 p.step_begin, p.step_end, h->T);
+    if (local) {
+        // A range that ends before T leaves its last partial errors in the mailbox for the range that continues it.  A
+        // launch that starts over instead (the pass was abandoned) must not find them: the mailbox is refilled.
+        CNT_REQUIRE(p.step_begin == 0 || p.step_begin == h->next_step, "lstm: the backward recursion stands at step %d, "
+                    "a range cannot start at step %d", h->next_step, p.step_begin);
+        if (p.step_begin == 0 && h->next_step != 0) h->bmail_dirty = 1;
+        h->next_step = p.step_end < h->T ? p.step_end : 0;
+    }
     const bool guard_rides = local && !fwd && h->warm && !resumes && !(h->bmail_dirty && h->lmail);
     if (!guard_rides) {
         hipLaunchKernelGGL(chain_guard, dim3(1), dim3(1024), 0, stream, g);
@@ -1230,6 +1244,8 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
         p.poll_delay = h->poll_delay_local;
         hipLaunchKernelGGL(k, dim3(blocks), dim3(local_threads(h->H)), 0, stream, p);
         CNT_HIP(hipGetLastError());
+        CNT_HIP(hipEventRecord(h->launch_done, stream));
+        h->launch_pending = 1;
         return CNT_OK;
     }
     const int G = h->H / h->JB;
@@ -1238,6 +1254,8 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     h->last_blocks = blocks;
     hipLaunchKernelGGL(k, dim3(blocks), dim3(fwd ? kThreads + 64 * ((h->JB * 16 * h->NT + 63) / 64) + 64 : kBwdThreads), 0, stream, p);
     CNT_HIP(hipGetLastError());
+    CNT_HIP(hipEventRecord(h->launch_done, stream));
+    h->launch_pending = 1;
     return CNT_OK;
 }
 
@@ -1416,6 +1434,7 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     if (err == hipSuccess && std::getenv("CNT_LSTM_TIMING"))
         err = hipMalloc(reinterpret_cast<void **>(&h->phase_ticks), 8 * 512 * 6 * sizeof(long long));
     if (err == hipSuccess && h->phase_ticks) err = hipMemset(h->phase_ticks, 0, 8 * 512 * 6 * sizeof(long long));
+    if (err == hipSuccess) err = hipEventCreateWithFlags(&h->launch_done, hipEventDisableTiming);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->abort_flag), sizeof(int));
     if (err == hipSuccess) err = hipMemset(h->abort_flag, 0, sizeof(int));
     // the word a kernel that gives up sets for the host: pinned, mapped, coherent host memory
@@ -1446,6 +1465,7 @@ int cnt_lstm_destroy(cnt_lstm *h) {
     if (h->lmail) (void)hipFree(h->lmail);
     if (h->ctl) (void)hipFree(h->ctl);
     if (h->latch_host) (void)hipHostFree(h->latch_host);
+    if (h->launch_done) (void)hipEventDestroy(h->launch_done);
     delete h;
     return CNT_OK;
 }
@@ -1457,6 +1477,7 @@ int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int
                 h->desc.maxT);
     CNT_REQUIRE(curMinT >= 0 && curMinT <= curMaxT, "lstm_load_sequences: curMinT %d outside 0..%d", curMinT, curMaxT);
     h->T = curMaxT; h->Tmin = curMinT; h->pat = patTypes;
+    if (h->next_step != 0) { h->bmail_dirty = 1; h->next_step = 0; }  // an abandoned partial backward pass
     const size_t nstate = (size_t)h->H * h->desc.maxT * h->desc.S;
     // stored output-gate deltas of both directions, one launch
     if (h->ndir == 2) CNT_TRY(fill_zero_pair(static_cast<hipStream_t>(stream), h->state[0][10], nstate, h->state[1][10], nstate));
@@ -1491,6 +1512,14 @@ extern "C++" int cnt::lstm_take_failure(cnt_lstm *h) {
     if (!h || !h->latch_host) return 0;
     volatile int *latch = h->latch_host;
     if (*latch == 0) return 0;
+    if (h->launch_pending) {
+        // the launch that set the mark may still be running: its other workgroups would set it again after the report
+        if (hipEventQuery(h->launch_done) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;  // reported by a later call, once the launch has ended
+        }
+        h->launch_pending = 0;
+    }
     *latch = 0;
     return 1;
 }
@@ -1563,6 +1592,7 @@ int cnt_lstm_forward(cnt_lstm *h, void *stream_, const float *weights, const flo
     CNT_REQUIRE(h && weights && x && outputs, "lstm_forward: null argument");
     CNT_REQUIRE(h->T > 0, "lstm_forward: load_sequences has not been called");
     CNT_LSTM_REPORT_FAILURE(h);
+    if (h->next_step != 0) { h->bmail_dirty = 1; h->next_step = 0; }  // new states: a partial backward pass is void
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const cnt_lstm_desc &d = h->desc;
     const int P = d.P, L = d.L, H = h->H, N = h->T * d.S;

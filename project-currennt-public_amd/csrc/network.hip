@@ -475,7 +475,7 @@ struct cnt_network {
     // optimizer state (allocated by the first update)
     float *cur_updates = nullptr, *deltas = nullptr, *stats = nullptr;
     int stats_option = -1;
-    float beta1_accum = 1.0f, beta2_accum = 1.0f;
+    float *adam_accum = nullptr;  // beta1^t, beta2^t of Adam's bias correction (device)
     int mdn_target_start = 0, mdn_classes = 0;
     // set on the device by an LSTM recursion that gives up; the optimizer step looks at it and leaves the weights alone
     int *veto = nullptr;
@@ -1175,7 +1175,7 @@ int cnt_network_load_sequences(cnt_network *net, void *stream_, int T, int Tmin,
                                const float *inputs, const float *targets) {
     using namespace cnt;
     CNT_REQUIRE(net && patTypes, "network_load_sequences: null argument");
-    CNT_TRY(report_failure(net));
+    CNT_TRY(report_failure(net, static_cast<hipStream_t>(stream_)));
     CNT_REQUIRE(T >= 1 && T <= net->maxT && Tmin >= 1 && Tmin <= T, "network_load_sequences: lengths %d / %d outside "
                 "1..%d", T, Tmin, net->maxT);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -1213,7 +1213,7 @@ int cnt_network_load_sequences(cnt_network *net, void *stream_, int T, int Tmin,
 int cnt_network_forward(cnt_network *net, void *stream_) {
     using namespace cnt;
     CNT_REQUIRE(net && net->T > 0, "network_forward: no fraction loaded");
-    CNT_TRY(report_failure(net));
+    CNT_TRY(report_failure(net, static_cast<hipStream_t>(stream_)));
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     // what the skip layers' forward passes clear (layers/SkipAddLayer.cu:195-205)
     if (net->skip_error_count) CNT_TRY(fill_zero(stream, net->skip_errors, net->skip_error_count));
@@ -1330,7 +1330,7 @@ int cnt_network_calculate_error(cnt_network *net, void *stream_, float *loss_dev
 int cnt_network_backward(cnt_network *net, void *stream_) {
     using namespace cnt;
     CNT_REQUIRE(net && net->T > 0, "network_backward: no fraction loaded");
-    CNT_TRY(report_failure(net));
+    CNT_TRY(report_failure(net, static_cast<hipStream_t>(stream_)));
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     int next_side = 0;
     bool side_used[cnt_network::kMaxSide] = {};
@@ -1701,12 +1701,16 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
 
 // CNT_ERR_DEVICE if a recursion of one of the network's LSTM layers has given up (and ended) since the last report;
 // clears every layer's mark and the device flag that holds the optimizer step back.
-extern "C++" int cnt::report_failure(cnt_network *net) {
+extern "C++" int cnt::report_failure(cnt_network *net, hipStream_t stream) {
     bool failed = false;
     for (auto &L : net->layers)
         if (L.lstm && cnt::lstm_take_failure(L.lstm)) failed = true;
     if (!failed) return CNT_OK;
-    if (net->veto) CNT_HIP(hipMemset(net->veto, 0, sizeof(int)));
+    // The launch that gave up has ended (lstm_take_failure reports nothing earlier), so nothing sets the flag again.
+    // The flag is cleared IN STREAM ORDER: an optimizer step of the failed pass that is already enqueued on this
+    // stream still finds it set, whatever kind of stream this is.
+    if (net->veto) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(net->veto), 1, 0u));
+
     set_error("network: an LSTM recursion gave up waiting for a neighbouring workgroup; the results of that pass are "
               "invalid and a weight update that followed it was skipped");
     return CNT_ERR_DEVICE;
@@ -1722,8 +1726,14 @@ int cnt_network_check(cnt_network *net, void *stream) {
             const int s = cnt_lstm_check(L.lstm, stream);
             if (s != CNT_OK && status == CNT_OK) status = s;
         }
-    if (status != CNT_OK && net->veto) CNT_HIP(hipMemset(net->veto, 0, sizeof(int)));
-    if (status == CNT_OK) status = report_failure(net);  // a layer whose launch ended on another stream
+    if (status != CNT_OK) {
+        // every stream of the network has been waited for: the flag is cleared on this stream and the clear awaited
+        if (net->veto) {
+            CNT_TRY(fill_words(static_cast<hipStream_t>(stream), reinterpret_cast<unsigned *>(net->veto), 1, 0u));
+            CNT_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+        }
+    }
+    if (status == CNT_OK) status = report_failure(net, static_cast<hipStream_t>(stream));  // a launch that ended on another stream
     return status;
 }
 
@@ -1743,7 +1753,7 @@ int cnt_network_update(cnt_network *net, void *stream_, int option, float learni
     // A pass whose recursion gave up must not reach the weights.  Two nets: launches that have already ended are
     // seen here, on the host; one that ends later sets the device flag the optimizer kernel looks at, and the next
     // call into the network reports it.
-    CNT_TRY(report_failure(net));
+    CNT_TRY(report_failure(net, static_cast<hipStream_t>(stream_)));
     const size_t n = (size_t)net->n_weights;
     if (!net->cur_updates) {
         CNT_TRY(device_alloc(net, (void **)&net->cur_updates, n * sizeof(float), true));
@@ -1760,15 +1770,22 @@ int cnt_network_update(cnt_network *net, void *stream_, int option, float learni
         net->stats_option = option;
     }
     if (adam) {
-        net->beta1_accum = cnt_opt_next_beta_accum(net->beta1_accum, 1);
-        net->beta2_accum = cnt_opt_next_beta_accum(net->beta2_accum, 2);
+        // beta1^t and beta2^t live in device memory and advance under the same flag as the step itself, so that a step
+        // the device-side veto skips leaves them untouched as well
+        if (!net->adam_accum) {
+            const float ones[2] = {1.0f, 1.0f};
+            CNT_TRY(device_alloc(net, (void **)&net->adam_accum, sizeof(ones), false));
+            CNT_HIP(hipMemcpy(net->adam_accum, ones, sizeof(ones), hipMemcpyHostToDevice));
+        }
+        CNT_TRY(opt_adam_advance(static_cast<hipStream_t>(stream_), net->adam_accum, net->veto));
     }
+    const float *accum_dev = adam ? net->adam_accum : nullptr;
     bool own_rates = false;
     for (const auto &L : net->layers) own_rates = own_rates || (L.weight_count() > 0 && L.learning_rate > -0.5f);
     if (!own_rates)
         return opt_step_guarded(static_cast<hipStream_t>(stream_), option, (long)n, net->weights, net->updates, net->cur_updates,
-                                net->stats, net->deltas, nullptr, frac_length, net->beta1_accum, net->beta2_accum, learning_rate,
-                                momentum, net->veto);
+                                net->stats, net->deltas, nullptr, frac_length, 0.0f, 0.0f, learning_rate, momentum, net->veto,
+                                accum_dev);
     // a layer's own "learningRate" replaces the optimizer's (optimizers/SteepestDescentOptimizer.cu:402-403, :425-426): one
     // launch per trainable layer
     for (const auto &L : net->layers) {
@@ -1777,9 +1794,8 @@ int cnt_network_update(cnt_network *net, void *stream_, int option, float learni
         const long o = L.w_off;
         float *st = net->stats ? net->stats + (adam ? 2 * o : o) : nullptr;
         CNT_TRY(opt_step_guarded(static_cast<hipStream_t>(stream_), option, c, net->weights + o, net->updates + o,
-                                 net->cur_updates + o, st, net->deltas + o, nullptr, frac_length, net->beta1_accum,
-                                 net->beta2_accum, L.learning_rate > -0.5f ? L.learning_rate : learning_rate, momentum,
-                                 net->veto));
+                                 net->cur_updates + o, st, net->deltas + o, nullptr, frac_length, 0.0f, 0.0f,
+                                 L.learning_rate > -0.5f ? L.learning_rate : learning_rate, momentum, net->veto, accum_dev));
     }
     return CNT_OK;
 }

@@ -31,6 +31,7 @@ struct OptArgs {
     int add;                     // accumulate: add to cur instead of overwriting it
     float frac_length, beta1_accum, beta2_accum, learning_rate, momentum;
     const int *veto;             // optional device flag: non-zero means the gradients are invalid, nothing is touched
+    const float *accum_dev;      // optional: Adam's two bias-correction products in device memory (replace the two floats)
 };
 
 __device__ __forceinline__ bool bad(float g) { return isnan(g) || isinf(g); }
@@ -46,8 +47,9 @@ __device__ __forceinline__ float adjust_one(const OptArgs &a, size_t i, float g)
         const float v = (float)(a.stats[2 * i + 1] * kBeta2 + (double)(ave * ave) * (1 - kBeta2));
         a.stats[2 * i] = m;
         a.stats[2 * i + 1] = v;
-        const float mh = m / (1 - a.beta1_accum);
-        const float vh = v / (1 - a.beta2_accum);
+        const float b1 = a.accum_dev ? a.accum_dev[0] : a.beta1_accum, b2 = a.accum_dev ? a.accum_dev[1] : a.beta2_accum;
+        const float mh = m / (1 - b1);
+        const float vh = v / (1 - b2);
         return (float)(mh / (sqrtf(vh) + kEps));
     }
     const float acc = a.stats[i] + (ave * ave);
@@ -78,6 +80,14 @@ __global__ __launch_bounds__(256) void optimizer_kernel(const OptArgs a) {
         if (MODE == 2 || MODE == 3) g = update_one(a, i, g);
         a.cur[i] = g;
     }
+}
+
+// Adam's bias-correction products beta1^t, beta2^t kept in device memory, advanced in stream order in front of a step
+// and under the same veto flag as the step: a step that the flag skips leaves them where they stood.
+__global__ void adam_advance_kernel(float *accum, const int *veto) {
+    if (veto && *veto != 0) return;
+    accum[0] = (float)(accum[0] * kBeta1);
+    accum[1] = (float)(accum[1] * kBeta2);
 }
 
 int blocks_for(size_t n) {
@@ -141,13 +151,20 @@ int cnt_opt_step(void *stream, int option, long n, float *weights, const float *
                  float *stats, float *weight_deltas, const float *mask, float frac_length, float beta1_accum,
                  float beta2_accum, float learning_rate, float momentum) {
     return cnt::opt_step_guarded(static_cast<hipStream_t>(stream), option, n, weights, layer_updates, cur_updates, stats,
-                                 weight_deltas, mask, frac_length, beta1_accum, beta2_accum, learning_rate, momentum, nullptr);
+                                 weight_deltas, mask, frac_length, beta1_accum, beta2_accum, learning_rate, momentum, nullptr,
+                                 nullptr);
+}
+
+extern "C++" int cnt::opt_adam_advance(hipStream_t stream, float *accum_dev, const int *veto) {
+    hipLaunchKernelGGL(adam_advance_kernel, dim3(1), dim3(1), 0, stream, accum_dev, veto);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
 }
 
 extern "C++" int cnt::opt_step_guarded(hipStream_t stream, int option, long n, float *weights, const float *layer_updates,
                                        float *cur_updates, float *stats, float *weight_deltas, const float *mask,
                                        float frac_length, float beta1_accum, float beta2_accum, float learning_rate,
-                                       float momentum, const int *veto) {
+                                       float momentum, const int *veto, const float *accum_dev) {
     using namespace cnt;
     CNT_REQUIRE(n >= 0 && (n == 0 || (weights && layer_updates && cur_updates && weight_deltas)), "opt_step: bad argument");
     CNT_REQUIRE(known_option(option), "opt_step: unknown optimizer option %d", option);
@@ -160,6 +177,7 @@ extern "C++" int cnt::opt_step_guarded(hipStream_t stream, int option, long n, f
     a.frac_length = frac_length; a.beta1_accum = beta1_accum; a.beta2_accum = beta2_accum;
     a.learning_rate = learning_rate; a.momentum = momentum;
     a.veto = veto;
+    a.accum_dev = accum_dev;
     ProfileScope prof(stream, "opt_step");
     hipLaunchKernelGGL(optimizer_kernel<3>, dim3(blocks_for(a.n)), dim3(256), 0, stream, a);
     CNT_HIP(hipGetLastError());

@@ -185,6 +185,67 @@ def test_lstm_recursion_in_several_launches_is_the_same_recursion(L, bidir, S, T
         assert np.array_equal(whole[k], parts[k]), k
 
 
+def test_lstm_abandoned_partial_recursion_does_not_leak_into_the_next_pass():
+    """A range of the backward recursion that ends before T leaves its last partial errors in the mailbox for the range
+    that continues it.  When the pass is abandoned instead -- the caller starts over at step 0, with or without a new
+    fraction in between -- the next recursion must not consume them: every result equals that of a clean pass, a range
+    that does not start where the last one ended is refused."""
+    import numpy as np
+    import torch
+
+    print("lstm abandoned partial recursion", flush=True)
+    capi = PC.pkg().capi
+    P, L, S, T = 40, 512, 6, 30
+    lengths = [T, 21, T, 17, 25, T]
+    W, x, outerr = PC.lstm_inputs(P, L, True, S, T, lengths, 4)
+    pat = PC.make_pat_types(lengths, T)
+    Wd, xd, pd, ed = PC.dev(W), PC.dev(x), PC.dev(pat), PC.dev(outerr)
+    out = torch.zeros(L * T * S, device="cuda")
+    layer = capi.Lstm(P, L, True, S, T)
+
+    def clean_pass():
+        layer.load_sequences(pd, T, min(lengths))
+        layer.forward(Wd, xd, out)
+        err, ex = ed.clone(), torch.zeros(P * T * S, device="cuda")
+        layer.backward_errors(Wd, err, ex)
+        layer.check()
+        torch.cuda.synchronize()
+        return ex.cpu().numpy().copy(), [layer.state(d, k).cpu().numpy().copy() for d in range(2) for k in ("dni", "dog", "cerr")]
+
+    ex0, st0 = clean_pass()
+    # abandoned after 11 steps, new fraction loaded
+    layer.load_sequences(pd, T, min(lengths))
+    layer.forward(Wd, xd, out)
+    layer.backward_errors_range(Wd, ed.clone(), 0, 11)
+    with pytest.raises(RuntimeError, match="stands at step"):
+        layer.backward_errors_range(Wd, ed.clone(), 14, T)   # not where the last range ended
+    ex1, st1 = clean_pass()
+    assert np.array_equal(ex0, ex1)
+    for a, b in zip(st0, st1):
+        assert np.array_equal(a, b)
+    # abandoned, then a full recursion on the same fraction (no load_sequences: the stored output-gate deltas of the
+    # eleven steps already done are added once more, as in the reference; every other array is that of a clean pass)
+    layer.load_sequences(pd, T, min(lengths))
+    layer.forward(Wd, xd, out)
+    layer.backward_errors_range(Wd, ed.clone(), 0, 11)
+    layer.load_sequences(pd, T, min(lengths))   # clears the stored output-gate deltas
+    err, ex = ed.clone(), torch.zeros(P * T * S, device="cuda")
+    layer.backward_errors(Wd, err, ex)
+    layer.check()
+    torch.cuda.synchronize()
+    assert np.array_equal(ex0, ex.cpu().numpy())
+    # a range after a forward pass has nothing to continue
+    layer.load_sequences(pd, T, min(lengths))
+    layer.forward(Wd, xd, out)
+    layer.backward_errors_range(Wd, ed.clone(), 0, 7)
+    layer.forward(Wd, xd, out)
+    with pytest.raises(RuntimeError, match="stands at step"):
+        layer.backward_errors_range(Wd, ed.clone(), 7, T)
+    ex2, _ = clean_pass()
+    assert np.array_equal(ex0, ex2)
+    layer.close()
+
+
 def test_lstm_config1_unidirectional():
     """benchmark config 1: P=382, H=256, T=200, S=4 with one sequence of 150 frames."""
     print("lstm config 1", flush=True)
