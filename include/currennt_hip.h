@@ -41,6 +41,11 @@ int cnt_profile_get(int index, char *label, int label_cap, int *launches, float 
  * a recursion step does between receiving and sending.  T times this is the floor of a T-step recursion spread
  * over compute units.  Synchronous; *hop_us (host memory) receives microseconds per hop. */
 int cnt_probe_hop_latency(void *stream, int same_xcd, int with_compute, int rounds, float *hop_us);
+/* Test hook: the scalar activation functions as the kernels evaluate them, out[i] = f(x[i]) for n device floats.
+ * which = 0: logistic, 1: tanh (activation_functions/Logistic.cuh, Tanh.cuh: exp and a true quotient, clamped at
+ * +-88.72); 2, 3: the same two from the hardware's exp2 and reciprocal, which only the forward LSTM recursion uses
+ * (within 4e-6 / 8e-6 absolute of the former, not bit-identical). */
+int cnt_probe_activation(void *stream, int which, long n, const float *x, float *out);
 
 /* ---- helpers::Matrix product seam -------------------------------------------------------------
  * Replaces helpers::Matrix<Gpu>::assignProduct / addProduct (helpers/Matrix.cu:353-377, which call

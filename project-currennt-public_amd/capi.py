@@ -69,6 +69,7 @@ _SIGNATURES = {
     "cnt_dense_backward_weights": (I, [VP, I, I, I, F, VP, VP, VP]),
     "cnt_dense_backward_weights_static": (I, [VP, I, I, I, F, VP, VP, VP]),
     "cnt_probe_hop_latency": (I, [VP, I, I, I, C.POINTER(F)]),
+    "cnt_probe_activation": (I, [VP, I, C.c_long, VP, VP]),
     "cnt_gemm_reserve": (I, [VP]),
     "cnt_gemm_release": (I, [VP]),
     "cnt_sse_backward": (I, [VP, I, I, VP, VP, VP, VP]),
@@ -237,6 +238,10 @@ def probe_hop_latency(same_xcd=True, with_compute=True, rounds=2000, stream=None
     out = F(0.0)
     check(lib().cnt_probe_hop_latency(stream_ptr(stream), int(same_xcd), int(with_compute), int(rounds), C.byref(out)))
     return float(out.value)
+
+
+def probe_activation(which, x, out, stream=None):
+    check(lib().cnt_probe_activation(stream_ptr(stream), int(which), x.numel(), ptr(x), ptr(out)))
 
 
 def gemm_reserve(stream=None):

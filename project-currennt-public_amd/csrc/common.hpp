@@ -60,9 +60,12 @@ __device__ __forceinline__ float logistic(float x) {
     }
     return 1.0f;
 }
-// The same functions from the hardware's exp2 and reciprocal (each within 1 ulp; the library routines above spend about
-// twenty instructions on denormal results and on an exactly rounded quotient), for the forward recursion, where the
-// five of them per cell and time step sit on the critical path of every step.
+// The same functions from the hardware's exp2 and reciprocal (the library routines above spend about twenty instructions
+// on denormal results and on an exactly rounded quotient), for the forward recursion, where the five of them per cell
+// and time step sit on the critical path of every step.  Not bit-identical to the functions above: exp2 and rcp are
+// good to 1 ulp each, but the argument -1.4427 * x is rounded to fp32 before the exponential, which alone is a
+// relative error of |x| * 6e-8 in exp(-x).  The result stays within 4e-6 absolute of the exact logistic function
+// (8e-6 for tanh) over the whole unclamped range, which tests/test_gpu_core.py checks against the CPU functions.
 __device__ __forceinline__ float logistic_quick(float x) {
     if (x < lim::kExpLimit) {
         if (x > -lim::kExpLimit) return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * x));

@@ -25,7 +25,7 @@ __global__ __launch_bounds__(64) void hop_probe_kernel(unsigned *ctl, unsigned *
         if (xcd == 0u) {
             const unsigned t = atomicAdd(&ctl[0], 1u);
             if (t == 0u || (same_xcd && t == 1u)) r = (int)t;
-        } else if (!same_xcd && xcd == 4u) {
+        } else if (!same_xcd) {  // any XCD other than the first role's
             if (atomicAdd(&ctl[1], 1u) == 0u) r = 1;
         }
         role_sh = r;
@@ -77,8 +77,27 @@ __global__ __launch_bounds__(64) void hop_probe_kernel(unsigned *ctl, unsigned *
     }
 }
 
+// the activation functions as the recursion kernels evaluate them, element by element (a test hook)
+__global__ void activations_kernel(size_t n, const float *__restrict__ x, float *__restrict__ out, int which) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = x[i];
+    out[i] = which == 0 ? logistic(v) : which == 1 ? tanh_act(v) : which == 2 ? logistic_quick(v) : tanh_quick(v);
+}
+
 }  // namespace
 }  // namespace cnt
+
+extern "C" int cnt_probe_activation(void *stream, int which, long n, const float *x, float *out) {
+    using namespace cnt;
+    CNT_REQUIRE(which >= 0 && which <= 3, "probe_activation: function %d, known 0..3", which);
+    CNT_REQUIRE(n >= 0 && (n == 0 || (x && out)), "probe_activation: bad argument");
+    if (n == 0) return CNT_OK;
+    hipLaunchKernelGGL(activations_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       (size_t)n, x, out, which);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
 
 extern "C" int cnt_probe_hop_latency(void *stream_, int same_xcd, int with_compute, int rounds, float *hop_us) {
     using namespace cnt;

@@ -246,6 +246,43 @@ def test_lstm_abandoned_partial_recursion_does_not_leak_into_the_next_pass():
     layer.close()
 
 
+def test_activation_functions_against_the_cpu_functions():
+    """The scalar semantics of the path (Logistic.cuh / Tanh.cuh with the clamps at +-88.72) and the quick forms the
+    forward recursion uses instead (hardware exp2 and reciprocal): swept over the whole unclamped range and across
+    the clamps, against the CPU oracle's scalar functions.  Tolerances: the exact forms 2e-7 absolute (one rounding of
+    exp and of the quotient) and 2e-5 relative, the quick forms 4e-6 (logistic) and 8e-6 (tanh) absolute and 1e-4 relative."""
+    import numpy as np
+    import torch
+
+    import oracle_lib as O
+
+    capi = PC.pkg().capi
+    xs = np.concatenate([np.linspace(-89.5, 89.5, 40001), np.linspace(-12, 12, 40001), np.linspace(-1, 1, 4001),
+                         np.array([-88.73, -88.72, -88.71, 88.71, 88.72, 88.73, 0.0, -0.0, 1e-30, -1e-30])]).astype(np.float32)
+    L = O.lib()
+    want_l = np.array([L.orc_logistic(float(v)) for v in xs], dtype=np.float32)
+    want_t = np.array([L.orc_tanh(float(v)) for v in xs], dtype=np.float32)
+    xd = PC.dev(xs)
+    out = torch.empty_like(xd)
+    got = []
+    for which in range(4):
+        capi.probe_activation(which, xd, out)
+        torch.cuda.synchronize()
+        got.append(out.cpu().numpy().copy())
+    for g, w, quick, tol in ((got[0], want_l, False, 2e-7), (got[1], want_t, False, 4e-7), (got[2], want_l, True, 4e-6),
+                             (got[3], want_t, True, 8e-6)):
+        assert np.abs(g - w).max() <= tol
+        big = np.abs(w) > 1e-30
+        rel = np.abs(g[big] - w[big]) / np.abs(w[big])
+        # tanh near 0 is a difference of nearly equal numbers in both forms: relative error only where |tanh| >= 0.01
+        if w is want_t:
+            rel = rel[np.abs(w[big]) >= 0.01]
+        assert rel.max() <= (1e-4 if quick else 2e-5)   # the device's and the host's expf differ by an ulp or two
+        # the clamps are exact in both forms
+        assert np.all(g[xs <= -88.73] == (0.0 if w is want_l else -1.0))
+        assert np.all(g[xs >= 88.73] == 1.0)
+
+
 def test_lstm_config1_unidirectional():
     """benchmark config 1: P=382, H=256, T=200, S=4 with one sequence of 150 frames."""
     print("lstm config 1", flush=True)

@@ -43,6 +43,34 @@ def test_static_scratch_entry_point_two_calls_second_smaller():
     _one_call(capi, 33, 7, 90, 1.0, seed=3)       # a single split
 
 
+def test_static_scratch_entry_point_takes_no_device_memory():
+    """The device's free memory as the driver reports it is the same before and after calls of the entry point (a first
+    call has been made, so the code object and its array are loaded); the allocating entry point beside it, called on a
+    stream that has no scratch buffer yet, is seen to take its 16 MB, which shows that the probe can see an allocation."""
+    import torch
+
+    capi = PC.pkg().capi
+    P, D, N = 128, 256, 6000
+    rng = np.random.default_rng(5)
+    xd = PC.dev(rng.standard_normal(P * N).astype(np.float32))
+    ed = PC.dev(rng.standard_normal(D * N).astype(np.float32))
+    dW = torch.zeros(P * D + D, dtype=torch.float32, device="cuda")
+    capi.dense_backward_weights_static(P, D, N, 1.0, xd, ed, dW)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        capi.dense_backward_weights_static(P, D, N, 1.0, xd, ed, dW)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0
+    stream = torch.cuda.Stream()   # a stream the library has not seen: its first split product allocates the scratch
+    capi.dense_backward_weights(P, D, N, 1.0, xd, ed, dW, stream=stream)
+    torch.cuda.synchronize()
+    free2, _ = torch.cuda.mem_get_info()
+    capi.gemm_release(stream)
+    assert free0 - free2 >= 16 << 20
+
+
 def test_static_scratch_entry_point_rejects_oversized_layers():
     import torch
 
