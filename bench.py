@@ -30,21 +30,46 @@ sys.path.insert(0, os.path.join(ROOT, "oracle"))  # the CPU checker: imported on
 
 import numpy as np  # noqa: E402
 
-# HBM bytes one launch of the backward recursion kernel moves on this workload (T=588, S=10, H=256, two directions),
+# HBM bytes one launch of the backward recursion kernel moves on this workload (T=600, S=10, H=256, two directions),
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a copy of known size; the figure and the command
 # that made it are in the profile named here.  Algorithmic bytes of the same launch: 120 MB.  None = not measured
 # for the kernel this tree runs.
 CHAIN_TRAFFIC_BYTES = 173.6e6  # (47 440 KiB x 2.00 fetched + 74 690 KiB written) per launch of lstm_backward_local<256, 8>
 CHAIN_TRAFFIC_SOURCE = "profiles/acoustic_backward_hbm_traffic.md"
+# The counters were read for this kernel, built from this source text (first 16 hex digits of the SHA-256 of
+# csrc/lstm_local.hpp); when the file has changed since, the figure no longer describes the kernel that runs and the
+# benchmark prints null for it.
+CHAIN_TRAFFIC_KERNEL = "lstm_backward_local<256, 8>"
+CHAIN_TRAFFIC_SOURCE_SHA16 = "5ff49375364c1571"
 
 METRIC = "BLSTM backward frames/sec at 1 MI355X; % HBM/MFMA roofline vs host CPU"
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
 
-def make_fraction(seed, S, Tmax, Tlo, in_dim, out_dim):
+def chain_traffic():
+    """(bytes per launch, what they were measured on), or (None, why not) when the kernel's source has changed since."""
+    import hashlib
+
+    path = os.path.join(ROOT, "project-currennt-public_amd", "csrc", "lstm_local.hpp")
+    try:
+        with open(path, "rb") as f:
+            now = hashlib.sha256(f.read()).hexdigest()[:16]
+    except OSError:
+        now = None
+    measured_on = {"kernel": CHAIN_TRAFFIC_KERNEL, "source_sha16": CHAIN_TRAFFIC_SOURCE_SHA16, "profile": CHAIN_TRAFFIC_SOURCE}
+    if now != CHAIN_TRAFFIC_SOURCE_SHA16:
+        measured_on["stale"] = "csrc/lstm_local.hpp is now %s: the counters have not been read for this kernel" % now
+        return None, measured_on
+    return CHAIN_TRAFFIC_BYTES, measured_on
+
+
+def make_fraction(seed, S, Tmax, Tlo, in_dim, out_dim, pin_longest=False):
     rng = np.random.default_rng(seed)
     lengths = [int(v) for v in rng.integers(Tlo, Tmax + 1, size=S)]
+    if pin_longest:
+        # the fraction is as long as the configuration says: the longest draw is made Tmax
+        lengths[lengths.index(max(lengths))] = Tmax
     T = max(lengths)
     x = rng.standard_normal((T, S, in_dim)).astype(np.float32)
     tgt = rng.standard_normal((T, S, out_dim)).astype(np.float32)
@@ -140,7 +165,7 @@ def main():
 
     S, Tmax, seed = 10, 600, 20240
     input_size, specs = pkg.specs.acoustic_model_spec()
-    lengths, T, x, tgt, pat = make_fraction(seed, S, Tmax, 300, input_size, 187)
+    lengths, T, x, tgt, pat = make_fraction(seed, S, Tmax, 300, input_size, 187, pin_longest=True)
     frames = sum(lengths)
 
     # the network file a user of the reference would write for this model, handed to the library's sequencer
@@ -216,8 +241,9 @@ def main():
         hop_bare_us = probe(same_xcd=True, with_compute=False)
         hop_far_us = probe(same_xcd=False, with_compute=False)
         us_per_step = 1e3 * kernels[dom]["avg_ms"] / T
+        traffic, measured_on = chain_traffic()
         roof = {"bound": "mfma", "achieved": flops / dom_avg_s / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "traffic": CHAIN_TRAFFIC_BYTES, "traffic_source": CHAIN_TRAFFIC_SOURCE,
+                "unit": "TFLOP/s", "traffic": traffic, "traffic_measured_on": measured_on,
                 "kernel": dom,
                 "us_per_step": us_per_step,
                 "latency_floor_us_per_step": hop_us,

@@ -204,7 +204,7 @@ def dft_c5(args, pkg):
     sec = _timed(step, args.steps, args.warmup)
     kernels = _profile(capi, step, args.steps)
     dom = "dft_loss"
-    nbytes = 12.0 * W * n  # per launch = one resolution: read source + target, write gradient
+    nbytes = 12.0 * W * n  # per launch (all three resolutions in it): read source + target once, write the gradient once
     ach = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
     # traffic: two rocprofv3 --pmc runs of this workload (FETCH_SIZE x 2.00 by a copy of known size, WRITE_SIZE x 1.00):
     # dft_loss_kernel 6.3 MB read (every sample is part of four frames per resolution) + 6.3 MB written (overlap-add)

@@ -86,6 +86,10 @@ int cnt_dense_backward_weights(void *stream, int P, int D, int N, float bias, co
  * memory, a stream under capture) adds its splits atomically instead. */
 int cnt_gemm_reserve(void *stream);
 int cnt_gemm_release(void *stream);
+/* How many such buffers the library holds at the moment.  That allocation is the only one any entry point other
+ * than a *_create call makes, so a caller (or a test) that sees the same number before and after a pass knows that
+ * the pass allocated nothing.  No counterpart in the reference. */
+int cnt_gemm_scratch_buffers(void);
 /* cnt_dense_backward_weights for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc): same arguments, same result, but the split partial products go
  * through an 8 MB array that is part of the library's code object (one copy per GPU, held until the process ends),

@@ -72,6 +72,7 @@ _SIGNATURES = {
     "cnt_probe_activation": (I, [VP, I, C.c_long, VP, VP]),
     "cnt_gemm_reserve": (I, [VP]),
     "cnt_gemm_release": (I, [VP]),
+    "cnt_gemm_scratch_buffers": (I, []),
     "cnt_sse_backward": (I, [VP, I, I, VP, VP, VP, VP]),
     "cnt_sse_error": (I, [VP, I, I, VP, VP, VP, VP]),
     "cnt_dataset_open": (I, [C.c_char_p, C.POINTER(DatasetDesc), C.POINTER(VP)]),

@@ -195,6 +195,8 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args);
 void gemm_release_stream(hipStream_t stream);
 // Allocates the split-K scratch buffer of `stream` now instead of inside the first product that wants it.
 int gemm_reserve_stream(hipStream_t stream);
+// number of split-K scratch buffers the library holds at the moment (one per stream that has needed or reserved one)
+int gemm_scratch_buffers();
 // cnt_dense_backward_weights with the partial products in a scratch array that is part of the code object
 int gemm_dense_weights_static(hipStream_t stream, int P, int D, int N, float bias, const float *x, const float *err,
                               float *weight_updates);

@@ -257,6 +257,8 @@ int cnt_dense_backward_weights_static(void *stream, int P, int D, int N, float b
 
 int cnt_gemm_reserve(void *stream) { return cnt::gemm_reserve_stream(static_cast<hipStream_t>(stream)); }
 
+int cnt_gemm_scratch_buffers(void) { return cnt::gemm_scratch_buffers(); }
+
 int cnt_gemm_release(void *stream) {
     cnt::gemm_release_stream(static_cast<hipStream_t>(stream));
     return CNT_OK;

@@ -190,6 +190,11 @@ int gemm_reserve_stream(hipStream_t stream) {
     return CNT_OK;
 }
 
+int gemm_scratch_buffers() {
+    std::lock_guard<std::mutex> lock(g_split_mu);
+    return (int)g_split_scratch.size();
+}
+
 void gemm_plan(GemmArgs &args, hipStream_t stream) {
     if (args.splitk != 0) return;
     // Long-K products with a small output (weight gradients): cut K so that the launch has about

@@ -10,6 +10,7 @@
 // (currennt/src/main.cpp:692-695 catches it).  Device memory is plain hipMalloc.
 #pragma once
 
+#include <cstdlib>
 #include <hip/hip_runtime.h>
 
 #include <cstddef>
@@ -136,7 +137,12 @@ public:
     TrainableLayer(const std::string &name, int size, int parallelSequences, int maxSeqLength, Layer *preceding,
                    hipStream_t stream, size_t weightCount, float bias)
         : Layer(name, size, parallelSequences, maxSeqLength, preceding, stream), m_bias(bias), m_weights(weightCount),
-          m_weightUpdates(weightCount) {}
+          m_weightUpdates(weightCount) {
+        // a weight gradient may go through split partial products: the stream's scratch buffer for them is allocated
+        // here, at construction (once per stream, later calls find it), so that no computeBackwardPass allocates
+        // (CNT_HOST_NO_RESERVE leaves it to the first product that needs it: how the test sees the difference)
+        if (!std::getenv("CNT_HOST_NO_RESERVE")) check(cnt_gemm_reserve(stream), "gemm reserve");
+    }
     real_vector &weights() { return m_weights; }
     real_vector &weightUpdates() { return m_weightUpdates; }
     float bias() const { return m_bias; }

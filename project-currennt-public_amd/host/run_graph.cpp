@@ -168,11 +168,20 @@ int main(int argc, char **argv) {
         fr.targets = read_file<float>(dir + "targets.bin", (size_t)post->size() * T * S);
         net.loadSequences(fr);
         if (first_core) first_core->loadContext(read_file<float>(dir + "context.bin", (size_t)context_dim * T * S));
+        // Everything is allocated at construction: the library's only allocation on the path of a pass is a stream's
+        // scratch buffer for split products, and the number of those it holds is the same before and after the passes.
+        // (The device's free memory still drops over a first pass: the runtime loads each code object of the library at
+        // the first launch of one of its kernels.)
+        hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize");
+        size_t free_before = 0, free_after = 0, total = 0;
+        hip_check(hipMemGetInfo(&free_before, &total), "hipMemGetInfo");
+        const int scratch_before = cnt_gemm_scratch_buffers();
         net.computeForwardPass();
         const float loss = post->calculateError();
         net.computeBackwardPass();
         for (LstmLayer *l : lstms) l->synchronizeAndCheck();
         hip_check(hipStreamSynchronize(stream), "hipStreamSynchronize");
+        hip_check(hipMemGetInfo(&free_after, &total), "hipMemGetInfo");
 
         {
             std::ofstream o(dir + "loss.txt");
@@ -186,7 +195,9 @@ int main(int argc, char **argv) {
             write_file(dir + l.name() + ".err.bin", l.outputErrors().to_host(), n);
         }
         for (TrainableLayer *t : trainable) write_file(dir + t->name() + ".dW.bin", t->weightUpdates().to_host(), t->weightUpdates().size());
-        std::printf("run_graph ok: %zu layers, loss %.6f\n", net.size(), loss);
+        std::printf("run_graph ok: %zu layers, loss %.6f, scratch buffers allocated during the passes: %d, device memory taken "
+                    "(code objects included): %lld bytes\n", net.size(), loss, cnt_gemm_scratch_buffers() - scratch_before,
+                    (long long)free_before - (long long)free_after);
         return 0;
     } catch (const std::exception &e) {
         // same wording as the reference's top-level handler (currennt/src/main.cpp:692-695)

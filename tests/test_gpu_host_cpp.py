@@ -90,15 +90,49 @@ def _graph_driver():
     return driver
 
 
-def _run_graph(tmp_path, statements, files):
+_last_stdout = [""]
+
+
+def _run_graph(tmp_path, statements, files, env=None):
     with open(tmp_path / "job.txt", "w") as f:
         f.write("\n".join(statements) + "\n")
     for name, arr in files.items():
         np.ascontiguousarray(arr).tofile(tmp_path / name)
-    r = subprocess.run([_graph_driver(), str(tmp_path)], capture_output=True, text=True, timeout=100)
+    r = subprocess.run([_graph_driver(), str(tmp_path)], capture_output=True, text=True, timeout=100,
+                       env=dict(os.environ, **(env or {})))
     print(r.stdout, r.stderr, flush=True)
     assert r.returncode == 0
+    _last_stdout[0] = r.stdout
     return float(open(tmp_path / "loss.txt").read())
+
+
+def _scratch_buffers_allocated():
+    import re
+
+    return int(re.search(r"scratch buffers allocated during the passes: (-?\d+)", _last_stdout[0]).group(1))
+
+
+def test_cpp_shells_allocate_at_construction_not_in_a_pass(tmp_path):
+    """A dense layer over 4096 slots: its weight gradient is a split product whose partial products go through the
+    stream's scratch buffer, the only allocation the library makes outside its *_create calls.  The shells reserve that
+    buffer when they are constructed, so the driver sees the library hold as many buffers after forward + backward as
+    before; with the reservation switched off the first backward pass allocates one, which shows that the driver would
+    see it."""
+    print("c++ shells: no allocation inside a pass", flush=True)
+    S, T, P, D = 2, 2048, 32, 48
+    rng = np.random.default_rng(11)
+    pat = np.full(T * S, 2, dtype=np.int8)
+    x = rng.standard_normal(P * T * S).astype(np.float32)
+    tgt = rng.standard_normal(D * T * S).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, P * D + D).astype(np.float32)
+    st = ["geometry %d %d %d" % (S, T, T), "input %d" % P, "ff out 0 %d 1.0" % D, "post sse"]
+    files = {"pat.bin": pat, "input.bin": x, "targets.bin": tgt, "out.W.bin": w}
+    _run_graph(tmp_path, st, files)
+    assert _scratch_buffers_allocated() == 0
+    dW = _result(tmp_path, "out", "dW")
+    _run_graph(tmp_path, st, files, env={"CNT_HOST_NO_RESERVE": "1"})
+    assert _scratch_buffers_allocated() == 1
+    assert PC.relerr(_result(tmp_path, "out", "dW"), dW) < 1e-6
 
 
 def _result(tmp_path, name, kind):
