@@ -221,8 +221,12 @@ typedef struct {
 /* MDNLayer::MDNLayer (layers/MDNLayer.cu:280-324, 457-545). */
 int cnt_mdn_create(const cnt_mdn_desc *desc, const float *config, int config_len, cnt_mdn **out);
 int cnt_mdn_destroy(cnt_mdn *h);
-/* Variance floor of a mixture unit (MDNUnit.cu:5233-5234 sets it when the network has no trained
- * weights; it is 0 otherwise). */
+/* Variance floor of a mixture unit.  The reference derives it from data -- MDNUnit_mixture::initPreOutput
+ * (layers/MDNUnit.cu:5146-5234: vFloorPara (1e-4) times the mean standard deviation of the target dimensions) --
+ * and only when the network file holds no "weights" section (NeuralNetwork.cpp:1047-1048, :3649-3664); it is 0 for
+ * a network that starts from trained weights.  That pass over the training targets is not part of this library: a
+ * caller that trains from scratch computes the statistic (the reference's own mean / variance file, e.g.) and hands
+ * the floor over here; left alone it is 0, as when training resumes from a weights file. */
 int cnt_mdn_set_var_floor(cnt_mdn *h, int unit, float var_floor);
 /* Layer::loadSequences: records the fraction's pattern types (device memory, char[curMaxT*S]). */
 int cnt_mdn_load_sequences(cnt_mdn *h, void *stream, const char *patTypes, int curMaxT);
@@ -506,6 +510,12 @@ typedef struct {
 } cnt_dataset_desc;
 int cnt_dataset_open(const char *nc_path, const cnt_dataset_desc *desc, cnt_dataset **out);
 int cnt_dataset_close(cnt_dataset *d);
+/* DataSet::_shuffleSequences and _shuffleFractions (data_sets/DataSet.cpp:491-514), which the reference runs at the
+ * start of every epoch when --shuffle_sequences / --shuffle_fractions are set (:1026-1031): the order of the
+ * sequences is permuted, then the order of the groups of parallel_sequences consecutive sequences.  One generator
+ * per data set, seeded by the first call (--random_seed); the permutations are seeded and repeatable but not the
+ * reference's own, whose draws come from boost's generators. */
+int cnt_dataset_shuffle(cnt_dataset *d, int shuffle_sequences, int shuffle_fractions, unsigned seed);
 /* DataSet::totalSequences / inputPatternSize / outputPatternSize / isClassificationData / totalTimesteps /
  * minSeqLength / maxSeqLength (data_sets/DataSet.hpp); any pointer may be NULL. */
 int cnt_dataset_info(cnt_dataset *d, int *num_sequences, int *input_size, int *output_size, int *is_classification,

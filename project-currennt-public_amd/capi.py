@@ -77,6 +77,7 @@ _SIGNATURES = {
     "cnt_sse_error": (I, [VP, I, I, VP, VP, VP, VP]),
     "cnt_dataset_open": (I, [C.c_char_p, C.POINTER(DatasetDesc), C.POINTER(VP)]),
     "cnt_dataset_close": (I, [VP]),
+    "cnt_dataset_shuffle": (I, [VP, I, I, C.c_uint]),
     "cnt_dataset_info": (I, [VP, C.POINTER(I), C.POINTER(I), C.POINTER(I), C.POINTER(I), C.POINTER(C.c_long),
                              C.POINTER(I), C.POINTER(I)]),
     "cnt_dataset_sequence": (I, [VP, I, C.POINTER(I), C.POINTER(I), C.c_char_p, I]),
@@ -276,6 +277,10 @@ class Dataset:
         self.num_sequences, self.input_size, self.output_size = n.value, p.value, q.value
         self.is_classification, self.total_timesteps = bool(cls.value), tot.value
         self.min_len, self.max_len = mn.value, mx.value
+
+    def shuffle(self, sequences, fractions, seed=0):
+        """What the reference does at the start of an epoch with --shuffle_sequences / --shuffle_fractions."""
+        check(lib().cnt_dataset_shuffle(self.handle, int(sequences), int(fractions), seed))
 
     def sequence(self, index):
         length, orig = I(), I()

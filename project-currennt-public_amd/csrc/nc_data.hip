@@ -19,6 +19,7 @@
 // noise injection, external / auxiliary data, sequence and fraction shuffling, ordered file lists.
 #include "common.hpp"
 
+#include <random>
 #include <algorithm>
 #include <cerrno>
 #include <cstring>
@@ -233,6 +234,8 @@ struct cnt_dataset {
     long total_timesteps;
     int min_len, max_len;
     std::vector<cnt::Sequence> sequences;
+    std::mt19937 shuffle_gen;  // one generator for every shuffle of this data set, seeded by the first one
+    bool shuffle_seeded = false;
 };
 
 namespace {
@@ -317,6 +320,48 @@ int cnt_dataset_open(const char *nc_path, const cnt_dataset_desc *desc, cnt_data
         std::stable_sort(d->sequences.begin(), d->sequences.end(),
                          [](const Sequence &a, const Sequence &b) { return a.length < b.length; });
     *out = d;
+    return CNT_OK;
+}
+
+// DataSet::_shuffleSequences / _shuffleFractions (data_sets/DataSet.cpp:491-514), run by the reference at the start of
+// every epoch (:1026-1031): first the sequences are shuffled, then the groups of parallel_sequences consecutive
+// sequences, whose concatenation becomes the new order (a last, shorter group may land in the middle, and the
+// fractions after it then straddle the old groups, as in the reference).  The shuffle is the one std::random_shuffle
+// of libstdc++ runs -- element i changes places with a uniformly drawn element of 0..i -- on one Mersenne twister per
+// data set that the first call seeds (the reference seeds one per process from --random_seed and draws through
+// boost::uniform_int, so the permutations themselves are not the reference's).
+int cnt_dataset_shuffle(cnt_dataset *d, int shuffle_sequences, int shuffle_fractions, unsigned seed) {
+    using namespace cnt;
+    CNT_REQUIRE(d, "dataset_shuffle: null handle");
+    if (!d->shuffle_seeded) {
+        d->shuffle_gen.seed(seed);
+        d->shuffle_seeded = true;
+    }
+    auto below = [&](size_t n) {  // uniform in 0 .. n-1, without modulo bias
+        const unsigned long long span = 0x100000000ull, lim = span - span % n;
+        unsigned long long r;
+        do r = d->shuffle_gen(); while (r >= lim);
+        return (size_t)(r % n);
+    };
+    auto shuffle = [&](auto &v) {
+        for (size_t i = 1; i < v.size(); ++i) {
+            const size_t j = below(i + 1);
+            if (i != j) std::swap(v[i], v[j]);
+        }
+    };
+    if (shuffle_sequences) shuffle(d->sequences);
+    if (shuffle_fractions) {
+        const size_t S = (size_t)d->desc.parallel_sequences;
+        std::vector<std::vector<Sequence>> groups;
+        for (size_t i = 0; i < d->sequences.size(); ++i) {
+            if (i % S == 0) groups.emplace_back();
+            groups.back().push_back(d->sequences[i]);
+        }
+        shuffle(groups);
+        d->sequences.clear();
+        for (const auto &g : groups)
+            for (const auto &q : g) d->sequences.push_back(q);
+    }
     return CNT_OK;
 }
 

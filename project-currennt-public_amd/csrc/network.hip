@@ -463,6 +463,7 @@ struct cnt_network {
     // conditioning sub-network: the layer flagged "wavenetConditionInputLayer" feeds the wavnetc layers
     int flagged = -1, first_wavnetc = -1;
     float *ctx_own = nullptr, *ctx_grad = nullptr;
+    float *ctx_mv = nullptr;  // the first wavnetc layer's "contextMV": [means | standard deviations] (device), or NULL
     struct LowRes { int res; char *pat; };
     std::vector<LowRes> low_res;
     std::vector<void *> allocations;
@@ -681,8 +682,27 @@ int build_layer_into(cnt_network *net, NetLayer &L, const json::Value &obj, cons
         CNT_REQUIRE(P == 2 * L.size, "network: wavnetc layer '%s' of size %d needs a preceding layer of size %d",
                     L.name.c_str(), L.size, 2 * L.size);
         CNT_REQUIRE(L.res == 1, "network: wavnetc layer '%s' must have resolution 1", L.name.c_str());
-        CNT_REQUIRE(get_str(obj, "contextMV").empty(), "network: wavnetc layer '%s': contextMV is not built",
-                    L.name.c_str());
+        // "contextMV": a file of contextDim means followed by contextDim standard deviations, raw float32
+        // (layers/wavNetCore.cu:322-332, :343-351); every such layer reads its file, the first one's is the one in use
+        // (:455-492: only the initial core fills the shared conditioning buffer)
+        const std::string mv_path = get_str(obj, "contextMV");
+        if (!mv_path.empty() && L.ctx_dim > 0) {
+            std::vector<float> mv;
+            if (FILE *f = std::fopen(mv_path.c_str(), "rb")) {
+                float v;
+                while (mv.size() <= 2 * (size_t)L.ctx_dim && std::fread(&v, sizeof(v), 1, f) == 1) mv.push_back(v);
+                std::fclose(f);
+            } else {
+                set_error("network: wavnetc layer '%s': cannot open contextMV file %s", L.name.c_str(), mv_path.c_str());
+                return CNT_ERR_ARG;
+            }
+            CNT_REQUIRE(mv.size() == 2 * (size_t)L.ctx_dim, "network: wavnetc layer '%s': context mean variance dim unequal "
+                        "(%s does not hold 2 x %d floats)", L.name.c_str(), mv_path.c_str(), L.ctx_dim);
+            if (net->first_wavnetc < 0) {
+                CNT_TRY(device_alloc(net, (void **)&net->ctx_mv, mv.size() * sizeof(float), false));
+                CNT_HIP(hipMemcpy(net->ctx_mv, mv.data(), mv.size() * sizeof(float), hipMemcpyHostToDevice));
+            }
+        }
         if (net->first_wavnetc < 0) net->first_wavnetc = index;
         NetLayer &before = net->layers[(size_t)index - 1];
         if (before.kind == K_CNN && before.cnn_tanh) before.delta_fused = true;
@@ -1152,6 +1172,10 @@ int cnt_network_set_context(cnt_network *net, const float *ctx) {
     CNT_REQUIRE(net, "network_set_context: null handle");
     CNT_REQUIRE(net->flagged < 0, "network_set_context: this network computes the conditioning features itself (layer "
                 "'%s')", net->layers[(size_t)net->flagged].name.c_str());
+    // features handed over one column per slot are used where they stand; mean and deviation of a "contextMV" file
+    // are applied where the library up-samples frame-rate features itself
+    CNT_REQUIRE(!net->ctx_mv, "network_set_context: the wavnetc layers name a contextMV file; hand over normalised features "
+                "and drop the key, or let the network up-sample them (layerFlag wavenetConditionInputLayer)");
     net->ctx = ctx;
     return CNT_OK;
 }
@@ -1277,7 +1301,7 @@ int cnt_network_forward(cnt_network *net, void *stream_) {
                     const NetLayer &f = net->layers[(size_t)net->flagged];
                     CNT_TRY(fill_zero(stream, net->ctx_grad, (size_t)L.ctx_dim * N));
                     CNT_TRY(cnt_wavnetc_load_context(stream, L.ctx_dim, net->S, N, f.T, f.res == 1 ? 1 : 0, f.out,
-                                                     net->layers.front().out, nullptr, L.pat, net->ctx_own));
+                                                     net->layers.front().out, net->ctx_mv, L.pat, net->ctx_own));
                 }
                 CNT_TRY(cnt_wavnetc_forward(stream, L.size, L.ctx_dim, N, L.pat, W, net->ctx, prev.out, L.core, L.cth,
                                             L.out));

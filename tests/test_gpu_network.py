@@ -389,13 +389,16 @@ class _CondOracleBackend(OM.OracleBackend):
         O.wavnetc_backward(D, C, N, pat, W, ctx, core, cth, err, prev_err, dW, self.ctx_grad)
 
 
-def test_wavenet_with_frame_rate_conditioning_network():
+@pytest.mark.parametrize("context_mv", [False, True])
+def test_wavenet_with_frame_rate_conditioning_network(context_mv, tmp_path):
     """The reference example's layout in full: externalloader -> skipini -> blstm -> cnn -> skipcat at one slot per
     R time steps, flagged as the wavnetc layers' input; the oracle side walks the same graph with the oracle's
-    primitives (conditioning part spelled out here, sample-rate part by the shared graph walk)."""
+    primitives (conditioning part spelled out here, sample-rate part by the shared graph walk).  With context_mv the
+    wavnetc layers name a "contextMV" file (means and standard deviations of the conditioning features, one of them
+    vanishing), which the first of them applies while it up-samples (layers/wavNetCore.cu:143-190, :322-351)."""
     import torch
 
-    print("wavenet network file with conditioning sub-network", flush=True)
+    print("wavenet network file with conditioning sub-network, contextMV", context_mv, flush=True)
     pkg = PC.pkg()
     capi, networks = pkg.capi, PC.networks()
     nb, Q, R, K = 3, 64, 32, 64
@@ -433,7 +436,12 @@ def test_wavenet_with_frame_rate_conditioning_network():
     O.cnn_forward(HB, DC, S, Tr, 0, 0, 1.0, hw, it, pat_r, w_cnn, l2, con, l3)
     cat = np.concatenate([l3.reshape(Nr, DC), ext.reshape(Nr, E)[:, 11:12]], axis=1).astype(np.float32)
     ctx = np.zeros(C * N, dtype=np.float32)
-    O.wavnetc_load_context(C, S, N, Tr, False, np.ascontiguousarray(cat.reshape(-1)), frame_index.reshape(-1), None, pat, ctx)
+    ctx_mv = None
+    if context_mv:
+        ctx_mv = np.concatenate([0.2 * rng.standard_normal(C), rng.uniform(0.4, 1.5, C)]).astype(np.float32)
+        ctx_mv[C + 2] = 1e-6   # a vanishing deviation counts as 1
+        ctx_mv.tofile(tmp_path / "context.mv")
+    O.wavnetc_load_context(C, S, N, Tr, False, np.ascontiguousarray(cat.reshape(-1)), frame_index.reshape(-1), ctx_mv, pat, ctx)
 
     # ---- oracle: sample-rate part --------------------------------------------------------------------------------
     backend = _CondOracleBackend()
@@ -473,6 +481,15 @@ def test_wavenet_with_frame_rate_conditioning_network():
              "preSkipLayer": "exL3,exSkip", "preSkipLayerDim": "0_%d_11_12" % DC,
              "layerFlag": "wavenetConditionInputLayer"}]
     doc["layers"] = doc["layers"][:1] + cond + doc["layers"][1:]
+    if context_mv:
+        for layer in doc["layers"]:
+            if layer["type"] == "wavnetc":
+                layer["contextMV"] = str(tmp_path / "context.mv")
+        bad = json.loads(json.dumps(doc))
+        (tmp_path / "short.mv").write_bytes(ctx_mv[:-1].tobytes())
+        [l for l in bad["layers"] if l["type"] == "wavnetc"][1]["contextMV"] = str(tmp_path / "short.mv")
+        with pytest.raises(RuntimeError, match="mean variance dim unequal"):
+            capi.Network(json.dumps(bad), S, T + 6, mdn_config=[1, 0, Q, 0, 1, -1])
     net = capi.Network(json.dumps(doc), S, T + 6, mdn_config=[1, 0, Q, 0, 1, -1])
     assert net.layer("exL2")["resolution"] == RES and net.layer("emb")["resolution"] == 1
     for L in net.layers:

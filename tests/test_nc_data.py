@@ -107,6 +107,60 @@ def test_reader_matches_oracle(tmp_path, version, classes, S, trunc, frac, train
         ds.close()
 
 
+def test_shuffling_permutes_sequences_and_fractions(tmp_path):
+    """DataSet::_shuffleSequences / _shuffleFractions (data_sets/DataSet.cpp:491-514): a sequence shuffle is a
+    permutation of the segment list, a fraction shuffle a permutation of the groups of S consecutive segments (the
+    short last group included, each group's inner order kept); both are repeatable for a seed, go on to another
+    permutation at the next epoch, and leave the fractions' contents those of the oracle for the new order."""
+    capi = load_package().capi
+    lengths = [5, 9, 3, 7, 11, 4, 8, 6, 10, 2, 12]
+    S = 3
+    p = str(tmp_path / "shuffle.nc")
+    write_nc(p, lengths, 4, 2, 1, seed=3)
+
+    def order(ds):
+        return [ds.sequence(i)[2] for i in range(ds.num_sequences)]
+
+    ds = capi.Dataset(p, S, training_mode=True)
+    base = order(ds)
+    groups = [tuple(base[i:i + S]) for i in range(0, len(base), S)]
+    ds.shuffle(False, True, seed=7)
+    after = order(ds)
+    assert sorted(after) == sorted(base) and after != base
+    # cut the new order back into the old groups: walk it group by group
+    seen, i = [], 0
+    while i < len(after):
+        g = next(g for g in groups if g[0] == after[i])
+        assert tuple(after[i:i + len(g)]) == g
+        seen.append(g)
+        i += len(g)
+    assert sorted(seen) == sorted(groups)
+    # the fractions of the new order are what the oracle builds for that order
+    by_tag = {s["tag"]: s for s in NF.segments(p, training_mode=True)}
+    new_segs = [by_tag[t] for t in after]
+    for first in range(0, ds.num_sequences, S):
+        got, want = ds.fraction(first), NF.make_fraction(p, new_segs, first, S)
+        for k in ("num_seqs", "max_len", "min_len", "total_length"):
+            assert got[k] == want[k], (first, k)
+        for k in ("patTypes", "inputs", "targets"):
+            assert np.array_equal(got[k], want[k]), (first, k)
+    ds.shuffle(True, False)
+    again = order(ds)
+    assert sorted(again) == sorted(base) and again != after
+    ds.close()
+    # repeatable: the same seed gives the same two epochs
+    twin = capi.Dataset(p, S, training_mode=True)
+    twin.shuffle(False, True, seed=7)
+    assert order(twin) == after
+    twin.shuffle(True, False)
+    assert order(twin) == again
+    twin.close()
+    other = capi.Dataset(p, S, training_mode=True)
+    other.shuffle(True, True, seed=8)
+    assert order(other) != after and sorted(order(other)) == sorted(base)
+    other.close()
+
+
 def test_reader_errors(tmp_path):
     capi = load_package().capi
     with pytest.raises(RuntimeError, match="Could not open"):
