@@ -78,3 +78,77 @@ def test_acoustic_model_forward_backward():
         worst = max(worst, e)
     net.close()
     assert worst < 1e-4
+
+
+def test_acoustic_model_full_size_against_oracle():
+    """benchmark configs[1] at its real size -- T = 600, S = 10, lengths drawn from 300..600 with one of them 600 --
+    through the library's network sequencer (the path bench.py times: side streams, split weight halves) against the
+    CPU oracle with its outputs shared out over the host's cores: the loss, every layer's outputs, errors and weight
+    gradients at 1e-4 L2-normalised."""
+    import json
+
+    import torch
+
+    import oracle_lib as O
+
+    print("acoustic model, full size, sequencer against the oracle", flush=True)
+    O.use_all_cores()
+    capi = PC.pkg().capi
+    input_size, specs = PC.pkg().specs.acoustic_model_spec()
+    S = 10
+    rng = np.random.default_rng(31)
+    lengths = [int(v) for v in rng.integers(300, 601, size=S)]
+    lengths[4] = 600
+    T = 600
+    x = rng.standard_normal((T, S, input_size)).astype(np.float32)
+    tgt = rng.standard_normal((T, S, 187)).astype(np.float32)
+    pat = np.zeros((T, S), dtype=np.int8)
+    for s_, n in enumerate(lengths):
+        x[n:, s_] = 0
+        tgt[n:, s_] = 0
+        pat[:n, s_] = 2
+        pat[0, s_] = 1
+        pat[n - 1, s_] = 3
+    x, tgt, pat = x.reshape(-1), tgt.reshape(-1), pat.reshape(-1)
+    weights = OM.init_weights(input_size, specs, 32, 0.08)
+
+    ref = OM.OracleNetwork(input_size, specs, S, T, min(lengths), pat, [w.copy() for w in weights])
+    ref.forward(x, tgt)
+    ref_loss = ref.error()
+    ref.backward()
+
+    layers = [{"size": input_size, "name": "input", "type": "input"}]
+    for i, sp in enumerate(specs):
+        layers.append(dict(sp, name="%s_%d" % (sp["type"], i + 1)))
+    net = capi.Network(json.dumps({"layers": layers}), S, T)
+    trainable = [L for L in net.layers if L["weight_count"]]
+    assert len(trainable) == len(weights)
+    for L, w in zip(trainable, weights):
+        L["weights"].copy_(torch.from_numpy(w))
+    net.load_sequences(torch.from_numpy(pat).cuda(), T, min(lengths), torch.from_numpy(x).cuda(), torch.from_numpy(tgt).cuda())
+    net.forward()
+    loss = float(net.calculate_error().item())
+    net.backward()
+    net.check()
+    torch.cuda.synchronize()
+    # The loss is a sum of 919 000 squares.  The reference's host path (and so the oracle) adds them one by one in fp32,
+    # which by itself is off by a few 1e-4 relative at this length; the library adds in a tree.  Both are therefore
+    # compared with the same sum in float64 over the oracle's outputs: the library at 1e-5, the oracle at 1e-3.
+    N = T * S
+    y64 = ref.layers[-2]["outputs"].astype(np.float64).reshape(N, 187)
+    valid = pat != 0
+    loss64 = 0.5 * float((((tgt.reshape(N, 187).astype(np.float64) - y64) ** 2)[valid]).sum())
+    assert abs(loss - loss64) <= 1e-5 * loss64
+    assert abs(ref_loss - loss64) <= 1e-3 * loss64
+    worst = 0.0
+    for g, r in zip(net.layers[1:], ref.layers):
+        if g["type"] == "sse":
+            continue
+        n = g["size"] * N
+        for what, a, b in (("outputs", g["outputs"][:n], r["outputs"]), ("errors", g["errors"][:n], r["errors"]),
+                           ("updates", g["updates"], r["updates"])):
+            e = PC.relerr(a.cpu().numpy(), b)
+            print("%-24s %-8s %.2e" % (g["name"], what, e), flush=True)
+            worst = max(worst, e)
+    net.close()
+    assert worst < 1e-4
