@@ -137,33 +137,32 @@ def mdn_c3(args, pkg):
     layer.calculate_error(td, res)
 
     def step():
-        # the gradient needs the posteriors the error pass leaves behind (MDNUnit.cu:6037-6193 before :6222), so a
-        # step is both
+        # the gradient needs the posteriors of the error pass (MDNUnit.cu:6037-6193 before :6222), so a step is both:
+        # one call, one pass over the parameters
+        layer.error_backward(td, res, err)
+
+    def step_two_calls():
         layer.calculate_error(td, res)
         layer.backward(td, err)
 
     sec = _timed(step, args.steps, args.warmup)
     kernels = _profile(capi, step, args.steps)
-    dom = max(("mdn_mixture_backward", "mdn_mixture_error"), key=lambda k: kernels[k]["avg_ms"])
-    # error pass: weights, means, deviations and targets in, M + 1 log-likelihood terms out;
-    # gradient pass: the same in plus those terms, Lp errors out
-    nbytes = F * ((Lp + D + M + 1) * 4 if dom == "mdn_mixture_error" else (Lp + M + 1 + D + Lp) * 4)
+    sec_two = _timed(step_two_calls, args.steps, args.warmup)
+    kernels.update(_profile(capi, step_two_calls, args.steps))
+    dom = "mdn_mixture_error_backward"
+    # weights, means, deviations and targets in; Lp errors and the M + 1 log-likelihood terms out
+    nbytes = F * (Lp + D + Lp + M + 1) * 4
     ach = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
     roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None,
             "kernel": dom}
-    if (F, M, D) == (6000, 16, 60):
-        # two rocprofv3 --pmc runs of this workload (FETCH_SIZE x 2.00 by a copy of known size, WRITE_SIZE x 1.00):
-        # error kernel 48.0 MB read + 0.4 MB written, gradient kernel 49.6 MB read + 47.3 MB written per launch
-        roof["traffic"] = 48.4e6 if dom == "mdn_mixture_error" else 96.9e6
-        roof["traffic_source"] = "profiles/mdn_c3_backward_kernel_stats.md"
 
     def full():
         layer.forward(xd)
-        layer.calculate_error(td, res)
-        layer.backward(td, err)
+        layer.error_backward(td, res, err)
 
     sec_full = _timed(full, args.steps, 1)
-    extra = {"roofline": roof, "kernels": kernels, "forward_error_backward_ms": 1e3 * sec_full}
+    extra = {"roofline": roof, "kernels": kernels, "forward_error_backward_ms": 1e3 * sec_full,
+             "error_then_backward_two_calls_ms": 1e3 * sec_two}
     if not args.no_cpu:
         import oracle_lib as O  # the checker, only for this reported baseline
 

@@ -239,6 +239,12 @@ int cnt_mdn_calculate_error(cnt_mdn *h, void *stream, const float *targets, floa
 /* MDNLayer::computeBackwardPass (layers/MDNLayer.cu:875-917): prev_errors is the preceding layer's
  * whole error buffer, Lp x (maxT*S); it is zero-filled and then receives every unit's gradient. */
 int cnt_mdn_backward(cnt_mdn *h, void *stream, const float *targets, float *prev_errors);
+/* MDNLayer::calculateError followed by MDNLayer::computeBackwardPass (layers/MDNLayer.cu:797-827, :875-917) as one
+ * call, for trainers that always run both: *result_dev, the units' buffers and prev_errors end up as after the two
+ * calls above.  A mixture unit of at most 16 components over at most 64 target dimensions (sizes and start columns
+ * multiples of four, buffers 16-byte aligned) reads its parameters once for both steps; any other layer runs the two
+ * calls one after the other. */
+int cnt_mdn_error_backward(cnt_mdn *h, void *stream, const float *targets, float *result_dev, float *prev_errors);
 /* Device pointer to a unit's buffer. which: 0 parameters (softmax: F*K probabilities; mixture:
  * [F*M weights | F*M*D means | F*M*D std]), 1 mixture log-likelihoods [F*M | F].  *count receives the
  * number of floats in use for the current fraction. */

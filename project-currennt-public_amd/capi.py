@@ -112,6 +112,7 @@ _SIGNATURES = {
     "cnt_mdn_forward": (I, [VP, VP, VP]),
     "cnt_mdn_calculate_error": (I, [VP, VP, VP, VP]),
     "cnt_mdn_backward": (I, [VP, VP, VP, VP]),
+    "cnt_mdn_error_backward": (I, [VP, VP, VP, VP, VP]),
     "cnt_mdn_unit_buffer": (VP, [VP, I, I, C.POINTER(C.c_long)]),
     "cnt_dft_create": (I, [C.POINTER(DftDesc), C.POINTER(VP)]),
     "cnt_dft_destroy": (I, [VP]),
@@ -676,6 +677,9 @@ class Mdn:
 
     def backward(self, targets, prev_errors, stream=None):
         check(lib().cnt_mdn_backward(self.handle, stream_ptr(stream), ptr(targets), ptr(prev_errors)))
+
+    def error_backward(self, targets, result, prev_errors, stream=None):
+        check(lib().cnt_mdn_error_backward(self.handle, stream_ptr(stream), ptr(targets), ptr(result), ptr(prev_errors)))
 
     def unit_buffer(self, unit, which):
         import torch

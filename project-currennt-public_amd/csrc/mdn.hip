@@ -413,6 +413,114 @@ __global__ void mixture_backward_kernel(UnitGeom g, const char *__restrict__ pat
     }
 }
 
+// Error and gradient of a mixture unit in ONE pass over its parameters (MDNUnit_mixture::calculateError followed by
+// ::computeBackward, layers/MDNUnit.cu:6036-6193, :6195-6416), for units of at most sixteen components and 64 target
+// dimensions whose data moves 16 bytes at a time.  A wave takes a frame; lane (m, p) holds the 16-byte vectors p, p+4,
+// p+8, p+12 of component m's means and deviations and of the targets in registers, so the 1936 parameters of a
+// benchmark frame are read once: the component's log-likelihood comes out of two quad steps, the frame's log-sum out
+// of a wave maximum and a wave sum, and the posterior turns the same registers into the errors.  What the two separate
+// kernels leave behind is left behind here as well (per-component log-likelihoods and log-sums in tmp, the summed
+// negative log-likelihood), with the same arithmetic as mixture_error_vec_kernel and mixture_backward_kernel<true>.
+constexpr int kFusedWaves = 8;  // measured on MI355X at 6000 frames: 4 -> 33.8 us, 8 -> 25.6 us, 16 -> 29.4 us
+__global__ __launch_bounds__(64 * kFusedWaves) void mixture_error_backward_kernel(UnitGeom g, const char *__restrict__ pat,
+                                                                                 const float *__restrict__ target,
+                                                                                 const float *__restrict__ para,
+                                                                                 float *__restrict__ tmp,
+                                                                                 float *__restrict__ result,
+                                                                                 float *__restrict__ errors) {
+    __shared__ float block_sum[kFusedWaves];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int M = g.M, D = g.D, MD = M * D, DV = D / 4, Lp = g.Lp;
+    const int p = lane & 3, m = lane >> 2;
+    const int unit_cols = M + 2 * MD;
+    const int f = blockIdx.x * kFusedWaves + wave;
+    float wave_total = 0.0f;
+    if (f < g.F) {
+        float *e = errors + (size_t)f * Lp + g.startD;
+        if (pat[f] == 0) {
+            // as in the two kernels: the distance pass leaves 0, the gradient pass the zeros described there
+            for (int k = lane; k < M; k += 64) {
+                tmp[(size_t)f * M + k] = 0.0f;
+                const long idx = (long)f * M + k;
+                const int col = (int)(idx % Lp);
+                if (col < g.startD || col >= g.startD + unit_cols) errors[idx] = 0.0f;
+            }
+            for (int i = lane; i < unit_cols; i += 64) e[i] = 0.0f;
+        } else {
+            const float gauss_const = (float)(D * log(2 * 3.141215) / 2.0);  // the reference's own value of pi
+            const float4 *t4 = reinterpret_cast<const float4 *>(target + (size_t)f * g.Lt + g.startDOut);
+            const float4 *mean4 = reinterpret_cast<const float4 *>(para + (size_t)g.F * M + (size_t)f * MD);
+            const float4 *sd4 = reinterpret_cast<const float4 *>(para + (size_t)g.F * M * (1 + D) + (size_t)f * MD);
+            const bool live = m < M;
+            const int mc = live ? m : 0;
+            float4 s[4], mu[4], tv[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int v = min(p + 4 * q, DV - 1);
+                s[q] = sd4[mc * DV + v]; mu[q] = mean4[mc * DV + v]; tv[q] = t4[v];
+            }
+            const float weight = para[(size_t)f * M + mc];
+            float dist = 0.0f, logsd = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (p + 4 * q >= DV) continue;
+                const float d0 = tv[q].x - mu[q].x, d1 = tv[q].y - mu[q].y, d2 = tv[q].z - mu[q].z, d3 = tv[q].w - mu[q].w;
+                dist += d0 * d0 / (s[q].x * s[q].x) * 0.5f; dist += d1 * d1 / (s[q].y * s[q].y) * 0.5f;
+                dist += d2 * d2 / (s[q].z * s[q].z) * 0.5f; dist += d3 * d3 / (s[q].w * s[q].w) * 0.5f;
+                logsd += safe_log(s[q].x) + safe_log(s[q].y) + safe_log(s[q].z) + safe_log(s[q].w);
+            }
+            dist += __shfl_xor(dist, 1); logsd += __shfl_xor(logsd, 1);
+            dist += __shfl_xor(dist, 2); logsd += __shfl_xor(logsd, 2);
+            float lp = logf(weight) - dist - gauss_const - logsd;
+            if (lp < lim::kLSmall) lp = lim::kLSmall;
+            if (live && p == 0) tmp[(size_t)f * M + m] = lp;
+            const float mx = wave_max(live ? lp : lim::kLogZero);
+            const float se = wave_sum((live && p == 0) ? expf(lp - mx) : 0.0f);
+            const float lsum = mx + logf(se);
+            if (lane == 0) {
+                tmp[(size_t)g.F * M + f] = lsum;
+                wave_total = -lsum;
+            }
+            const float post = safe_exp(lp - lsum);
+            if (live) {
+                if (p == 0) {
+                    float v = weight - post;
+                    // a padding frame fd with fd*M + m' == this index overwrites the value with 0 afterwards
+                    const long idx = (long)f * Lp + g.startD + m;
+                    const long fd = idx / M;
+                    if (fd < g.F && pat[fd] == 0) v = 0.0f;
+                    e[m] = v;
+                }
+                float4 *em4 = reinterpret_cast<float4 *>(e + M + (size_t)m * D);
+                float4 *es4 = reinterpret_cast<float4 *>(e + M + MD + (size_t)m * D);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int v = p + 4 * q;
+                    if (v >= DV) continue;
+                    const float muv[4] = {mu[q].x, mu[q].y, mu[q].z, mu[q].w}, sv[4] = {s[q].x, s[q].y, s[q].z, s[q].w};
+                    const float tt[4] = {tv[q].x, tv[q].y, tv[q].z, tv[q].w};
+                    float em[4], es[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        em[k] = post * (muv[k] - tt[k]) / sv[k] / sv[k];
+                        es[k] = (sv[k] > g.var_floor) ? post - em[k] * (muv[k] - tt[k]) : 0.0f;
+                    }
+                    em4[v] = make_float4(em[0], em[1], em[2], em[3]);
+                    es4[v] = make_float4(es[0], es[1], es[2], es[3]);
+                }
+            }
+        }
+    }
+    if (lane == 0) block_sum[wave] = wave_total;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kFusedWaves; w += 2) v += block_sum[w] + block_sum[w + 1];
+        if (v != 0.0f) atomicAdd(result, v);
+    }
+}
+
 }  // namespace
 }  // namespace cnt
 
@@ -617,6 +725,43 @@ int cnt_mdn_calculate_error(cnt_mdn *h, void *stream_, const float *targets, flo
                                    result_dev);
             }
         }
+        CNT_HIP(hipGetLastError());
+    }
+    return CNT_OK;
+}
+
+// calculateError and computeBackwardPass of the layer in one call: the same results in result_dev, the units' buffers
+// and prev_errors as cnt_mdn_calculate_error followed by cnt_mdn_backward.  A mixture unit of at most sixteen components
+// and 64 target dimensions with 16-byte aligned data takes both steps in one pass over its parameters; every other
+// unit runs its two kernels one after the other.
+int cnt_mdn_error_backward(cnt_mdn *h, void *stream_, const float *targets, float *result_dev, float *prev_errors) {
+    using namespace cnt;
+    CNT_REQUIRE(h && targets && result_dev && prev_errors, "mdn_error_backward: null argument");
+    CNT_REQUIRE(h->T > 0, "mdn_error_backward: load_sequences has not been called");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    bool all_fused = true;
+    for (auto &u : h->units) {
+        const UnitGeom g = unit_geom(h, u);
+        const bool fused = u.type > 0 && g.M <= 16 && g.D <= 64 && g.D % 4 == 0 && g.M % 4 == 0 && g.Lp % 4 == 0 &&
+                           g.Lt % 4 == 0 && g.startD % 4 == 0 && g.startDOut % 4 == 0 && aligned(targets) &&
+                           aligned(u.para) && aligned(prev_errors);
+        all_fused = all_fused && fused;
+    }
+    if (!all_fused) {
+        CNT_TRY(cnt_mdn_calculate_error(h, stream_, targets, result_dev));
+        return cnt_mdn_backward(h, stream_, targets, prev_errors);
+    }
+    const size_t used = (size_t)h->T * h->desc.S * h->desc.Lp;
+    const size_t cap = (size_t)h->desc.maxT * h->desc.S * h->desc.Lp;
+    CNT_TRY(fill_zero(stream, result_dev, 1));
+    if (!h->covers_all_columns) CNT_TRY(fill_zero(stream, prev_errors, used));
+    if (cap > used) CNT_TRY(fill_zero(stream, prev_errors + used, cap - used));
+    for (auto &u : h->units) {
+        const UnitGeom g = unit_geom(h, u);
+        ProfileScope prof(stream, "mdn_mixture_error_backward");
+        hipLaunchKernelGGL(mixture_error_backward_kernel, dim3((g.F + kFusedWaves - 1) / kFusedWaves), dim3(64 * kFusedWaves), 0,
+                           stream, g, h->pat, targets, u.para, u.tmp, result_dev, prev_errors);
         CNT_HIP(hipGetLastError());
     }
     return CNT_OK;

@@ -214,6 +214,7 @@ struct NetLayer {
     std::vector<int> cat_lo, cat_hi;         // skipcat: dimension range taken from each source
     const float *ext_data = nullptr;         // externalloader: [frame][sequence][dimension], set by the caller
     const float *ext_mean_std = nullptr;
+    bool mdn_errors_done = false;            // mdn: calculate_error has already written the preceding layer's errors
     int ext_frames = 0, index_load_method = 0;
     int cnn_tanh = 0;                        // cnn: "tanhoutput"
     bool delta_fused = false;                // cnn followed by a wavnetc layer: that layer writes this layer's delta
@@ -1317,6 +1318,7 @@ int cnt_network_forward(cnt_network *net, void *stream_) {
             }
             case K_MDN:
                 CNT_TRY(cnt_mdn_forward(L.mdn, stream, prev.out));
+                L.mdn_errors_done = false;  // new parameters: errors written for the old ones do not count
                 break;
             case K_GATED:
                 CNT_TRY(cnt_gatedact_forward(stream, L.size, N, L.pat, prev.out, L.out));
@@ -1346,6 +1348,14 @@ int cnt_network_calculate_error(cnt_network *net, void *stream_, float *loss_dev
         // distances of every resolution
         hipLaunchKernelGGL(sum_few_kernel, dim3(1), dim3(64), 0, stream, post.dft_error_count, post.dft_errors, loss_dev);
         CNT_HIP(hipGetLastError());
+        return CNT_OK;
+    }
+    // The error pass and the gradient pass of a mixture layer read the same parameters: with an error buffer to write
+    // to, both happen here, in one pass (cnt_mdn_error_backward), and the backward pass finds the layer's step done.
+    // The preceding layer's error buffer has no other writer between the forward pass and the backward pass.
+    if (last.err) {
+        CNT_TRY(cnt_mdn_error_backward(post.mdn, stream, post.out, loss_dev, last.err));
+        post.mdn_errors_done = true;
         return CNT_OK;
     }
     return cnt_mdn_calculate_error(post.mdn, stream, post.out, loss_dev);
@@ -1522,7 +1532,9 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                 CNT_TRY(cnt_sse_backward(stream, L.size, N, L.pat, prev.out, L.out, prev.err));
                 break;
             case K_MDN:
-                CNT_TRY(cnt_mdn_backward(L.mdn, stream, L.out, prev.err));
+                // already written by cnt_network_calculate_error of this fraction's forward pass
+                if (L.mdn_errors_done) L.mdn_errors_done = false;
+                else CNT_TRY(cnt_mdn_backward(L.mdn, stream, L.out, prev.err));
                 break;
             case K_DFT:
                 // writes the whole preceding error buffer: gradients up to the waveform's length, zeros beyond

@@ -263,7 +263,7 @@ def run_sse_case(D, lengths, seed):
     return abs(float(res.item()) - e_o) / max(abs(e_o), 1e-30)
 
 
-def run_mdn_mixture_case(lengths, M, D, extra, seed, var_floor=0.0, maxT=None):
+def run_mdn_mixture_case(lengths, M, D, extra, seed, var_floor=0.0, maxT=None, one_call=False):
     """Mixture unit at column `extra` of the feeding layer; returns worst error over parameters,
     log-likelihoods, loss and gradients.  Padding handling (exact zeros, the index collision) is part of
     the gradient comparison because the oracle reproduces the reference's sequential outcome."""
@@ -293,8 +293,11 @@ def run_mdn_mixture_case(lengths, M, D, extra, seed, var_floor=0.0, maxT=None):
     err_d = torch.full((maxT * S * Lp,), 9.0, dtype=torch.float32, device="cuda")
     layer.load_sequences(pd, T)
     layer.forward(xd)
-    layer.calculate_error(td, res)
-    layer.backward(td, err_d)
+    if one_call:
+        layer.error_backward(td, res, err_d)   # cnt_mdn_error_backward: both steps, one pass where the unit allows it
+    else:
+        layer.calculate_error(td, res)
+        layer.backward(td, err_d)
     torch.cuda.synchronize()
     valid = np.repeat(pat != 0, 1)
     para_d = layer.unit_buffer(0, 0).cpu().numpy()

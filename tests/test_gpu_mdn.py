@@ -18,14 +18,18 @@ TOL = 1e-4
     ([12, 7, 12], 8, 12, 4),       # every size a multiple of four behind four leading columns: the 16-byte path
     ([12, 7, 12], 8, 12, 2),       # the same unit two columns further on: not aligned, scalar path
 ])
-def test_mixture_unit(lengths, M, D, extra):
-    print("mdn mixture case", lengths, M, D, extra, flush=True)
-    assert PC.run_mdn_mixture_case(lengths, M, D, extra, seed=M + D) < TOL
+@pytest.mark.parametrize("one_call", [False, True])
+def test_mixture_unit(lengths, M, D, extra, one_call):
+    # one_call: error and gradient through cnt_mdn_error_backward (one pass over the parameters for the units of at most
+    # sixteen components whose data is 16-byte aligned, the two kernels in turn for the others)
+    print("mdn mixture case", lengths, M, D, extra, one_call, flush=True)
+    assert PC.run_mdn_mixture_case(lengths, M, D, extra, seed=M + D, one_call=one_call) < TOL
 
 
-def test_mixture_unit_variance_floor_and_short_fraction():
-    print("mdn floor case", flush=True)
-    assert PC.run_mdn_mixture_case([7, 5], 3, 4, 0, seed=3, var_floor=0.8, maxT=12) < TOL
+@pytest.mark.parametrize("M,D,one_call", [(3, 4, False), (3, 4, True), (4, 8, True)])
+def test_mixture_unit_variance_floor_and_short_fraction(M, D, one_call):
+    print("mdn floor case", M, D, one_call, flush=True)
+    assert PC.run_mdn_mixture_case([7, 5], M, D, 0, seed=3, var_floor=0.8, maxT=12, one_call=one_call) < TOL
 
 
 @pytest.mark.parametrize("lengths,K,extra", [([6, 6], 10, 0), ([9, 5, 7], 257, 3), ([30, 17], 1024, 0)])
