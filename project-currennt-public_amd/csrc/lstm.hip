@@ -31,6 +31,9 @@
 #include <new>
 #include <type_traits>
 #include <vector>
+#include <utility>
+#include <algorithm>
+#include <mutex>
 
 namespace cnt {
 namespace {
@@ -1069,6 +1072,7 @@ struct cnt_lstm {
     size_t lmail_words;
     int last_blocks;       // workgroups of the last recursion launch
     int warm;  // read the recursion's inputs once before the XCD-local backward recursion (CNT_LSTM_WARM=0: off)
+    int spread_lds;  // dynamic LDS the XCD-local recursion asks for so that a compute unit takes one of its workgroups
     int poll_delay_local;  // pause before the first poll of a step in the XCD-local recursion, units of 64 clocks
     // recorded behind every recursion launch: the failure latch is taken only once the launch that may have set it has
     // ended, so that no workgroup of that launch can set it (or the veto) again after the report
@@ -1182,7 +1186,12 @@ int warm_backward_inputs(const cnt_lstm *h, hipStream_t stream, const ChainParam
 }
 
 chain_kernel_t pick_local_kernel(int H, int &JB) {
-    if (H == 256) { JB = 8; return (chain_kernel_t)lstm_backward_local<256, 8>; }
+    if (H == 256) {
+        static const int wide = [] { const char *e = std::getenv("CNT_LSTM_LOCAL_JB"); return e ? std::atoi(e) : 8; }();
+        if (wide == 16) { JB = 16; return (chain_kernel_t)lstm_backward_local<256, 16>; }
+        JB = 8;
+        return (chain_kernel_t)lstm_backward_local<256, 8>;
+    }
     if (H == 128) { JB = 4; return (chain_kernel_t)lstm_backward_local<128, 4>; }
     if (H == 64) { JB = 4; return (chain_kernel_t)lstm_backward_local<64, 4>; }
     return nullptr;
@@ -1242,7 +1251,25 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
         const int blocks = (h->njobs * G + 8 * (G - 1) + 7) / 8 * 8;
         h->last_blocks = blocks;
         p.poll_delay = h->poll_delay_local;
-        hipLaunchKernelGGL(k, dim3(blocks), dim3(local_threads(h->H)), 0, stream, p);
+        // One workgroup per compute unit.  A team's workgroups take a step in lock-step, and two of them on one compute
+        // unit share its four matrix pipes and its path to the L2 at exactly the same moments: the dispatcher, left to
+        // itself, puts the 32 workgroups of a 256-cell team on 16-17 compute units, and a step then takes 1.55 us instead
+        // of 1.30 us (measured on MI355X, benchmark layer: 932 -> 781 us per launch).  What keeps a second workgroup of
+        // this kernel off a compute unit is its LDS request: the launch asks for a little more than half of a compute
+        // unit's LDS (unused dynamic shared memory), which still leaves room for two workgroups of a matrix product
+        // beside it.  CNT_LSTM_SPREAD_LDS sets the request in bytes (0: none).
+        const int spread_lds = h->spread_lds;
+        if (spread_lds > 0) {
+            static std::mutex mu;
+            static std::vector<std::pair<int, const void *>> done;
+            std::lock_guard<std::mutex> lock(mu);
+            const std::pair<int, const void *> key(h->device, reinterpret_cast<const void *>(k));
+            if (std::find(done.begin(), done.end(), key) == done.end()) {
+                CNT_HIP(hipFuncSetAttribute(key.second, hipFuncAttributeMaxDynamicSharedMemorySize, spread_lds));
+                done.push_back(key);
+            }
+        }
+        hipLaunchKernelGGL(k, dim3(blocks), dim3(local_threads(h->H)), (size_t)spread_lds, stream, p);
         CNT_HIP(hipGetLastError());
         CNT_HIP(hipEventRecord(h->launch_done, stream));
         h->launch_pending = 1;
@@ -1385,6 +1412,17 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     h->poll_delay_local = 11;
     h->warm = 1;
     if (const char *e = std::getenv("CNT_LSTM_WARM")) h->warm = std::atoi(e) != 0;
+    {
+        // a little more than half of a compute unit's LDS (160 KB on gfx950: 82 KB); the kernel's own few KB come on top
+        int per_cu = 0, dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&per_cu, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            per_cu = 0;
+        }
+        h->spread_lds = per_cu >= (64 << 10) ? per_cu / 2 + 2048 : 0;
+        if (const char *e = std::getenv("CNT_LSTM_SPREAD_LDS")) h->spread_lds = std::atoi(e);
+    }
     if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY")) h->poll_delay = h->poll_delay_local = std::atoi(e);
     // forward recursion: the senders' cell update (a few hundred clocks) plus store visibility
     // measured optima on MI355X: 26 at H=256 (S=10 and S=4), 25-26 at H=128 (S=8), 24 at H=64 (S=6); two units early
@@ -1560,7 +1598,7 @@ int cnt_lstm_check(cnt_lstm *h, void *stream) {
             for (int b = 0; b < blocks; ++b) {
                 if (t[(size_t)b * stride + 3] == 0) continue;
                 const long long *r = &tr[(size_t)b * kTraceStride];
-                std::fprintf(stderr, "trace block %d job %lld member %lld xcd %lld:", b, r[0], r[1], r[2]);
+                std::fprintf(stderr, "trace block %d job %lld member %lld xcd %lld hwid %lld:", b, r[0], r[1], r[2], r[3]);
                 for (int q = 0; q < 5 * kTraceSteps; ++q) std::fprintf(stderr, " %lld", r[4 + q]);
                 std::fprintf(stderr, "\n");
             }

@@ -100,11 +100,11 @@ __device__ int local_claim_role(const ChainParams &p, int G) {
 // v[lane] + v[lane ^ 32].
 template <int JB>
 __device__ __forceinline__ float sender_sum(float v) {
-    static_assert(JB == 4 || JB == 8, "cells per workgroup");
+    static_assert(JB == 4 || JB == 8 || JB == 16, "cells per workgroup");
     auto dpp = [](float x, auto ctrl) {
         return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xF, 0xF, false));
     };
-    v += dpp(v, std::integral_constant<int, 0x128>{});                // row_ror:8
+    if (JB <= 8) v += dpp(v, std::integral_constant<int, 0x128>{});   // row_ror:8
     if (JB == 4) v += dpp(v, std::integral_constant<int, 0x124>{});   // row_ror:4
     {
         const unsigned u = __builtin_bit_cast(unsigned, v);
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
     constexpr int DP = KW + 4;        // pitch of a sequence's deltas in LDS (16-byte reads of four sequences: no bank shared)
     constexpr int PAIR = NSQ * JB;    // words of one (receiver, sender) pair
     constexpr int RECV = G * PAIR;    // words one receiver gets per step
-    static_assert((JB == 4 || JB == 8) && EL <= 64 && G % SPW == 0 && NL == PW, "local recursion geometry");
+    static_assert((JB == 4 || JB == 8 || JB == 16) && EL <= 64 && G % SPW == 0 && NL == PW, "local recursion geometry");
     enum { C_OG = 0, C_CE, C_NI, C_FG, C_IG, C_E, C_DOG, C_FGACT, C_DUMMY, NCOEF };
 
     __shared__ __attribute__((aligned(16))) float dl[2][NSQ][DP];
@@ -400,5 +400,6 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
         o[0] = ph0; o[1] = ph1; o[3] = ph3; o[4] = poll_rounds; o[6] = ph6;
         long long *tr = p.phase_ticks + kTraceBase + (size_t)blockIdx.x * kTraceStride;
         tr[0] = job; tr[1] = me; tr[2] = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u;
+        tr[3] = __builtin_amdgcn_s_getreg((31 << 11) | (0 << 6) | 4);  // HW_ID: cu_id [11:8], sh_id [12], se_id [15:13]
     }
 }
