@@ -75,6 +75,7 @@ struct ChainParams {
     struct { int dir, seq0, nseq; } job[8];
     unsigned *ctl;   // placement counters, zero at launch
     float *lmail;    // one mailbox per job
+    float *flmail;   // the same for the XCD-local forward recursion
     // XCD-local backward recursion over a range of its steps: [step_begin, step_end) of 0 .. T.  A launch that starts
     // at a later step takes what the step before it left: the carried cell-state terms from the state arrays, the
     // partial errors from the mailbox (which nothing may touch in between).
@@ -813,6 +814,7 @@ __global__ __launch_bounds__(kBwdThreads) void lstm_backward_chain(const ChainPa
 }
 
 #include "lstm_local.hpp"
+#include "lstm_local_fwd.hpp"
 
 // Runs in front of every recursion launch (one workgroup).  If the launch before gave up, the device flag is still
 // set and mailbox words may be left over: refill the mailboxes and clear the flag, so that a handle heals without
@@ -1070,10 +1072,14 @@ struct cnt_lstm {
     unsigned *ctl;
     float *lmail;
     size_t lmail_words;
+    float *flmail;         // XCD-local forward recursion: one mailbox per job
+    size_t flmail_words;
+    int fwd_local;
     int last_blocks;       // workgroups of the last recursion launch
     int warm;  // read the recursion's inputs once before the XCD-local backward recursion (CNT_LSTM_WARM=0: off)
     int spread_lds;  // dynamic LDS the XCD-local recursion asks for so that a compute unit takes one of its workgroups
     int poll_delay_local;  // pause before the first poll of a step in the XCD-local recursion, units of 64 clocks
+    int poll_delay_fwd_local;  // the same for the XCD-local forward recursion
     // recorded behind every recursion launch: the failure latch is taken only once the launch that may have set it has
     // ended, so that no workgroup of that launch can set it (or the veto) again after the report
     hipEvent_t launch_done;
@@ -1140,6 +1146,7 @@ void fill_chain_params(const cnt_lstm *h, const float *weights, ChainParams &p) 
     for (int j = 0; j < h->njobs; ++j) { p.job[j].dir = h->job[j].dir; p.job[j].seq0 = h->job[j].seq0; p.job[j].nseq = h->job[j].nseq; }
     p.ctl = h->ctl;
     p.lmail = h->lmail;
+    p.flmail = h->flmail;
     p.phase_ticks = h->phase_ticks;
     p.poll_delay = h->poll_delay; p.poll_gap = h->poll_gap; p.poll_delay_fwd = h->poll_delay_fwd;
 }
@@ -1197,6 +1204,28 @@ chain_kernel_t pick_local_kernel(int H, int &JB) {
     return nullptr;
 }
 
+// the forward recursion's kernel with the backward recursion's cells per workgroup (one mailbox geometry for both)
+chain_kernel_t pick_local_forward_kernel(int H, int &JB) {
+    if (H == 256) { JB = 8; return (chain_kernel_t)lstm_forward_local<256, 8>; }
+    if (H == 128) { JB = 4; return (chain_kernel_t)lstm_forward_local<128, 4>; }
+    if (H == 64) { JB = 4; return (chain_kernel_t)lstm_forward_local<64, 4>; }
+    return nullptr;
+}
+
+// allows a kernel the dynamic LDS of the launches below (once per device and kernel)
+int set_spread_lds(const cnt_lstm *h, const void *kernel) {
+    if (h->spread_lds <= 0) return CNT_OK;
+    static std::mutex mu;
+    static std::vector<std::pair<int, const void *>> done;
+    std::lock_guard<std::mutex> lock(mu);
+    const std::pair<int, const void *> key(h->device, kernel);
+    if (std::find(done.begin(), done.end(), key) == done.end()) {
+        CNT_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, h->spread_lds));
+        done.push_back(key);
+    }
+    return CNT_OK;
+}
+
 int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     const bool local = !fwd && h->local;
     int local_jb = 0;
@@ -1245,6 +1274,21 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
         CNT_TRY(warm_backward_inputs(h, stream, p, guard_rides ? g : none));
     }
     ProfileScope prof(stream, fwd ? "lstm_forward_chain" : "lstm_backward_chain");
+    if (fwd && h->fwd_local) {
+        CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->flmail), h->flmail_words, kEmpty));
+        int fjb = 0;
+        chain_kernel_t fk = pick_local_forward_kernel(h->H, fjb);
+        const int G = h->H / fjb;
+        const int blocks = (h->njobs * G + 8 * (G - 1) + 7) / 8 * 8;
+        h->last_blocks = blocks;
+        CNT_TRY(set_spread_lds(h, reinterpret_cast<const void *>(fk)));
+        p.poll_delay_fwd = h->poll_delay_fwd_local;
+        hipLaunchKernelGGL(fk, dim3(blocks), dim3(local_threads(h->H)), (size_t)h->spread_lds, stream, p);
+        CNT_HIP(hipGetLastError());
+        CNT_HIP(hipEventRecord(h->launch_done, stream));
+        h->launch_pending = 1;
+        return CNT_OK;
+    }
     if (local) {
         // enough workgroups that njobs complete teams form on any spread over the XCDs
         const int G = h->H / local_jb;
@@ -1258,18 +1302,8 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
         // this kernel off a compute unit is its LDS request: the launch asks for a little more than half of a compute
         // unit's LDS (unused dynamic shared memory), which still leaves room for two workgroups of a matrix product
         // beside it.  CNT_LSTM_SPREAD_LDS sets the request in bytes (0: none).
-        const int spread_lds = h->spread_lds;
-        if (spread_lds > 0) {
-            static std::mutex mu;
-            static std::vector<std::pair<int, const void *>> done;
-            std::lock_guard<std::mutex> lock(mu);
-            const std::pair<int, const void *> key(h->device, reinterpret_cast<const void *>(k));
-            if (std::find(done.begin(), done.end(), key) == done.end()) {
-                CNT_HIP(hipFuncSetAttribute(key.second, hipFuncAttributeMaxDynamicSharedMemorySize, spread_lds));
-                done.push_back(key);
-            }
-        }
-        hipLaunchKernelGGL(k, dim3(blocks), dim3(local_threads(h->H)), (size_t)spread_lds, stream, p);
+        CNT_TRY(set_spread_lds(h, reinterpret_cast<const void *>(k)));
+        hipLaunchKernelGGL(k, dim3(blocks), dim3(local_threads(h->H)), (size_t)h->spread_lds, stream, p);
         CNT_HIP(hipGetLastError());
         CNT_HIP(hipEventRecord(h->launch_done, stream));
         h->launch_pending = 1;
@@ -1428,7 +1462,10 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     // measured optima on MI355X: 26 at H=256 (S=10 and S=4), 25-26 at H=128 (S=8), 24 at H=64 (S=6); two units early
     // cost a second poll round (+0.2 us per step), every unit late costs its 0.027 us
     h->poll_delay_fwd = H <= 64 ? 24 : 26;
-    if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY_FWD")) h->poll_delay_fwd = std::atoi(e);
+    // the same pause for the forward recursion on XCD-local teams: measured optima 24 at 256 cells (876 us per benchmark
+    // layer; 14: 887, 18: 916, 30: 963), 14-18 at 128 cells, 18 at 64 cells
+    h->poll_delay_fwd_local = H >= 256 ? 24 : H >= 128 ? 16 : 18;
+    if (const char *e = std::getenv("CNT_LSTM_POLL_DELAY_FWD")) h->poll_delay_fwd = h->poll_delay_fwd_local = std::atoi(e);
     if (const char *e = std::getenv("CNT_LSTM_POLL_GAP")) h->poll_gap = std::atoi(e);
     hipError_t err = hipGetDevice(&h->device);
     const size_t nstate = (size_t)H * desc->maxT * desc->S;
@@ -1465,6 +1502,17 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
             }
             h->lmail_words = (size_t)h->njobs * (size_t)kMailSlots * (H / local_jb) * (H / local_jb) * kLocalSeqs * local_jb;
             if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->lmail), h->lmail_words * sizeof(float));
+            // the forward recursion on the same teams (lstm_local_fwd.hpp); CNT_LSTM_FWD_LOCAL=0: the kernel across XCDs
+            h->fwd_local = 1;
+            if (const char *fe = std::getenv("CNT_LSTM_FWD_LOCAL")) h->fwd_local = std::atoi(fe) != 0;
+            if (h->fwd_local) {
+                int fjb = 0;
+                h->fwd_local = pick_local_forward_kernel(H, fjb) != nullptr;
+                if (h->fwd_local) {
+                    h->flmail_words = (size_t)h->njobs * local_job_words(H, fjb);
+                    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->flmail), h->flmail_words * sizeof(float));
+                }
+            }
             if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->ctl), kCtlWords * sizeof(unsigned));
             if (err == hipSuccess) err = hipMemset(h->ctl, 0, kCtlWords * sizeof(unsigned));
         }
@@ -1501,6 +1549,7 @@ int cnt_lstm_destroy(cnt_lstm *h) {
     if (h->abort_flag) (void)hipFree(h->abort_flag);
     if (h->phase_ticks) (void)hipFree(h->phase_ticks);
     if (h->lmail) (void)hipFree(h->lmail);
+    if (h->flmail) (void)hipFree(h->flmail);
     if (h->ctl) (void)hipFree(h->ctl);
     if (h->latch_host) (void)hipHostFree(h->latch_host);
     if (h->launch_done) (void)hipEventDestroy(h->launch_done);
@@ -1532,6 +1581,7 @@ int cnt_lstm_set_wait_bounds(cnt_lstm *h, unsigned spin_limit, int poll_delay_ba
     h->poll_delay = poll_delay_backward;
     h->poll_delay_local = poll_delay_backward < 11 ? poll_delay_backward : 11;
     h->poll_delay_fwd = poll_delay_forward;
+    h->poll_delay_fwd_local = poll_delay_forward < 24 ? poll_delay_forward : h->poll_delay_fwd_local;
     return CNT_OK;
 }
 
