@@ -32,15 +32,15 @@ import numpy as np  # noqa: E402
 
 # HBM bytes one launch of the backward recursion kernel moves on this workload (T=600, S=10, H=256, two directions),
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a copy of known size; the figure and the command
-# that made it are in the profile named here.  Algorithmic bytes of the same launch: 120 MB.  None = not measured
+# that made it are in the profile named here.  Algorithmic bytes of the same launch (T = 600): 123 MB.  None = not measured
 # for the kernel this tree runs.
-CHAIN_TRAFFIC_BYTES = 173.6e6  # (47 440 KiB x 2.00 fetched + 74 690 KiB written) per launch of lstm_backward_local<256, 8>
+CHAIN_TRAFFIC_BYTES = 176.8e6  # (48 280 KiB x 2.00 fetched + 76 128 KiB written) per launch of lstm_backward_local<256, 8>
 CHAIN_TRAFFIC_SOURCE = "profiles/acoustic_backward_hbm_traffic.md"
 # The counters were read for this kernel, built from this source text (first 16 hex digits of the SHA-256 of
 # csrc/lstm_local.hpp); when the file has changed since, the figure no longer describes the kernel that runs and the
 # benchmark prints null for it.
 CHAIN_TRAFFIC_KERNEL = "lstm_backward_local<256, 8>"
-CHAIN_TRAFFIC_SOURCE_SHA16 = "5ff49375364c1571"
+CHAIN_TRAFFIC_SOURCE_SHA16 = "1de15ab35991987c"
 
 METRIC = "BLSTM backward frames/sec at 1 MI355X; % HBM/MFMA roofline vs host CPU"
 PEAK_FP32_MFMA_TFLOPS = 157.3
@@ -131,7 +131,7 @@ def main():
                     help="acoustic = benchmark configs[1] (the headline metric); the others are the remaining configs")
     ap.add_argument("--via-layer-calls", action="store_true",
                     help="also time the same backward pass through one C-ABI call per layer on one stream (the binding "
-                         "INTEGRATION.md shows for the reference's Layer classes) and print it as `via_layer_calls`")
+                         "a shell around the reference's Layer classes would use) and print it as `via_layer_calls`")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters)")
@@ -240,6 +240,12 @@ def main():
         hop_us = probe(same_xcd=True, with_compute=True)
         hop_bare_us = probe(same_xcd=True, with_compute=False)
         hop_far_us = probe(same_xcd=False, with_compute=False)
+
+        def message(kb):
+            try:
+                return capi.probe_hop_message(kb, rounds=2000)
+            except RuntimeError:
+                return None
         us_per_step = 1e3 * kernels[dom]["avg_ms"] / T
         traffic, measured_on = chain_traffic()
         roof = {"bound": "mfma", "achieved": flops / dom_avg_s / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS,
@@ -248,7 +254,9 @@ def main():
                 "us_per_step": us_per_step,
                 "latency_floor_us_per_step": hop_us,
                 "frac_of_latency_floor": hop_us / us_per_step if hop_us else None,
-                "hop_us": {"same_xcd": hop_bare_us, "same_xcd_with_step_arithmetic": hop_us, "across_xcds": hop_far_us},
+                "hop_us": {"same_xcd": hop_bare_us, "same_xcd_with_step_arithmetic": hop_us, "across_xcds": hop_far_us,
+                           # what a workgroup receives per step: 4 KB today, 16 KB if partial pre-activations travelled
+                           "message_4kb_same_xcd": message(4), "message_16kb_same_xcd": message(16)},
                 "note": "latency-bound recursion: T sequential steps, each a 256x1024x%d product cut into (direction, "
                         "sequence group) jobs of 32 workgroups per XCD plus one exchange through that XCD's L2; `frac` is "
                         "against the fp32 MFMA peak as the metric asks, `frac_of_latency_floor` against T x (one measured "

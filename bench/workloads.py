@@ -153,8 +153,11 @@ def mdn_c3(args, pkg):
     # weights, means, deviations and targets in; Lp errors and the M + 1 log-likelihood terms out
     nbytes = F * (Lp + D + Lp + M + 1) * 4
     ach = nbytes / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
-    roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None,
-            "kernel": dom}
+    # traffic: two rocprofv3 --pmc runs of this workload (FETCH_SIZE 23 975 KiB x 2.00 by a copy of known size, WRITE_SIZE
+    # 54 442 KiB x 1.00) for the benchmark size; other sizes have not been read
+    roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
+            "traffic": 104.8e6 if (F, M, D) == (6000, 16, 60) else None,
+            "traffic_source": "profiles/mdn_c3_backward_kernel_stats.md", "kernel": dom}
 
     def full():
         layer.forward(xd)

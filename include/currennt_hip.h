@@ -41,6 +41,11 @@ int cnt_profile_get(int index, char *label, int label_cap, int *launches, float 
  * a recursion step does between receiving and sending.  T times this is the floor of a T-step recursion spread
  * over compute units.  Synchronous; *hop_us (host memory) receives microseconds per hop. */
 int cnt_probe_hop_latency(void *stream, int same_xcd, int with_compute, int rounds, float *hop_us);
+/* The same hop for a message of `kilobytes` (4, 8, 12 or 16) between two workgroups of four waves on one XCD: every
+ * lane polls its 16-byte pieces until all carry the round's tag, the waves meet at a barrier, the workgroup answers.
+ * 4 KB is what a workgroup of a 256-cell recursion receives per step today; 16 KB is what the forward recursion would
+ * receive if it exchanged partial pre-activations of the four gates instead of outputs. */
+int cnt_probe_hop_message(void *stream, int kilobytes, int rounds, float *hop_us);
 /* Test hook: the scalar activation functions as the kernels evaluate them, out[i] = f(x[i]) for n device floats.
  * which = 0: logistic, 1: tanh (activation_functions/Logistic.cuh, Tanh.cuh: exp and a true quotient, clamped at
  * +-88.72); 2, 3: the same two from the hardware's exp2 and reciprocal, which only the forward LSTM recursion uses
@@ -128,7 +133,15 @@ typedef struct {
 /* LstmLayer::LstmLayer (layers/LstmLayer.cu:1078-1268): allocates the per-direction state.  Layers with 64, 128,
  * 256 or 512 cells per direction and at most 32 parallel sequences run their recursions as persistent kernels;
  * any other geometry runs them step by step (one batched recurrent product and one cell kernel per time step, the
- * reference's own schedule), with the same results. */
+ * reference's own schedule), with the same results.
+ * With 64, 128 or 256 cells per direction both recursions run on teams of workgroups that share one XCD's L2: a job
+ * is a direction and up to four sequences, its team exchanges each step's outputs (forward) or partial errors
+ * (backward) through that L2, and the launch asks for a little more than half of a compute unit's LDS so that every
+ * workgroup of a team gets a compute unit of its own (two on one unit take their steps at the same moments and cost
+ * a fifth of the step time).  Environment, read when a handle is created: CNT_LSTM_LOCAL=0 / CNT_LSTM_FWD_LOCAL=0
+ * (the kernels that exchange across XCDs instead), CNT_LSTM_SPREAD_LDS=<bytes> (the LDS request, 0: none),
+ * CNT_LSTM_LOCAL_JB=16 (16 instead of 8 cells per workgroup for 256-cell layers), CNT_LSTM_WARM=0 (no read of the
+ * states into the memory-side cache in front of the backward recursion), CNT_LSTM_STEPWISE=1. */
 int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out);
 int cnt_lstm_destroy(cnt_lstm *h);
 /* LstmLayer::loadSequences (layers/LstmLayer.cu:1488-1533): records the fraction's geometry and
@@ -163,8 +176,9 @@ int cnt_lstm_backward_prev_errors(cnt_lstm *h, void *stream, const float *weight
  * ranges of one pass must be launched in order on one stream, the first from step 0.  The handle keeps the step the
  * pass stands at: a range that starts anywhere else is refused (CNT_ERR_ARG), and a pass that is abandoned half way
  * -- a range from step 0, cnt_lstm_backward_errors, cnt_lstm_forward or cnt_lstm_load_sequences before step curMaxT
- * was reached -- is dropped cleanly (the partial errors it left in the mailbox are discarded).  Only where cnt_lstm_backward_can_split returns 1 (layers whose backward recursion runs as one
- * persistent kernel per group of sequences); elsewhere it is an error.
+ * was reached -- is dropped cleanly (the partial errors it left in the mailbox are discarded).  Only where
+ * cnt_lstm_backward_can_split returns 1 (layers whose backward recursion runs as one persistent kernel per group of
+ * sequences); elsewhere it is an error.
  * cnt_lstm_backward_steps_done: the time steps [t_begin, t_end) whose deltas are final once `steps` steps have run
  * (both directions have passed them), i.e. what cnt_lstm_backward_prev_errors_range may already compute:
  * prev_errors columns of the time steps [t_begin, t_end) only.

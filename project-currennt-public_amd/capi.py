@@ -69,6 +69,7 @@ _SIGNATURES = {
     "cnt_dense_backward_weights": (I, [VP, I, I, I, F, VP, VP, VP]),
     "cnt_dense_backward_weights_static": (I, [VP, I, I, I, F, VP, VP, VP]),
     "cnt_probe_hop_latency": (I, [VP, I, I, I, C.POINTER(F)]),
+    "cnt_probe_hop_message": (I, [VP, I, I, C.POINTER(F)]),
     "cnt_probe_activation": (I, [VP, I, C.c_long, VP, VP]),
     "cnt_gemm_reserve": (I, [VP]),
     "cnt_gemm_release": (I, [VP]),
@@ -240,6 +241,13 @@ def probe_hop_latency(same_xcd=True, with_compute=True, rounds=2000, stream=None
     """Microseconds per hop of a word between two workgroups (see cnt_probe_hop_latency)."""
     out = F(0.0)
     check(lib().cnt_probe_hop_latency(stream_ptr(stream), int(same_xcd), int(with_compute), int(rounds), C.byref(out)))
+    return float(out.value)
+
+
+def probe_hop_message(kilobytes=4, rounds=2000, stream=None):
+    """Microseconds per hop of a message of 4..16 KB between two four-wave workgroups on one XCD."""
+    out = F(0.0)
+    check(lib().cnt_probe_hop_message(stream_ptr(stream), int(kilobytes), int(rounds), C.byref(out)))
     return float(out.value)
 
 

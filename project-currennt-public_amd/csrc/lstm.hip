@@ -1868,7 +1868,7 @@ extern "C++" int cnt::lstm_backward_weights_parts(cnt_lstm *h, hipStream_t strea
     if (H % 4 == 0) {
         SmallGradDirs sp;
         sp.H = H; sp.L = L; sp.S = S; sp.N = N; sp.bias = d.bias;
-        sp.chunk = 64;
+        sp.chunk = N >= 4096 ? 64 : 16;  // a short fraction still fills some tens of workgroups
         for (int dir = 0; dir < 2; ++dir) {
             const int sd = dir < h->ndir ? dir : 0;
             sp.dni[dir] = h->state[sd][7]; sp.dig[dir] = h->state[sd][8]; sp.dfg[dir] = h->state[sd][9];

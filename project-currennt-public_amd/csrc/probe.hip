@@ -77,6 +77,69 @@ __global__ __launch_bounds__(64) void hop_probe_kernel(unsigned *ctl, unsigned *
     }
 }
 
+// The same hop for a message of `pieces` x 4 KB between two workgroups of four waves on one XCD, the way a recursion
+// step receives: every lane polls its 16-byte pieces (all in flight together) until each carries the round's tag, the
+// waves meet at a barrier, then the workgroup answers with a message of the same size.  4 KB is what a workgroup of a
+// 256-cell recursion receives per step when outputs (forward, gather form) or partial errors (backward) travel;
+// 16 KB is what it would receive if the forward recursion sent partial pre-activations of four gates instead.
+__global__ __launch_bounds__(256) void hop_message_kernel(unsigned *ctl, unsigned *mail, int rounds, int pieces, long long *ticks) {
+    __shared__ int role_sh;
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    if (threadIdx.x == 0) {
+        const unsigned xcd = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u;  // XCC_ID
+        int r = -1;
+        if (xcd == 0u) {
+            const unsigned t = atomicAdd(&ctl[0], 1u);
+            if (t < 2u) r = (int)t;
+        }
+        role_sh = r;
+    }
+    __syncthreads();
+    const int r = role_sh;
+    if (r < 0) return;
+    const size_t words = (size_t)pieces * 1024;  // per direction
+    unsigned *mine = mail + (r ? words : 0), *theirs = mail + (r ? 0 : words);
+    const long long t0 = wall_clock64();
+    bool ok = true;
+    for (int i = 1; i <= rounds && ok; ++i) {
+        for (int half = 0; half < 2; ++half) {
+            const bool sender = (half == 0) == (r == 0);
+            if (sender) {
+                const u32x4 v = {(unsigned)i, (unsigned)i, (unsigned)i, (unsigned)i};
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (q < pieces)
+                        asm volatile("global_store_dwordx4 %0, %1, off" ::"v"(mine + (size_t)q * 1024 + threadIdx.x * 4), "v"(v) : "memory");
+            } else {
+                unsigned spins = 0;
+                bool all = false;
+                do {
+                    u32x4 w[4];
+                    unsigned worst = (unsigned)i;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        if (q < pieces)
+                            asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(w[q]) : "v"(theirs + (size_t)q * 1024 + threadIdx.x * 4) : "memory");
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (q >= pieces) continue;
+                        asm volatile("" : "+v"(w[q]));
+                        if (w[q].x != (unsigned)i || w[q].y != (unsigned)i || w[q].z != (unsigned)i || w[q].w != (unsigned)i) worst = 0u;
+                    }
+                    all = __builtin_amdgcn_ballot_w64(worst != (unsigned)i) == 0;
+                } while (!all && ++spins < (1u << 20));
+                if (!all) ok = false;  // every wait is bounded: the kernel always ends
+                __syncthreads();
+            }
+        }
+    }
+    if (threadIdx.x == 0) {
+        ticks[r] = wall_clock64() - t0;
+        if (!ok) ticks[2] = 1;
+    }
+}
+
 // the activation functions as the recursion kernels evaluate them, element by element (a test hook)
 __global__ void activations_kernel(size_t n, const float *__restrict__ x, float *__restrict__ out, int which) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -129,6 +192,40 @@ extern "C" int cnt_probe_hop_latency(void *stream_, int same_xcd, int with_compu
         return CNT_ERR_DEVICE;
     }
     // 100 MHz clock; a round is two hops
+    *hop_us = (float)((double)(host_ticks[0] > host_ticks[1] ? host_ticks[0] : host_ticks[1]) * 0.01 / rounds / 2.0);
+    return CNT_OK;
+}
+
+extern "C" int cnt_probe_hop_message(void *stream_, int kilobytes, int rounds, float *hop_us) {
+    using namespace cnt;
+    CNT_REQUIRE(hop_us, "probe_hop_message: null argument");
+    CNT_REQUIRE(rounds >= 1 && rounds <= 100000, "probe_hop_message: 1..100000 rounds");
+    CNT_REQUIRE(kilobytes == 4 || kilobytes == 8 || kilobytes == 12 || kilobytes == 16, "probe_hop_message: 4, 8, 12 or 16 KB");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int pieces = kilobytes / 4;
+    const size_t bytes = 8192 + (size_t)2 * pieces * 4096;
+    unsigned *buf = nullptr;
+    CNT_HIP(hipMalloc(reinterpret_cast<void **>(&buf), bytes));
+    int status = CNT_OK;
+    long long host_ticks[3] = {0, 0, 0};
+    do {
+        if (hipMemsetAsync(buf, 0, bytes, stream) != hipSuccess) { status = CNT_ERR_HIP; break; }
+        unsigned *ctl = buf, *mail = buf + 2048;
+        long long *ticks = reinterpret_cast<long long *>(buf + 512);
+        hipLaunchKernelGGL(hop_message_kernel, dim3(256), dim3(256), 0, stream, ctl, mail, rounds, pieces, ticks);
+        if (hipGetLastError() != hipSuccess || hipStreamSynchronize(stream) != hipSuccess ||
+            hipMemcpy(host_ticks, ticks, sizeof(host_ticks), hipMemcpyDeviceToHost) != hipSuccess)
+            status = CNT_ERR_HIP;
+    } while (false);
+    (void)hipFree(buf);
+    if (status != CNT_OK) {
+        set_error("probe_hop_message: HIP call failed: %s", hipGetErrorString(hipGetLastError()));
+        return status;
+    }
+    if (host_ticks[2] != 0 || host_ticks[0] == 0 || host_ticks[1] == 0) {
+        set_error("probe_hop_message: the two workgroups did not meet (placement or visibility)");
+        return CNT_ERR_DEVICE;
+    }
     *hop_us = (float)((double)(host_ticks[0] > host_ticks[1] ? host_ticks[0] : host_ticks[1]) * 0.01 / rounds / 2.0);
     return CNT_OK;
 }

@@ -246,6 +246,22 @@ def test_lstm_abandoned_partial_recursion_does_not_leak_into_the_next_pass():
     layer.close()
 
 
+def test_hop_probes_measure_a_plausible_exchange():
+    """The measurement hooks behind the benchmark's latency floor: a word between two workgroups of one XCD takes a
+    fraction of a microsecond, across XCDs longer, and a 16 KB message longer than a 4 KB one (the reason the forward
+    recursion exchanges outputs, 4 KB per workgroup and step, and not partial pre-activations, 16 KB)."""
+    capi = PC.pkg().capi
+    print("hop probes: word same XCD / across XCDs, message 4 KB / 16 KB", flush=True)
+    near = capi.probe_hop_latency(True, False, 500)
+    far = capi.probe_hop_latency(False, False, 500)
+    m4 = capi.probe_hop_message(4, 500)
+    m16 = capi.probe_hop_message(16, 500)
+    assert 0.05 < near < 5.0 and near < far < 20.0
+    assert near < m4 < m16 < 10.0
+    with pytest.raises(RuntimeError, match="4, 8, 12 or 16 KB"):
+        capi.probe_hop_message(5, 10)
+
+
 def test_activation_functions_against_the_cpu_functions():
     """The scalar semantics of the path (Logistic.cuh / Tanh.cuh with the clamps at +-88.72) and the quick forms the
     forward recursion uses instead (hardware exp2 and reciprocal): swept over the whole unclamped range and across
