@@ -1080,9 +1080,9 @@ struct cnt_lstm {
     int spread_lds;  // dynamic LDS the XCD-local recursion asks for so that a compute unit takes one of its workgroups
     int poll_delay_local;  // pause before the first poll of a step in the XCD-local recursion, units of 64 clocks
     int poll_delay_fwd_local;  // the same for the XCD-local forward recursion
-    // recorded behind every recursion launch: the failure latch is taken only once the launch that may have set it has
-    // ended, so that no workgroup of that launch can set it (or the veto) again after the report
-    hipEvent_t launch_done;
+    // set by every recursion launch: the failure latch is taken only once the launch that may have set it has ended
+    // (the device's recursion-order event, see launch_in_order), so that no workgroup of that launch can set it (or the
+    // veto) again after the report
     int launch_pending;
     // backward recursion run as ranges of steps: the step the next range has to start at (0: a fresh pass)
     int next_step;
@@ -1226,6 +1226,38 @@ int set_spread_lds(const cnt_lstm *h, const void *kernel) {
     return CNT_OK;
 }
 
+// Persistent recursion launches of one process run one at a time on a device.  Every workgroup of a team has to be
+// resident before the team can take a step, and an XCD-local launch takes a compute unit per workgroup: two such
+// launches that start together on different streams can each hold half of an XCD's compute units with half a team and
+// wait for the other half until their bounded waits give up.  A launch therefore waits, in stream order, for the
+// recursion launched before it (from whatever handle or stream); launches on one stream are ordered anyway and skip
+// the wait.  The mutex keeps wait, launch and record of one launch together when several host threads launch.
+struct RecursionOrder {
+    std::mutex mu;
+    hipEvent_t done = nullptr;
+    hipStream_t last = nullptr;
+    bool any = false;
+};
+RecursionOrder &recursion_order(int device) {
+    static RecursionOrder order[64];
+    return order[device >= 0 && device < 64 ? device : 0];
+}
+template <typename Launch>
+int launch_in_order(cnt_lstm *h, hipStream_t stream, Launch launch) {
+    RecursionOrder &o = recursion_order(h->device);
+    std::lock_guard<std::mutex> lock(o.mu);
+    if (!o.done) CNT_HIP(hipEventCreateWithFlags(&o.done, hipEventDisableTiming));
+    if (o.any && o.last != stream) CNT_HIP(hipStreamWaitEvent(stream, o.done, 0));
+    launch();
+    CNT_HIP(hipGetLastError());
+    // Also what lstm_take_failure asks: once this record (or a later one, which waited for it) has completed, every
+    // recursion launched so far has ended.
+    CNT_HIP(hipEventRecord(o.done, stream));
+    o.last = stream; o.any = true;
+    h->launch_pending = 1;
+    return CNT_OK;
+}
+
 int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     const bool local = !fwd && h->local;
     int local_jb = 0;
@@ -1283,11 +1315,9 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
         h->last_blocks = blocks;
         CNT_TRY(set_spread_lds(h, reinterpret_cast<const void *>(fk)));
         p.poll_delay_fwd = h->poll_delay_fwd_local;
-        hipLaunchKernelGGL(fk, dim3(blocks), dim3(local_threads(h->H)), (size_t)h->spread_lds, stream, p);
-        CNT_HIP(hipGetLastError());
-        CNT_HIP(hipEventRecord(h->launch_done, stream));
-        h->launch_pending = 1;
-        return CNT_OK;
+        return launch_in_order(h, stream, [&] {
+            hipLaunchKernelGGL(fk, dim3(blocks), dim3(local_threads(h->H)), (size_t)h->spread_lds, stream, p);
+        });
     }
     if (local) {
         // enough workgroups that njobs complete teams form on any spread over the XCDs
@@ -1303,21 +1333,17 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
         // unit's LDS (unused dynamic shared memory), which still leaves room for two workgroups of a matrix product
         // beside it.  CNT_LSTM_SPREAD_LDS sets the request in bytes (0: none).
         CNT_TRY(set_spread_lds(h, reinterpret_cast<const void *>(k)));
-        hipLaunchKernelGGL(k, dim3(blocks), dim3(local_threads(h->H)), (size_t)h->spread_lds, stream, p);
-        CNT_HIP(hipGetLastError());
-        CNT_HIP(hipEventRecord(h->launch_done, stream));
-        h->launch_pending = 1;
-        return CNT_OK;
+        return launch_in_order(h, stream, [&] {
+            hipLaunchKernelGGL(k, dim3(blocks), dim3(local_threads(h->H)), (size_t)h->spread_lds, stream, p);
+        });
     }
     const int G = h->H / h->JB;
     p.xcd_pack = fwd ? h->xcd_pack : 0;
     const int blocks = p.xcd_pack ? 8 * G : h->ndir * G;
     h->last_blocks = blocks;
-    hipLaunchKernelGGL(k, dim3(blocks), dim3(fwd ? kThreads + 64 * ((h->JB * 16 * h->NT + 63) / 64) + 64 : kBwdThreads), 0, stream, p);
-    CNT_HIP(hipGetLastError());
-    CNT_HIP(hipEventRecord(h->launch_done, stream));
-    h->launch_pending = 1;
-    return CNT_OK;
+    return launch_in_order(h, stream, [&] {
+        hipLaunchKernelGGL(k, dim3(blocks), dim3(fwd ? kThreads + 64 * ((h->JB * 16 * h->NT + 63) / 64) + 64 : kBwdThreads), 0, stream, p);
+    });
 }
 
 // The recursions of both directions step by step (see lstm_forward_step): per step the recurrent products of all
@@ -1520,7 +1546,6 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     if (err == hipSuccess && std::getenv("CNT_LSTM_TIMING"))
         err = hipMalloc(reinterpret_cast<void **>(&h->phase_ticks), 8 * 512 * 6 * sizeof(long long));
     if (err == hipSuccess && h->phase_ticks) err = hipMemset(h->phase_ticks, 0, 8 * 512 * 6 * sizeof(long long));
-    if (err == hipSuccess) err = hipEventCreateWithFlags(&h->launch_done, hipEventDisableTiming);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->abort_flag), sizeof(int));
     if (err == hipSuccess) err = hipMemset(h->abort_flag, 0, sizeof(int));
     // the word a kernel that gives up sets for the host: pinned, mapped, coherent host memory
@@ -1552,7 +1577,6 @@ int cnt_lstm_destroy(cnt_lstm *h) {
     if (h->flmail) (void)hipFree(h->flmail);
     if (h->ctl) (void)hipFree(h->ctl);
     if (h->latch_host) (void)hipHostFree(h->latch_host);
-    if (h->launch_done) (void)hipEventDestroy(h->launch_done);
     delete h;
     return CNT_OK;
 }
@@ -1602,7 +1626,9 @@ extern "C++" int cnt::lstm_take_failure(cnt_lstm *h) {
     if (*latch == 0) return 0;
     if (h->launch_pending) {
         // the launch that set the mark may still be running: its other workgroups would set it again after the report
-        if (hipEventQuery(h->launch_done) != hipSuccess) {
+        RecursionOrder &o = recursion_order(h->device);
+        std::lock_guard<std::mutex> lock(o.mu);
+        if (o.done && hipEventQuery(o.done) != hipSuccess) {
             (void)hipGetLastError();
             return 0;  // reported by a later call, once the launch has ended
         }

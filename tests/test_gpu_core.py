@@ -358,6 +358,57 @@ def test_lstm_gives_up_cleanly_and_recovers():
     layer.close()
 
 
+def test_lstm_layers_on_two_streams_at_once():
+    """Two layers of the benchmark's size driven from two non-blocking streams at the same time.  Each XCD-local
+    recursion wants a compute unit per workgroup and all of them at once; the library orders recursion launches of
+    different streams one behind the other, so both passes run to their end with the results each gives alone."""
+    import numpy as np
+    import torch
+
+    print("two lstm layers on two streams", flush=True)
+    capi = PC.pkg().capi
+    P, L, S, T = 64, 512, 10, 200
+    N = T * S
+    rng = np.random.default_rng(9)
+    pat = torch.full((N,), 2, dtype=torch.int8, device="cuda")
+    layers, data, alone = [], [], []
+    for k in range(2):
+        W = torch.from_numpy(rng.uniform(-0.08, 0.08, capi.lib().cnt_lstm_weight_count(P, L, 1)).astype(np.float32)).cuda()
+        x = torch.from_numpy(rng.standard_normal(P * N).astype(np.float32)).cuda()
+        err = torch.from_numpy((0.1 * rng.standard_normal(L * N)).astype(np.float32)).cuda()
+        layer = capi.Lstm(P, L, True, S, T)
+        out = torch.zeros(L * N, device="cuda"); ex = torch.zeros(P * N, device="cuda"); dW = torch.zeros_like(W)
+        layer.load_sequences(pat, T, T)
+        layer.forward(W, x, out)
+        layer.backward(W, x, out, err.clone(), ex, dW)
+        layer.check()
+        layers.append(layer); data.append((W, x, err)); alone.append((out.clone(), ex.clone(), dW.clone()))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = []
+    for k in range(2):
+        W, x, err = data[k]
+        out = torch.zeros(L * N, device="cuda"); ex = torch.zeros(P * N, device="cuda"); dW = torch.zeros_like(W)
+        got.append((out, ex, dW))
+    torch.cuda.synchronize()
+    for _ in range(3):   # forward and backward recursions of the two layers interleaved on the two streams
+        for k in range(2):
+            W, x, _ = data[k]
+            layers[k].load_sequences(pat, T, T, stream=streams[k])
+            layers[k].forward(W, x, got[k][0], stream=streams[k])
+        for k in range(2):
+            W, x, err = data[k]
+            # a bidirectional layer leaves its output errors as they are: the same buffer serves every pass
+            layers[k].backward(W, x, got[k][0], err, got[k][1], got[k][2], stream=streams[k])
+    torch.cuda.synchronize()
+    for k in range(2):
+        layers[k].check()
+        assert PC.relerr(got[k][0].cpu().numpy(), alone[k][0].cpu().numpy()) < 1e-6
+        assert PC.relerr(got[k][1].cpu().numpy(), alone[k][1].cpu().numpy()) < 1e-6
+        assert PC.relerr(got[k][2].cpu().numpy(), alone[k][2].cpu().numpy()) < 1e-5
+        layers[k].close()
+
+
 def test_lstm_step_by_step_recursion_equals_the_persistent_kernels(monkeypatch):
     """The two implementations of the recursion on a geometry both cover (clip active, ragged lengths): the handle
     created with CNT_LSTM_STEPWISE set runs step by step."""
