@@ -1682,8 +1682,9 @@ int cnt_lstm_check(cnt_lstm *h, void *stream) {
         CNT_HIP(hipMemset(h->phase_ticks, 0, 8 * 512 * 6 * sizeof(long long)));
         const double us = active ? 0.01 / active / h->T : 0.0;
         if (h->last_was_forward)
-            std::fprintf(stderr, "lstm forward per step [us]: gather waves wait+product %.3f loop %.3f poll rounds %.2f "
-                         "(T=%d, %d workgroups)\n", m[0] * us, m[3] * us, active ? m[4] / active / h->T : 0.0, h->T, active);
+            std::fprintf(stderr, "lstm forward per step [us]: gather waves pause+poll %.3f product %.3f barrier %.3f loop %.3f "
+                         "poll rounds %.2f (T=%d, %d workgroups)\n", m[1] * us, (m[0] - m[1] - m[2]) * us, m[2] * us, m[3] * us,
+                         active ? m[4] / active / h->T : 0.0, h->T, active);
         else if (local)
             std::fprintf(stderr, "lstm backward per step [us], XCD-local: cell wave wait+poll %.3f (lane 0's polls %.3f in %.2f rounds) "
                          "update+barrier %.3f loop %.3f | product waves busy %.3f | memory wave busy %.3f (T=%d, %d workgroups)\n",

@@ -36,7 +36,9 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_forward_local(const Cha
     enum { R_NI = 0, R_IG, R_FG, R_OG, R_C, R_H, NRES };
 
     __shared__ float red[2][PW][ROWS][NSQ];   // recurrent sums of the step, one share per gather wave
-    __shared__ __attribute__((aligned(16))) float hstage[PW][NSQ][16 / (ROWS / 4)][64 / (16 / (ROWS / 4))];
+    // a gather wave's 64 source cells per sequence, in cell order; the pitch keeps the four sequences' 16-byte reads
+    // off each other's banks
+    __shared__ __attribute__((aligned(16))) float hstage[PW][NSQ][64 + 4];
     __shared__ float pre[2][4][64];       // input projections of the step
     __shared__ int pre_dummy[2][64];
     __shared__ float res[2][NRES][64];    // results of the step
@@ -212,8 +214,10 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_forward_local(const Cha
 
     // ---------------------------------------------------------------------- gather waves
     // Wave pw takes the source cells 64*pw .. 64*pw + 63 for ALL of the workgroup's rows.  MFMA blocks: block = kq * RG + rg
-    // multiplies the four rows 4*rg .. + 3 with the source cells of residue kq (cell = KQ * i + kq in instruction i), so the
-    // sum over a block's cells happens inside the accumulator and only the KQ residues meet across lanes afterwards.
+    // multiplies the four rows 4*rg .. + 3 with the kq-th run of NI source cells (cell = NI * kq + i in instruction i), so
+    // the sum over a block's cells happens inside the accumulator and only the KQ runs meet across lanes afterwards.  A
+    // lane's polled vector (four neighbouring cells of one sequence) goes to LDS as it is, and a lane's B operands are
+    // NI neighbouring cells of its sequence: 16-byte LDS accesses on both sides.
     const int pw = wave;
     constexpr int RG = ROWS / 4;         // groups of four rows
     constexpr int KQ = 16 / RG;          // residues of the source cell index dealt to the blocks
@@ -226,10 +230,10 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_forward_local(const Cha
         const int o = rg * 4 + sub, g = o / JB, jj = o % JB;
         const float *wg = D.w_int + (size_t)g * p.L * H + (size_t)(j0 + jj) * H + 64 * pw;
 #pragma unroll
-        for (int i = 0; i < NI; ++i) wreg[i] = wg[KQ * i + kq];
+        for (int i = 0; i < NI; ++i) wreg[i] = wg[NI * kq + i];
     }
-    // the wave's own staging buffer: [sequence][residue][i], written as the words arrive, read back as B operands
-    float (*hb)[KQ][NI] = hstage[pw];
+    // the wave's own staging buffer: [sequence][cell], written as the words arrive, read back as B operands
+    float (*hb)[64 + 4] = hstage[pw];
     const unsigned poll_off = ((unsigned)me * RECV + (unsigned)(64 * pw + lane) * 4u) * 4u;
     long long ph0 = 0, ph1 = 0, ph2 = 0, ph3 = 0, poll_rounds = 0;
     const bool timing = p.phase_ticks != nullptr;
@@ -259,21 +263,14 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_forward_local(const Cha
             for (int d = 0; d < p.poll_gap; ++d) __builtin_amdgcn_s_sleep(1);
         }
         if (timing) ph1 += wall_clock64() - tk0;
-        {
-            // this lane's vector: sequence sub, source cells 4*blk .. + 3 of the wave's 64
-            const f32x4 hv = __builtin_bit_cast(f32x4, w[0]);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int lc = 4 * blk + e;
-                hb[sub][lc % KQ][lc / KQ] = hv[e];
-            }
-        }
+        // this lane's vector: sequence sub, source cells 4*blk .. + 3 of the wave's 64
+        *reinterpret_cast<f32x4 *>(&hb[sub][4 * blk]) = __builtin_bit_cast(f32x4, w[0]);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         f32x4 acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
 #pragma unroll
         for (int i4 = 0; i4 < NI; i4 += 4) {
-            const f32x4 hv = *reinterpret_cast<const f32x4 *>(&hb[sub][kq][i4]);
+            const f32x4 hv = *reinterpret_cast<const f32x4 *>(&hb[sub][NI * kq + i4]);
             acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(wreg[i4 + 0], hv[0], acc0, 0, 0, 0);
             acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(wreg[i4 + 1], hv[1], acc1, 0, 0, 0);
             acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(wreg[i4 + 2], hv[2], acc0, 0, 0, 0);
