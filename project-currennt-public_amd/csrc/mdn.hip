@@ -427,7 +427,10 @@ __global__ __launch_bounds__(64 * kFusedWaves) void mixture_error_backward_kerne
                                                                                  const float *__restrict__ para,
                                                                                  float *__restrict__ tmp,
                                                                                  float *__restrict__ result,
-                                                                                 float *__restrict__ errors) {
+                                                                                 float *__restrict__ errors,
+                                                                                 float *__restrict__ loss_acc,
+                                                                                 unsigned *__restrict__ loss_ticket,
+                                                                                 unsigned total_workgroups) {
     __shared__ float block_sum[kFusedWaves];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int M = g.M, D = g.D, MD = M * D, DV = D / 4, Lp = g.Lp;
@@ -517,7 +520,18 @@ __global__ __launch_bounds__(64 * kFusedWaves) void mixture_error_backward_kerne
         float v = 0.0f;
 #pragma unroll
         for (int w = 0; w < kFusedWaves; w += 2) v += block_sum[w] + block_sum[w + 1];
-        if (v != 0.0f) atomicAdd(result, v);
+        // The workgroups of a call (of all its units' launches) add into an accumulator of the handle; the one that
+        // finishes last hands the sum to the caller and leaves accumulator and ticket counter at zero for the next
+        // call, so that no launch has to clear the caller's result first.
+        // No fence (a device-scope fence writes the L2 back, which costs more than the kernel): the ticket is taken
+        // only after the add has returned its old value, i.e. has been performed where every XCD's atomics meet.
+        const float before = __hip_atomic_fetch_add(loss_acc, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned one = 1u;
+        asm volatile("" : "+v"(one) : "v"(before));  // the ticket's operand depends on the returned value
+        if (__hip_atomic_fetch_add(loss_ticket, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == total_workgroups - 1u) {
+            *result = __hip_atomic_exchange(loss_acc, 0.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(loss_ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 }
 
@@ -542,6 +556,8 @@ struct cnt_mdn {
     const char *pat;
     int T;
     bool covers_all_columns;
+    float *loss_acc;         // cnt_mdn_error_backward: the call's running sum (device), zero between calls
+    unsigned *loss_ticket;   // and the count of workgroups that have added to it
 };
 
 extern "C" {
@@ -552,6 +568,7 @@ int cnt_mdn_destroy(cnt_mdn *h) {
         if (u.para) (void)hipFree(u.para);
         if (u.tmp) (void)hipFree(u.tmp);
     }
+    if (h->loss_acc) (void)hipFree(h->loss_acc);
     delete h;
     return CNT_OK;
 }
@@ -620,6 +637,16 @@ int cnt_mdn_create(const cnt_mdn_desc *desc, const float *config, int config_len
     }
     h->covers_all_columns = true;
     for (char c : covered) h->covers_all_columns = h->covers_all_columns && c;
+    {
+        hipError_t err = hipMalloc(reinterpret_cast<void **>(&h->loss_acc), 256);
+        if (err == hipSuccess) err = hipMemset(h->loss_acc, 0, 256);
+        if (err != hipSuccess) {
+            set_error("mdn_create: %s", hipGetErrorString(err));
+            cnt_mdn_destroy(h);
+            return CNT_ERR_HIP;
+        }
+        h->loss_ticket = reinterpret_cast<unsigned *>(h->loss_acc) + 32;
+    }
     *out = h;
     return CNT_OK;
 }
@@ -754,14 +781,15 @@ int cnt_mdn_error_backward(cnt_mdn *h, void *stream_, const float *targets, floa
     }
     const size_t used = (size_t)h->T * h->desc.S * h->desc.Lp;
     const size_t cap = (size_t)h->desc.maxT * h->desc.S * h->desc.Lp;
-    CNT_TRY(fill_zero(stream, result_dev, 1));
     if (!h->covers_all_columns) CNT_TRY(fill_zero(stream, prev_errors, used));
     if (cap > used) CNT_TRY(fill_zero(stream, prev_errors + used, cap - used));
+    unsigned total = 0;
+    for (auto &u : h->units) total += (unsigned)((unit_geom(h, u).F + kFusedWaves - 1) / kFusedWaves);
     for (auto &u : h->units) {
         const UnitGeom g = unit_geom(h, u);
         ProfileScope prof(stream, "mdn_mixture_error_backward");
         hipLaunchKernelGGL(mixture_error_backward_kernel, dim3((g.F + kFusedWaves - 1) / kFusedWaves), dim3(64 * kFusedWaves), 0,
-                           stream, g, h->pat, targets, u.para, u.tmp, result_dev, prev_errors);
+                           stream, g, h->pat, targets, u.para, u.tmp, result_dev, prev_errors, h->loss_acc, h->loss_ticket, total);
         CNT_HIP(hipGetLastError());
     }
     return CNT_OK;
