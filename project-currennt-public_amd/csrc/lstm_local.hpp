@@ -47,21 +47,24 @@ constexpr size_t local_job_words(int H, int JB) {
     return (size_t)kMailSlots * (H / JB) * (H / JB) * kLocalSeqs * JB;
 }
 
+// The placement counters carry nothing but their own values (everything else a workgroup reads was written by earlier
+// launches), so every access to them is a relaxed device-scope atomic: acquire or release at that scope would write
+// back and invalidate the XCD's L2 at every access, also under the launches that run beside this one.
 __device__ __forceinline__ unsigned ctl_load(const unsigned *p) {
-    return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Role of this workgroup: job * 64 + member, or -1.  Called by one thread.
 __device__ int local_claim_role(const ChainParams &p, int G) {
     const unsigned xcd = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u;  // XCC_ID, bits 3:0
     if (xcd >= 8u) return -1;
-    const unsigned ticket = __hip_atomic_fetch_add(p.ctl + kCtlTickets + xcd, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned ticket = __hip_atomic_fetch_add(p.ctl + kCtlTickets + xcd, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const unsigned team = ticket / (unsigned)G, member = ticket % (unsigned)G;
     if (team >= (unsigned)kLocalTeams) return -1;
     unsigned *arrived = p.ctl + kCtlArrived + xcd * kLocalTeams + team;
     unsigned *team_job = p.ctl + kCtlTeamJob + xcd * kLocalTeams + team;
     unsigned *claimed = p.ctl + kCtlClaimed;
-    const unsigned before = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned before = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     unsigned job = 0;  // 0: undecided, j + 1: job j, kNoJob: none
     if (before == (unsigned)G - 1u) {
         // this arrival completes the team
@@ -70,9 +73,9 @@ __device__ int local_claim_role(const ChainParams &p, int G) {
             const long long t0 = wall_clock64();
             while (ctl_load(claimed) < (unsigned)p.njobs && wall_clock64() - t0 < 2000) __builtin_amdgcn_s_sleep(8);
         }
-        const unsigned c = __hip_atomic_fetch_add(claimed, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned c = __hip_atomic_fetch_add(claimed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         job = c < (unsigned)p.njobs ? c + 1u : kNoJob;
-        __hip_atomic_store(team_job, job, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(team_job, job, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
         unsigned spins = 0;
         for (;;) {
@@ -203,8 +206,13 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
         };
         StepIn in;
         const int sb = p.step_begin;
-        load_step(sb, in); wait_all_vmem(); put_coef(sb, in);
-        load_step(sb + 1, in); wait_all_vmem(); put_coef(sb + 1, in);
+        {
+            // the first two steps' inputs together: one trip to memory instead of two before the recursion starts
+            StepIn first, second;
+            load_step(sb, first); load_step(sb + 1, second);
+            wait_all_vmem();
+            put_coef(sb, first); put_coef(sb + 1, second);
+        }
         load_step(sb + 2, in);
         const bool mtiming = p.phase_ticks != nullptr;
         long long mbusy = 0;
