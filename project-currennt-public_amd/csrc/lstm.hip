@@ -823,14 +823,14 @@ struct GuardParams {
     int *abort_flag;
     unsigned *ctl;
     int nctl;
-    unsigned *mail[3];
-    size_t words[3];
+    unsigned *mail[4];
+    size_t words[4];
 };
 // the work of one workgroup (any size)
 __device__ __forceinline__ void guard_body(const GuardParams &g) {
     const bool heal = __hip_atomic_load(g.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
     if (heal) {
-        for (int m = 0; m < 3; ++m)
+        for (int m = 0; m < 4; ++m)
             for (size_t i = threadIdx.x; i < g.words[m]; i += blockDim.x) g.mail[m][i] = kEmpty;
     }
     for (int i = threadIdx.x; i < g.nctl; i += blockDim.x) g.ctl[i] = 0u;
@@ -1062,6 +1062,7 @@ struct cnt_lstm {
     int poll_delay, poll_gap, poll_delay_fwd;
     int last_was_forward;  // which recursion the diagnostic buffer describes
     int bmail_dirty;       // the backward mailbox may hold words that are not empty
+    int flmail_dirty;      // the same for the XCD-local forward recursion's mailbox
     int stepwise;          // no persistent recursion kernel for this geometry: one product + one cell kernel per step
     int *latch_host, *latch_dev;  // pinned host word a kernel that gives up sets; read by the host without a sync
     int *veto;             // a network's shared flag (device), or NULL
@@ -1271,6 +1272,7 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     g.mail[0] = reinterpret_cast<unsigned *>(h->bmail[0]); g.words[0] = h->bmail[0] ? h->bmail_words : 0;
     g.mail[1] = reinterpret_cast<unsigned *>(h->bmail[1]); g.words[1] = h->bmail[1] ? h->bmail_words : 0;
     g.mail[2] = reinterpret_cast<unsigned *>(h->lmail); g.words[2] = h->lmail ? h->lmail_words : 0;
+    g.mail[3] = reinterpret_cast<unsigned *>(h->flmail); g.words[3] = h->flmail ? h->flmail_words : 0;
     // a launch that continues a recursion in the middle: the counters are zeroed, nothing is refilled or warmed
     const bool resumes = local && p.step_begin > 0;
     CNT_REQUIRE(local || (p.step_begin == 0 && p.step_end == h->T), "lstm: only the XCD-local backward recursion runs a "
@@ -1290,10 +1292,11 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
         hipLaunchKernelGGL(chain_guard, dim3(1), dim3(1024), 0, stream, g);
         CNT_HIP(hipGetLastError());
     }
-    // Every word of a mailbox starts out empty.  The forward recursion leaves its last outputs behind; the
+    // Every word of a mailbox starts out empty.  The forward recursion across XCDs leaves its last outputs behind; the
     // backward recursions hand every word back, so their mailboxes need the fill once (and the guard above refills
     // them after a recursion that gave up).
     for (int dir = 0; dir < h->ndir; ++dir) {
+        if (fwd && h->fwd_local) continue;  // that kernel's mailbox is looked after below
         if (fwd) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->fmail[dir]), h->fmail_words, kEmpty));
         else if (h->bmail_dirty && h->bmail[dir]) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->bmail[dir]), h->bmail_words, kEmpty));
     }
@@ -1307,7 +1310,10 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
     }
     ProfileScope prof(stream, fwd ? "lstm_forward_chain" : "lstm_backward_chain");
     if (fwd && h->fwd_local) {
-        CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->flmail), h->flmail_words, kEmpty));
+        // like the backward recursions, this one hands every word back as empty: the fill is needed once (the guard
+        // refills after a launch that gave up)
+        if (h->flmail_dirty) CNT_TRY(fill_words(stream, reinterpret_cast<unsigned *>(h->flmail), h->flmail_words, kEmpty));
+        h->flmail_dirty = 0;
         int fjb = 0;
         chain_kernel_t fk = pick_local_forward_kernel(h->H, fjb);
         const int G = h->H / fjb;
@@ -1449,6 +1455,7 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     h->desc = *desc; h->ndir = ndir; h->H = H; h->JB = JB; h->NT = NT;
     h->stepwise = stepwise ? 1 : 0;
     h->bmail_dirty = 1;
+    h->flmail_dirty = 1;
     h->spin_limit = 1u << 22;
     if (const char *e = std::getenv("CNT_LSTM_SPIN_LIMIT")) h->spin_limit = (unsigned)std::strtoul(e, nullptr, 10);
     h->xcd_pack = 0;
