@@ -220,6 +220,11 @@ void lstm_set_veto(cnt_lstm *h, int *veto);
 // cnt_lstm_backward_weights in two parts that write disjoint ranges (1: input weights, 2: the rest)
 int lstm_backward_weights_parts(cnt_lstm *h, hipStream_t stream, const float *x, float *weight_updates, int parts);
 int lstm_take_failure(cnt_lstm *h);
+// makes `other` wait for the recursion launched last on this handle's device (the event the library records behind
+// every recursion launch anyway): what a stream needs that consumes the recursion's results, without another event
+// record on the launching stream
+int lstm_wait_recursion(cnt_lstm *h, hipStream_t other);
+int lstm_is_persistent(const cnt_lstm *h);  // its recursions are single launches (not the step-by-step schedule)
 int report_failure(cnt_network *net, hipStream_t stream);
 
 // ----- error halves that also do the backward step of the skip layer in front of them ----------------

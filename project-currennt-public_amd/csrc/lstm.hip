@@ -1627,6 +1627,16 @@ extern "C++" void cnt::lstm_set_veto(cnt_lstm *h, int *veto) {
     if (h) h->veto = veto;
 }
 
+extern "C++" int cnt::lstm_is_persistent(const cnt_lstm *h) { return h && !h->stepwise ? 1 : 0; }
+
+extern "C++" int cnt::lstm_wait_recursion(cnt_lstm *h, hipStream_t other) {
+    CNT_REQUIRE(h, "lstm_wait_recursion: null handle");
+    RecursionOrder &o = recursion_order(h->device);
+    std::lock_guard<std::mutex> lock(o.mu);
+    if (o.done && o.any) CNT_HIP(hipStreamWaitEvent(other, o.done, 0));
+    return CNT_OK;
+}
+
 extern "C++" int cnt::lstm_take_failure(cnt_lstm *h) {
     if (!h || !h->latch_host) return 0;
     volatile int *latch = h->latch_host;

@@ -1421,13 +1421,18 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     // layers' weight gradients end the pass side by side) and loses 2% on the WaveNet stack (three batched products
     // at once crowd the error chain on the main stream).
     int next_small = 0;
+    cnt_lstm *after_recursion = nullptr;  // set: the side stream waits for this layer's recursion, just launched
     auto next_side_stream = [&](hipStream_t *ws, bool large) -> int {
         int &cursor = large ? next_side : next_small;
         const int span = large ? net->n_side : std::min(net->n_side, 2);
         cursor %= span;
         *ws = net->side[cursor];
-        CNT_HIP(hipEventRecord(net->ev_main, stream));
-        CNT_HIP(hipStreamWaitEvent(*ws, net->ev_main, 0));
+        if (after_recursion) {
+            CNT_TRY(lstm_wait_recursion(after_recursion, *ws));
+        } else {
+            CNT_HIP(hipEventRecord(net->ev_main, stream));
+            CNT_HIP(hipStreamWaitEvent(*ws, net->ev_main, 0));
+        }
         side_used[cursor] = true;
         cursor = (cursor + 1) % span;
         return CNT_OK;
@@ -1633,7 +1638,10 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                         // further along when the next layer's recursion starts: acoustic model 2.88 -> 2.78 ms.
                         CNT_TRY(cnt_lstm_backward_errors(L.lstm, stream, W, L.err, nullptr));
                         pending.push_back(i);
-                        CNT_TRY(hand_over(true));
+                        after_recursion = lstm_is_persistent(L.lstm) ? L.lstm : nullptr;
+                        const int handed = hand_over(true);
+                        after_recursion = nullptr;
+                        CNT_TRY(handed);
                         CNT_TRY(cnt_lstm_backward_prev_errors(L.lstm, stream, W, prev_err));
                         break;
                     }
