@@ -1474,9 +1474,11 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     }
     // XCD-local recursion: product (about 0.3 us) and one hop through the L2 (about 0.45 us) pass between a step's
     // barrier and the arrival of the next partial errors
-    // (fitted on the benchmark models: 10-12 give the acoustic model's pass 2.65 ms where 8 gives 2.68 and 16 gives 2.69;
-    // the same recursion alone is best at 8, 0.92 against 0.94 ms -- beside other streams' products the words arrive later)
-    h->poll_delay_local = 11;
+    // (fitted on the benchmark models with one workgroup of a team per compute unit: the acoustic model's pass takes
+    // 2.41 / 2.38 / 2.35 / 2.39 / 2.47 / 2.50 ms at 8 / 9 / 10 / 11 / 12 / 13 units, the single 256-cell layer 0.355 /
+    // 0.353 / 0.361 ms at 9 / 10 / 11: a pause that ends after the words have arrived costs a whole poll round less,
+    // one that ends too late costs its own length)
+    h->poll_delay_local = 10;
     h->warm = 1;
     if (const char *e = std::getenv("CNT_LSTM_WARM")) h->warm = std::atoi(e) != 0;
     {
@@ -1610,7 +1612,7 @@ int cnt_lstm_set_wait_bounds(cnt_lstm *h, unsigned spin_limit, int poll_delay_ba
                 poll_delay_forward <= 4096, "lstm_set_wait_bounds: poll delays must be within 0..4096");
     h->spin_limit = spin_limit;
     h->poll_delay = poll_delay_backward;
-    h->poll_delay_local = poll_delay_backward < 11 ? poll_delay_backward : 11;
+    h->poll_delay_local = poll_delay_backward < 10 ? poll_delay_backward : 10;
     h->poll_delay_fwd = poll_delay_forward;
     h->poll_delay_fwd_local = poll_delay_forward < 24 ? poll_delay_forward : h->poll_delay_fwd_local;
     return CNT_OK;
