@@ -67,6 +67,7 @@ struct ChainParams {
     int xcd_pack;
     long long *phase_ticks;  // optional diagnostic: per workgroup accumulated phase durations (100 MHz ticks)
     int poll_delay, poll_gap;  // s_sleep units before the first poll of a step / between polls
+    int mem_delay;             // XCD-local backward recursion: s_sleep units before the memory wave's work of a step
     int poll_delay_fwd;
     int *latch;  // host-visible mark "a recursion of this handle gave up" (pinned host memory), never cleared by kernels
     int *veto;   // optional device flag shared by a network's handles, set together with the latch
@@ -1080,6 +1081,7 @@ struct cnt_lstm {
     int warm;  // read the recursion's inputs once before the XCD-local backward recursion (CNT_LSTM_WARM=0: off)
     int spread_lds;  // dynamic LDS the XCD-local recursion asks for so that a compute unit takes one of its workgroups
     int poll_delay_local;  // pause before the first poll of a step in the XCD-local recursion, units of 64 clocks
+    int mem_delay_local;   // pause of that recursion's memory wave after the step barrier, same units
     int poll_delay_fwd_local;  // the same for the XCD-local forward recursion
     // set by every recursion launch: the failure latch is taken only once the launch that may have set it has ended
     // (the device's recursion-order event, see launch_in_order), so that no workgroup of that launch can set it (or the
@@ -1331,6 +1333,7 @@ int launch_chain(cnt_lstm *h, hipStream_t stream, bool fwd, ChainParams &p) {
         const int blocks = (h->njobs * G + 8 * (G - 1) + 7) / 8 * 8;
         h->last_blocks = blocks;
         p.poll_delay = h->poll_delay_local;
+        p.mem_delay = h->mem_delay_local;
         // One workgroup per compute unit.  A team's workgroups take a step in lock-step, and two of them on one compute
         // unit share its four matrix pipes and its path to the L2 at exactly the same moments: the dispatcher, left to
         // itself, puts the 32 workgroups of a 256-cell team on 16-17 compute units, and a step then takes 1.55 us instead
@@ -1479,6 +1482,13 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     // 0.353 / 0.361 ms at 9 / 10 / 11: a pause that ends after the words have arrived costs a whole poll round less,
     // one that ends too late costs its own length)
     h->poll_delay_local = 10;
+    // The memory wave's loads and stores of a step are issued once the first poll is expected back: pause of the poll
+    // plus one poll round (four 16-byte loads per lane at 256 cells, two or one below).  Measured on MI355X: acoustic
+    // model 2.39 / 2.53 / 2.52 / 2.36 / 2.31 / 2.32 / 2.34 / 2.36 ms at 0 / 12 / 14 / 16 / 17 / 18 / 19 / 24 units (a wave that
+    // wakes while the poll is in flight is the worst case); a 128- or 64-cell BLSTM layer alone 716 / 661 / 695 / 722 us
+    // and 688 / 641 / 678 / 713 us at 0 / 15 / 17 / 19 units.
+    h->mem_delay_local = h->poll_delay_local + (H >= 256 ? 7 : 5);
+    if (const char *e = std::getenv("CNT_LSTM_MEM_DELAY")) h->mem_delay_local = std::atoi(e);
     h->warm = 1;
     if (const char *e = std::getenv("CNT_LSTM_WARM")) h->warm = std::atoi(e) != 0;
     {
@@ -1613,6 +1623,7 @@ int cnt_lstm_set_wait_bounds(cnt_lstm *h, unsigned spin_limit, int poll_delay_ba
     h->spin_limit = spin_limit;
     h->poll_delay = poll_delay_backward;
     h->poll_delay_local = poll_delay_backward < 10 ? poll_delay_backward : 10;
+    if (poll_delay_backward < 10) h->mem_delay_local = poll_delay_backward;
     h->poll_delay_fwd = poll_delay_forward;
     h->poll_delay_fwd_local = poll_delay_forward < 24 ? poll_delay_forward : h->poll_delay_fwd_local;
     return CNT_OK;

@@ -221,6 +221,11 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
             const int t = slot_of(step), b = step & 1;
             lds_barrier();  // results of this step are in LDS; the cell wave is done with this parity's coefficients
             if (wait_failed) return;
+            // This wave's loads and stores have a whole step to complete, but a compute unit returns its vector-memory
+            // accesses in order over all of its waves: issued while the cell wave's poll for the next step is in flight
+            // they hold that poll back.  The wave sleeps until the first poll is expected back (its coefficient
+            // arithmetic then also stays off the SIMD of a product wave while the products run).
+            for (int d = 0; d < p.mem_delay; ++d) __builtin_amdgcn_s_sleep(1);
             const long long tm0 = mtiming ? wall_clock64() : 0;
             wait_all_vmem();  // inputs requested a step ago are there, state stores of the step before are done
             put_coef(step + 2, in);
