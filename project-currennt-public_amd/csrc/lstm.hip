@@ -1078,7 +1078,7 @@ struct cnt_lstm {
     size_t flmail_words;
     int fwd_local;
     int last_blocks;       // workgroups of the last recursion launch
-    int warm;  // read the recursion's inputs once before the XCD-local backward recursion (CNT_LSTM_WARM=0: off)
+    int warm;  // read the recursion's inputs once before the XCD-local backward recursion (off; CNT_LSTM_WARM=1: on)
     int spread_lds;  // dynamic LDS the XCD-local recursion asks for so that a compute unit takes one of its workgroups
     int poll_delay_local;  // pause before the first poll of a step in the XCD-local recursion, units of 64 clocks
     int mem_delay_local;   // pause of that recursion's memory wave after the step barrier, same units
@@ -1486,10 +1486,14 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     // plus one poll round (four 16-byte loads per lane at 256 cells, two or one below).  Measured on MI355X: acoustic
     // model 2.39 / 2.53 / 2.52 / 2.36 / 2.31 / 2.32 / 2.34 / 2.36 ms at 0 / 12 / 14 / 16 / 17 / 18 / 19 / 24 units (a wave that
     // wakes while the poll is in flight is the worst case); a 128- or 64-cell BLSTM layer alone 716 / 661 / 695 / 722 us
-    // and 688 / 641 / 678 / 713 us at 0 / 15 / 17 / 19 units.
-    h->mem_delay_local = h->poll_delay_local + (H >= 256 ? 7 : 5);
+    // and 688 / 641 / 678 / 713 us at 0 / 15 / 17 / 19 units.  One unit more than the best value: the step from 16 to 17
+    // units is a cliff (2.45 -> 2.28 ms without the cache-warming read), the one from 17 to 18 costs 0.4 %.
+    h->mem_delay_local = h->poll_delay_local + (H >= 256 ? 8 : 6);
     if (const char *e = std::getenv("CNT_LSTM_MEM_DELAY")) h->mem_delay_local = std::atoi(e);
-    h->warm = 1;
+    // The full-bandwidth read of the recursion's inputs in front of it (warm_cache) was worth 0.15 ms per model pass
+    // while the memory wave's loads were issued in front of the polls; with that wave's pause it costs more than it
+    // gains (2.290 -> 2.282 ms without it, 0.355 -> 0.352 ms for the single layer).  CNT_LSTM_WARM=1 turns it on.
+    h->warm = 0;
     if (const char *e = std::getenv("CNT_LSTM_WARM")) h->warm = std::atoi(e) != 0;
     {
         // a little more than half of a compute unit's LDS (160 KB on gfx950: 82 KB); the kernel's own few KB come on top
