@@ -140,8 +140,9 @@ typedef struct {
  * workgroup of a team gets a compute unit of its own (two on one unit take their steps at the same moments and cost
  * a fifth of the step time).  Environment, read when a handle is created: CNT_LSTM_LOCAL=0 / CNT_LSTM_FWD_LOCAL=0
  * (the kernels that exchange across XCDs instead), CNT_LSTM_SPREAD_LDS=<bytes> (the LDS request, 0: none),
- * CNT_LSTM_LOCAL_JB=16 (16 instead of 8 cells per workgroup for 256-cell layers), CNT_LSTM_WARM=0 (no read of the
- * states into the memory-side cache in front of the backward recursion), CNT_LSTM_STEPWISE=1. */
+ * CNT_LSTM_LOCAL_JB=16 (16 instead of 8 cells per workgroup for 256-cell layers), CNT_LSTM_WARM=1 (a full-bandwidth
+ * read of the states into the memory-side cache in front of the backward recursion), CNT_LSTM_MEM_DELAY=<units of 64
+ * clocks> (how long the backward recursion's memory wave sleeps after a step's barrier), CNT_LSTM_STEPWISE=1. */
 int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out);
 int cnt_lstm_destroy(cnt_lstm *h);
 /* LstmLayer::loadSequences (layers/LstmLayer.cu:1488-1533): records the fraction's geometry and

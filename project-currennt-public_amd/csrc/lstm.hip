@@ -1486,9 +1486,12 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     // plus one poll round (four 16-byte loads per lane at 256 cells, two or one below).  Measured on MI355X: acoustic
     // model 2.39 / 2.53 / 2.52 / 2.36 / 2.31 / 2.32 / 2.34 / 2.36 ms at 0 / 12 / 14 / 16 / 17 / 18 / 19 / 24 units (a wave that
     // wakes while the poll is in flight is the worst case); a 128- or 64-cell BLSTM layer alone 716 / 661 / 695 / 722 us
-    // and 688 / 641 / 678 / 713 us at 0 / 15 / 17 / 19 units.  One unit more than the best value: the step from 16 to 17
-    // units is a cliff (2.45 -> 2.28 ms without the cache-warming read), the one from 17 to 18 costs 0.4 %.
-    h->mem_delay_local = h->poll_delay_local + (H >= 256 ? 8 : 6);
+    // and 688 / 641 / 678 / 713 us at 0 / 15 / 17 / 19 units.  With the mailbox hand-back stores in this wave as well the
+    // landscape moves by one unit (2.51 / 2.35 / 2.28 / 2.30 / 2.31 / 2.34 ms at 16 / 17 / 18 / 19 / 20 / 21).  The value kept
+    // is one unit behind the best one: the step in front of the best value is a cliff, the step behind it costs 0.2 %.
+    // (128- and 64-cell layers alone, hand-back stores included: 679 / 647 / 657 / 676 us and 683 / 648 / 662 / 672 us at
+    // 14 / 15 / 16 / 17 units.)
+    h->mem_delay_local = h->poll_delay_local + (H >= 256 ? 9 : 6);
     if (const char *e = std::getenv("CNT_LSTM_MEM_DELAY")) h->mem_delay_local = std::atoi(e);
     // The full-bandwidth read of the recursion's inputs in front of it (warm_cache) was worth 0.15 ms per model pass
     // while the memory wave's loads were issued in front of the polls; with that wave's pause it costs more than it

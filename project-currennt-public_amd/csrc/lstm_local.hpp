@@ -238,6 +238,16 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
                 if (p.herr_out) p.herr_out[gi] = res[b][0][lane];
                 else D.herr[gi] = res[b][0][lane];
             }
+            if (step > 0) {
+                // The words the cell wave consumed in this step (before the barrier) are empty again.  The slot is used
+                // again three steps from now, so this hand-back can wait for this wave's turn instead of sitting in
+                // front of the next poll in the compute unit's queue.
+                const u32x4 empty = {kEmpty, kEmpty, kEmpty, kEmpty};
+#pragma unroll
+                for (int q = 0; q < RECV / 256; ++q)
+                    __builtin_amdgcn_raw_buffer_store_b128(empty, mail, (int)((unsigned)((step - 1) % kMailSlots) * slot_words * 4u +
+                                                           ((unsigned)me * RECV + (unsigned)(q * 64 + lane) * 4u) * 4u), 0, 0);
+            }
             if (mtiming) mbusy += wall_clock64() - tm0;
         }
         if (mtiming && lane == 0) {
@@ -260,8 +270,6 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
         const int bj = lane & 3, first_cell = 64 * pw + 4 * (lane >> 2);
         const unsigned pub_off = ((unsigned)(first_cell / JB) * RECV + (unsigned)me * PAIR + (unsigned)bj * JB +
                                   (unsigned)(first_cell % JB)) * 4u;
-        // reset role: sixteen bytes of the block this workgroup's cell wave polls
-        const unsigned reset_off = ((unsigned)me * RECV + (unsigned)(tid - 64) * 4u) * 4u;
         wait_all_vmem();
         lds_barrier();  // start of the recursion
         const bool timing = p.phase_ticks != nullptr;
@@ -293,11 +301,6 @@ __global__ __launch_bounds__(local_threads(H)) void lstm_backward_local(const Ch
                 v.x = v.x == kEmpty ? 0x7FC00000u : v.x; v.y = v.y == kEmpty ? 0x7FC00000u : v.y;
                 v.z = v.z == kEmpty ? 0x7FC00000u : v.z; v.w = v.w == kEmpty ? 0x7FC00000u : v.w;
                 __builtin_amdgcn_raw_buffer_store_b128(v, mail, (int)((unsigned)(step % kMailSlots) * slot_words * 4u + pub_off), 0, 0);
-            }
-            if (step > 0) {
-                // the words the cell wave consumed in this step (before the barrier) are empty again
-                const u32x4 empty = {kEmpty, kEmpty, kEmpty, kEmpty};
-                __builtin_amdgcn_raw_buffer_store_b128(empty, mail, (int)((unsigned)((step - 1) % kMailSlots) * slot_words * 4u + reset_off), 0, 0);
             }
             if (tid == 64) trace_stamp(p, step, 4);
             if (failed) return;
