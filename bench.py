@@ -40,7 +40,7 @@ CHAIN_TRAFFIC_SOURCE = "profiles/acoustic_backward_hbm_traffic.md"
 # csrc/lstm_local.hpp); when the file has changed since, the figure no longer describes the kernel that runs and the
 # benchmark prints null for it.
 CHAIN_TRAFFIC_KERNEL = "lstm_backward_local<256, 8>"
-CHAIN_TRAFFIC_SOURCE_SHA16 = "fa4ad345c470a9d0"
+CHAIN_TRAFFIC_SOURCE_SHA16 = "1e7524efa6f2effe"
 
 METRIC = "BLSTM backward frames/sec at 1 MI355X; % HBM/MFMA roofline vs host CPU"
 PEAK_FP32_MFMA_TFLOPS = 157.3
