@@ -135,6 +135,8 @@ enum GemmEpilogue {
     EPI_CONTEXT = 5,        // th = tanh(acc); aux_out = th; C = aux_in + th; both 0 on "none" columns
     EPI_PARTIAL = 6,        // split-K without atomics: every split stores its m x n partial product into the
                             // launcher's scratch, and a second kernel sums the splits into C (set by gemm_plan)
+    EPI_STORE_DELTA = 8,    // C = acc * act'(aux_in): the product that writes a dense layer's output errors turns them
+                            // into that layer's deltas on the way out (aux_in = the layer's outputs, layout of C)
     EPI_FAN = 7             // a skip layer's backward step in the epilogue of the product that writes the layer's
                             // errors: e = aux_in + acc (aux_in may be NULL), C = e, and e goes on to fan_n buffers of
                             // C's layout -- added to those flagged in fan_is_skip, stored over the others
@@ -146,7 +148,7 @@ struct GemmProblem {
     int b_shift[kGemmMaxSeg];  // masked mode: time-slot shift of the B operand per operand pair
     float *C;
     const float *bias_vec;
-    const float *aux_in;  // EPI_CONTEXT, same layout as C
+    const float *aux_in;  // EPI_CONTEXT, EPI_STORE_DELTA: same layout as C
     float *aux_out;       // EPI_CONTEXT, may be NULL
     float *rowsum_out;    // GemmArgs::rowsum: receives rowsum_scale * sum_k B(j, k), j < n
     float rowsum_scale;
@@ -241,7 +243,13 @@ struct FanOut {
 // *fused tells whether the step was done (operands that the fan epilogue does not exist for, or a convolution
 // with several filter groups, leave it to the caller).
 int dense_backward_errors_fan(hipStream_t stream, int P, int D, int N, int act, const float *weights, const float *y,
-                              float *err, float *prev_err, const FanOut *fan, bool *fused);
+                              float *err, float *prev_err, const FanOut *fan, bool *fused, int prev_act = ACT_IDENTITY,
+                              const float *prev_y = nullptr);
+// (prev_act, prev_y): the preceding layer is a dense layer with that activation and those outputs, and nothing but
+// this product writes its output errors: the product stores act'(prev_y) * error, the preceding layer's deltas, and
+// that layer's own backward step then runs with ACT_IDENTITY.  The same for a recurrent layer's error product:
+int lstm_prev_errors_delta(cnt_lstm *h, hipStream_t stream, const float *weights, float *prev_errors, int prev_act,
+                           const float *prev_y);
 // Error path of one WaveNet residual block in one launch (skip 1x1 layer, the skip layer in front of it, the 1x1
 // layer behind the gated unit, the gated unit): see wavenet_block_errors_kernel.
 bool wavenet_block_errors_supported(int R, int K);

@@ -174,7 +174,7 @@ int cnt_dense_backward_errors(void *stream, int P, int D, int N, int act, const 
 
 extern "C++" int cnt::dense_backward_errors_fan(hipStream_t stream, int P, int D, int N, int act, const float *weights,
                                                 const float *y, float *err, float *prev_err, const FanOut *fan,
-                                                bool *fused) {
+                                                bool *fused, int prev_act, const float *prev_y) {
     if (fused) *fused = false;
     CNT_REQUIRE(weights && y && err, "dense_backward_errors: null argument");
     CNT_REQUIRE(P > 0 && D > 0 && N > 0, "dense_backward_errors: non-positive size");
@@ -195,6 +195,11 @@ extern "C++" int cnt::dense_backward_errors_fan(hipStream_t stream, int P, int D
         ga.ldc = P;
         ga.nseg = 1; ga.nprob = 1; ga.splitk = 1; ga.epilogue = EPI_STORE;
         ga.prob[0].A[0] = weights; ga.prob[0].B[0] = err; ga.prob[0].C = prev_err;
+        if (prev_act != ACT_IDENTITY && prev_y && !fan) {
+            ga.epilogue = EPI_STORE_DELTA;
+            ga.act = prev_act;
+            ga.prob[0].aux_in = prev_y;
+        }
         if (fan && fused && gemm_fan_supported(ga)) {
             ga.epilogue = EPI_FAN;
             ga.fan_n = fan->n; ga.fan_targets = fan->targets; ga.fan_is_skip = fan->is_skip;

@@ -246,6 +246,8 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
                 args.nprob, kGemmMaxProb);
     CNT_REQUIRE(args.splitk >= 0 && (args.splitk == 1 || args.epilogue == EPI_ATOMIC || args.epilogue == EPI_PARTIAL),
                 "gemm: split-K needs the atomic epilogue");
+    CNT_REQUIRE(args.epilogue != EPI_STORE_DELTA || (args.splitk == 1 && args.prob[0].aux_in != nullptr),
+                "gemm: the delta epilogue needs the preceding layer's outputs and no split");
     CNT_REQUIRE(args.epilogue != EPI_FAN || (gemm_fan_supported(args) && args.splitk == 1),
                 "gemm: the fan epilogue exists for one unsplit problem with 16-byte row-contiguous A and k-contiguous B");
     CNT_REQUIRE(args.epilogue != EPI_PARTIAL || (args.splitk >= 1 && args.partial_stride > 0 && args.partial),

@@ -391,6 +391,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
                 const float v = acc[i][j][r];
                 switch (args.epilogue) {
                     case EPI_STORE: *dst = v; break;
+                    case EPI_STORE_DELTA: *dst = v * act_deriv(args.act, pb.aux_in[idx]); break;
                     case EPI_ADD: *dst = *dst + v; break;
                     case EPI_ATOMIC: atomicAdd(dst, v); break;
 

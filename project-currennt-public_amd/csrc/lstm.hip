@@ -1863,6 +1863,32 @@ int cnt_lstm_backward_prev_errors_range(cnt_lstm *h, void *stream_, const float 
     return CNT_OK;
 }
 
+// cnt_lstm_backward_prev_errors whose product also applies the derivative of the preceding (dense) layer's activation
+extern "C++" int cnt::lstm_prev_errors_delta(cnt_lstm *h, hipStream_t stream, const float *weights, float *prev_errors,
+                                             int prev_act, const float *prev_y) {
+    CNT_REQUIRE(h && weights && prev_errors && prev_y, "lstm_prev_errors_delta: null argument");
+    CNT_REQUIRE(h->T > 0, "lstm_prev_errors_delta: load_sequences has not been called");
+    CNT_LSTM_REPORT_FAILURE(h);
+    const cnt_lstm_desc &d = h->desc;
+    const int P = d.P, L = d.L, H = h->H, N = h->T * d.S;
+    GemmArgs ga = {};
+    ga.m = P; ga.n = N; ga.k = H;
+    ga.a_kcontig = 0; ga.lda = P;
+    ga.b_kcontig = 1; ga.ldb = H;
+    ga.ldc = P;
+    ga.nseg = 4 * h->ndir; ga.nprob = 1; ga.splitk = 1; ga.epilogue = EPI_STORE_DELTA;
+    ga.act = prev_act;
+    for (int dir = 0; dir < h->ndir; ++dir)
+        for (int g = 0; g < 4; ++g) {
+            ga.prob[0].A[dir * 4 + g] = weights + (size_t)g * P * L + (size_t)dir * P * H;
+            ga.prob[0].B[dir * 4 + g] = h->state[dir][7 + g];
+        }
+    ga.prob[0].C = prev_errors;
+    ga.prob[0].aux_in = prev_y;
+    ga.label = "gemm:lstm_prev_errors";
+    return gemm_launch(stream, ga);
+}
+
 int cnt_lstm_backward_weights(cnt_lstm *h, void *stream, const float *x, float *weight_updates) {
     return cnt::lstm_backward_weights_parts(h, static_cast<hipStream_t>(stream), x, weight_updates, 3);
 }

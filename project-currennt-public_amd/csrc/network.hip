@@ -1375,6 +1375,21 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
     // weight halves of small layers are collected and handed over a few at a time, those of large layers at once.
     std::vector<char> fan_done(net->layers.size(), 0);
     std::vector<char> errors_done(net->layers.size(), 0);  // error step done by the block launch of a later layer
+    // A dense layer whose output errors are written by the one product of the layer above it (no skip layer links to
+    // it): that product's epilogue multiplies with the derivative of the dense layer's activation, so the errors
+    // arrive as deltas and the layer's own delta launch is left out.
+    std::vector<char> delta_done(net->layers.size(), 0);
+    std::vector<char> feeds_skip(net->layers.size(), 0);
+    for (const NetLayer &S : net->layers)
+        for (int x : S.pre)
+            if (x >= 0 && (size_t)x < feeds_skip.size()) feeds_skip[(size_t)x] = 1;
+    static const bool fuse_delta = [] { const char *e = std::getenv("CNT_NET_FUSE_DELTA"); return !e || std::atoi(e) != 0; }();
+    auto delta_target = [&](size_t below) {
+        const NetLayer &B = net->layers[below];
+        // (the layer that feeds the conditioning of wavnetc layers gets their share of the gradient added later)
+        return fuse_delta && below >= 1 && B.kind == K_DENSE && B.act != ACT_IDENTITY && B.err && !feeds_skip[below] &&
+               (int)below != net->flagged && !is_skip_kind(net->layers[below + 1].kind);
+    };
     for (auto &L : net->layers) L.colsum_rows = 0;
     static const bool fuse_blocks = [] { const char *e = std::getenv("CNT_NET_FUSE_BLOCKS"); return !e || std::atoi(e) != 0; }();
     // WaveNet residual block seen from its skip 1x1 layer i: [cnn 2R][wavnetc R][dense R, identity][skipadd, shares
@@ -1613,19 +1628,25 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                     if (L.kind == K_DENSE && early && net->overlap && prev_err && (double)prev.size * L.size * N >= 4e8) {
                         // a large dense layer: deltas first, then its weight half starts on a side stream next to the
                         // product for the preceding layer's errors instead of after it
-                        CNT_TRY(dense_backward_errors_fan(stream, prev.size, L.size, N, L.act, W, L.out, L.err, nullptr, nullptr,
-                                                          nullptr));
+                        CNT_TRY(dense_backward_errors_fan(stream, prev.size, L.size, N, delta_done[i] ? ACT_IDENTITY : L.act, W,
+                                                          L.out, L.err, nullptr, nullptr, nullptr));
                         pending.push_back(i);
                         CNT_TRY(hand_over(true));
+                        const bool below = !wanted && prev_err == prev.err && prev.N == N && delta_target(i - 1);
                         CNT_TRY(dense_backward_errors_fan(stream, prev.size, L.size, N, ACT_IDENTITY, W, L.out, L.err, prev_err,
-                                                          wanted ? &fan : nullptr, &fused));
+                                                          wanted ? &fan : nullptr, &fused, below ? prev.act : ACT_IDENTITY,
+                                                          below ? prev.out : nullptr));
+                        if (below) delta_done[i - 1] = 1;
                         fan_done[i - 1] = fused ? 1 : 0;
                         break;
                     }
-                    if (L.kind == K_DENSE)
-                        CNT_TRY(dense_backward_errors_fan(stream, prev.size, L.size, N, L.act, W, L.out, L.err, prev_err,
-                                                          wanted ? &fan : nullptr, &fused));
-                    else
+                    if (L.kind == K_DENSE) {
+                        const bool below = !wanted && prev_err && prev_err == prev.err && prev.N == N && delta_target(i - 1);
+                        CNT_TRY(dense_backward_errors_fan(stream, prev.size, L.size, N, delta_done[i] ? ACT_IDENTITY : L.act, W,
+                                                          L.out, L.err, prev_err, wanted ? &fan : nullptr, &fused,
+                                                          below ? prev.act : ACT_IDENTITY, below ? prev.out : nullptr));
+                        if (below) delta_done[i - 1] = 1;
+                    } else
                         CNT_TRY(cnn_backward_errors_fan(L.cnn, stream, L.pat, L.T, W, L.out, L.err, prev_err,
                                                         L.delta_fused ? 1 : 0, wanted ? &fan : nullptr, &fused));
                     fan_done[i - 1] = fused ? 1 : 0;
@@ -1642,7 +1663,12 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
                         const int handed = hand_over(true);
                         after_recursion = nullptr;
                         CNT_TRY(handed);
-                        CNT_TRY(cnt_lstm_backward_prev_errors(L.lstm, stream, W, prev_err));
+                        if (prev_err == prev.err && prev.N == N && delta_target(i - 1)) {
+                            CNT_TRY(lstm_prev_errors_delta(L.lstm, stream, W, prev_err, prev.act, prev.out));
+                            delta_done[i - 1] = 1;
+                        } else {
+                            CNT_TRY(cnt_lstm_backward_prev_errors(L.lstm, stream, W, prev_err));
+                        }
                         break;
                     }
                     CNT_TRY(cnt_lstm_backward_errors(L.lstm, stream, W, L.err, prev_err));
