@@ -168,6 +168,90 @@ struct TileStage {
     }
 };
 
+// The unmasked loader.  What a thread loads differs from tile to tile only by the tile's k
+// offset, so everything per thread is computed once: `voff`, the byte offset of its vector inside the operand at k = 0
+// (row clamped into the matrix), as a 32-bit offset beside a 64-bit base that is uniform over the workgroup -- the
+// address form that costs no vector arithmetic per load -- and which of its vectors lie inside the matrix.  A tile
+// needs masking only at the matrix edge or in the last, partly filled k tile of an operand pair; both are uniform over
+// the workgroup (`special`), every other tile is stored as it arrived.
+template <int VEC, bool KCONTIG, int ROWS>
+struct FastStage {
+    static constexpr int NLOAD = (ROWS * BK) / (NTHREADS * VEC);
+    typedef typename VecT<VEC>::type vec_t;
+    vec_t r[NLOAD];
+    unsigned voff[NLOAD];    // byte offsets at k = 0
+    unsigned koff[NLOAD];    // what has to be taken off voff to reach k position 0 of the tile (used in a k tail only)
+    int kpos[NLOAD];         // first k of the vector inside the tile
+    bool row_ok[NLOAD];
+    bool edge;               // uniform: some row of this tile lies outside the matrix
+    int k_valid;             // uniform: k values of the tile in registers that lie inside the operand pair
+
+    __device__ __forceinline__ void init(int ld, int row0, int rows_total, int tid) {
+        edge = row0 + ROWS > rows_total;
+        if (KCONTIG) {
+            constexpr int TPR = BK / VEC, RPP = NTHREADS / TPR;
+            const int kq = (tid % TPR) * VEC, rr = tid / TPR;
+#pragma unroll
+            for (int p = 0; p < NLOAD; ++p) {
+                const int row = row0 + rr + p * RPP;
+                row_ok[p] = row < rows_total;
+                voff[p] = (unsigned)(((size_t)min(row, rows_total - 1) * ld + kq) * sizeof(float));
+                koff[p] = (unsigned)(kq * sizeof(float));
+                kpos[p] = kq;
+            }
+        } else {
+            constexpr int TPK = ROWS / VEC, KPP = NTHREADS / TPK;
+            const int rq = (tid % TPK) * VEC, kk = tid / TPK;
+#pragma unroll
+            for (int p = 0; p < NLOAD; ++p) {
+                const int k = kk + p * KPP;
+                row_ok[p] = (row0 + rq) < rows_total;
+                const int rc = row_ok[p] ? row0 + rq : 0;
+                voff[p] = (unsigned)(((size_t)k * ld + rc) * sizeof(float));
+                koff[p] = (unsigned)((size_t)k * ld * sizeof(float));
+                kpos[p] = k;
+            }
+        }
+    }
+    // base = the operand at the tile's first k (uniform), kv = valid k values of the tile
+    __device__ __forceinline__ void load(const float *__restrict__ base, int kv) {
+        k_valid = kv;
+        const char *b = reinterpret_cast<const char *>(base);
+        if (kv >= BK) {
+#pragma unroll
+            for (int p = 0; p < NLOAD; ++p) r[p] = *reinterpret_cast<const vec_t *>(b + voff[p]);
+        } else {
+            // partly filled tile: a vector beyond the operand's k extent is read from k position 0 instead (in bounds)
+            // and dropped at the store
+#pragma unroll
+            for (int p = 0; p < NLOAD; ++p)
+                r[p] = *reinterpret_cast<const vec_t *>(b + (kpos[p] < kv ? voff[p] : voff[p] - koff[p]));
+        }
+    }
+    __device__ __forceinline__ void store(float *__restrict__ lds, int tid) const {
+        const bool special = edge || k_valid < BK;
+        if (KCONTIG) {
+            constexpr int TPR = BK / VEC, RPP = NTHREADS / TPR;
+            const int kq = (tid % TPR) * VEC, rr = tid / TPR;
+#pragma unroll
+            for (int p = 0; p < NLOAD; ++p) {
+                vec_t v = r[p];
+                if (special && !(row_ok[p] && kpos[p] < k_valid)) v = vec_t{};
+                *reinterpret_cast<vec_t *>(lds + (rr + p * RPP) * PITCH + kq) = v;
+            }
+        } else {
+            constexpr int TPK = ROWS / VEC, KPP = NTHREADS / TPK;
+            const int rq = (tid % TPK) * VEC, kk = tid / TPK;
+#pragma unroll
+            for (int p = 0; p < NLOAD; ++p) {
+                vec_t v = r[p];
+                if (special && !(row_ok[p] && kpos[p] < k_valid)) v = vec_t{};
+                *reinterpret_cast<vec_t *>(lds + (kk + p * KPP) * ROWS + rq) = v;
+            }
+        }
+    }
+};
+
 // MASKED selects the time-shifted, padding-masked B loader at compile time: its per-element predication is a lot
 // of code, and four copies of it (two prologue fetches, two in the unrolled loop) inside the plain kernels would
 // push their hot loop out of the instruction cache.
@@ -232,16 +316,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     // workgroup per compute unit, which is what the benchmark's shapes give, nothing else hides that latency.
     // The loop is unrolled by two so that the sets swap roles without register copies, and its barrier orders
     // LDS only (__syncthreads() would also drain the loads in flight).
-    TileStage<VA, AK, TILE> sa0, sa1;
-    TileStage<VB, BK_, TILE> sb0, sb1;
     const char *mask_pat = MASKED ? args.pat : nullptr;
-    auto fetch = [&](int it, TileStage<VA, AK, TILE> &ra, TileStage<VB, BK_, TILE> &rb) __attribute__((always_inline)) {
-        const int seg = it / kt_per_seg;
-        const int k0 = (it % kt_per_seg) * BK;
-        ra.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
-        rb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid, mask_pat, pb.b_shift[seg], args.n_slots,
-                args.b_time_on_k != 0);
-    };
 
     // sum of the B operand over this split's k range, per row (dense bias gradient); kept by the waves with wm == 0
     const bool rowsum = args.rowsum != 0;
@@ -249,55 +324,93 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
 #pragma unroll
     for (int j = 0; j < NB; ++j) rs[j] = 0.0f;
 
-    fetch(it_begin, sa0, sb0);
-    fetch(min(it_begin + 1, it_end - 1), sa1, sb1);
-    sa0.store(lds_a[0], tid);
-    sb0.store(lds_b[0], tid);
-    lds_only_barrier();
-
     const int frag_row = lane & 31;
     constexpr int FK = BK / 2;  // k values per half-wave and tile
     const int frag_k = (lane >> 5) * FK;
 
-    // one k-iteration on LDS buffer `cur`; `held` carries tile it+1, `recv` receives tile it+2
-    auto iterate = [&](int it, int cur, TileStage<VA, AK, TILE> &held_a, TileStage<VB, BK_, TILE> &held_b,
-                       TileStage<VA, AK, TILE> &recv_a, TileStage<VB, BK_, TILE> &recv_b) __attribute__((always_inline)) {
-        // always issued (the last iterations refetch the final tile) so that the count of loads in flight is
-        // the same on every path
-        fetch(min(it + 2, it_end - 1), recv_a, recv_b);
-        __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMA block: the scheduler would sink them
+    // `fetch_next(a, b)` loads the next tile of the walk into a pair of register sets; after the last tile it loads
+    // that one again, so that the count of loads in flight is the same on every path.
+    auto run = [&](auto &a0, auto &b0, auto &a1, auto &b1, auto &fetch_next) __attribute__((always_inline)) {
+        fetch_next(a0, b0);
+        fetch_next(a1, b1);
+        a0.store(lds_a[0], tid);
+        b0.store(lds_b[0], tid);
+        lds_only_barrier();
+        // one k-iteration on LDS buffer `cur`; `held` carries tile it+1, `recv` receives tile it+2
+        auto iterate = [&](int it, int cur, auto &held_a, auto &held_b, auto &recv_a, auto &recv_b) __attribute__((always_inline)) {
+            fetch_next(recv_a, recv_b);
+            __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMA block: the scheduler would sink them
 
-        float fa[NB][FK], fb[NB][FK];
-#pragma unroll
-        for (int i = 0; i < NB; ++i) {
-            TileStage<VA, AK, TILE>::fragment(lds_a[cur], wm * WT + i * 32 + frag_row, frag_k, fa[i]);
-            TileStage<VB, BK_, TILE>::fragment(lds_b[cur], wn * WT + i * 32 + frag_row, frag_k, fb[i]);
-        }
-#pragma unroll
-        for (int kk = 0; kk < FK; ++kk) {
+            float fa[NB][FK], fb[NB][FK];
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
+                TileStage<VA, AK, TILE>::fragment(lds_a[cur], wm * WT + i * 32 + frag_row, frag_k, fa[i]);
+                TileStage<VB, BK_, TILE>::fragment(lds_b[cur], wn * WT + i * 32 + frag_row, frag_k, fb[i]);
+            }
+#pragma unroll
+            for (int kk = 0; kk < FK; ++kk) {
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+#pragma unroll
+                    for (int j = 0; j < NB; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][kk], fa[i][kk], acc[i][j], 0, 0, 0);
+                }
+            }
+            if (rowsum) {
 #pragma unroll
                 for (int j = 0; j < NB; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][kk], fa[i][kk], acc[i][j], 0, 0, 0);
+#pragma unroll
+                    for (int kk = 0; kk < FK; ++kk) rs[j] += fb[j][kk];
             }
-        }
-        if (rowsum) {
-#pragma unroll
-            for (int j = 0; j < NB; ++j)
-#pragma unroll
-                for (int kk = 0; kk < FK; ++kk) rs[j] += fb[j][kk];
-        }
 
-        if (it + 1 < it_end) {
-            held_a.store(lds_a[cur ^ 1], tid);
-            held_b.store(lds_b[cur ^ 1], tid);
+            if (it + 1 < it_end) {
+                held_a.store(lds_a[cur ^ 1], tid);
+                held_b.store(lds_b[cur ^ 1], tid);
+            }
+            lds_only_barrier();
+        };
+        for (int it = it_begin; it < it_end; it += 2) {
+            iterate(it, 0, a1, b1, a0, b0);
+            if (it + 1 < it_end) iterate(it + 1, 1, a0, b0, a1, b1);
         }
-        lds_only_barrier();
     };
-    for (int it = it_begin; it < it_end; it += 2) {
-        iterate(it, 0, sa1, sb1, sa0, sb0);
-        if (it + 1 < it_end) iterate(it + 1, 1, sa0, sb0, sa1, sb1);
+    if constexpr (MASKED) {
+        TileStage<VA, AK, TILE> sa0, sa1;
+        TileStage<VB, BK_, TILE> sb0, sb1;
+        int next_it = it_begin;
+        auto fetch_next = [&](TileStage<VA, AK, TILE> &ra, TileStage<VB, BK_, TILE> &rb) __attribute__((always_inline)) {
+            const int it = min(next_it, it_end - 1);
+            ++next_it;
+            const int seg = it / kt_per_seg;
+            const int k0 = (it % kt_per_seg) * BK;
+            ra.load(pb.A[seg], args.lda, m0, k0, args.m, args.k, tid);
+            rb.load(pb.B[seg], args.ldb, n0, k0, args.n, args.k, tid, mask_pat, pb.b_shift[seg], args.n_slots,
+                    args.b_time_on_k != 0);
+        };
+        run(sa0, sb0, sa1, sb1, fetch_next);
+    } else {
+        // the tile cursor: operand pair `seg`, k tile `kin` inside it; the operands' base pointers are looked up only
+        // when the pair changes
+        FastStage<VA, AK, TILE> qa0, qa1;
+        FastStage<VB, BK_, TILE> qb0, qb1;
+        qa0.init(args.lda, m0, args.m, tid); qa1.init(args.lda, m0, args.m, tid);
+        qb0.init(args.ldb, n0, args.n, tid); qb1.init(args.ldb, n0, args.n, tid);
+        int seg = it_begin / kt_per_seg, kin = it_begin % kt_per_seg, left = it_end - it_begin - 1;
+        const float *pa = pb.A[seg], *pbb = pb.B[seg];
+        const size_t ka = AK ? 1 : (size_t)args.lda, kb = BK_ ? 1 : (size_t)args.ldb;  // floats per k step
+        auto fetch_next = [&](FastStage<VA, AK, TILE> &qa, FastStage<VB, BK_, TILE> &qb) __attribute__((always_inline)) {
+            const int kv = min(BK, args.k - kin * BK);
+            qa.load(pa + (size_t)kin * BK * ka, kv);
+            qb.load(pbb + (size_t)kin * BK * kb, kv);
+            if (left > 0) {
+                --left;
+                if (++kin == kt_per_seg) {
+                    kin = 0; ++seg;
+                    pa = pb.A[seg]; pbb = pb.B[seg];
+                }
+            }
+        };
+        run(qa0, qb0, qa1, qb1, fetch_next);
     }
 
     // epilogue: lane%32 runs along m (contiguous), the 16 accumulators along n
