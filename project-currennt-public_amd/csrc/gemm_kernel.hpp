@@ -317,6 +317,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     // The loop is unrolled by two so that the sets swap roles without register copies, and its barrier orders
     // LDS only (__syncthreads() would also drain the loads in flight).
     const char *mask_pat = MASKED ? args.pat : nullptr;
+    constexpr bool kStoreEarly = true;
 
     // sum of the B operand over this split's k range, per row (dense bias gradient); kept by the waves with wm == 0
     const bool rowsum = args.rowsum != 0;
@@ -340,6 +341,13 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
         auto iterate = [&](int it, int cur, auto &held_a, auto &held_b, auto &recv_a, auto &recv_b) __attribute__((always_inline)) {
             fetch_next(recv_a, recv_b);
             __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMA block: the scheduler would sink them
+            if (kStoreEarly && it + 1 < it_end) {
+                // the tile that arrived during the last iteration goes to the other LDS buffer (free since the barrier)
+                // while this iteration's fragments are on their way, not behind the last MFMA
+                held_a.store(lds_a[cur ^ 1], tid);
+                held_b.store(lds_b[cur ^ 1], tid);
+                __builtin_amdgcn_sched_barrier(0);
+            }
 
             float fa[NB][FK], fb[NB][FK];
 #pragma unroll
@@ -363,7 +371,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
                     for (int kk = 0; kk < FK; ++kk) rs[j] += fb[j][kk];
             }
 
-            if (it + 1 < it_end) {
+            if (!kStoreEarly && it + 1 < it_end) {
                 held_a.store(lds_a[cur ^ 1], tid);
                 held_b.store(lds_b[cur ^ 1], tid);
             }
