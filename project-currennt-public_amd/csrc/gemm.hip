@@ -204,10 +204,13 @@ void gemm_plan(GemmArgs &args, hipStream_t stream) {
     // Outputs of one or two tiles per problem (the WaveNet layers' 64 x 64 ... 80 x 128 weights) take twice the
     // workgroups: measured on MI355X next to the error chain of the same pass, 1024 workgroups end the stack's backward
     // pass 4% sooner than 512, and 1536 or more (where the partial products no longer fit the scratch buffer and the
-    // launch adds atomically) 4-8% later; the acoustic model's wide outputs are best at 512.
+    // launch adds atomically) 4-8% later; the acoustic model's wide outputs are best at 768 (2.249 / 2.232 / 2.219 / 2.246 /
+    // 2.243 ms at 512 / 640 / 768 / 896 / 1024 with the loader of constant offsets; they were best at 512 before it).
     static const int forced_target = [] { const char *e = std::getenv("CNT_GEMM_SPLIT_TARGET"); return e ? std::atoi(e) : 0; }();
-    const int target = forced_target > 0 ? forced_target : ((long)args.m * args.n <= 16384 ? 1024 : 512);
     const long tiles = (long)((args.m + 63) / 64) * ((args.n + 63) / 64) * args.nprob;
+    // (768 only where a launch has at least 64 tiles to begin with: the WaveNet stack's 256 x 256 output layers over
+    // 32 000 samples, 16 tiles, are better off with 512: 2.724 against 2.736 ms)
+    const int target = forced_target > 0 ? forced_target : ((long)args.m * args.n <= 16384 ? 1024 : tiles >= 64 ? 768 : 512);
     const long kt = ((long)args.k + BK - 1) / BK * args.nseg;
     long s = (target + tiles - 1) / tiles;
     s = std::min(s, std::max(1L, kt / 8));
