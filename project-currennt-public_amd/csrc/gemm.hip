@@ -260,6 +260,13 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
         for (int s = 0; s < args.nseg; ++s)
             CNT_REQUIRE(args.prob[p].A[s] && args.prob[p].B[s], "gemm: null operand");
     }
+    // the unmasked loaders address an operand through 32-bit byte offsets beside a base that moves along k
+    const auto reachable = [](long rows, long ld, int kcontig) {
+        return (kcontig ? rows * ld : BK * ld + rows) * (long)sizeof(float) < (1L << 32);
+    };
+    CNT_REQUIRE(args.masked || (reachable(args.m, args.lda, args.a_kcontig) && reachable(args.n, args.ldb, args.b_kcontig)),
+                "gemm: operands of 4 GiB and more are not supported (%d x %d x %d, lda %d, ldb %d)", args.m, args.n, args.k,
+                args.lda, args.ldb);
     const int va = pick_vec(args, true), vb = pick_vec(args, false);
     gemm_plan(args, stream);
     if (args.epilogue != EPI_PARTIAL) args.rowsum = 0;
