@@ -152,7 +152,18 @@ struct GemmProblem {
     float *aux_out;       // EPI_CONTEXT, may be NULL
     float *rowsum_out;    // GemmArgs::rowsum: receives rowsum_scale * sum_k B(j, k), j < n
     float rowsum_scale;
+    int k_trim;           // GemmArgs::k_order: 0 all listed k lines, 1 without those of the first time step, 2 without the last one's
+    int k_shift;          // GemmArgs::k_order: added to every listed line (an operand pair that starts at a later slot)
 };
+
+// The slots of a fraction in the order "valid ones first, ascending; then the padding slots, ascending" (device
+// memory: n_slots indices and three counts), made from the pattern types by slot_order_build.  The errors
+// and deltas of every layer are zero on padding slots, so a sum over the slots may skip them.
+struct SlotOrder {
+    const int *order;
+    const int *count;  // [0] valid slots, [1] those of the first time step, [2] those of the last time step
+};
+int slot_order_build(hipStream_t stream, const char *pat, int n_slots, int slots_per_step, int *order, int *count);
 
 // Masked mode (dilated convolutions without a materialised column buffer): one index of the B operand is a
 // time slot u -- its row index (b_time_on_k = 0) or its k index (b_time_on_k = 1).  The element is read from
@@ -183,6 +194,14 @@ struct GemmArgs {
     float *partial;        // scratch of splitk * partial_stride floats: the stream's buffer (set by gemm_plan) or the caller's
     size_t partial_stride;  // floats per split: nprob * m * n (+ nprob * n with rowsum)
     int xcd_map;            // set by gemm_launch: workgroups pick their tile by XCD (gemm_kernel.hpp)
+    // A product over the slots of a fraction (weight gradients) that leaves the padding slots out (both in device memory,
+    // or both NULL): only the k lines k_order[lo .. lo + n) of the operands are read, the others being all zero in at least
+    // one operand.  k_count[0] = number of listed lines; with GemmProblem::k_trim = 1 the problem leaves out the first
+    // k_count[1] of them (the lines of the first time step), with 2 the last k_count[2] (those of the last time step).  The
+    // launcher uses the list where both operands are row-contiguous and 16-byte aligned and the tile is 64 x 64, and
+    // multiplies all k lines otherwise -- so the operands' base pointers must be valid for both readings.
+    const int *k_order;
+    const int *k_count;
 };
 
 // Resolves splitk = 0 (chosen by the launcher) and, where the arguments allow it and it pays, switches an
@@ -250,6 +269,9 @@ int dense_backward_errors_fan(hipStream_t stream, int P, int D, int N, int act, 
 // that layer's own backward step then runs with ACT_IDENTITY.  The same for a recurrent layer's error product:
 int lstm_prev_errors_delta(cnt_lstm *h, hipStream_t stream, const float *weights, float *prev_errors, int prev_act,
                            const float *prev_y);
+// The slots of the fraction a recurrent layer has loaded, valid ones first (nullptr: none known); the layer's weight
+// gradients then skip the padding slots.  cnt_lstm_load_sequences forgets it.
+void lstm_set_slot_order(cnt_lstm *h, const SlotOrder *order);
 // Error path of one WaveNet residual block in one launch (skip 1x1 layer, the skip layer in front of it, the 1x1
 // layer behind the gated unit, the gated unit): see wavenet_block_errors_kernel.
 bool wavenet_block_errors_supported(int R, int K);
@@ -273,7 +295,7 @@ int cnn_backward_errors_fan(cnt_cnn *h, hipStream_t stream, const char *patTypes
 // same D, C, N and one context buffer, as the problems of one product.  Same results as `count` calls of
 // cnt_dense_backward_weights / cnt_wavnetc_backward_weights.
 int dense_backward_weights_batch(hipStream_t stream, int P, int D, int N, int count, const float *bias,
-                                 const float *const *x, const float *const *err, float *const *weight_updates);
+                                 const float *const *x, const float *const *err, float *const *weight_updates, const SlotOrder *order = nullptr);
 int wavnetc_backward_weights_batch(hipStream_t stream, int D, int C, int N, int count, const float *ctx,
                                    const float *const *ctx_tanh, float *const *weight_updates);
 // Convolution layers with one filter group each and the same sizes, window and causality (dilations may differ):

@@ -108,7 +108,63 @@ inline int stream_blocks(size_t count) {
     return (int)b;
 }
 
+// One workgroup: every thread counts the valid slots of its contiguous share, the counts are scanned (inside a wave by
+// shuffles, the waves' totals through LDS), and the thread then writes its valid slots from its offset among the valid
+// ones and its padding slots from its offset among the padding ones, behind all valid ones.
+constexpr int kOrderThreads = 256;
+__global__ __launch_bounds__(kOrderThreads) void slot_order_kernel(const char *__restrict__ pat, int n, int per_step,
+                                                                   int *__restrict__ order, int *__restrict__ count) {
+    __shared__ int wave_total[kOrderThreads / 64];
+    __shared__ int edge_count[2];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int share = (n + kOrderThreads - 1) / kOrderThreads;
+    const int lo = min(tid * share, n), hi = min(lo + share, n);
+    if (tid < 2) edge_count[tid] = 0;
+    __syncthreads();
+    int valid = 0, in_first = 0, in_last = 0;
+    for (int i = lo; i < hi; ++i) {
+        const int v = pat[i] != 0;
+        valid += v;
+        in_first += v && i < per_step;
+        in_last += v && i >= n - per_step;
+    }
+    if (in_first) atomicAdd(&edge_count[0], in_first);
+    if (in_last) atomicAdd(&edge_count[1], in_last);
+    int incl = valid;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int v = __shfl_up(incl, d);
+        if (lane >= d) incl += v;
+    }
+    if (lane == 63) wave_total[wave] = incl;
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kOrderThreads / 64; ++w) {
+        if (w < wave) before += wave_total[w];
+        total += wave_total[w];
+    }
+    int at_valid = before + incl - valid;      // valid slots before this thread's share
+    int at_pad = total + (lo - at_valid);      // padding slots before it, behind all valid ones
+    for (int i = lo; i < hi; ++i) {
+        if (pat[i] != 0) order[at_valid++] = i;
+        else order[at_pad++] = i;
+    }
+    if (tid == 0) {
+        count[0] = total;
+        count[1] = edge_count[0];
+        count[2] = edge_count[1];
+    }
+}
+
 }  // namespace
+
+int slot_order_build(hipStream_t stream, const char *pat, int n_slots, int slots_per_step, int *order, int *count) {
+    CNT_REQUIRE(pat && order && count && n_slots > 0 && slots_per_step > 0, "slot_order_build: bad argument");
+    hipLaunchKernelGGL(slot_order_kernel, dim3(1), dim3(kOrderThreads), 0, stream, pat, n_slots, slots_per_step, order, count);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
 
 int fill_zero(hipStream_t stream, float *p, size_t count) {
     if (count == 0) return CNT_OK;
@@ -220,7 +276,7 @@ int cnt_dense_backward_weights(void *stream, int P, int D, int N, float bias, co
 
 extern "C++" int cnt::dense_backward_weights_batch(hipStream_t stream, int P, int D, int N, int count, const float *bias,
                                                    const float *const *x, const float *const *err,
-                                                   float *const *weight_updates) {
+                                                   float *const *weight_updates, const SlotOrder *order) {
     CNT_REQUIRE(count >= 1 && count <= kGemmMaxProb, "dense_backward_weights: %d layers in one launch, supported 1..%d",
                 count, kGemmMaxProb);
     CNT_REQUIRE(bias && x && err && weight_updates, "dense_backward_weights: null argument");
@@ -237,6 +293,11 @@ extern "C++" int cnt::dense_backward_weights_batch(hipStream_t stream, int P, in
         ga.prob[z].A[0] = x[z]; ga.prob[z].B[0] = err[z]; ga.prob[z].C = weight_updates[z];
         ga.prob[z].rowsum_out = weight_updates[z] + (size_t)P * D;
         ga.prob[z].rowsum_scale = bias[z];
+    }
+    if (order && order->order) {
+        // the deltas are zero on padding slots: the sum over the slots leaves them out
+        ga.k_order = order->order;
+        ga.k_count = order->count;
     }
     ga.label = "gemm:dense_dW";
     // narrow layers: the launcher sums partial products instead of adding atomically, which overwrites the

@@ -271,6 +271,13 @@ int gemm_launch(hipStream_t stream, const GemmArgs &args_in) {
     gemm_plan(args, stream);
     if (args.epilogue != EPI_PARTIAL) args.rowsum = 0;
     const int tile = pick_tile(args);
+    static const bool use_lines = [] { const char *e = std::getenv("CNT_GEMM_K_ORDER"); return !e || std::atoi(e) != 0; }();
+    if (!use_lines) args.k_order = nullptr;
+    // a list of k lines is used where the kernel that reads through it exists, and ignored otherwise (the lines it leaves
+    // out are zero)
+    if (args.k_order && !(args.k_count && !args.masked && !args.a_kcontig && !args.b_kcontig && va == 4 && vb == 4 && tile == 64 &&
+                          args.epilogue != EPI_FAN && args.k < (1 << 24) && args.lda < (1 << 22) && args.ldb < (1 << 22)))
+        args.k_order = nullptr;
     const int tiles = ((args.m + tile - 1) / tile) * ((args.n + tile - 1) / tile);
     dim3 grid(tiles, args.splitk, args.nprob);
     // XCD-aware placement (gemm_kernel.hpp) for launches of several problems: measured with FETCH_SIZE on MI355X it

@@ -252,12 +252,55 @@ struct FastStage {
     }
 };
 
+// The unmasked loader for row-contiguous operands whose k lines are picked through a list (16-byte vectors only): tile k
+// line j is line idx[j] of the operand.  The indices of a tile are loaded one iteration ahead by the kernel (both operands
+// share them) and handed to load(); everything else is FastStage.
+template <int ROWS>
+struct GatherStage {
+    static constexpr int NLOAD = (ROWS * BK) / (NTHREADS * 4);
+    static constexpr int TPK = ROWS / 4, KPP = NTHREADS / TPK;
+    float4 r[NLOAD];
+    unsigned roff;   // byte offset of the thread's four rows inside a k line (clamped into the matrix)
+    int kk;          // the thread's first k line inside a tile; its others follow at a distance of KPP
+    bool row_ok;
+    bool edge;       // uniform: some row of this tile lies outside the matrix
+    int k_valid;     // uniform: k lines of the tile in registers that are listed
+
+    __device__ __forceinline__ void init(int row0, int rows_total, int tid) {
+        edge = row0 + ROWS > rows_total;
+        const int rq = (tid % TPK) * 4;
+        kk = tid / TPK;
+        row_ok = (row0 + rq) < rows_total;
+        roff = (unsigned)((row_ok ? row0 + rq : 0) * sizeof(float));
+    }
+    // line_bytes and the indices are below 2^24 and the operand below 4 GiB (checked by the launcher): a 24-bit multiply-add
+    // gives the 32-bit offset beside the uniform base
+    __device__ __forceinline__ void load(const float *__restrict__ operand, unsigned line_bytes, const int (&idx)[NLOAD], int kv) {
+        k_valid = kv;
+        const char *b = reinterpret_cast<const char *>(operand);
+#pragma unroll
+        for (int p = 0; p < NLOAD; ++p)
+            r[p] = *reinterpret_cast<const float4 *>(b + (__umul24((unsigned)idx[p], line_bytes) + roff));
+    }
+    __device__ __forceinline__ void store(float *__restrict__ lds, int tid) const {
+        const bool special = edge || k_valid < BK;
+        const int rq = (tid % TPK) * 4;
+#pragma unroll
+        for (int p = 0; p < NLOAD; ++p) {
+            float4 v = r[p];
+            if (special && !(row_ok && kk + p * KPP < k_valid)) v = float4{0.0f, 0.0f, 0.0f, 0.0f};
+            *reinterpret_cast<float4 *>(lds + (kk + p * KPP) * ROWS + rq) = v;
+        }
+    }
+};
+
 // MASKED selects the time-shifted, padding-masked B loader at compile time: its per-element predication is a lot
 // of code, and four copies of it (two prologue fetches, two in the unrolled loop) inside the plain kernels would
 // push their hot loop out of the instruction cache.
 // FAN: the EPI_FAN epilogue, a kernel of its own (instantiated for 16-byte row-contiguous A and k-contiguous B only,
 // the shapes of the error products that use it) so that its registers and code stay out of every other product.
-template <int VA, bool AK, int VB, bool BK_, bool MASKED, int TILE, bool FAN = false>
+// GATHER: the k lines of both (row-contiguous, 16-byte aligned) operands are those a list names (GemmArgs::k_order).
+template <int VA, bool AK, int VB, bool BK_, bool MASKED, int TILE, bool FAN = false, bool GATHER = false>
 __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args) {
     constexpr int BM = TILE, BN = TILE;
     constexpr int WT = TILE / 2;   // edge of a wave's block (waves are arranged 2 x 2)
@@ -296,12 +339,21 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
     const GemmProblem &pb = args.prob[prob_id];
 
     // iteration space: segments x k-tiles, cut into splitk contiguous ranges
-    const int kt_per_seg = (args.k + BK - 1) / BK;
+    // the listed k lines this problem takes: all of them, or all but the first / last time step's
+    int k_extent = args.k, k_lo = 0;
+    if (GATHER) {
+        k_extent = args.k_count[0];
+        if (pb.k_trim == 1) { k_lo = args.k_count[1]; k_extent -= k_lo; }
+        else if (pb.k_trim == 2) k_extent -= args.k_count[2];
+        k_extent = max(k_extent, 0);
+    }
+    const int kt_per_seg = (k_extent + BK - 1) / BK;
     const int total_it = kt_per_seg * args.nseg;
     const int per_split = (total_it + args.splitk - 1) / args.splitk;
     const int it_begin = split_id * per_split;
     const int it_end = min(total_it, it_begin + per_split);
-    if (it_begin >= it_end) return;
+    // (a split left without k lines by a short list still has its partial product to write)
+    if (it_begin >= it_end && !(GATHER && args.epilogue == EPI_PARTIAL)) return;
 
     f32x16 acc[NB][NB];
 #pragma unroll
@@ -382,7 +434,39 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(const GemmArgs args)
             if (it + 1 < it_end) iterate(it + 1, 1, a0, b0, a1, b1);
         }
     };
-    if constexpr (MASKED) {
+    if constexpr (GATHER) {
+        static_assert(VA == 4 && VB == 4 && !AK && !BK_ && !MASKED, "the gathering loader is for two row-contiguous operands");
+        GatherStage<TILE> ga0, ga1, gb0, gb1;
+        ga0.init(m0, args.m, tid); ga1.init(m0, args.m, tid);
+        gb0.init(n0, args.n, tid); gb1.init(n0, args.n, tid);
+        constexpr int NL = GatherStage<TILE>::NLOAD, KPP = GatherStage<TILE>::KPP;
+        const int *__restrict__ order = args.k_order + k_lo;
+        const int k_shift = pb.k_shift;
+        const unsigned a_line = (unsigned)(args.lda * sizeof(float)), b_line = (unsigned)(args.ldb * sizeof(float));
+        int seg = it_begin / kt_per_seg, kin = it_begin % kt_per_seg, left = it_end - it_begin - 1;
+        const float *pa = pb.A[seg], *pbb = pb.B[seg];
+        // the k lines of the cursor's tile, loaded while the tile before it is being requested
+        int idx[NL];
+        auto lines_of = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+            for (int p = 0; p < NL; ++p) idx[p] = order[max(min(tile * BK + ga0.kk + p * KPP, k_extent - 1), 0)] + k_shift;
+        };
+        lines_of(kin);
+        auto fetch_next = [&](GatherStage<TILE> &qa, GatherStage<TILE> &qb) __attribute__((always_inline)) {
+            const int kv = min(BK, k_extent - kin * BK);
+            qa.load(pa, a_line, idx, kv);
+            qb.load(pbb, b_line, idx, kv);
+            if (left > 0) {
+                --left;
+                if (++kin == kt_per_seg) {
+                    kin = 0; ++seg;
+                    pa = pb.A[seg]; pbb = pb.B[seg];
+                }
+            }
+            lines_of(kin);
+        };
+        if (it_begin < it_end) run(ga0, gb0, ga1, gb1, fetch_next);
+    } else if constexpr (MASKED) {
         TileStage<VA, AK, TILE> sa0, sa1;
         TileStage<VB, BK_, TILE> sb0, sb1;
         int next_it = it_begin;
@@ -542,6 +626,12 @@ void launch_m(const GemmArgs &a, dim3 grid, hipStream_t s) {
             else
                 hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, false, TILE, true>), grid, dim3(NTHREADS), 0, s, a);
         }
+        return;
+    }
+    if (a.k_order) {
+        // gemm_launch has checked that the operands are of the one kind this exists for
+        if constexpr (VA == 4 && !AK && VB == 4 && !BK_ && TILE == 64)
+            hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, false, TILE, false, true>), grid, dim3(NTHREADS), 0, s, a);
         return;
     }
     if (a.masked) hipLaunchKernelGGL((gemm_f32_kernel<VA, AK, VB, BK_, true, TILE>), grid, dim3(NTHREADS), 0, s, a);

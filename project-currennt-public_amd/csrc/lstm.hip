@@ -1064,6 +1064,7 @@ struct cnt_lstm {
     int last_was_forward;  // which recursion the diagnostic buffer describes
     int bmail_dirty;       // the backward mailbox may hold words that are not empty
     int flmail_dirty;      // the same for the XCD-local forward recursion's mailbox
+    cnt::SlotOrder slot_order;  // the loaded fraction's slots, valid ones first (set by the owner of the pattern types, or null)
     int stepwise;          // no persistent recursion kernel for this geometry: one product + one cell kernel per step
     int *latch_host, *latch_dev;  // pinned host word a kernel that gives up sets; read by the host without a sync
     int *veto;             // a network's shared flag (device), or NULL
@@ -1614,6 +1615,7 @@ int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int
                 h->desc.maxT);
     CNT_REQUIRE(curMinT >= 0 && curMinT <= curMaxT, "lstm_load_sequences: curMinT %d outside 0..%d", curMinT, curMaxT);
     h->T = curMaxT; h->Tmin = curMinT; h->pat = patTypes;
+    h->slot_order = SlotOrder{nullptr, nullptr};
     if (h->next_step != 0) { h->bmail_dirty = 1; h->next_step = 0; }  // an abandoned partial backward pass
     const size_t nstate = (size_t)h->H * h->desc.maxT * h->desc.S;
     // stored output-gate deltas of both directions, one launch
@@ -1648,6 +1650,10 @@ extern "C++" void cnt::lstm_set_veto(cnt_lstm *h, int *veto) {
 }
 
 extern "C++" int cnt::lstm_is_persistent(const cnt_lstm *h) { return h && !h->stepwise ? 1 : 0; }
+
+extern "C++" void cnt::lstm_set_slot_order(cnt_lstm *h, const SlotOrder *order) {
+    if (h) h->slot_order = order ? *order : SlotOrder{nullptr, nullptr};
+}
 
 extern "C++" int cnt::lstm_wait_recursion(cnt_lstm *h, hipStream_t other) {
     CNT_REQUIRE(h, "lstm_wait_recursion: null handle");
@@ -1929,6 +1935,11 @@ extern "C++" int cnt::lstm_backward_weights_parts(cnt_lstm *h, hipStream_t strea
                 pb.B[0] = h->state[dir][7 + g];
                 pb.C = weight_updates + (size_t)g * P * L + (size_t)dir * P * H;
             }
+        if (h->slot_order.order) {
+            // the deltas are zero on padding slots: the sum over the slots leaves them out
+            ga.k_order = h->slot_order.order;
+            ga.k_count = h->slot_order.count;
+        }
         ga.label = "gemm:lstm_dW_input";
         CNT_TRY(gemm_launch(stream, ga));
     }
@@ -1951,7 +1962,15 @@ extern "C++" int cnt::lstm_backward_weights_parts(cnt_lstm *h, hipStream_t strea
                 pb.A[0] = dir ? hbuf + (size_t)S * H : hbuf;
                 pb.B[0] = dir ? dl : dl + (size_t)S * H;
                 pb.C = weight_updates + off_int + (size_t)g * L * H + (size_t)dir * H * H;
+                // with the list of valid slots: a forward state's pairs are the valid slots from the second time step on,
+                // counted from there; a backward state's are the valid slots before the last time step
+                pb.k_trim = dir ? 2 : 1;
+                pb.k_shift = dir ? 0 : -S;
             }
+        if (h->slot_order.order) {
+            ga.k_order = h->slot_order.order;
+            ga.k_count = h->slot_order.count;
+        }
         ga.label = "gemm:lstm_dW_internal";
         CNT_TRY(gemm_launch(stream, ga));
     }

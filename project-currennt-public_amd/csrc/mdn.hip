@@ -188,6 +188,30 @@ __global__ void softmax_backward_kernel(UnitGeom g, const char *__restrict__ pat
     }
 }
 
+// the same with 16-byte accesses (M, the row pitches and the unit's first column multiples of four): an item is four
+// classes of one frame, and a thread has several items in flight
+__global__ __launch_bounds__(256) void softmax_backward_vec4_kernel(UnitGeom g, const char *__restrict__ pat,
+                                                                    const float *__restrict__ target,
+                                                                    const float *__restrict__ prob, float *__restrict__ errors) {
+    const int per_frame = g.M / 4;
+    const size_t items = (size_t)g.F * per_frame;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < items; i += stride) {
+        const size_t f = i / per_frame;
+        const int k = (int)(i % per_frame) * 4;
+        float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (pat[f] != 0) {
+            const float t = target[f * g.Lt + g.startDOut];
+            v = *reinterpret_cast<const float4 *>(prob + f * g.M + k);
+            float *e = reinterpret_cast<float *>(&v);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if ((double)((t - (k + q)) * (t - (k + q))) < 0.0001) e[q] += -1.0f;
+        }
+        *reinterpret_cast<float4 *>(errors + f * g.Lp + g.startD + k) = v;
+    }
+}
+
 // ---- mixture unit -----------------------------------------------------------------------------------
 // para = [F*M weights | F*M*D means | F*M*D std], offsets by the CURRENT frame count F.
 __global__ void mixture_forward_kernel(UnitGeom g, const char *__restrict__ pat, const float *__restrict__ x,
@@ -816,8 +840,16 @@ int cnt_mdn_backward(cnt_mdn *h, void *stream_, const float *targets, float *pre
                                stream, g, h->desc.sigmoid_continuous, h->pat, targets, u.para, prev_errors);
         } else if (u.type == -1) {
             ProfileScope prof(stream, "mdn_softmax_backward");
-            hipLaunchKernelGGL(softmax_backward_kernel, grid, block, 0, stream, g, h->pat, targets, u.para,
-                               prev_errors);
+            const bool vec4 = g.M % 4 == 0 && g.Lp % 4 == 0 && g.startD % 4 == 0 &&
+                              (reinterpret_cast<uintptr_t>(u.para) & 15) == 0 && (reinterpret_cast<uintptr_t>(prev_errors) & 15) == 0;
+            if (vec4) {
+                const size_t items = (size_t)g.F * (g.M / 4);
+                hipLaunchKernelGGL(softmax_backward_vec4_kernel, dim3((unsigned)std::min<size_t>((items + 255) / 256, 2048)),
+                                   dim3(256), 0, stream, g, h->pat, targets, u.para, prev_errors);
+            } else {
+                hipLaunchKernelGGL(softmax_backward_kernel, grid, block, 0, stream, g, h->pat, targets, u.para,
+                                   prev_errors);
+            }
         } else {
             ProfileScope prof(stream, "mdn_mixture_backward");
             auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };

@@ -210,6 +210,7 @@ struct NetLayer {
     int res = 1, maxTr = 0;
     int T = 0, Tmin = 0, N = 0;              // of the current fraction, at this layer's resolution
     const char *pat = nullptr;               // pattern types at this layer's resolution
+    SlotOrder order = {nullptr, nullptr};    // the fraction's slots at this layer's resolution, valid ones first (or none)
     std::string flag;                        // "layerFlag"
     std::vector<int> cat_lo, cat_hi;         // skipcat: dimension range taken from each source
     const float *ext_data = nullptr;         // externalloader: [frame][sequence][dimension], set by the caller
@@ -465,7 +466,9 @@ struct cnt_network {
     int flagged = -1, first_wavnetc = -1;
     float *ctx_own = nullptr, *ctx_grad = nullptr;
     float *ctx_mv = nullptr;  // the first wavnetc layer's "contextMV": [means | standard deviations] (device), or NULL
-    struct LowRes { int res; char *pat; };
+    struct LowRes { int res; char *pat; int *order; int *order_count; bool order_built; };
+    int *order = nullptr, *order_count = nullptr;  // the fraction's slots at resolution 1, valid ones first (slot_order_build)
+    bool skip_padding = true;
     std::vector<LowRes> low_res;
     std::vector<void *> allocations;
     // weight gradients go round-robin to these streams (default priority); CNT_NET_SIDE_STREAMS overrides the count
@@ -1000,14 +1003,24 @@ int finish_build(cnt_network *net, const json::Value *weights) {
         const size_t rows = ((size_t)net->S * C.maxTr + 63) / 64;
         CNT_TRY(device_alloc(net, (void **)&C.colsum, rows * C.size * sizeof(float), false));
     }
+    // the slots of a fraction with the valid ones first: the weight gradients of the dense and recurrent layers sum over
+    // those only (CNT_NET_SKIP_PADDING=0: over all slots)
+    {
+        const char *e = std::getenv("CNT_NET_SKIP_PADDING");
+        net->skip_padding = !e || std::atoi(e) != 0;
+        CNT_TRY(device_alloc(net, (void **)&net->order, ((size_t)net->S * net->maxT + 4) * sizeof(int), true));
+        net->order_count = net->order + (size_t)net->S * net->maxT;
+    }
     // pattern types of the lower time resolutions, one buffer per resolution
     for (auto &L : net->layers) {
         if (L.res == 1) continue;
         bool have = false;
         for (auto &lr : net->low_res) have = have || lr.res == L.res;
         if (have) continue;
-        cnt_network::LowRes lr = {L.res, nullptr};
+        cnt_network::LowRes lr = {L.res, nullptr, nullptr, nullptr, false};
         CNT_TRY(device_alloc(net, (void **)&lr.pat, (size_t)net->S * L.maxTr, true));
+        CNT_TRY(device_alloc(net, (void **)&lr.order, ((size_t)net->S * L.maxTr + 4) * sizeof(int), true));
+        lr.order_count = lr.order + (size_t)net->S * L.maxTr;
         net->low_res.push_back(lr);
     }
     // conditioning sub-network (NeuralNetwork.cpp:544-561, layers/wavNetCore.cu:455-492, :895-913): the wavnetc
@@ -1222,14 +1235,38 @@ int cnt_network_load_sequences(cnt_network *net, void *stream_, int T, int Tmin,
                            patTypes, lr.pat);
         CNT_HIP(hipGetLastError());
     }
+    // which time bases have a layer whose weight gradient can use the slot order; a fraction whose sequences all have the
+    // full length has no padding slots
+    bool wanted_main = false;
+    for (size_t i = 1; i < net->layers.size(); ++i) {
+        const NetLayer &L = net->layers[i];
+        if (net->skip_padding && Tmin < T && (L.kind == K_DENSE || L.kind == K_LSTM) && L.res == 1) wanted_main = true;
+    }
+    if (wanted_main) CNT_TRY(slot_order_build(stream, patTypes, (int)slots, net->S, net->order, net->order_count));
+    for (auto &lr : net->low_res) {
+        bool wanted = false;
+        for (size_t i = 1; i < net->layers.size(); ++i) {
+            const NetLayer &L = net->layers[i];
+            if (net->skip_padding && Tmin < T && (L.kind == K_DENSE || L.kind == K_LSTM) && L.res == lr.res) wanted = true;
+        }
+        lr.order_built = wanted;
+        if (wanted) CNT_TRY(slot_order_build(stream, lr.pat, ((T + lr.res - 1) / lr.res) * net->S, net->S, lr.order, lr.order_count));
+    }
     for (auto &L : net->layers) {
         L.T = (T + L.res - 1) / L.res;
         L.Tmin = (Tmin + L.res - 1) / L.res;
         L.N = L.T * net->S;
         L.pat = patTypes;
+        L.order = wanted_main && L.res == 1 ? SlotOrder{net->order, net->order_count} : SlotOrder{nullptr, nullptr};
         for (auto &lr : net->low_res)
-            if (lr.res == L.res) L.pat = lr.pat;
-        if (L.lstm) CNT_TRY(cnt_lstm_load_sequences(L.lstm, stream, L.pat, L.T, L.Tmin));
+            if (lr.res == L.res) {
+                L.pat = lr.pat;
+                L.order = lr.order_built ? SlotOrder{lr.order, lr.order_count} : SlotOrder{nullptr, nullptr};
+            }
+        if (L.lstm) {
+            CNT_TRY(cnt_lstm_load_sequences(L.lstm, stream, L.pat, L.T, L.Tmin));
+            lstm_set_slot_order(L.lstm, &L.order);
+        }
         if (L.mdn) CNT_TRY(cnt_mdn_load_sequences(L.mdn, stream, L.pat, L.T));
     }
     return CNT_OK;
@@ -1425,8 +1462,10 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
         NetLayer &L = net->layers[i];
         NetLayer &prev = net->layers[i - 1];
         float *dW = net->updates + L.w_off;
-        if (L.kind == K_DENSE)
-            return cnt_dense_backward_weights(ws, prev.size, L.size, L.N, L.bias, prev.out, L.err, dW);
+        if (L.kind == K_DENSE) {
+            const float *x = prev.out, *e = L.err;
+            return dense_backward_weights_batch(ws, prev.size, L.size, L.N, 1, &L.bias, &x, &e, &dW, &L.order);
+        }
         if (L.kind == K_LSTM) return cnt_lstm_backward_weights(L.lstm, ws, prev.out, dW);
         if (L.kind == K_CNN) return cnt_cnn_backward_weights(L.cnn, ws, L.pat, L.T, prev.out, L.err, dW);
         return cnt_wavnetc_backward_weights(ws, L.size, L.ctx_dim, L.N, net->ctx, L.cth, dW);
@@ -1507,7 +1546,7 @@ int cnt_network_backward(cnt_network *net, void *stream_) {
             colsum[z] = L.colsum; colsum_rows[z] = L.colsum_rows;
         }
         g.layers.clear();
-        if (g.kind == K_DENSE) return dense_backward_weights_batch(ws, g.a, g.b, g.n, count, bias, in0, in1, dW);
+        if (g.kind == K_DENSE) return dense_backward_weights_batch(ws, g.a, g.b, g.n, count, bias, in0, in1, dW, &first.order);
         if (g.kind == K_CNN) return cnn_backward_weights_batch(cnn, count, ws, first.pat, first.T, in0, in1, dW, colsum, colsum_rows);
         return wavnetc_backward_weights_batch(ws, g.a, g.b, g.n, count, net->ctx, in0, dW);
     };

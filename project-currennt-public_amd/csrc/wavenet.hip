@@ -458,29 +458,33 @@ __global__ __launch_bounds__(CONV ? 512 : 256, (CONV || K > 128) ? 1 : 2) void w
 
 // out[d] = scale * sum over rows of partial[row][d] (the second half of a column sum whose first half rode in
 // wavenet_block_errors_kernel); overwrites
-__global__ __launch_bounds__(1024) void colsum_finish_kernel(const float *__restrict__ partial, int rows, int D, float scale,
-                                                             float *__restrict__ out) {
-    // 64 columns per block, sixteen groups of lanes over the rows, eight loads in flight per lane
-    __shared__ float part[16][64];
+constexpr int kColsumGroups = 4;
+__global__ __launch_bounds__(64 * kColsumGroups) void colsum_finish_kernel(const float *__restrict__ partial, int rows, int D,
+                                                                           float scale, float *__restrict__ out) {
+    // 64 columns per block, four groups of lanes over the rows, eight loads in flight per lane.  Four waves and few registers:
+    // a block finds room on a compute unit that a block-error workgroup (which leaves a tenth of the registers) occupies;
+    // with sixteen waves it waited for that launch to end.
+    constexpr int G = kColsumGroups;
+    __shared__ float part[G][64];
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     const int d = blockIdx.x * 64 + tx;
     float acc = 0.0f;
     if (d < D) {
         int r = ty;
-        for (; r + 7 * 16 < rows; r += 8 * 16) {
+        for (; r + 7 * G < rows; r += 8 * G) {
             float x[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) x[u] = partial[(size_t)(r + 16 * u) * D + d];
+            for (int u = 0; u < 8; ++u) x[u] = partial[(size_t)(r + G * u) * D + d];
             acc += ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
         }
-        for (; r < rows; r += 16) acc += partial[(size_t)r * D + d];
+        for (; r < rows; r += G) acc += partial[(size_t)r * D + d];
     }
     part[ty][tx] = acc;
     __syncthreads();
     if (ty == 0 && d < D) {
         float v = 0.0f;
 #pragma unroll
-        for (int q = 0; q < 16; ++q) v += part[q][tx];
+        for (int q = 0; q < G; ++q) v += part[q][tx];
         out[d] = scale * v;
     }
 }
@@ -785,7 +789,7 @@ extern "C++" int cnt::cnn_backward_weights_batch(cnt_cnn *const *h, int count, h
         float *bias_grad = weight_updates[z] + (size_t)P * h[z]->Lw;
         if (colsum_partial && colsum_partial[z] && colsum_rows[z] > 0) {
             // the launch that wrote these deltas summed them per workgroup
-            hipLaunchKernelGGL(colsum_finish_kernel, dim3((D + 63) / 64), dim3(1024), 0, stream, colsum_partial[z],
+            hipLaunchKernelGGL(colsum_finish_kernel, dim3((D + 63) / 64), dim3(64 * kColsumGroups), 0, stream, colsum_partial[z],
                                colsum_rows[z], D, h[z]->desc.bias, bias_grad);
             CNT_HIP(hipGetLastError());
         } else {

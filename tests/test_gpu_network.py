@@ -101,6 +101,57 @@ def test_stacked_network_trains_like_the_oracle(option, momentum, overlap):
     net.close()
 
 
+def test_weight_gradients_of_a_fraction_that_is_mostly_padding():
+    """One long sequence beside seven of a single frame: the weight gradients sum over the valid slots only (a list of them,
+    made when the fraction is loaded), a recurrent layer's recurrent weights over the list without the first or the last
+    time step, and most splits of the narrow layers' split-K products are left without a single slot."""
+    import torch
+
+    print("network case: mostly padding", flush=True)
+    capi, networks = PC.pkg().capi, PC.networks()
+    P, Q, S, T = 16, 8, 8, 600
+    lengths = [T, 1, 1, 1, 1, 1, 1, 1]
+    specs = [{"name": "ff1", "type": "feedforward_tanh", "size": 64, "bias": 1.0},
+             {"name": "bl1", "type": "blstm", "size": 128, "bias": 1.0},
+             {"name": "out", "type": "feedforward_identity", "size": Q, "bias": 1.0},
+             {"name": "postoutput", "type": "sse", "size": Q}]
+    weights = OM.init_weights(P, specs, 9, 0.1)
+    doc = {"layers": [{"size": P, "name": "input", "type": "input"}] + specs, "weights": {}}
+    wi, prev = iter(weights), P
+    for sp in specs:
+        n_in, n_bias, _ = networks.weight_sections(sp, prev)
+        if n_in:
+            _sections(doc["weights"], sp["name"], next(wi), n_in, n_bias)
+        prev = sp["size"]
+    net = capi.Network(json.dumps(doc), S, T)
+    rng = np.random.default_rng(10)
+    # a fraction without padding first: every split of the split-K products leaves its partial sums in the scratch buffer,
+    # where a split of the next pass that wrote nothing would let them be counted again
+    full = make_pat_types([T] * S, T)
+    net.load_sequences(PC.dev(full), T, T, PC.dev(rng.standard_normal(T * S * P).astype(np.float32)),
+                       PC.dev(rng.standard_normal(T * S * Q).astype(np.float32)))
+    net.forward()
+    net.backward()
+    pat = make_pat_types(lengths, T)
+    x = rng.standard_normal((T, S, P)).astype(np.float32)
+    tgt = (0.3 * rng.standard_normal((T, S, Q))).astype(np.float32)
+    valid = (pat != 0).reshape(T, S)
+    x[~valid] = 0
+    tgt[~valid] = 0
+    net.load_sequences(PC.dev(pat), T, 1, PC.dev(x.reshape(-1)), PC.dev(tgt.reshape(-1)))
+    net.forward()
+    net.backward()
+    net.check()
+    ref = OM.OracleNetwork(P, specs, S, T, 1, pat, [w.copy() for w in weights])
+    ref.forward(x.reshape(-1), tgt.reshape(-1))
+    ref.backward()
+    grads = [L["updates"] for L in ref.layers if "updates" in L]
+    torch.cuda.synchronize()
+    for L, g in zip([L for L in net.layers if L["weight_count"]], grads):
+        assert PC.relerr(L["updates"].cpu().numpy(), g) < TOL, L["name"]
+    net.close()
+
+
 def test_network_reports_a_later_lstm_layer_that_gave_up_and_keeps_the_weights():
     """Failure handling at network level, forced from the host: the SECOND recurrent layer's recursions get a spin
     limit of zero, the first layer's stay as they are.  Every kernel still ends normally; the failure is reported by
