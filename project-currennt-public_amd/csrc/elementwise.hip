@@ -110,8 +110,9 @@ inline int stream_blocks(size_t count) {
 
 // One workgroup: every thread counts the valid slots of its contiguous share, the counts are scanned (inside a wave by
 // shuffles, the waves' totals through LDS), and the thread then writes its valid slots from its offset among the valid
-// ones and its padding slots from its offset among the padding ones, behind all valid ones.
-constexpr int kOrderThreads = 256;
+// ones and its padding slots from its offset among the padding ones, behind all valid ones.  The pattern types are read
+// eight at a time, so that a thread waits for memory once per eight slots and not once per slot.
+constexpr int kOrderThreads = 1024;
 __global__ __launch_bounds__(kOrderThreads) void slot_order_kernel(const char *__restrict__ pat, int n, int per_step,
                                                                    int *__restrict__ order, int *__restrict__ count) {
     __shared__ int wave_total[kOrderThreads / 64];
@@ -122,11 +123,18 @@ __global__ __launch_bounds__(kOrderThreads) void slot_order_kernel(const char *_
     if (tid < 2) edge_count[tid] = 0;
     __syncthreads();
     int valid = 0, in_first = 0, in_last = 0;
-    for (int i = lo; i < hi; ++i) {
-        const int v = pat[i] != 0;
-        valid += v;
-        in_first += v && i < per_step;
-        in_last += v && i >= n - per_step;
+    for (int c = lo; c < hi; c += 8) {
+        char v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = pat[min(c + j, n - 1)];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int i = c + j;
+            const int is = i < hi && v[j] != 0;
+            valid += is;
+            in_first += is && i < per_step;
+            in_last += is && i >= n - per_step;
+        }
     }
     if (in_first) atomicAdd(&edge_count[0], in_first);
     if (in_last) atomicAdd(&edge_count[1], in_last);
@@ -146,9 +154,17 @@ __global__ __launch_bounds__(kOrderThreads) void slot_order_kernel(const char *_
     }
     int at_valid = before + incl - valid;      // valid slots before this thread's share
     int at_pad = total + (lo - at_valid);      // padding slots before it, behind all valid ones
-    for (int i = lo; i < hi; ++i) {
-        if (pat[i] != 0) order[at_valid++] = i;
-        else order[at_pad++] = i;
+    for (int c = lo; c < hi; c += 8) {
+        char v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = pat[min(c + j, n - 1)];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int i = c + j;
+            if (i >= hi) continue;
+            if (v[j] != 0) order[at_valid++] = i;
+            else order[at_pad++] = i;
+        }
     }
     if (tid == 0) {
         count[0] = total;
