@@ -451,7 +451,11 @@ int cnt_network_set_external_input(cnt_network *net, int layer_index, const floa
                                    const float *mean_std);
 /* NeuralNetwork::loadSequences (NeuralNetwork.cpp:1367-1417): records the fraction's geometry and pattern types
  * (device memory, char[T*S], kept by pointer), copies inputs (input size x T*S) and targets (post-output size x T*S)
- * when given, and passes the call on to the layers that keep per-fraction state. */
+ * when given, and passes the call on to the layers that keep per-fraction state.  When Tmin < T (some sequence is
+ * shorter than the fraction) it also lists the fraction's valid slots from the pattern types, on the stream: the
+ * weight gradients of the dense and recurrent layers then sum over those slots only, which changes no result (every
+ * layer's deltas are zero on padding slots).  The pattern types are therefore read at this call as well as during the
+ * passes: change them only through another cnt_network_load_sequences. */
 int cnt_network_load_sequences(cnt_network *net, void *stream, int T, int Tmin, const char *patTypes,
                                const float *inputs, const float *targets);
 /* NeuralNetwork::computeForwardPass in training mode (NeuralNetwork.cpp:1419-1471, :1734-1760). */
