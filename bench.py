@@ -287,7 +287,10 @@ def main():
                           "frac": step_flops / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
                           "flops_per_frame": backward_flops_per_slot(input_size, specs),
                           "counted": "valid frames (%d of %d slots)" % (frames, slots),
-                          "frac_over_padded_slots": step_flops_padded / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS},
+                          "frac_over_padded_slots": step_flops_padded / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+                          "note": "frac_over_padded_slots prices every slot, as the reference's schedule multiplies them; "
+                                  "the library's weight gradients sum over the valid slots only, its other products "
+                                  "over all slots"},
         "forward_backward_ms": fb_ms,
         "kernels": kernels,
     }
