@@ -147,7 +147,10 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out);
 int cnt_lstm_destroy(cnt_lstm *h);
 /* LstmLayer::loadSequences (layers/LstmLayer.cu:1488-1533): records the fraction's geometry and
  * zero-fills the stored output-gate deltas.  patTypes is device memory, char[curMaxT*S], and must
- * stay valid until the next call of this function. */
+ * stay valid until the next call of this function.  For a fraction with much padding (curMinT at most 3/4 of
+ * curMaxT, at least 2048 slots) it also lists the valid slots, on the stream, and cnt_lstm_backward_weights then sums
+ * over those only -- the deltas are zero on padding slots, so no result changes (CNT_LSTM_SKIP_PADDING=0, read at
+ * cnt_lstm_create: never). */
 int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int curMaxT, int curMinT);
 /* LstmLayer::computeForwardPass(nnState) (layers/LstmLayer.cu:1743-1949).
  * x is P x (T*S); outputs is L x (T*S). */

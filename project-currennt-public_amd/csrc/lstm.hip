@@ -1065,6 +1065,8 @@ struct cnt_lstm {
     int bmail_dirty;       // the backward mailbox may hold words that are not empty
     int flmail_dirty;      // the same for the XCD-local forward recursion's mailbox
     cnt::SlotOrder slot_order;  // the loaded fraction's slots, valid ones first (set by the owner of the pattern types, or null)
+    int *own_order;             // maxT * S indices + 4 counts: the list the handle makes itself for a fraction with much padding
+    bool make_order;            // false inside a network, whose sequencer makes one list for all layers
     int stepwise;          // no persistent recursion kernel for this geometry: one product + one cell kernel per step
     int *latch_host, *latch_dev;  // pinned host word a kernel that gives up sets; read by the host without a sync
     int *veto;             // a network's shared flag (device), or NULL
@@ -1497,6 +1499,8 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     // The full-bandwidth read of the recursion's inputs in front of it (warm_cache) was worth 0.15 ms per model pass
     // while the memory wave's loads were issued in front of the polls; with that wave's pause it costs more than it
     // gains (2.290 -> 2.282 ms without it, 0.355 -> 0.352 ms for the single layer).  CNT_LSTM_WARM=1 turns it on.
+    h->make_order = true;
+    if (const char *e = std::getenv("CNT_LSTM_SKIP_PADDING")) h->make_order = std::atoi(e) != 0;
     h->warm = 0;
     if (const char *e = std::getenv("CNT_LSTM_WARM")) h->warm = std::atoi(e) != 0;
     {
@@ -1573,6 +1577,7 @@ int cnt_lstm_create(const cnt_lstm_desc *desc, cnt_lstm **out) {
     if (err == hipSuccess && std::getenv("CNT_LSTM_TIMING"))
         err = hipMalloc(reinterpret_cast<void **>(&h->phase_ticks), 8 * 512 * 6 * sizeof(long long));
     if (err == hipSuccess && h->phase_ticks) err = hipMemset(h->phase_ticks, 0, 8 * 512 * 6 * sizeof(long long));
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->own_order), ((size_t)h->desc.maxT * h->desc.S + 4) * sizeof(int));
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&h->abort_flag), sizeof(int));
     if (err == hipSuccess) err = hipMemset(h->abort_flag, 0, sizeof(int));
     // the word a kernel that gives up sets for the host: pinned, mapped, coherent host memory
@@ -1603,6 +1608,7 @@ int cnt_lstm_destroy(cnt_lstm *h) {
     if (h->lmail) (void)hipFree(h->lmail);
     if (h->flmail) (void)hipFree(h->flmail);
     if (h->ctl) (void)hipFree(h->ctl);
+    if (h->own_order) (void)hipFree(h->own_order);
     if (h->latch_host) (void)hipHostFree(h->latch_host);
     delete h;
     return CNT_OK;
@@ -1616,6 +1622,15 @@ int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int
     CNT_REQUIRE(curMinT >= 0 && curMinT <= curMaxT, "lstm_load_sequences: curMinT %d outside 0..%d", curMinT, curMaxT);
     h->T = curMaxT; h->Tmin = curMinT; h->pat = patTypes;
     h->slot_order = SlotOrder{nullptr, nullptr};
+    // A fraction with much padding (the shortest sequence at most 3/4 of the longest, and enough slots for the list's one
+    // launch to pay): the weight gradients sum over its valid slots only (GemmArgs::k_order).  The owner of a network's
+    // pattern types hands its own list over instead (lstm_set_slot_order).
+    if (h->make_order && h->own_order && (long)curMaxT * h->desc.S >= 2048 && (curMaxT - curMinT) * 4 >= curMaxT) {
+        const int n = curMaxT * h->desc.S;
+        int *count = h->own_order + (size_t)h->desc.maxT * h->desc.S;
+        CNT_TRY(slot_order_build(static_cast<hipStream_t>(stream), patTypes, n, h->desc.S, h->own_order, count));
+        h->slot_order = SlotOrder{h->own_order, count};
+    }
     if (h->next_step != 0) { h->bmail_dirty = 1; h->next_step = 0; }  // an abandoned partial backward pass
     const size_t nstate = (size_t)h->H * h->desc.maxT * h->desc.S;
     // stored output-gate deltas of both directions, one launch
@@ -1652,7 +1667,9 @@ extern "C++" void cnt::lstm_set_veto(cnt_lstm *h, int *veto) {
 extern "C++" int cnt::lstm_is_persistent(const cnt_lstm *h) { return h && !h->stepwise ? 1 : 0; }
 
 extern "C++" void cnt::lstm_set_slot_order(cnt_lstm *h, const SlotOrder *order) {
-    if (h) h->slot_order = order ? *order : SlotOrder{nullptr, nullptr};
+    if (!h) return;
+    h->make_order = false;  // from now on the caller's lists (or none) are the ones that count: no list of the handle's own
+    h->slot_order = order ? *order : SlotOrder{nullptr, nullptr};
 }
 
 extern "C++" int cnt::lstm_wait_recursion(cnt_lstm *h, hipStream_t other) {

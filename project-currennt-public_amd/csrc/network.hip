@@ -571,6 +571,7 @@ int build_layer_into(cnt_network *net, NetLayer &L, const json::Value &obj, cons
         CNT_TRY(cnt_lstm_create(&d, &L.lstm));
         if (!net->veto) CNT_TRY(device_alloc(net, (void **)&net->veto, sizeof(int), true));
         cnt::lstm_set_veto(L.lstm, net->veto);
+        cnt::lstm_set_slot_order(L.lstm, nullptr);  // the sequencer lists a fraction's valid slots once for all layers
     } else if (t == "skipini" || t == "skipadd") {
         // NeuralNetwork.cpp:470-530 offers every earlier skip layer plus the layer right before; SkipAddLayer.cu:
         // 96-138 keeps those named by preSkipLayer, or by default the last two of the offer (a skipini, and the

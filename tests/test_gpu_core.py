@@ -70,6 +70,9 @@ def test_sse():
     (16, 128, True, [1, 1]),               # a single time step, two sequences
     (24, 256, True, [7, 4, 7] * 6),        # 18 parallel sequences, bidirectional: the recursion that spans the XCDs
     (24, 128, False, [3, 9, 1, 9, 2]),     # very ragged, one sequence of a single step among longer ones
+    # 2400 slots of which a third is valid: the layer lists the valid slots itself and its weight gradients sum over those
+    (24, 128, True, [300, 50, 300, 20, 100, 300, 7, 1]),
+    (20, 64, False, [1, 600, 1, 1]),       # the same for a forward-only layer: one long sequence beside three single frames
     # geometries without a persistent recursion kernel: step-by-step recursion
     (12, 64, True, [30, 23]),              # 32 cells per direction (the reference example's conditioning BLSTM)
     (7, 20, False, [9, 4, 9]),             # 20 cells, sizes that are no multiple of anything
