@@ -311,6 +311,21 @@ int cnn_backward_weights_batch(cnt_cnn *const *h, int count, hipStream_t stream,
 int fill_zero(hipStream_t stream, float *p, size_t count);
 // two buffers in one launch
 int fill_zero_pair(hipStream_t stream, float *p, size_t count, float *q, size_t count_q);
+// What a network does on the device when a fraction is loaded, as ONE launch: up to kLoadClears buffers zeroed (the
+// recurrent layers' stored output-gate deltas) and, when `order` is given, the fraction's slot order built (as
+// slot_order_build does).
+constexpr int kLoadClears = 8;
+struct LoadClears {
+    float *ptr[kLoadClears];
+    unsigned long long count[kLoadClears];  // floats, multiples of four, 16-byte aligned buffers
+    int n;
+};
+int load_clear_and_order(hipStream_t stream, const LoadClears &clears, const char *pat, int n_slots, int slots_per_step,
+                         int *order, int *count);
+// cnt_lstm_load_sequences without the clearing launch: the caller clears what `clears` lists afterwards (false: the list
+// is full or a buffer does not qualify, and the handle has launched its own clear)
+int lstm_load_sequences_collect(cnt_lstm *h, hipStream_t stream, const char *patTypes, int curMaxT, int curMinT,
+                                LoadClears &clears);
 int fill_words(hipStream_t stream, unsigned *p, size_t count, unsigned word);
 // out[d] += scale * sum over the N columns of a D x N column-major matrix (out pre-zeroed by the caller)
 int column_sum(hipStream_t stream, const float *v, int D, int N, float scale, float *out);

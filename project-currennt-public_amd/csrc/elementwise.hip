@@ -113,8 +113,8 @@ inline int stream_blocks(size_t count) {
 // ones and its padding slots from its offset among the padding ones, behind all valid ones.  The pattern types are read
 // eight at a time, so that a thread waits for memory once per eight slots and not once per slot.
 constexpr int kOrderThreads = 1024;
-__global__ __launch_bounds__(kOrderThreads) void slot_order_kernel(const char *__restrict__ pat, int n, int per_step,
-                                                                   int *__restrict__ order, int *__restrict__ count) {
+__device__ __forceinline__ void slot_order_block(const char *__restrict__ pat, int n, int per_step, int *__restrict__ order,
+                                                 int *__restrict__ count) {
     __shared__ int wave_total[kOrderThreads / 64];
     __shared__ int edge_count[2];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -173,7 +173,43 @@ __global__ __launch_bounds__(kOrderThreads) void slot_order_kernel(const char *_
     }
 }
 
+__global__ __launch_bounds__(kOrderThreads) void slot_order_kernel(const char *__restrict__ pat, int n, int per_step,
+                                                                   int *__restrict__ order, int *__restrict__ count) {
+    slot_order_block(pat, n, per_step, order, count);
+}
+
+// workgroup 0 builds the slot order (when there is one to build), the others zero the listed buffers with 16-byte stores
+__global__ __launch_bounds__(kOrderThreads) void load_clear_and_order_kernel(const LoadClears c, const char *__restrict__ pat,
+                                                                             int n, int per_step, int *__restrict__ order,
+                                                                             int *__restrict__ count) {
+    if (blockIdx.x == 0) {
+        if (order) slot_order_block(pat, n, per_step, order, count);
+        return;
+    }
+    const size_t first = (size_t)(blockIdx.x - 1) * kOrderThreads + threadIdx.x;
+    const size_t stride = (size_t)(gridDim.x - 1) * kOrderThreads;
+    for (int b = 0; b < c.n; ++b) {
+        float4 *p = reinterpret_cast<float4 *>(c.ptr[b]);
+        const size_t n4 = c.count[b] / 4;
+        for (size_t i = first; i < n4; i += stride) p[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+}
+
 }  // namespace
+
+int load_clear_and_order(hipStream_t stream, const LoadClears &clears, const char *pat, int n_slots, int slots_per_step,
+                         int *order, int *count) {
+    CNT_REQUIRE(clears.n >= 0 && clears.n <= kLoadClears, "load_clear_and_order: %d buffers", clears.n);
+    CNT_REQUIRE(!order || (pat && count && n_slots > 0 && slots_per_step > 0), "load_clear_and_order: bad slot order argument");
+    if (clears.n == 0 && !order) return CNT_OK;
+    size_t floats = 0;
+    for (int b = 0; b < clears.n; ++b) floats += clears.count[b];
+    const unsigned fill_blocks = clears.n ? (unsigned)std::min<size_t>((floats / 4 + kOrderThreads - 1) / kOrderThreads, 1024) : 0;
+    hipLaunchKernelGGL(load_clear_and_order_kernel, dim3(1 + fill_blocks), dim3(kOrderThreads), 0, stream, clears, pat, n_slots,
+                       slots_per_step, order, count);
+    CNT_HIP(hipGetLastError());
+    return CNT_OK;
+}
 
 int slot_order_build(hipStream_t stream, const char *pat, int n_slots, int slots_per_step, int *order, int *count) {
     CNT_REQUIRE(pat && order && count && n_slots > 0 && slots_per_step > 0, "slot_order_build: bad argument");

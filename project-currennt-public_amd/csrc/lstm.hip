@@ -1614,7 +1614,9 @@ int cnt_lstm_destroy(cnt_lstm *h) {
     return CNT_OK;
 }
 
-int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int curMaxT, int curMinT) {
+namespace {
+// everything cnt_lstm_load_sequences does; the stored output-gate deltas are cleared here, or listed in `collect` for the caller
+int load_sequences_impl(cnt_lstm *h, hipStream_t stream, const char *patTypes, int curMaxT, int curMinT, cnt::LoadClears *collect) {
     using namespace cnt;
     CNT_REQUIRE(h && patTypes, "lstm_load_sequences: null argument");
     CNT_REQUIRE(curMaxT >= 1 && curMaxT <= h->desc.maxT, "lstm_load_sequences: curMaxT %d outside 1..%d", curMaxT,
@@ -1628,15 +1630,33 @@ int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int
     if (h->make_order && h->own_order && (long)curMaxT * h->desc.S >= 2048 && (curMaxT - curMinT) * 4 >= curMaxT) {
         const int n = curMaxT * h->desc.S;
         int *count = h->own_order + (size_t)h->desc.maxT * h->desc.S;
-        CNT_TRY(slot_order_build(static_cast<hipStream_t>(stream), patTypes, n, h->desc.S, h->own_order, count));
+        CNT_TRY(slot_order_build(stream, patTypes, n, h->desc.S, h->own_order, count));
         h->slot_order = SlotOrder{h->own_order, count};
     }
     if (h->next_step != 0) { h->bmail_dirty = 1; h->next_step = 0; }  // an abandoned partial backward pass
     const size_t nstate = (size_t)h->H * h->desc.maxT * h->desc.S;
+    if (collect && nstate % 4 == 0 && collect->n + h->ndir <= kLoadClears) {
+        for (int dir = 0; dir < h->ndir; ++dir) {
+            collect->ptr[collect->n] = h->state[dir][10];
+            collect->count[collect->n] = nstate;
+            ++collect->n;
+        }
+        return CNT_OK;
+    }
     // stored output-gate deltas of both directions, one launch
-    if (h->ndir == 2) CNT_TRY(fill_zero_pair(static_cast<hipStream_t>(stream), h->state[0][10], nstate, h->state[1][10], nstate));
-    else CNT_TRY(fill_zero(static_cast<hipStream_t>(stream), h->state[0][10], nstate));
+    if (h->ndir == 2) CNT_TRY(fill_zero_pair(stream, h->state[0][10], nstate, h->state[1][10], nstate));
+    else CNT_TRY(fill_zero(stream, h->state[0][10], nstate));
     return CNT_OK;
+}
+}  // namespace
+
+int cnt_lstm_load_sequences(cnt_lstm *h, void *stream, const char *patTypes, int curMaxT, int curMinT) {
+    return load_sequences_impl(h, static_cast<hipStream_t>(stream), patTypes, curMaxT, curMinT, nullptr);
+}
+
+extern "C++" int cnt::lstm_load_sequences_collect(cnt_lstm *h, hipStream_t stream, const char *patTypes, int curMaxT,
+                                                  int curMinT, LoadClears &clears) {
+    return load_sequences_impl(h, stream, patTypes, curMaxT, curMinT, &clears);
 }
 
 int cnt_lstm_set_wait_bounds(cnt_lstm *h, unsigned spin_limit, int poll_delay_backward, int poll_delay_forward) {

@@ -1243,7 +1243,7 @@ int cnt_network_load_sequences(cnt_network *net, void *stream_, int T, int Tmin,
         const NetLayer &L = net->layers[i];
         if (net->skip_padding && Tmin < T && (L.kind == K_DENSE || L.kind == K_LSTM) && L.res == 1) wanted_main = true;
     }
-    if (wanted_main) CNT_TRY(slot_order_build(stream, patTypes, (int)slots, net->S, net->order, net->order_count));
+    LoadClears clears = {};  // the recurrent layers' per-fraction clears, done with the slot order in one launch below
     for (auto &lr : net->low_res) {
         bool wanted = false;
         for (size_t i = 1; i < net->layers.size(); ++i) {
@@ -1265,11 +1265,13 @@ int cnt_network_load_sequences(cnt_network *net, void *stream_, int T, int Tmin,
                 L.order = lr.order_built ? SlotOrder{lr.order, lr.order_count} : SlotOrder{nullptr, nullptr};
             }
         if (L.lstm) {
-            CNT_TRY(cnt_lstm_load_sequences(L.lstm, stream, L.pat, L.T, L.Tmin));
+            CNT_TRY(lstm_load_sequences_collect(L.lstm, stream, L.pat, L.T, L.Tmin, clears));
             lstm_set_slot_order(L.lstm, &L.order);
         }
         if (L.mdn) CNT_TRY(cnt_mdn_load_sequences(L.mdn, stream, L.pat, L.T));
     }
+    CNT_TRY(load_clear_and_order(stream, clears, patTypes, (int)slots, net->S, wanted_main ? net->order : nullptr,
+                                 net->order_count));
     return CNT_OK;
 }
 
